@@ -1,0 +1,93 @@
+/* sqhip: C ABI of the MI355X (gfx950) codebook-linear kernels.
+ *
+ * One shared library, libsqhip.so, replaces every GPU launch site of the reference's
+ * codebook linear layer.  All pointers inside sq_matrix and all x / y / out / workspace
+ * pointers are DEVICE pointers owned by the caller; nothing here allocates or frees
+ * device memory and nothing synchronises the host: every call only enqueues kernels on
+ * `stream` (a hipStream_t passed as void*; NULL = the default stream), so calls can be
+ * recorded into a HIP graph.  Functions return SQ_OK or a negative SQ_E* code and keep a
+ * message for sq_last_error() (thread local).
+ *
+ * Data layout is the packed file's own (reference shapequant/packed.py:1-42): per matrix
+ * an int32 [R, W] little-endian bit stream of log2(K)-bit tags (W = ceil(C/d * bits / 32)),
+ * an fp16 [G*K, d] table, an fp16 [R] row scale, optional uint8 [R] row_book (G > 1) and
+ * uint8 [R] row_mask (M > 1).  Column orders are int32 [M, C] (regenerated from the seed by
+ * the host, reference shapequant/masks.py:334-342).  Row r decodes as
+ *     u[r, j*d + k] = f32(table[row_book[r]*K + tag[r, j]][k]) * f32(row_scale[r])
+ *     w[r, perms[row_mask[r]][c]] = u[r, c]
+ * and the layer computes Y[t, y_off + r] = sum_c X[t, c] * w[r, c] with fp32 accumulation.
+ */
+#ifndef SQHIP_H
+#define SQHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { SQ_OK = 0, SQ_EINVAL = -1, SQ_EUNSUPPORTED = -2, SQ_EWORKSPACE = -3, SQ_ELAUNCH = -4 };
+enum { SQ_F32 = 0, SQ_F16 = 1, SQ_BF16 = 2 };
+
+/* One packed matrix resident in device memory (the tensors the reference keeps in
+ * kernels/gemv.py:107-131 PackedLinear, same meaning, file layout unchanged). */
+typedef struct sq_matrix {
+    const int32_t*  tags;       /* [R, W] */
+    const uint16_t* table;      /* fp16 bits [G*K, d] */
+    const uint16_t* row_scale;  /* fp16 bits [R] */
+    const uint8_t*  row_book;   /* [R] or NULL when G == 1 */
+    const uint8_t*  row_mask;   /* [R] or NULL when M == 1 */
+    const int32_t*  perms;      /* [M, C] or NULL when M == 1 */
+    const int32_t*  row_order;  /* optional [R]: row ids sorted by row_mask (stable); NULL = natural */
+    int32_t R, C, d, bits, G, M, W;
+    int32_t y_off;              /* first output column of this piece in the stacked Y */
+} sq_matrix;
+
+/* Library / device identification.  sq_version: ABI version (major*100 + minor). */
+int sq_version(void);
+const char* sq_last_error(void);
+
+/* Dense weight rows [r0, r1) of one matrix into out[(r - r0) * ld_out + c], original column
+ * order, out_dtype SQ_F32 (exact product), SQ_F16 or SQ_BF16 (one round-to-nearest-even).
+ * Replaces cuda_dequant.dequant(rl, out, rows) (reference shapequant/kernels/cuda_dequant.py:79-103)
+ * and batched_runs.dequant_tile (reference shapequant/kernels/batched_runs.py:935-961); unlike
+ * those it also applies column orders, i.e. it is packed.decode_tensors (reference
+ * shapequant/packed.py:259-270) on the device. */
+int sq_dequant(const sq_matrix* m, void* out, int out_dtype, int64_t ld_out, int32_t r0, int32_t r1,
+               void* stream);
+
+/* Decode-time product for B = 1..SQ_SMALL_BMAX activation rows over n_mats stacked pieces that
+ * share C: Y[b, y_off + r] for every piece, X [B, C] with row stride ldx, Y row stride ldy
+ * (elements).  x_dtype / y_dtype: SQ_F16 or SQ_BF16 (y may also be SQ_F32).
+ * Replaces proto_runs.gemv (reference shapequant/kernels/proto_runs.py:505-571), cuda_gemv.gemv
+ * (cuda_gemv.py:148-172), PackedLinear.gemv (gemv.py:142-156) and RunsBatch.run
+ * (batched_runs.py:745-771).  Pieces with M > 1 need workspace (see sq_workspace_bytes). */
+#define SQ_SMALL_BMAX 32
+int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx,
+                    void* y, int y_dtype, int64_t ldy, int32_t B, void* workspace, size_t ws_bytes,
+                    void* stream);
+
+/* Prefill product for T activation rows: dequantise-into-LDS tile GEMM on fp16 MFMA with fp32
+ * accumulation, row scale applied to the accumulator.  Same argument meaning as sq_linear_small.
+ * Replaces runs_gemm.gemm (reference shapequant/kernels/runs_gemm.py:471-514).  Pieces with
+ * M > 1 are decoded with their column orders into workspace and multiplied from there. */
+int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx,
+                   void* y, int y_dtype, int64_t ldy, int32_t T, void* workspace, size_t ws_bytes,
+                   void* stream);
+
+/* Dense fp16/bf16 weight [R, C] (row stride ldw) times X: the GEMM half of the reference's
+ * "dequant + GEMM" large-M route (reference shapequant/vllm_ext/core.py:396-406, where it is a
+ * cuBLAS call).  w_dtype: SQ_F16 or SQ_BF16, independent of x_dtype (both are multiplied as fp16). */
+int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype,
+                  int64_t ldx, void* y, int y_dtype, int64_t ldy, int32_t T, void* stream);
+
+/* Bytes of workspace sq_linear_small (which = 0) or sq_linear_gemm (which = 1) needs for these
+ * pieces at `rows` activation rows; the caller grows its buffer before any graph capture
+ * (the reference grows its buffers the same way: batched_runs.py:628-640, runs_gemm.py:396-404). */
+size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SQHIP_H */

@@ -1,0 +1,81 @@
+"""ctypes binding of libsqhip.so (the C ABI declared in include/sqhip.h)."""
+
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+import torch
+
+_HERE = Path(__file__).resolve().parent
+LIB_PATH = _HERE / "libsqhip.so"
+
+SQ_F32, SQ_F16, SQ_BF16 = 0, 1, 2
+SQ_OK, SQ_EINVAL, SQ_EUNSUPPORTED, SQ_EWORKSPACE, SQ_ELAUNCH = 0, -1, -2, -3, -4
+SMALL_BMAX = 32
+
+DTYPES = {torch.float32: SQ_F32, torch.float16: SQ_F16, torch.bfloat16: SQ_BF16}
+
+
+class SqMatrix(ctypes.Structure):
+    """struct sq_matrix of include/sqhip.h."""
+    _fields_ = [("tags", ctypes.c_void_p), ("table", ctypes.c_void_p), ("row_scale", ctypes.c_void_p),
+                ("row_book", ctypes.c_void_p), ("row_mask", ctypes.c_void_p), ("perms", ctypes.c_void_p),
+                ("row_order", ctypes.c_void_p),
+                ("R", ctypes.c_int32), ("C", ctypes.c_int32), ("d", ctypes.c_int32), ("bits", ctypes.c_int32),
+                ("G", ctypes.c_int32), ("M", ctypes.c_int32), ("W", ctypes.c_int32), ("y_off", ctypes.c_int32)]
+
+
+class SqError(RuntimeError):
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"sqhip error {code}: {msg}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library.  Raises (never falls back) when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m quantexperiments_amd.build` "
+                "(hipcc --offload-arch=gfx950); there is no fallback path")
+        L = ctypes.CDLL(str(LIB_PATH))
+        vp, i32, i64, sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_size_t
+        mp = ctypes.POINTER(SqMatrix)
+        L.sq_version.restype = ctypes.c_int
+        L.sq_last_error.restype = ctypes.c_char_p
+        L.sq_dequant.argtypes = [mp, vp, ctypes.c_int, i64, i32, i32, vp]
+        L.sq_linear_small.argtypes = [mp, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
+        L.sq_linear_gemm.argtypes = [mp, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
+        L.sq_gemm_dense.argtypes = [vp, ctypes.c_int, i64, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp]
+        L.sq_workspace_bytes.argtypes = [mp, i32, i32, ctypes.c_int]
+        L.sq_workspace_bytes.restype = sz
+        for f in (L.sq_dequant, L.sq_linear_small, L.sq_linear_gemm, L.sq_gemm_dense):
+            f.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
+           "sq_workspace_bytes")
+
+
+def check(rc: int) -> None:
+    if rc != SQ_OK:
+        raise SqError(rc, lib().sq_last_error().decode())
+
+
+def stream_ptr(device) -> int:
+    """torch's current HIP stream on `device` as the void* the C ABI takes."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def matrix_array(mats) -> ctypes.Array:
+    arr = (SqMatrix * len(mats))()
+    for i, m in enumerate(mats):
+        arr[i] = m
+    return arr

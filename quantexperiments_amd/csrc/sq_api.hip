@@ -1,0 +1,123 @@
+// extern "C" surface of libsqhip.so: argument checks, error text, dispatch to the launchers.
+#include <stdarg.h>
+#include <stdio.h>
+#include "sq_common.h"
+
+namespace sq {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SQ_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return SQ_OK;
+}
+
+int device_cus() {
+    static int cus[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        cus[dev] = v;
+    }
+    return cus[dev];
+}
+
+static int check_matrix(const sq_matrix& m, const char* who) {
+    if (!m.tags || !m.table || !m.row_scale) return fail(SQ_EINVAL, "%s: null tags/table/row_scale", who);
+    if (m.R < 0 || m.C <= 0 || m.d <= 0 || m.C % m.d) return fail(SQ_EINVAL, "%s: R %d C %d d %d", who, m.R, m.C, m.d);
+    if (m.bits < 1 || m.bits > 16) return fail(SQ_EINVAL, "%s: tag bits %d outside 1..16", who, m.bits);
+    if (m.G < 1 || m.G > 256 || (m.G > 1 && !m.row_book)) return fail(SQ_EINVAL, "%s: G %d needs row_book", who, m.G);
+    if (m.M > 1 && (!m.row_mask || !m.perms)) return fail(SQ_EINVAL, "%s: M %d needs row_mask and perms", who, m.M);
+    if (m.M > 256) return fail(SQ_EINVAL, "%s: M %d > 256", who, m.M);
+    if ((int64_t)m.W * 32 < (int64_t)(m.C / m.d) * m.bits) return fail(SQ_EINVAL, "%s: W %d too small", who, m.W);
+    if (((uintptr_t)m.tags & 3) || ((uintptr_t)m.table & 1) || ((uintptr_t)m.row_scale & 1))
+        return fail(SQ_EINVAL, "%s: misaligned tensor", who);
+    if ((m.d * 2) % 8 == 0 && ((uintptr_t)m.table & 15)) return fail(SQ_EINVAL, "%s: table must be 16-byte aligned", who);
+    return SQ_OK;
+}
+
+static int check_xy(const char* who, const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, const void* y,
+                    int y_dtype, int64_t ldy, int rows) {
+    if (n < 0 || (n > 0 && !mats)) return fail(SQ_EINVAL, "%s: n_mats %d", who, n);
+    if (rows < 0) return fail(SQ_EINVAL, "%s: %d activation rows", who, rows);
+    if (x_dtype != SQ_F16 && x_dtype != SQ_BF16) return fail(SQ_EINVAL, "%s: x_dtype %d", who, x_dtype);
+    if (y_dtype != SQ_F16 && y_dtype != SQ_BF16 && y_dtype != SQ_F32) return fail(SQ_EINVAL, "%s: y_dtype %d", who, y_dtype);
+    if (y_dtype != SQ_F32 && y_dtype != x_dtype) return fail(SQ_EINVAL, "%s: y_dtype %d != x_dtype %d", who, y_dtype, x_dtype);
+    if (rows > 0 && n > 0 && (!x || !y)) return fail(SQ_EINVAL, "%s: null x / y", who);
+    int64_t need = 0;
+    for (int i = 0; i < n; ++i) {
+        int rc = check_matrix(mats[i], who);
+        if (rc) return rc;
+        if (mats[i].C != mats[0].C) return fail(SQ_EINVAL, "%s: stacked pieces disagree on the input size (%d vs %d)", who, mats[i].C, mats[0].C);
+        if (mats[i].y_off < 0) return fail(SQ_EINVAL, "%s: y_off %d", who, mats[i].y_off);
+        if ((int64_t)mats[i].y_off + mats[i].R > need) need = (int64_t)mats[i].y_off + mats[i].R;
+    }
+    if (n > 0 && rows > 1 && (ldx < mats[0].C || ldy < need)) return fail(SQ_EINVAL, "%s: ldx %lld / ldy %lld too small", who, (long long)ldx, (long long)ldy);
+    return SQ_OK;
+}
+
+}  // namespace sq
+
+using namespace sq;
+
+extern "C" {
+
+int sq_version(void) { return 100; }
+
+const char* sq_last_error(void) { return g_err; }
+
+int sq_dequant(const sq_matrix* m, void* out, int out_dtype, int64_t ld_out, int32_t r0, int32_t r1, void* stream) {
+    if (!m) return fail(SQ_EINVAL, "sq_dequant: null matrix");
+    int rc = check_matrix(*m, "sq_dequant");
+    if (rc) return rc;
+    if (r0 < 0 || r1 < r0 || r1 > m->R) return fail(SQ_EINVAL, "sq_dequant: rows [%d, %d) outside [0, %d)", r0, r1, m->R);
+    if (r1 == r0) return SQ_OK;
+    if (!out || ld_out < m->C) return fail(SQ_EINVAL, "sq_dequant: out %p ld_out %lld", out, (long long)ld_out);
+    return launch_dequant(*m, out, out_dtype, ld_out, r0, r1, (hipStream_t)stream);
+}
+
+int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                    int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream) {
+    int rc = check_xy("sq_linear_small", mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B);
+    if (rc) return rc;
+    if (B > SQ_SMALL_BMAX) return fail(SQ_EINVAL, "sq_linear_small: B %d > %d", B, SQ_SMALL_BMAX);
+    if (B == 0 || n_mats == 0) return SQ_OK;
+    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, workspace, ws_bytes, (hipStream_t)stream);
+}
+
+int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                   int64_t ldy, int32_t T, void* workspace, size_t ws_bytes, void* stream) {
+    int rc = check_xy("sq_linear_gemm", mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T);
+    if (rc) return rc;
+    if (T == 0 || n_mats == 0) return SQ_OK;
+    return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T, workspace, ws_bytes, (hipStream_t)stream);
+}
+
+int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype, int64_t ldx,
+                  void* y, int y_dtype, int64_t ldy, int32_t T, void* stream) {
+    if (x_dtype != SQ_F16 && x_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense: x_dtype %d", x_dtype);
+    if (w_dtype != SQ_F16 && w_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense: w_dtype %d", w_dtype);
+    if (y_dtype != SQ_F32 && y_dtype != x_dtype) return fail(SQ_EINVAL, "sq_gemm_dense: y_dtype %d", y_dtype);
+    if (R < 0 || C <= 0 || T < 0) return fail(SQ_EINVAL, "sq_gemm_dense: R %d C %d T %d", R, C, T);
+    if (R == 0 || T == 0) return SQ_OK;
+    if (!w || !x || !y || ldw < C || ldx < C || ldy < R) return fail(SQ_EINVAL, "sq_gemm_dense: bad pointer or stride");
+    return launch_gemm_dense(w, w_dtype, ldw, R, C, x, x_dtype, ldx, y, y_dtype, ldy, T, (hipStream_t)stream);
+}
+
+size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which) {
+    if (!mats || n_mats <= 0 || rows <= 0) return 0;
+    return which == 0 ? small_workspace(mats, n_mats, rows) : gemm_workspace(mats, n_mats, rows);
+}
+
+}  // extern "C"

@@ -1,0 +1,80 @@
+// Shared device helpers for the gfx950 codebook-linear kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/sqhip.h"
+
+namespace sq {
+
+typedef _Float16 half_t;
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ float h2f(uint16_t b) { return (float)__builtin_bit_cast(half_t, b); }
+__device__ __forceinline__ float bf2f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+// fp32 -> bf16 bits, round to nearest even, NaN stays NaN.
+__device__ __forceinline__ uint16_t f2bf(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ uint16_t f2h(float f) { return __builtin_bit_cast(uint16_t, (half_t)f); }
+
+// bf16 bits -> fp16 value (through fp32; exact whenever the value is an fp16 normal,
+// rounds to nearest even in the fp16 subnormal range, +-inf beyond 65504).
+__device__ __forceinline__ half_t bf2h(uint16_t b) { return (half_t)bf2f(b); }
+
+// two packed bf16 (one dword) -> two packed fp16
+__device__ __forceinline__ uint32_t bf2h_x2(uint32_t v) {
+    half2v h;
+    h.x = (half_t)__builtin_bit_cast(float, v << 16);
+    h.y = (half_t)__builtin_bit_cast(float, v & 0xFFFF0000u);
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+template <int DT> struct store_as;
+template <> struct store_as<SQ_F32> { typedef float type; static __device__ __forceinline__ float cvt(float f) { return f; } };
+template <> struct store_as<SQ_F16> { typedef uint16_t type; static __device__ __forceinline__ uint16_t cvt(float f) { return f2h(f); } };
+template <> struct store_as<SQ_BF16> { typedef uint16_t type; static __device__ __forceinline__ uint16_t cvt(float f) { return f2bf(f); } };
+
+// Tag j of a row's little-endian bit stream (any width 1..16).  `W` bounds the second word.
+__device__ __forceinline__ uint32_t tag_at(const uint32_t* __restrict__ row, int W, int bits, int j) {
+    const int p = j * bits, w = p >> 5, s = p & 31;
+    const uint32_t lo = row[w];
+    const uint32_t hi = (s + bits > 32 && w + 1 < W) ? row[w + 1] : 0u;
+    const uint64_t v = ((uint64_t)hi << 32) | lo;
+    return (uint32_t)(v >> s) & ((1u << bits) - 1u);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// error plumbing shared by the launchers (defined in sq_api.hip)
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+// launchers implemented in the kernel translation units
+int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s,
+                   bool raw = false);
+int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s);
+size_t small_workspace(const sq_matrix* mats, int n, int B);
+int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s);
+size_t gemm_workspace(const sq_matrix* mats, int n, int T);
+int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, const void* x, int x_dtype, int64_t ldx,
+                      void* y, int y_dtype, int64_t ldy, int T, hipStream_t s);
+
+}  // namespace sq

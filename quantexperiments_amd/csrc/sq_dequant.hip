@@ -1,0 +1,75 @@
+// Dense decode of a packed codebook matrix: one thread per chunk.
+//   out[r, perm[mask[r]][j*d + k]] = rn_T( f32(table[book[r]*K + tag[r, j]][k]) * f32(row_scale[r]) )
+// The fp32 product of two fp16 values is exact, so T = fp32 reproduces the CPU decode bit
+// for bit and T = fp16 / bf16 differ from it by exactly one round-to-nearest-even.
+#include "sq_common.h"
+
+namespace sq {
+
+template <int DT, int D>   // D = 0: any chunk width (scalar path)
+__global__ __launch_bounds__(256) void dequant_kernel(sq_matrix m, typename store_as<DT>::type* __restrict__ out,
+                                                      int64_t ld_out, int r0, int r1, int raw) {
+    typedef typename store_as<DT>::type T;
+    const int d = D ? D : m.d;
+    const int nch = m.C / d;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)(r1 - r0) * nch) return;
+    const int rr = (int)(idx / nch), j = (int)(idx - (int64_t)rr * nch);
+    const int r = r0 + rr;
+    const uint32_t* row = reinterpret_cast<const uint32_t*>(m.tags) + (int64_t)r * m.W;
+    uint32_t tag = tag_at(row, m.W, m.bits, j);
+    if (m.row_book) tag += (uint32_t)m.row_book[r] << m.bits;
+    const float s = raw ? 1.f : h2f(m.row_scale[r]);     // raw: unscaled codewords (exact in fp16)
+    const uint16_t* cw = m.table + (int64_t)tag * d;
+    T* o = out + (int64_t)rr * ld_out;
+    // a perms array without row_mask is one matrix-wide column order
+    const int32_t* pm = m.perms ? m.perms + (int64_t)(m.row_mask ? m.row_mask[r] : 0) * m.C : nullptr;
+    if (D == 8 && !pm) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(cw);
+        T t[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            t[2 * k] = store_as<DT>::cvt(h2f((uint16_t)(v[k] & 0xFFFFu)) * s);
+            t[2 * k + 1] = store_as<DT>::cvt(h2f((uint16_t)(v[k] >> 16)) * s);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o[j * 8 + k] = t[k];
+        return;
+    }
+    if (D == 4 && !pm) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(cw);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            o[j * 4 + 2 * k] = store_as<DT>::cvt(h2f((uint16_t)(v[k] & 0xFFFFu)) * s);
+            o[j * 4 + 2 * k + 1] = store_as<DT>::cvt(h2f((uint16_t)(v[k] >> 16)) * s);
+        }
+        return;
+    }
+    for (int k = 0; k < d; ++k) {
+        const int c = j * d + k;
+        o[pm ? pm[c] : c] = store_as<DT>::cvt(h2f(cw[k]) * s);
+    }
+}
+
+template <int DT>
+static int launch_dt(const sq_matrix& m, void* out, int64_t ld_out, int r0, int r1, hipStream_t s, int raw) {
+    typedef typename store_as<DT>::type T;
+    const int64_t n = (int64_t)(r1 - r0) * (m.C / m.d);
+    if (n == 0) return SQ_OK;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (m.d == 8) hipLaunchKernelGGL((dequant_kernel<DT, 8>), dim3(grid), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw);
+    else if (m.d == 4) hipLaunchKernelGGL((dequant_kernel<DT, 4>), dim3(grid), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw);
+    else hipLaunchKernelGGL((dequant_kernel<DT, 0>), dim3(grid), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw);
+    return check_launch("sq_dequant");
+}
+
+int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s, bool raw) {
+    switch (out_dtype) {
+        case SQ_F32: return launch_dt<SQ_F32>(m, out, ld_out, r0, r1, s, raw ? 1 : 0);
+        case SQ_F16: return launch_dt<SQ_F16>(m, out, ld_out, r0, r1, s, raw ? 1 : 0);
+        case SQ_BF16: return launch_dt<SQ_BF16>(m, out, ld_out, r0, r1, s, raw ? 1 : 0);
+    }
+    return fail(SQ_EINVAL, "sq_dequant: out_dtype %d", out_dtype);
+}
+
+}  // namespace sq

@@ -1,0 +1,217 @@
+// Prefill product Y[T, R] = X[T, C] . W^T on fp16 MFMA (v_mfma_f32_32x32x16_f16), fp32 accumulate.
+//
+// The MFMA's B operand wants, per lane, 8 consecutive k of one weight row: exactly one d = 8
+// codeword (or two d = 4 codewords), so a weight tile is "dequantised" by gathering raw fp16
+// codewords into an LDS tile; the row scale multiplies the fp32 accumulator in the epilogue,
+// which keeps the tile exact.  bf16 activations are converted to fp16 while they are staged
+// (exact for every fp16-normal value); fp16 MFMA runs at the bf16 rate on gfx950 and keeps the
+// codewords' 11-bit significands, which bf16 tiles would cut to 8.
+//
+// Operand layout of v_mfma_f32_32x32x16_f16 (A: 32 x 16, B: 16 x 32, D: 32 x 32), lane l:
+//   A: row l % 32, k = 8 * (l / 32) .. + 7        (tokens)
+//   B: col l % 32, k = 8 * (l / 32) .. + 7        (weight rows)
+//   D[v], v = 0..15: row 8 * (v / 4) + 4 * (l / 32) + v % 4, col l % 32
+#include "sq_common.h"
+
+namespace sq {
+
+constexpr int BM = 128, BN = 128, BK = 32, LDT = BK + 8;   // LDT: padded LDS row stride (halves)
+
+struct GemmArgs {
+    sq_matrix m;          // codebook piece (fused) ...
+    const uint16_t* wd;   // ... or dense weight [R, C] with row stride ldw (m.R, m.C, m.y_off still valid)
+    int64_t ldw;
+    const uint16_t* x;
+    int64_t ldx;
+    void* y;
+    int64_t ldy;
+    int T;
+    int x_dtype, y_dtype, w_dtype;   // w_dtype: element type of wd
+};
+
+// 8 consecutive halves of activation row t starting at column k (zeros outside the matrix)
+__device__ __forceinline__ u32x4 load_x8(const GemmArgs& a, int t, int k) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (t < a.T && k < a.m.C) {
+        v = *reinterpret_cast<const u32x4*>(a.x + (int64_t)t * a.ldx + k);
+        if (a.x_dtype == SQ_BF16) { v.x = bf2h_x2(v.x); v.y = bf2h_x2(v.y); v.z = bf2h_x2(v.z); v.w = bf2h_x2(v.w); }
+    }
+    return v;
+}
+
+// 8 consecutive raw weights (unscaled codewords, or dense halves) of row r starting at column k
+template <int D, bool DENSE>
+__device__ __forceinline__ u32x4 load_w8(const GemmArgs& a, int r, int k) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (r >= a.m.R || k >= a.m.C) return v;
+    if (DENSE) {
+        v = *reinterpret_cast<const u32x4*>(a.wd + (int64_t)r * a.ldw + k);
+        if (a.w_dtype == SQ_BF16) { v.x = bf2h_x2(v.x); v.y = bf2h_x2(v.y); v.z = bf2h_x2(v.z); v.w = bf2h_x2(v.w); }
+        return v;
+    }
+    const sq_matrix& m = a.m;
+    const uint32_t* row = reinterpret_cast<const uint32_t*>(m.tags) + (int64_t)r * m.W;
+    const uint32_t boff = m.row_book ? (uint32_t)m.row_book[r] << m.bits : 0u;
+    if (D == 8) {
+        const uint32_t tag = tag_at(row, m.W, m.bits, k >> 3) + boff;
+        v = *reinterpret_cast<const u32x4*>(m.table + (size_t)tag * 8);
+    } else {
+        const uint32_t t0 = tag_at(row, m.W, m.bits, k >> 2) + boff;
+        const uint32_t t1 = tag_at(row, m.W, m.bits, (k >> 2) + 1) + boff;
+        const u32x2 c0 = *reinterpret_cast<const u32x2*>(m.table + (size_t)t0 * 4);
+        const u32x2 c1 = *reinterpret_cast<const u32x2*>(m.table + (size_t)t1 * 4);
+        v.x = c0.x; v.y = c0.y; v.z = c1.x; v.w = c1.y;
+    }
+    return v;
+}
+
+template <int D, bool DENSE>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
+    __shared__ __attribute__((aligned(16))) uint16_t sx[BM * LDT];
+    __shared__ __attribute__((aligned(16))) uint16_t sw[BN * LDT];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t0 = blockIdx.y * BM, r0 = blockIdx.x * BN;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;     // wave tile origin inside the block tile
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // staging assignment: 512 16-byte pieces per tile, two per thread
+    const int sr0 = tid >> 2, sk = (tid & 3) * 8;              // rows sr0 and sr0 + 64, columns sk .. sk + 7
+    u32x4 px[2], pw[2];
+    px[0] = load_x8(a, t0 + sr0, sk);
+    px[1] = load_x8(a, t0 + sr0 + 64, sk);
+    pw[0] = load_w8<D, DENSE>(a, r0 + sr0, sk);
+    pw[1] = load_w8<D, DENSE>(a, r0 + sr0 + 64, sk);
+
+    for (int k0 = 0; k0 < a.m.C; k0 += BK) {
+        __syncthreads();
+        *reinterpret_cast<u32x4*>(sx + sr0 * LDT + sk) = px[0];
+        *reinterpret_cast<u32x4*>(sx + (sr0 + 64) * LDT + sk) = px[1];
+        *reinterpret_cast<u32x4*>(sw + sr0 * LDT + sk) = pw[0];
+        *reinterpret_cast<u32x4*>(sw + (sr0 + 64) * LDT + sk) = pw[1];
+        __syncthreads();
+        if (k0 + BK < a.m.C) {                                  // next tile's loads fly during the MFMAs
+            px[0] = load_x8(a, t0 + sr0, k0 + BK + sk);
+            px[1] = load_x8(a, t0 + sr0 + 64, k0 + BK + sk);
+            pw[0] = load_w8<D, DENSE>(a, r0 + sr0, k0 + BK + sk);
+            pw[1] = load_w8<D, DENSE>(a, r0 + sr0 + 64, k0 + BK + sk);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            half8v fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                fa[i] = *reinterpret_cast<const half8v*>(sx + (wm + i * 32 + (lane & 31)) * LDT + kk + (lane >> 5) * 8);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                fb[j] = *reinterpret_cast<const half8v*>(sw + (wn + j * 32 + (lane & 31)) * LDT + kk + (lane >> 5) * 8);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // epilogue: row scale on the accumulator, one rounding to the output type
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int r = r0 + wn + j * 32 + (lane & 31);
+        if (r >= a.m.R) continue;
+        const float sc = a.m.row_scale ? h2f(a.m.row_scale[r]) : 1.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int t = t0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (t >= a.T) continue;
+                const float val = acc[i][j][v] * sc;
+                const int64_t o = (int64_t)t * a.ldy + a.m.y_off + r;
+                if (a.y_dtype == SQ_BF16) reinterpret_cast<uint16_t*>(a.y)[o] = f2bf(val);
+                else if (a.y_dtype == SQ_F16) reinterpret_cast<uint16_t*>(a.y)[o] = f2h(val);
+                else reinterpret_cast<float*>(a.y)[o] = val;
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ host
+
+int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y,
+                         int y_dtype, int64_t ldy, int B, hipStream_t s);
+
+static bool x_vec_ok(const void* x, int64_t ldx, int C) { return C % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x & 15) == 0; }
+static bool fused_ok(const sq_matrix& m) { return (m.d == 8 || m.d == 4) && !m.perms && ((uintptr_t)m.table & 15) == 0; }
+static size_t dense_bytes(const sq_matrix& m) { return (((size_t)m.R * m.C * 2) + 255) & ~(size_t)255; }
+
+size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
+    (void)T;
+    size_t need = 0;
+    for (int i = 0; i < n; ++i)
+        if (!fused_ok(mats[i]) && dense_bytes(mats[i]) > need) need = dense_bytes(mats[i]);
+    return need;
+}
+
+static int run(const GemmArgs& a, int d, bool dense, hipStream_t s) {
+    const dim3 grid((a.m.R + BN - 1) / BN, (a.T + BM - 1) / BM);
+    if (dense) hipLaunchKernelGGL((gemm_kernel<8, true>), grid, dim3(256), 0, s, a);
+    else if (d == 8) hipLaunchKernelGGL((gemm_kernel<8, false>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((gemm_kernel<4, false>), grid, dim3(256), 0, s, a);
+    return check_launch("sq_linear_gemm");
+}
+
+int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, const void* x, int x_dtype, int64_t ldx,
+                      void* y, int y_dtype, int64_t ldy, int T, hipStream_t s) {
+    if (!x_vec_ok(x, ldx, C) || !x_vec_ok(w, ldw, C))
+        return fail(SQ_EUNSUPPORTED, "sq_gemm_dense: C, ldx, ldw must be multiples of 8 and pointers 16-byte aligned");
+    GemmArgs a{};
+    a.m.R = R; a.m.C = C; a.m.y_off = 0;
+    a.wd = (const uint16_t*)w; a.ldw = ldw;
+    a.x = (const uint16_t*)x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.T = T; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+    a.w_dtype = w_dtype;
+    return run(a, 8, true, s);
+}
+
+int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (!x_vec_ok(x, ldx, mats[0].C)) {
+        // odd strides: the any-shape kernel, SQ_SMALL_BMAX activation rows at a time
+        for (int t = 0; t < T; t += SQ_SMALL_BMAX) {
+            const int nb = T - t < SQ_SMALL_BMAX ? T - t : SQ_SMALL_BMAX;
+            const size_t es = 2, ys = y_dtype == SQ_F32 ? 4 : 2;
+            int rc = launch_small_generic(mats, n, (const char*)x + (size_t)t * ldx * es, x_dtype, ldx,
+                                          (char*)y + (size_t)t * ldy * ys, y_dtype, ldy, nb, s);
+            if (rc) return rc;
+        }
+        return SQ_OK;
+    }
+    if (gemm_workspace(mats, n, T) > ws_bytes)
+        return fail(SQ_EWORKSPACE, "sq_linear_gemm: workspace %zu < %zu", ws_bytes, gemm_workspace(mats, n, T));
+    for (int i = 0; i < n; ++i) {
+        const sq_matrix& m = mats[i];
+        if (m.R == 0) continue;
+        GemmArgs a{};
+        a.m = m;
+        a.x = (const uint16_t*)x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.T = T; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+        int rc;
+        if (fused_ok(m)) {
+            rc = run(a, m.d, false, s);
+        } else {
+            // column orders or an unusual chunk width: gather the raw codewords (with the column
+            // scatter) into the workspace as fp16, which is exact, and multiply from there with the row scale
+            // applied to the accumulator as in the fused kernel; the stream orders the two kernels and the next piece
+            rc = launch_dequant(m, ws, SQ_F16, m.C, 0, m.R, s, /*raw=*/true);
+            if (rc) return rc;
+            a.wd = (const uint16_t*)ws; a.ldw = m.C; a.w_dtype = SQ_F16;
+            rc = run(a, 8, true, s);
+        }
+        if (rc) return rc;
+    }
+    return SQ_OK;
+}
+
+}  // namespace sq

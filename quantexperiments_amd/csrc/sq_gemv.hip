@@ -1,0 +1,180 @@
+// Host side of the decode-time product: picks the team geometry per shape, fuses stacked pieces
+// into one persistent launch, prepares permuted activations for pieces with column orders.
+#include "sq_gemv_kernel.h"
+
+namespace sq {
+
+int launch_gemv_b16d8(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_gemv_b12d4(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_gemv_b10d4(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_gemv_b8d4(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+
+// xp[m, b, c] = fp16(x[b, perms[m, c]])
+__global__ __launch_bounds__(256) void permute_x_kernel(const uint16_t* __restrict__ x, int64_t ldx, int x_dtype,
+                                                        const int32_t* __restrict__ perms, int M, int B, int C,
+                                                        uint16_t* __restrict__ xp) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)M * B * C) return;
+    const int c = (int)(i % C);
+    const int b = (int)((i / C) % B);
+    const int mk = (int)(i / ((int64_t)C * B));
+    const uint16_t v = x[(int64_t)b * ldx + perms[(int64_t)mk * C + c]];
+    xp[i] = x_dtype == SQ_BF16 ? __builtin_bit_cast(uint16_t, bf2h(v)) : v;
+}
+
+// ------------------------------------------------------------------------------------------ host
+
+int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y,
+                         int y_dtype, int64_t ldy, int B, hipStream_t s);
+int device_cus();
+
+static int unit_dwords(int bits) { return bits == 12 ? 3 : bits == 10 ? 5 : 4; }
+
+static bool fast_shape(const sq_matrix& m) {
+    const bool fmt = (m.d == 8 && m.bits == 16) || (m.d == 4 && (m.bits == 12 || m.bits == 10 || m.bits == 8));
+    if (!fmt) return false;
+    if (m.W % unit_dwords(m.bits)) return false;                 // rows must be whole units
+    if (((uintptr_t)m.tags & 15) || ((uintptr_t)m.table & 15)) return false;
+    if ((int64_t)(m.C / m.d) * m.bits != (int64_t)m.W * 32) return false;   // no pad bits inside the last unit
+    return true;
+}
+
+static size_t xp_bytes(const sq_matrix& m, int B) {
+    return (((size_t)(m.M > 1 ? m.M : 1) * B * m.C * 2) + 255) & ~(size_t)255;
+}
+
+struct Plan { int TS, S, nwaves; };
+
+// Host mirror of gemv_cfg<>::REGS / LB.
+static int cfg_regs(int bits, int d, int S, int NB) {
+    const int ud = unit_dwords(bits), xh = ud * 32 / bits * d / 2;
+    return NB * S * xh + GEMV_PF * S * ud + 56;
+}
+static int cfg_lb(int bits, int d, int S, int NB) { return cfg_regs(bits, d, S, NB) <= 256 ? 512 : 256; }
+
+// Team size / slots for U units per row: fewest idle lanes, then fewest slots.
+static Plan plan_for(int U, int bits, int d) {
+    Plan best{0, 0, 0};
+    double best_eff = -1.0;
+    const int cands[] = {16, 32, 64, 128, 192, 256, 320, 384, 448, 512};
+    const int slots[] = {1, 2, 3, 5};
+    for (int ts : cands)
+        for (int s : slots) {
+            if (ts * s < U) continue;
+            if (cfg_regs(bits, d, s, 1) > 440) break;
+            if (ts > cfg_lb(bits, d, s, 1)) break;
+            const double eff = (double)U / (ts * s) - 0.02 * (s - 1) - (ts > 64 ? 0.01 : 0.0);
+            if (eff > best_eff + 1e-9) { best_eff = eff; best.TS = ts; best.S = s; }
+            break;
+        }
+    if (best.TS == 0) return best;
+    const int lb = cfg_lb(bits, d, best.S, 1);
+    if (best.TS >= 64) {
+        const int wpr = best.TS / 64;
+        int rg = (lb / 64) / wpr;
+        if (rg < 1) rg = 1;
+        best.nwaves = wpr * rg;
+    } else best.nwaves = lb / 64;
+    return best;
+}
+
+size_t small_workspace(const sq_matrix* mats, int n, int B) {
+    size_t tot = 0;
+    for (int i = 0; i < n; ++i)
+        if (mats[i].perms && fast_shape(mats[i])) tot += xp_bytes(mats[i], B);
+    return tot;
+}
+
+int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (small_workspace(mats, n, B) > ws_bytes)
+        return fail(SQ_EWORKSPACE, "sq_linear_small: workspace %zu < %zu", ws_bytes, small_workspace(mats, n, B));
+    const int cus = device_cus();
+    const bool x_ok = (ldx % 2 == 0) && (((uintptr_t)x & 3) == 0);
+    size_t ws_off = 0;
+    int i = 0;
+    while (i < n) {
+        const sq_matrix& m0 = mats[i];
+        if (m0.R == 0) { ++i; continue; }
+        const int ud = unit_dwords(m0.bits);
+        const Plan pl = (fast_shape(m0) && x_ok) ? plan_for(m0.W / ud, m0.bits, m0.d) : Plan{0, 0, 0};
+        if (pl.TS == 0) {
+            int rc = launch_small_generic(mats + i, 1, x, x_dtype, ldx, y, y_dtype, ldy, B, s);
+            if (rc) return rc;
+            if (m0.perms && fast_shape(m0)) ws_off += xp_bytes(m0, B);
+            ++i;
+            continue;
+        }
+        // pieces i .. j-1 share one launch when their format, geometry and codebook size agree
+        const int U = m0.W / ud;
+        const size_t tab0 = (size_t)m0.G * ((size_t)1 << m0.bits) * m0.d * 2;
+        int j = i + 1;
+        while (j < n && j - i < GEMV_MAX_PIECES && fast_shape(mats[j]) && mats[j].bits == m0.bits && mats[j].d == m0.d &&
+               mats[j].W == m0.W && mats[j].G == m0.G && mats[j].R > 0)
+            ++j;
+        GemvArgs a;
+        a.n = j - i;
+        a.x = (const uint16_t*)x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.B = B;
+        a.x_dtype = x_dtype; a.y_dtype = y_dtype; a.TS = pl.TS;
+        a.table_bytes = tab0 <= 128 * 1024 ? (int)tab0 : 0;
+        const int wpr = pl.TS > 64 ? pl.TS / 64 : 1;
+        int64_t rows_total = 0;
+        for (int k = i; k < j; ++k) rows_total += mats[k].R;
+        for (int k = i; k < j; ++k) {
+            GemvPiece& P = a.p[k - i];
+            P.m = mats[k];
+            P.U = U;
+            P.xp = nullptr;
+            if (mats[k].perms) {
+                uint16_t* xp = (uint16_t*)((char*)ws + ws_off);
+                ws_off += xp_bytes(mats[k], B);
+                const int Mx = mats[k].M > 1 ? mats[k].M : 1;
+                const int64_t tot = (int64_t)Mx * B * mats[k].C;
+                hipLaunchKernelGGL(permute_x_kernel, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, s,
+                                   (const uint16_t*)x, ldx, x_dtype, mats[k].perms, Mx, B, mats[k].C, xp);
+                int rc = check_launch("sq_linear_small(permute_x)");
+                if (rc) return rc;
+                P.xp = xp;
+            }
+        }
+        for (int k = j - i; k < GEMV_MAX_PIECES; ++k) a.p[k] = a.p[0];
+        for (int b0 = 0; b0 < B;) {
+            const int left = B - b0;
+            int nbt = left >= 4 ? 4 : left >= 2 ? 2 : 1;
+            // fewer activation rows per pass when the registers or the workgroup width do not allow more
+            while (nbt > 1 && (cfg_regs(m0.bits, m0.d, pl.S, nbt) > 440 || cfg_lb(m0.bits, m0.d, pl.S, nbt) < wpr * 64)) nbt >>= 1;
+            const int lb = cfg_lb(m0.bits, m0.d, pl.S, nbt);
+            int nwaves = pl.nwaves;
+            if (nwaves * 64 > lb) nwaves = (lb / 64) / wpr * wpr;
+            const int ngrp = pl.TS > 64 ? nwaves / wpr : nwaves * (64 / pl.TS);
+            const size_t smem = (size_t)a.table_bytes + (wpr > 1 ? (size_t)GEMV_PF * ngrp * wpr * nbt * sizeof(float) : 0);
+            // persistent grid: workgroups per CU bounded by LDS and wave slots, split over the pieces by rows
+            int per_cu = smem > 80 * 1024 ? 1 : smem > 40 * 1024 ? 2 : smem > 20 * 1024 ? 4 : 8;
+            if (nwaves * per_cu > 16) per_cu = 16 / nwaves > 0 ? 16 / nwaves : 1;
+            const int64_t row_quant = (int64_t)ngrp * GEMV_PF;
+            const int grid_target = cus * per_cu;
+            int wg_begin = 0;
+            for (int k = i; k < j; ++k) {
+                GemvPiece& P = a.p[k - i];
+                int cnt = (int)((mats[k].R * (int64_t)grid_target + rows_total - 1) / rows_total);
+                const int most = (int)((mats[k].R + row_quant - 1) / row_quant);
+                if (cnt > most) cnt = most;
+                if (cnt < 1) cnt = 1;
+                P.wg_begin = wg_begin;
+                P.wg_count = cnt;
+                wg_begin += cnt;
+            }
+            a.b0 = b0;
+            int rc = SQ_EUNSUPPORTED;
+#define SQ_CASE(BI, DD) if (m0.bits == BI && m0.d == DD) rc = launch_gemv_b##BI##d##DD(a, pl.S, nbt, wg_begin, nwaves * 64, smem, s)
+            SQ_CASE(16, 8); SQ_CASE(12, 4); SQ_CASE(10, 4); SQ_CASE(8, 4);
+#undef SQ_CASE
+            if (rc) return rc;
+            b0 += nbt;
+        }
+        i = j;
+    }
+    return SQ_OK;
+}
+
+}  // namespace sq

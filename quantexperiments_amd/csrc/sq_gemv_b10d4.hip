@@ -1,0 +1,5 @@
+// Decode-time kernels for 10-bit tags, chunk width 4.
+#include "sq_gemv_kernel.h"
+namespace sq {
+SQ_GEMV_FORMAT(10, 4)
+}

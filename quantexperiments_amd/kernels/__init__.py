@@ -1,0 +1,196 @@
+"""Device-side holder of one packed matrix and the Python face of the HIP kernels.
+
+`PackedLinear` mirrors the reference's class of the same name (reference
+shapequant/kernels/gemv.py:107-175): it keeps the packed file's tensors on the GPU unchanged
+(words, table, row_scale, row_book, row_mask, column orders) and offers gemv / dense / forward /
+stored_bytes.  Every method launches kernels of libsqhip.so on torch's current stream; nothing
+here computes on the CPU and nothing falls back to PyTorch ops.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from .. import _lib
+from .._lib import SqMatrix
+
+
+class _Workspace:
+    """One growable byte buffer per device shared by every layer (layers run one at a time on
+    one stream).  It must be grown before a HIP graph that uses it is captured: callers run each
+    shape once eagerly first, as with the reference's shared buffers (reference
+    shapequant/vllm_ext/core.py:198-209, shapequant/kernels/batched_runs.py:628-640)."""
+    bufs: dict = {}
+
+    @classmethod
+    def get(cls, nbytes: int, dev) -> torch.Tensor:
+        key = str(dev)
+        b = cls.bufs.get(key)
+        if b is None or b.numel() < nbytes:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("sqhip workspace must grow outside graph capture: run this shape once eagerly first")
+            b = cls.bufs[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        return b
+
+
+class PackedLinear(torch.nn.Module):
+    """A block linear run from packed tensors."""
+
+    def __init__(self, words, table, row_scale, row_book, row_mask, perms, K: int, d: int, bias=None):
+        super().__init__()
+        R, W = words.shape
+        dev = words.device
+        if dev.type != "cuda":
+            raise ValueError("PackedLinear holds device tensors: pass cuda tensors")
+        C = perms.shape[1]
+        if K < 2 or K & (K - 1):
+            raise ValueError(f"K={K} is not a power of two")
+        if C % d:
+            raise ValueError(f"C={C} not divisible by d={d}")
+        self.R, self.C, self.K, self.d, self.W = R, C, K, d, W
+        self.bits = K.bit_length() - 1
+        self.nch = C // d
+        if W * 32 < self.nch * self.bits:
+            raise ValueError("tag words too short for C/d tags")
+        if table.shape[0] % K or table.shape[1] != d:
+            raise ValueError(f"table shape {tuple(table.shape)} does not hold whole codebooks of [{K}, {d}]")
+        self.G = table.shape[0] // K
+        if (self.G > 1) != (row_book is not None):
+            raise ValueError("row_book is needed exactly when the table holds several codebooks")
+        self.register_buffer("words", words.to(torch.int32).contiguous())
+        self.register_buffer("table", table.to(torch.float16).contiguous())
+        self.register_buffer("row_scale", row_scale.to(torch.float16).contiguous())
+        self.register_buffer("row_book", None if row_book is None else row_book.to(torch.uint8).contiguous())
+        self.has_mask = row_mask is not None and perms.shape[0] > 1
+        self.M = perms.shape[0] if self.has_mask else 1
+        if self.has_mask:
+            rm = row_mask.to(torch.uint8).contiguous()
+            self.register_buffer("row_mask", rm)
+            self.register_buffer("perms", perms.to(torch.int32).contiguous())
+            # rows regrouped by column order (stable), so a workgroup sees one order at a time
+            self.register_buffer("row_order", torch.sort(rm.to(torch.int32), stable=True).indices.to(torch.int32))
+        else:
+            self.register_buffer("row_mask", None)
+            self.register_buffer("perms", None)
+            self.register_buffer("row_order", None)
+        self.bias = bias
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_packed(cls, pf, name: str, device="cuda", bias=None):
+        m = pf.meta[name]
+        t = pf.tensors(name)
+        dev = torch.device(device)
+        return cls(t["tags"].to(dev), t["table"].to(dev), t["row_scale"].to(dev),
+                   t["row_book"].to(dev) if "row_book" in t else None,
+                   t["row_mask"].to(dev) if "row_mask" in t else None,
+                   pf.perms(name).to(dev), m["K"], m["d"], bias=bias)
+
+    @property
+    def device(self):
+        return self.words.device
+
+    def descriptor(self, y_off: int = 0) -> SqMatrix:
+        p = lambda t: None if t is None else t.data_ptr()
+        return SqMatrix(p(self.words), p(self.table), p(self.row_scale), p(self.row_book), p(self.row_mask),
+                        p(self.perms), p(self.row_order), self.R, self.C, self.d, self.bits, self.G, self.M, self.W,
+                        y_off)
+
+    # ------------------------------------------------------------------ kernels
+    def dense(self, dtype=torch.float32, out: torch.Tensor | None = None, rows: tuple | None = None) -> torch.Tensor:
+        """[R, C] decoded weight (rows r0:r1 if given) in the original column order."""
+        r0, r1 = rows if rows is not None else (0, self.R)
+        n = (r1 - r0) * self.C
+        if out is None:
+            w = torch.empty(r1 - r0, self.C, dtype=dtype, device=self.device)
+        else:
+            if out.dtype != dtype or out.numel() < n or not out.is_contiguous():
+                raise ValueError("out must be a contiguous buffer of `dtype` with at least rows * C elements")
+            w = out.view(-1)[:n].view(r1 - r0, self.C)
+        m = self.descriptor()
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.lib().sq_dequant(ctypes.byref(m), w.data_ptr(), _lib.DTYPES[dtype], self.C, r0, r1,
+                                             _lib.stream_ptr(self.device)))
+        return w
+
+    def gemv(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """x [C] (fp16 / bf16) -> y [R] in x's dtype."""
+        if x.shape != (self.C,):
+            raise ValueError(f"x shape {tuple(x.shape)} != ({self.C},)")
+        y = out if out is not None else torch.empty(self.R, dtype=x.dtype, device=x.device)
+        linear_small([self], x.view(1, self.C), y.view(1, self.R))
+        return y
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.C)
+        if x2.dtype not in (torch.float16, torch.bfloat16):
+            x2 = x2.to(torch.float16)
+        y = torch.empty(x2.shape[0], self.R, dtype=x2.dtype, device=x2.device)
+        if x2.shape[0] <= _lib.SMALL_BMAX:
+            linear_small([self], x2, y)
+        else:
+            linear_gemm([self], x2, y)
+        y = y.to(x.dtype).reshape(*lead, self.R)
+        return y if self.bias is None else y + self.bias
+
+    def stored_bytes(self) -> int:
+        """Bytes the product must stream from HBM: tags + table + scales (as the reference counts)."""
+        return sum(t.numel() * t.element_size() for t in (self.words, self.table, self.row_scale))
+
+
+def _prep(pieces, x: torch.Tensor, y: torch.Tensor):
+    if x.dim() != 2 or y.dim() != 2 or x.shape[0] != y.shape[0]:
+        raise ValueError("x must be [B, C] and y [B, sum R]")
+    if x.stride(1) != 1 or y.stride(1) != 1:
+        raise ValueError("x and y need unit column stride")
+    offs, off = [], 0
+    for p in pieces:
+        offs.append(off)
+        off += p.R
+    if y.shape[1] != off:
+        raise ValueError(f"y has {y.shape[1]} columns, pieces make {off}")
+    mats = _lib.matrix_array([p.descriptor(o) for p, o in zip(pieces, offs)])
+    return mats, x.stride(0) if x.shape[0] > 1 else max(x.stride(0), x.shape[1]), \
+        y.stride(0) if y.shape[0] > 1 else max(y.stride(0), y.shape[1])
+
+
+def linear_small(pieces, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """Y[b, off_i + r] for every stacked piece, B = x.shape[0] <= 32 (sq_linear_small)."""
+    mats, ldx, ldy = _prep(pieces, x, y)
+    dev = x.device
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        need = L.sq_workspace_bytes(mats, len(pieces), x.shape[0], 0)
+        ws = _Workspace.get(need, dev) if need else None
+        _lib.check(L.sq_linear_small(mats, len(pieces), x.data_ptr(), _lib.DTYPES[x.dtype], ldx, y.data_ptr(),
+                                     _lib.DTYPES[y.dtype], ldy, x.shape[0], None if ws is None else ws.data_ptr(),
+                                     0 if ws is None else ws.numel(), _lib.stream_ptr(dev)))
+    return y
+
+
+def linear_gemm(pieces, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """Y = X . W^T for T = x.shape[0] activation rows on the MFMA tile kernel (sq_linear_gemm)."""
+    mats, ldx, ldy = _prep(pieces, x, y)
+    dev = x.device
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        need = L.sq_workspace_bytes(mats, len(pieces), x.shape[0], 1)
+        ws = _Workspace.get(need, dev) if need else None
+        _lib.check(L.sq_linear_gemm(mats, len(pieces), x.data_ptr(), _lib.DTYPES[x.dtype], ldx, y.data_ptr(),
+                                    _lib.DTYPES[y.dtype], ldy, x.shape[0], None if ws is None else ws.data_ptr(),
+                                    0 if ws is None else ws.numel(), _lib.stream_ptr(dev)))
+    return y
+
+
+def gemm_dense(w: torch.Tensor, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """Y = X . W^T for a dense fp16 / bf16 weight [R, C] (sq_gemm_dense)."""
+    dev = x.device
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().sq_gemm_dense(w.data_ptr(), _lib.DTYPES[w.dtype], w.stride(0), w.shape[0], w.shape[1], x.data_ptr(),
+                                            _lib.DTYPES[x.dtype], x.stride(0), y.data_ptr(), _lib.DTYPES[y.dtype],
+                                            y.stride(0), x.shape[0], _lib.stream_ptr(dev)))
+    return y

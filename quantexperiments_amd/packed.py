@@ -1,0 +1,218 @@
+"""Packed file format "shapequant-stack-v1": same tensors, names and metadata as the reference
+(reference shapequant/packed.py:1-42), so files written by either side load on the other.
+
+Per matrix `name` ([R, C] weight, d-wide chunks, G codebooks of K entries, M column orders):
+
+  {name}.tags       int32 [R, W]    log2(K)-bit local tags, little-endian bit stream per row,
+                                    W = ceil(C/d * log2(K) / 32)
+  {name}.table      fp16  [G*K, d]
+  {name}.row_scale  fp16  [R]
+  {name}.row_book   uint8 [R]       only if G > 1
+  {name}.row_mask   uint8 [R]       only if M > 1
+
+File metadata: "summary" and "matrices" (JSON strings; "aux" is passed through untouched).
+Column orders are regenerated from each matrix's seed and checked against its CRC.
+
+This module is host logic (bit packing, file I/O, validation).  Decoding a matrix to a dense
+weight runs on the GPU through libsqhip.so; there is no CPU decode here.
+"""
+
+from __future__ import annotations
+
+import json
+import math
+import zlib
+from pathlib import Path
+
+import torch
+
+from . import masks as mk
+
+FORMAT = "shapequant-stack-v1"
+
+
+def words_per_row(n: int, bits: int) -> int:
+    return (n * bits + 31) // 32
+
+
+def pack_bits(vals: torch.Tensor, bits: int) -> torch.Tensor:
+    """[R, n] integers in [0, 2**bits) -> int32 [R, W] (reference shapequant/packed.py:61-77).
+    Each value is shifted to its bit position inside a 64-bit window and OR-ed into the one or
+    two words it touches, so the cost is O(R * n) with no per-bit expansion."""
+    if vals.dim() != 2:
+        raise ValueError("vals must be [R, n]")
+    R, n = vals.shape
+    W = words_per_row(n, bits)
+    v = vals.to(torch.int64).cpu()
+    if v.numel() and (int(v.min()) < 0 or int(v.max()) >= (1 << bits)):
+        raise ValueError(f"values out of range for {bits} bits")
+    pos = torch.arange(n, dtype=torch.int64) * bits
+    wi, sh = pos >> 5, pos & 31
+    wide = v << sh                                             # < 2**(bits + 31)
+    acc = torch.zeros(R, W + 1, dtype=torch.int64)
+    # values that share a word occupy disjoint bits, so adding equals OR-ing
+    acc.scatter_add_(1, wi.expand(R, n), wide & 0xFFFFFFFF)
+    acc.scatter_add_(1, (wi + 1).expand(R, n), wide >> 32)
+    acc = acc[:, :W]
+    return torch.where(acc >= (1 << 31), acc - (1 << 32), acc).to(torch.int32)
+
+
+def unpack_bits(words: torch.Tensor, bits: int, n: int) -> torch.Tensor:
+    """int32 [R, W] -> int64 [R, n] on words' device (reference shapequant/packed.py:80-90)."""
+    R, W = words.shape
+    if W * 32 < n * bits:
+        raise ValueError("too few words for n values")
+    dev = words.device
+    w = words.to(torch.int64) & 0xFFFFFFFF
+    w = torch.cat([w, torch.zeros(R, 1, dtype=torch.int64, device=dev)], 1)
+    pos = torch.arange(n, dtype=torch.int64, device=dev) * bits
+    wi, sh = pos >> 5, pos & 31
+    both = w[:, wi] | (w[:, wi + 1] << 32)                     # 64-bit window starting at word wi
+    return (both >> sh) & ((1 << bits) - 1)
+
+
+def perm_crc(perms: torch.Tensor) -> int:
+    """CRC32 of the orders as little-endian int64 (reference shapequant/packed.py:93-94)."""
+    return zlib.crc32(perms.to(torch.int64).cpu().contiguous().numpy().tobytes())
+
+
+def storage_bits(tensors: dict) -> int:
+    """Real tensor bytes plus 32 bits for the seed."""
+    return sum(t.numel() * t.element_size() * 8 for t in tensors.values()) + 32
+
+
+def pack_tensors(local_tags: torch.Tensor, table: torch.Tensor, row_scale: torch.Tensor, *, d: int, K: int,
+                 G: int = 1, M: int = 1, seed: int = 0, row_book: torch.Tensor | None = None,
+                 row_mask: torch.Tensor | None = None) -> tuple[dict, dict]:
+    """Tensors + metadata of one matrix from its parts: local_tags [R, C/d] in [0, K), table
+    [G*K, d], row_scale [R], row_book [R] (G > 1), row_mask [R] (M > 1).  Same validation and
+    metadata as the reference's pack_matrix (reference shapequant/packed.py:97-131)."""
+    if K < 2 or K & (K - 1):
+        raise ValueError(f"K={K} is not a power of two")
+    R, nch = local_tags.shape
+    C = nch * d
+    if tuple(table.shape) != (G * K, d):
+        raise ValueError(f"table shape {tuple(table.shape)} != ({G * K}, {d})")
+    if row_scale.shape != (R,):
+        raise ValueError(f"row_scale shape {tuple(row_scale.shape)} != ({R},)")
+    if (G > 1) != (row_book is not None):
+        raise ValueError("row_book is needed exactly when G > 1")
+    if (M > 1) != (row_mask is not None):
+        raise ValueError("row_mask is needed exactly when M > 1")
+    if G > 256 or M > 256:
+        raise ValueError("row_book / row_mask are stored as uint8")
+    b = K.bit_length() - 1
+    t = {"tags": pack_bits(local_tags, b), "table": table.to(torch.float16).cpu().contiguous(),
+         "row_scale": row_scale.to(torch.float16).cpu().contiguous()}
+    if G > 1:
+        if int(row_book.min()) < 0 or int(row_book.max()) >= G:
+            raise ValueError("row_book out of range")
+        t["row_book"] = row_book.cpu().to(torch.uint8)
+    if M > 1:
+        if int(row_mask.min()) < 0 or int(row_mask.max()) >= M:
+            raise ValueError("row_mask out of range")
+        t["row_mask"] = row_mask.cpu().to(torch.uint8)
+    perms = mk.seeded_perms(C, M, torch.Generator(device="cpu").manual_seed(seed))
+    meta = {"R": R, "C": C, "d": d, "K": K, "G": G, "M": M, "seed": seed, "perm_crc": perm_crc(perms),
+            "bits": storage_bits(t)}
+    return t, meta
+
+
+def pack_matrix(fit, *, d: int, K: int, G: int, M: int, seed: int) -> tuple[dict, dict]:
+    """The reference's entry point (reference shapequant/packed.py:97-131): `fit` is a quantiser
+    result with .tags (one stage of global tags), .row_scale, .perms, .row_mask and
+    .stats["books"][0]; global tags are split into (row_book, local tag)."""
+    if fit.tags is None or len(fit.tags) != 1:
+        raise ValueError("pack_matrix needs single-stage global tags (keep_tags=True)")
+    if K & (K - 1):
+        raise ValueError(f"K={K} is not a power of two")
+    R = fit.row_scale.shape[0]
+    C = fit.perms.shape[1]
+    if C % d:
+        raise ValueError(f"C={C} not divisible by d={d}")
+    gt = fit.tags[0].to(torch.int64).view(R, C // d).cpu()
+    book = torch.div(gt, K, rounding_mode="floor")
+    if not bool((book == book[:, :1]).all()):
+        raise ValueError("a row's tags span several codebooks")
+    t, meta = pack_tensors(gt - book[:, :1] * K, fit.stats["books"][0], fit.row_scale, d=d, K=K, G=G, M=M, seed=seed,
+                           row_book=book[:, 0] if G > 1 else None,
+                           row_mask=fit.row_mask if M > 1 else None)
+    perms = mk.seeded_perms(C, M, torch.Generator(device="cpu").manual_seed(seed))
+    if not torch.equal(perms, fit.perms.cpu()):
+        raise ValueError("fit's column orders do not regenerate from its seed")
+    return t, meta
+
+
+def save(path, packed: dict, *, base_model: str, extra: dict | None = None, aux: tuple | None = None) -> dict:
+    """Write {name: (tensors, meta)} to one safetensors file; returns the summary
+    (reference shapequant/packed.py:186-214).  `aux` = (tensors, meta) is stored as given."""
+    from safetensors.torch import save_file
+    tensors, metas = {}, {}
+    for name, (t, m) in packed.items():
+        for k, v in t.items():
+            tensors[f"{name}.{k}"] = v.contiguous()
+        metas[name] = m
+    bits = sum(m["bits"] for m in metas.values())
+    numel = sum(m["R"] * m["C"] for m in metas.values())
+    summary = {"format": FORMAT, "base_model": base_model, "matrices": len(metas), "bits": bits, "numel": numel,
+               "bpw": bits / numel if numel else 0.0, **(extra or {})}
+    md = {"matrices": json.dumps(metas)}
+    if aux is not None:
+        at, am = aux
+        tensors.update(at)
+        md["aux"] = json.dumps(am, default=str)
+        summary["aux"] = True
+    md["summary"] = json.dumps(summary)
+    Path(path).parent.mkdir(parents=True, exist_ok=True)
+    save_file(tensors, str(path), metadata=md)
+    return summary
+
+
+class PackedFile:
+    """Read access to a packed file (reference shapequant/packed.py:217-256): metadata, raw
+    tensors, regenerated column orders, unpacked tags, and the dense decode (on the GPU)."""
+
+    def __init__(self, path):
+        from safetensors import safe_open
+        self.path = str(path)
+        self.f = safe_open(self.path, framework="pt", device="cpu")
+        md = self.f.metadata() or {}
+        if "summary" not in md or "matrices" not in md:
+            raise ValueError(f"{path}: not a {FORMAT} file (no summary / matrices metadata)")
+        self.summary = json.loads(md["summary"])
+        if self.summary.get("format") != FORMAT:
+            raise ValueError(f"{path}: format {self.summary.get('format')!r} != {FORMAT}")
+        self.meta = json.loads(md["matrices"])
+        self.aux = json.loads(md["aux"]) if "aux" in md else None
+
+    def aux_tensor(self, name: str) -> torch.Tensor:
+        return self.f.get_tensor(f"aux.{name}")
+
+    def tensors(self, name: str) -> dict:
+        m = self.meta[name]
+        keys = ["tags", "table", "row_scale"]
+        if m["G"] > 1:
+            keys.append("row_book")
+        if m["M"] > 1:
+            keys.append("row_mask")
+        return {k: self.f.get_tensor(f"{name}.{k}") for k in keys}
+
+    def perms(self, name: str) -> torch.Tensor:
+        m = self.meta[name]
+        p = mk.seeded_perms(m["C"], m["M"], torch.Generator(device="cpu").manual_seed(m["seed"]))
+        if perm_crc(p) != m["perm_crc"]:
+            raise RuntimeError(f"{name}: regenerated column orders do not match the file (torch RNG changed?)")
+        return p
+
+    def local_tags(self, name: str, device="cpu") -> torch.Tensor:
+        m = self.meta[name]
+        return unpack_bits(self.f.get_tensor(f"{name}.tags").to(device), int(math.log2(m["K"])), m["C"] // m["d"])
+
+    def decode(self, name: str, device="cuda") -> torch.Tensor:
+        """Dense float32 [R, C] weight in the original row and column order, decoded by the HIP
+        dequant kernel on `device` (a GPU; bit-identical to the reference's CPU decode)."""
+        from .kernels import PackedLinear
+        dev = torch.device(device)
+        if dev.type != "cuda":
+            raise RuntimeError("PackedFile.decode runs on the GPU (libsqhip.so); pass a cuda device")
+        return PackedLinear.from_packed(self, name, device=dev).dense()

@@ -1,0 +1,248 @@
+"""vLLM-independent half of the integration: packed codebook matrices as linear layers.
+
+Same surface as the reference module (reference shapequant/vllm_ext/core.py): a vLLM linear
+layer may be several checkpoint matrices stacked along the output dimension; `PackedShards`
+holds one `PackedLinear` per stacked piece and computes Y[M, sum R] = X[M, C] . W^T
+
+  M <= cross (decode, small batches): sq_linear_small, every stacked piece written straight
+      into its column slice of Y, tags read in place from the packed layout;
+  M >  cross (prefill): sq_linear_gemm ("fused": codewords gathered into LDS tiles feeding
+      fp16 MFMA), or "dequant" / "chunked": sq_dequant into a shared scratch + sq_gemm_dense.
+
+Activations stay in their own dtype (bf16 or fp16) end to end; everything launches on torch's
+current stream, allocates only outside graph capture and never synchronises, so the calls are
+HIP-graph capturable after one eager call per shape.  `linear_op` exposes the forward as the
+torch custom op `shapequant::linear` (integer layer handle in, opaque to torch.compile).
+"""
+
+from __future__ import annotations
+
+import contextlib
+import re
+
+import torch
+
+from .. import _lib
+from ..kernels import PackedLinear, _Workspace, gemm_dense, linear_gemm, linear_small
+
+BMAX = _lib.SMALL_BMAX
+
+# checkpoint suffix of each vLLM (possibly stacked) linear -> the packed pieces, in output order
+STACKED = {
+    "self_attn.qkv_proj": ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj"),
+    "mlp.gate_up_proj": ("mlp.gate_proj", "mlp.up_proj"),
+    "linear_attn.in_proj_qkvz": ("linear_attn.in_proj_qkv", "linear_attn.in_proj_z"),
+}
+
+_LAYER = re.compile(r"(?:^|\.)layers\.(\d+)\.(.+)$")
+
+
+def packed_pieces(prefix: str, names) -> list | None:
+    """Packed matrix names (model.layers.N.<kind>) behind the vLLM layer at `prefix`, or None when
+    the layer is not packed; ValueError when only some of its pieces are
+    (reference shapequant/vllm_ext/core.py:127-142)."""
+    if prefix.startswith("mtp.") or ".mtp." in prefix:
+        return None
+    m = _LAYER.search(prefix)
+    if m is None:
+        return None
+    idx, kind = m.group(1), m.group(2)
+    pieces = [f"model.layers.{idx}.{s}" for s in STACKED.get(kind, (kind,))]
+    present = [p in names for p in pieces]
+    if all(present):
+        return pieces
+    if any(present):
+        raise ValueError(f"{prefix}: only some of its pieces are packed ({pieces})")
+    return None
+
+
+@contextlib.contextmanager
+def neutral_defaults():
+    """torch's stock defaults (CPU device, float32) while the layer's tensors are built: vLLM
+    constructs models under a GPU default device and a bf16 default dtype
+    (reference shapequant/vllm_ext/core.py:145-156)."""
+    dt = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float32)
+    try:
+        with torch.device("cpu"):
+            yield
+    finally:
+        torch.set_default_dtype(dt)
+
+
+_TUNED: dict = {}
+_TIME_STREAM: dict = {}
+
+
+def _time(fn, reps: int, n: int = 10) -> float:
+    """GPU ms per call: HIP-graph replay of n calls, median of reps
+    (reference shapequant/vllm_ext/core.py:168-195)."""
+    dev = torch.cuda.current_device()
+    s = _TIME_STREAM.setdefault(dev, torch.cuda.Stream())
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn()
+        fn()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(n):
+            fn()
+    ts = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        ts.append(a.elapsed_time(b) / n)
+    del g
+    return sorted(ts)[len(ts) // 2]
+
+
+class PackedShards:
+    def __init__(self, rls: list, *, bmax: int = BMAX, layout: str = "file", warps: int = 8, bps: int = 2,
+                 xs: bool = False, max_split: int = 8, large: str = "fused", chunk_bytes: int = 24 << 20,
+                 dequant_from: int = 1 << 30, compact: bool = False):
+        # layout / warps / bps / xs / max_split / compact tune the reference's CUDA launchers; the HIP
+        # library plans its own launches and reads the file layout in place (one copy of the tags, which
+        # is what `compact` asks for), so they are accepted and ignored.
+        if large not in ("dequant", "chunked", "fused"):
+            raise ValueError(f"large={large!r}: dequant | chunked | fused")
+        if not rls:
+            raise ValueError("no pieces")
+        if bmax < 1 or bmax > BMAX:
+            raise ValueError(f"bmax={bmax} outside 1..{BMAX}")
+        for rl in rls:
+            if not isinstance(rl, PackedLinear):
+                raise ValueError("pieces must be PackedLinear objects")
+        C = {rl.C for rl in rls}
+        if len(C) != 1:
+            raise ValueError(f"stacked pieces disagree on the input size: {sorted(C)}")
+        dev = {str(rl.device) for rl in rls}
+        if len(dev) != 1:
+            raise ValueError(f"stacked pieces live on different devices: {sorted(dev)}")
+        self.rls = list(rls)
+        self.C = C.pop()
+        self.Rs = [rl.R for rl in rls]
+        self.R = sum(self.Rs)
+        self.offs = [sum(self.Rs[:i]) for i in range(len(rls))]
+        self.large, self.chunk_bytes, self.dequant_from = large, chunk_bytes, dequant_from
+        self.layout, self.compact = layout, compact
+        self.bmax = bmax
+        self.cross = bmax            # M <= cross: small path, else the large-M path (tune() moves it)
+        self.device = rls[0].device
+        self.sq_name = ""            # set by the vLLM plugin (layer prefix)
+
+    @classmethod
+    def from_packed(cls, pf, names: list, dev="cuda", **kw) -> "PackedShards":
+        with neutral_defaults():
+            return cls([PackedLinear.from_packed(pf, n, device=dev) for n in names], **kw)
+
+    # ------------------------------------------------------------------ bookkeeping
+    def key(self) -> tuple:
+        return (tuple(self.Rs), self.C, tuple((rl.bits, rl.d, rl.G, rl.M) for rl in self.rls), self.large, self.bmax)
+
+    def nbytes(self) -> int:
+        n = 0
+        for rl in self.rls:
+            for t in (rl.words, rl.table, rl.row_scale, rl.row_book, rl.row_mask, rl.perms, rl.row_order):
+                if t is not None:
+                    n += t.numel() * t.element_size()
+        return n
+
+    def dense(self) -> torch.Tensor:
+        """fp16 [R, C] (testing)."""
+        return torch.cat([rl.dense(torch.float16) for rl in self.rls])
+
+    def tune_launch(self, reps: int = 3) -> list:
+        """Launch geometry is planned inside the library per shape; nothing to search here."""
+        return []
+
+    @torch.no_grad()
+    def tune(self, Ms=(8, 16, 24, 32), reps: int = 5) -> int:
+        """Measure the small path against the large-M path at each M <= bmax and set cross = the
+        largest M before the large path first wins; cached per shape
+        (reference shapequant/vllm_ext/core.py:308-328)."""
+        k = self.key()
+        if k in _TUNED:
+            self.cross = _TUNED[k]
+            return self.cross
+        cross = 0
+        for M in Ms:
+            if M > self.bmax:
+                break
+            x = torch.randn(M, self.C, device=self.device, dtype=torch.bfloat16)
+            t_small = _time(lambda: self._small(x, M), reps)
+            t_large = _time(lambda: self._large(x), reps)
+            if t_large < t_small:
+                break
+            cross = M
+        self.cross = _TUNED[k] = cross
+        return cross
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x [..., C] -> [..., R] in x's dtype."""
+        shp = x.shape
+        if shp[-1] != self.C:
+            raise ValueError(f"input size {shp[-1]} != {self.C}")
+        x2 = x.reshape(-1, self.C)
+        M = x2.shape[0]
+        if M == 0:
+            return x2.new_empty(0, self.R).view(*shp[:-1], self.R)
+        xin = x2 if x2.dtype in (torch.float16, torch.bfloat16) else x2.to(torch.float16)
+        if xin.stride(1) != 1 or xin.stride(0) % 8 or xin.data_ptr() % 16:
+            xin = xin.contiguous()
+        y = self._small(xin, M) if M <= self.cross else self._large(xin)
+        return y.to(x.dtype).view(*shp[:-1], self.R)
+
+    def _small(self, x: torch.Tensor, M: int) -> torch.Tensor:
+        y = torch.empty(M, self.R, dtype=x.dtype, device=x.device)
+        return linear_small(self.rls, x, y)
+
+    def _large(self, x: torch.Tensor) -> torch.Tensor:
+        M = x.shape[0]
+        y = torch.empty(M, self.R, dtype=x.dtype, device=x.device)
+        if self.large == "fused" and M < self.dequant_from:
+            return linear_gemm(self.rls, x, y)
+        # dequant + GEMM: whole pieces ("dequant") or row chunks of ~chunk_bytes ("chunked") decoded to
+        # fp16 in the shared scratch, each multiplied into its column slice of Y
+        rows = max(self.Rs)
+        if self.large == "chunked":
+            rows = min(rows, max(128, (self.chunk_bytes // (2 * self.C)) // 128 * 128))
+        scratch = _Workspace.get(rows * self.C * 2, x.device).view(torch.float16)
+        for rl, off in zip(self.rls, self.offs):
+            for r0 in range(0, rl.R, rows):
+                r1 = min(rl.R, r0 + rows)
+                w = rl.dense(torch.float16, out=scratch, rows=(r0, r1))
+                gemm_dense(w, x, y[:, off + r0:off + r1])
+        return y
+
+
+# ------------------------------------------------------------------ torch custom op
+
+_REGISTRY: list = []
+
+
+def register(ps) -> int:
+    _REGISTRY.append(ps)
+    return len(_REGISTRY) - 1
+
+
+def pool_tile_words() -> int:
+    """The reference pools its per-matrix tile-word copies here (reference
+    shapequant/vllm_ext/core.py:630-670).  The HIP kernels read the file layout in place and keep
+    no second copy, so there is nothing to pool: returns 0 bytes."""
+    return 0
+
+
+@torch.library.custom_op("shapequant::linear", mutates_args=())
+def linear_op(x: torch.Tensor, handle: int) -> torch.Tensor:
+    return _REGISTRY[handle].forward(x)
+
+
+@linear_op.register_fake
+def _(x: torch.Tensor, handle: int) -> torch.Tensor:
+    return x.new_empty(*x.shape[:-1], _REGISTRY[handle].R)

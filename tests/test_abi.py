@@ -1,0 +1,75 @@
+"""The C-ABI library loads, exports every function include/sqhip.h declares, and rejects bad
+arguments on the host before any GPU work.  CPU only: no kernel is launched here."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from quantexperiments_amd import _lib
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def _declared():
+    text = (ROOT / "include" / "sqhip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sq_[a-z_]+)\s*\(", text)))
+
+
+def test_header_and_loader_agree():
+    assert _declared() == sorted(_lib.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib.lib()
+    for name in _declared():
+        assert getattr(L, name) is not None, name
+    assert L.sq_version() == 100
+
+
+def test_struct_layout_matches_header():
+    # 7 pointers + 8 int32
+    assert ctypes.sizeof(_lib.SqMatrix) == 7 * 8 + 8 * 4
+    assert _lib.SqMatrix.R.offset == 56 and _lib.SqMatrix.y_off.offset == 56 + 28
+
+
+def test_host_side_argument_checks():
+    L = _lib.lib()
+    m = _lib.SqMatrix()                       # all null
+    assert L.sq_dequant(ctypes.byref(m), None, _lib.SQ_F32, 0, 0, 0, None) == _lib.SQ_EINVAL
+    assert b"null" in L.sq_last_error()
+    m = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 4, 30, 4, 8, 1, 1, 2, 0)
+    assert L.sq_dequant(ctypes.byref(m), None, _lib.SQ_F32, 30, 0, 4, None) == _lib.SQ_EINVAL   # C % d
+    m.C = 32
+    m.bits = 17
+    assert L.sq_dequant(ctypes.byref(m), None, _lib.SQ_F32, 32, 0, 4, None) == _lib.SQ_EINVAL
+    m.bits = 8
+    m.W = 1                                   # 8 tags of 8 bits need 2 words
+    assert L.sq_dequant(ctypes.byref(m), None, _lib.SQ_F32, 32, 0, 4, None) == _lib.SQ_EINVAL
+    m.W = 2
+    assert L.sq_dequant(ctypes.byref(m), None, _lib.SQ_F32, 32, 3, 9, None) == _lib.SQ_EINVAL   # rows outside
+    assert L.sq_dequant(ctypes.byref(m), None, _lib.SQ_F32, 32, 2, 2, None) == _lib.SQ_OK       # empty range
+    m.M = 4                                   # masks without row_mask / perms
+    arr = _lib.matrix_array([m])
+    assert L.sq_linear_small(arr, 1, 0x4000, _lib.SQ_BF16, 32, 0x5000, _lib.SQ_BF16, 4, 1, None, 0, None) == _lib.SQ_EINVAL
+    m.M = 1
+    arr = _lib.matrix_array([m])
+    assert L.sq_linear_small(arr, 1, 0x4000, _lib.SQ_F32, 32, 0x5000, _lib.SQ_F32, 4, 1, None, 0, None) == _lib.SQ_EINVAL
+    assert L.sq_linear_small(arr, 1, 0x4000, _lib.SQ_BF16, 32, 0x5000, _lib.SQ_BF16, 4, 33, None, 0, None) == _lib.SQ_EINVAL
+    assert L.sq_linear_small(arr, 1, 0x4000, _lib.SQ_BF16, 32, 0x5000, _lib.SQ_BF16, 4, 0, None, 0, None) == _lib.SQ_OK
+    assert L.sq_linear_gemm(arr, 1, 0x4000, _lib.SQ_BF16, 16, 0x5000, _lib.SQ_BF16, 4, 64, None, 0, None) == _lib.SQ_EINVAL
+    assert L.sq_gemm_dense(0x1000, 5, 32, 8, 32, 0x4000, _lib.SQ_F16, 32, 0x5000, _lib.SQ_F16, 8, 4, None) == _lib.SQ_EINVAL
+    with pytest.raises(_lib.SqError):
+        _lib.check(_lib.SQ_EINVAL)
+
+
+def test_workspace_sizes_are_host_arithmetic():
+    L = _lib.lib()
+    plain = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 8, 16, 1, 1, 32, 0)
+    masked = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, 0x6000, 0x7000, None, 64, 512, 8, 16, 1, 16, 32, 0)
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 1, 0) == 0
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 0
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == 16 * 2 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2048, 1) == 64 * 512 * 2

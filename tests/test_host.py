@@ -1,0 +1,176 @@
+"""Host logic of the shipped package against the oracle and the reference's CPU-side tests:
+bit packing, packed files, column orders, piece naming, defaults.  CPU only, no kernels."""
+
+import json
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sq_oracle as O
+from quantexperiments_amd import codebook as cb
+from quantexperiments_amd import masks as mk
+from quantexperiments_amd import packed
+from tests.helpers import synth
+
+
+@pytest.mark.parametrize("bits", [1, 8, 10, 12, 13, 14, 16])
+def test_pack_bits_matches_oracle(bits):
+    g = torch.Generator().manual_seed(bits)
+    v = torch.randint(0, 1 << bits, (70, 37), generator=g)
+    words = packed.pack_bits(v, bits)
+    assert words.dtype == torch.int32 and words.shape == (70, math.ceil(37 * bits / 32))
+    assert np.array_equal(words.numpy(), O.pack_bits(v.numpy(), bits))
+    assert torch.equal(packed.unpack_bits(words, bits, 37), v)
+
+
+def test_pack_bits_known_answers():
+    w = packed.pack_bits(torch.tensor([[1, 1, 0, 0]]), 10)
+    assert int(w[0, 0]) == (1 | (1 << 10))
+    w = packed.pack_bits(torch.tensor([[0, 0, 0, 1023]]), 10).to(torch.int64) & 0xFFFFFFFF
+    assert int(w[0, 0]) == 0b11 << 30 and int(w[0, 1]) == 0xFF
+
+
+def test_pack_bits_errors_and_empty():
+    with pytest.raises(ValueError):
+        packed.pack_bits(torch.tensor([[16]]), 4)
+    with pytest.raises(ValueError):
+        packed.pack_bits(torch.tensor([[-1]]), 4)
+    assert packed.pack_bits(torch.zeros(0, 5, dtype=torch.int64), 7).shape == (0, 2)
+    assert packed.unpack_bits(torch.zeros(3, 2, dtype=torch.int32), 7, 0).shape == (3, 0)
+
+
+def test_seeded_perms_and_crc_match_reference_golden(golden_dir):
+    gold = json.loads((golden_dir / "seeded_perms.json").read_text())
+    for c in gold["cases"]:
+        p = mk.seeded_perms(c["C"], c["M"], torch.Generator(device="cpu").manual_seed(c["seed"]))
+        assert p.dtype == torch.int64 and list(p.shape) == c["shape"]
+        assert packed.perm_crc(p) == c["crc"]
+        assert np.array_equal(p.numpy(), O.seeded_perms(c["C"], c["M"], c["seed"]))
+
+
+def _file(tmp_path, **kw):
+    s = synth(kw.get("R", 24), kw.get("C", 64), kw.get("d", 4), kw.get("bits", 6), kw.get("G", 1), kw.get("M", 1), seed=3)
+    t, meta = packed.pack_tensors(torch.from_numpy(s.tags), torch.from_numpy(s.table), torch.from_numpy(s.row_scale),
+                                  d=s.d, K=s.K, G=s.G, M=s.M, seed=4,       # helpers use seed + 1 for the orders
+                                  row_book=None if s.row_book is None else torch.from_numpy(s.row_book),
+                                  row_mask=None if s.row_mask is None else torch.from_numpy(s.row_mask))
+    path = tmp_path / "q.safetensors"
+    summary = packed.save(path, {"model.layers.0.mlp.up_proj": (t, meta)}, base_model="test/base")
+    return s, t, meta, summary, path
+
+
+@pytest.mark.parametrize("G,M", [(1, 1), (4, 1), (1, 8), (4, 8)])
+def test_packed_file_round_trip(tmp_path, G, M):
+    s, t, meta, summary, path = _file(tmp_path, G=G, M=M)
+    assert meta["bits"] == O.storage_bits(s.R, s.C, s.d, s.K, G, M) == summary["bits"]
+    assert summary["format"] == "shapequant-stack-v1" and summary["matrices"] == 1
+    assert abs(summary["bpw"] - meta["bits"] / (s.R * s.C)) < 1e-12
+    pf = packed.PackedFile(path)
+    name = "model.layers.0.mlp.up_proj"
+    assert pf.meta[name] == meta
+    got = pf.tensors(name)
+    assert set(got) == {"tags", "table", "row_scale"} | ({"row_book"} if G > 1 else set()) | ({"row_mask"} if M > 1 else set())
+    assert got["tags"].dtype == torch.int32 and np.array_equal(got["tags"].numpy(), s.words)
+    assert got["table"].dtype == torch.float16 and got["row_scale"].dtype == torch.float16
+    assert np.array_equal(pf.local_tags(name).numpy(), s.tags)
+    assert np.array_equal(pf.perms(name).numpy(), s.perms)
+    with pytest.raises(RuntimeError, match="GPU"):
+        pf.decode(name, device="cpu")
+
+
+def test_packed_file_guards(tmp_path):
+    s, t, meta, summary, path = _file(tmp_path, M=4)
+    bad = dict(meta, perm_crc=meta["perm_crc"] ^ 1)
+    packed.save(tmp_path / "bad.safetensors", {"m": (t, bad)}, base_model="x")
+    with pytest.raises(RuntimeError, match="column orders"):
+        packed.PackedFile(tmp_path / "bad.safetensors").perms("m")
+    from safetensors.torch import save_file
+    save_file({"a": torch.zeros(1)}, str(tmp_path / "other.safetensors"),
+              metadata={"summary": json.dumps({"format": "something-else"}), "matrices": "{}"})
+    with pytest.raises(ValueError, match="format"):
+        packed.PackedFile(tmp_path / "other.safetensors")
+
+
+def test_pack_tensors_validation():
+    s = synth(8, 32, 4, 4, seed=1)
+    tg, tb, rs = torch.from_numpy(s.tags), torch.from_numpy(s.table), torch.from_numpy(s.row_scale)
+    with pytest.raises(ValueError, match="power of two"):
+        packed.pack_tensors(tg, tb[:12], rs, d=4, K=12)
+    with pytest.raises(ValueError, match="table shape"):
+        packed.pack_tensors(tg, tb[:8], rs, d=4, K=16)
+    with pytest.raises(ValueError, match="row_book"):
+        packed.pack_tensors(tg, tb, rs, d=4, K=16, row_book=torch.zeros(8))
+    with pytest.raises(ValueError, match="row_mask"):
+        packed.pack_tensors(tg, tb, rs, d=4, K=16, M=4)
+
+
+def test_pack_matrix_takes_a_fit_like_object():
+    class Fit:
+        pass
+    s = synth(10, 32, 4, 4, G=2, M=4, seed=6)
+    f = Fit()
+    f.tags = [torch.from_numpy(s.tags + s.row_book.astype(np.int64)[:, None] * s.K).reshape(-1)]
+    f.row_scale, f.row_mask = torch.from_numpy(s.row_scale), torch.from_numpy(s.row_mask)
+    f.perms = torch.from_numpy(s.perms)
+    f.stats = {"books": [torch.from_numpy(s.table)]}
+    t, meta = packed.pack_matrix(f, d=4, K=16, G=2, M=4, seed=7)
+    assert np.array_equal(t["tags"].numpy(), s.words) and np.array_equal(t["row_book"].numpy(), s.row_book)
+    assert meta["perm_crc"] == O.perm_crc(s.perms)
+    with pytest.raises(ValueError, match="regenerate"):
+        packed.pack_matrix(f, d=4, K=16, G=2, M=4, seed=8)
+    f.tags[0][1] += 16       # a row whose tags leave its codebook
+    with pytest.raises(ValueError, match="several codebooks"):
+        packed.pack_matrix(f, d=4, K=16, G=2, M=4, seed=7)
+
+
+def test_codebook_host_helpers():
+    assert cb.layer_seed(3, "a.b") == O.layer_seed(3, "a.b")
+    w = torch.arange(20.0).view(2, 10)
+    ch, pad = cb.chunk_rows(w, 8)
+    ref, rpad = O.chunk_rows(w.numpy(), 8)
+    assert pad == rpad == 6 and np.array_equal(ch.numpy(), ref)
+    cm = cb.CodebookMatrix(torch.zeros(2, 2, dtype=torch.int64), torch.ones(4, 8).half(), torch.ones(2).half(), 6, 10)
+    assert cm.d == 8 and cm.K == 4
+    with pytest.raises(RuntimeError, match="GPU"):
+        cb.decode(cm, device="cpu")
+
+
+def test_packed_pieces():
+    # reference tests/test_vllm_ext_core.py:14-29
+    from quantexperiments_amd.vllm_ext import core
+    names = {"model.layers.3.self_attn.q_proj", "model.layers.3.self_attn.k_proj", "model.layers.3.self_attn.v_proj",
+             "model.layers.0.linear_attn.in_proj_qkv", "model.layers.0.linear_attn.in_proj_z",
+             "model.layers.0.mlp.down_proj"}
+    assert core.packed_pieces("model.layers.3.self_attn.qkv_proj", names) == [
+        "model.layers.3.self_attn.q_proj", "model.layers.3.self_attn.k_proj", "model.layers.3.self_attn.v_proj"]
+    assert core.packed_pieces("language_model.model.layers.0.linear_attn.in_proj_qkvz", names) == [
+        "model.layers.0.linear_attn.in_proj_qkv", "model.layers.0.linear_attn.in_proj_z"]
+    assert core.packed_pieces("model.layers.0.mlp.down_proj", names) == ["model.layers.0.mlp.down_proj"]
+    assert core.packed_pieces("model.layers.0.linear_attn.in_proj_ba", names) is None
+    assert core.packed_pieces("model.layers.0.linear_attn.conv1d", names) is None
+    assert core.packed_pieces("lm_head", names) is None
+    assert core.packed_pieces("mtp.layers.0.mlp.down_proj", names) is None
+    assert core.packed_pieces("model.mtp.layers.0.mlp.down_proj", names) is None
+    with pytest.raises(ValueError):
+        core.packed_pieces("model.layers.0.mlp.gate_up_proj", names | {"model.layers.0.mlp.gate_proj"})
+
+
+def test_neutral_defaults_and_registry():
+    from quantexperiments_amd.vllm_ext import core
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with core.neutral_defaults():
+            assert torch.get_default_dtype() == torch.float32 and torch.zeros(1).device.type == "cpu"
+        assert torch.get_default_dtype() == torch.bfloat16
+    finally:
+        torch.set_default_dtype(torch.float32)
+
+    class Stub:
+        R = 7
+    h = core.register(Stub())
+    assert core._REGISTRY[h].R == 7 and core.pool_tile_words() == 0
+    # the fake (meta) implementation gives the output shape without touching a kernel
+    y = torch.ops.shapequant.linear(torch.empty(2, 3, 5, device="meta"), h)
+    assert y.shape == (2, 3, 7) and y.device.type == "meta"
