@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Headline benchmark of the codebook linear hot path on one MI355X.
+
+A "step" is one batch-1 pass over the 7 block linears of one Qwen2.5-7B-shaped layer
+(q/o 3584x3584, k/v 512x3584, gate/up 18944x3584, down 3584x18944; d = 8, K = 65,536 fp16
+codebook per matrix, uint16 tags = 2 bits per weight, fp16 row scales, bf16 activations), run as
+the serving path runs it: 4 launches (q|k|v stacked, o, gate|up stacked, down) through the C ABI.
+Steps rotate over enough distinct layers (>= 4x the 256 MB last-level cache) that tags stream from
+HBM.  K steps are captured in one HIP graph and timed between device synchronisations.
+
+value = packed (algorithmic) bytes of a layer / time per layer, in GB/s.  The same JSON line
+carries us_per_layer, the roofline of the dominant kernel (gate|up launch, HIP events around graph
+replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s, and the CPU baseline (the
+reference's CPU route, oracle port, on the host cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16
+
+SHAPES_7B = {"q": (3584, 3584), "k": (512, 3584), "v": (512, 3584), "o": (3584, 3584),
+             "gate": (18944, 3584), "up": (18944, 3584), "down": (3584, 18944)}
+LAUNCHES = (("q", "k", "v"), ("o",), ("gate", "up"), ("down",))
+D, BITS = 8, 16
+
+
+def algorithmic_bytes(names, B=1):
+    """tags + table + row scales + x + y of the pieces of one launch, each counted once."""
+    n = 0
+    C = SHAPES_7B[names[0]][1]
+    for nm in names:
+        R, C = SHAPES_7B[nm]
+        n += R * (C // D) * BITS // 8 + (1 << BITS) * D * 2 + R * 2 + B * R * 2
+    return n + B * C * 2
+
+
+def make_layer(torch, dev, gen):
+    """One layer of PackedLinear pieces with seeded synthetic contents, generated on the device."""
+    from quantexperiments_amd.kernels import PackedLinear
+    out = {}
+    for nm, (R, C) in SHAPES_7B.items():
+        W = (C // D) * BITS // 32
+        words = torch.randint(-2 ** 31, 2 ** 31, (R, W), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
+        table = torch.randn(1 << BITS, D, device=dev, generator=gen).to(torch.float16)
+        rs = (torch.randn(R, device=dev, generator=gen) * 0.005 + 0.02).abs().to(torch.float16)
+        out[nm] = PackedLinear(words, table, rs, None, None, torch.arange(C, device=dev)[None], 1 << BITS, D)
+    return out
+
+
+def timed_graph(torch, fn, reps=5):
+    """ms per replay of a HIP graph of fn(), median of reps; events on torch's current stream."""
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        ts.append(a.elapsed_time(b))
+    return sorted(ts)[len(ts) // 2], g
+
+
+def cpu_baseline(torch, layer, x):
+    """The reference's CPU route (unpack, gather, scale, fp32 matmul, bf16) on the host cores:
+    one full layer, after a warm-up on k_proj."""
+    from oracle import sq_oracle as O
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    host = {nm: (p.words.cpu(), p.table.cpu(), p.row_scale.cpu()) for nm, p in layer.items()}
+    xs = {C: x[C].cpu() for C in x}
+    w, t, rs = host["k"]
+    O.torch_cpu_layer(w, t, rs, None, None, BITS, xs[3584])
+    dec = mm = 0.0
+    t0 = time.perf_counter()
+    for nm, (w, t, rs) in host.items():
+        _, a, b = O.torch_cpu_layer(w, t, rs, None, None, BITS, xs[SHAPES_7B[nm][1]])
+        dec += a
+        mm += b
+    total = time.perf_counter() - t0
+    nbytes = sum(algorithmic_bytes(l) for l in LAUNCHES)
+    return {"value": nbytes / total / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "one full 7B-shaped layer (7 matrices, bs=1), 1 repetition after a k_proj warm-up; "
+                      "torch gather + scale + fp32 matmul + bf16 round",
+            "us_per_layer": total * 1e6, "decode_s": dec, "matmul_s": mm}
+
+
+def prefill(torch, dev, layer, steps=3):
+    """M = 2048 prefill GEMM at gate/up (18944x3584) and down (3584x18944)."""
+    from quantexperiments_amd.kernels import linear_gemm
+    res = {}
+    for nm in ("gate", "down"):
+        R, C = SHAPES_7B[nm]
+        x = torch.randn(2048, C, device=dev).to(torch.bfloat16)
+        y = torch.empty(2048, R, device=dev, dtype=torch.bfloat16)
+        ms, g = timed_graph(torch, lambda: linear_gemm([layer[nm]], x, y), reps=steps)
+        del g
+        res[nm] = {"ms": ms, "tflops": 2.0 * 2048 * R * C / (ms * 1e-3) / 1e12}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=280)
+    ap.add_argument("--warmup", type=int, default=28)
+    ap.add_argument("--layers", type=int, default=28, help="distinct layers the steps rotate over")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures the one-GPU hot path; multi-GPU runs are not part of this build (use --gpus 1)")
+
+    import torch
+    from quantexperiments_amd.kernels import linear_small
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X (no CPU fallback)")
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    layers = [make_layer(torch, dev, gen) for _ in range(args.layers)]
+    x = {C: torch.randn(1, C, device=dev, generator=gen).to(torch.bfloat16) for C in (3584, 18944)}
+    y = {l: torch.empty(1, sum(SHAPES_7B[n][0] for n in l), device=dev, dtype=torch.bfloat16) for l in LAUNCHES}
+
+    def step(i):
+        L = layers[i % len(layers)]
+        for l in LAUNCHES:
+            linear_small([L[n] for n in l], x[SHAPES_7B[l[0]][1]], y[l])
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(args.steps):
+            step(i)
+    g.replay()                                   # graph upload / first-launch costs stay outside the timed region
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    g.replay()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    layer_bytes = sum(algorithmic_bytes(l) for l in LAUNCHES)
+    tag_bytes = sum(R * (C // D) * BITS // 8 for R, C in SHAPES_7B.values())
+    value = layer_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # dominant kernel: the gate|up launch alone, over all layers, HIP events around graph replays
+    gu = LAUNCHES[2]
+
+    def gate_up_all():
+        for L in layers:
+            linear_small([L[n] for n in gu], x[3584], y[gu])
+    ms, g2 = timed_graph(torch, gate_up_all)
+    del g2
+    dur_us = ms * 1e3 / len(layers)
+    gu_bytes = algorithmic_bytes(gu)
+    achieved = gu_bytes / (dur_us * 1e-6) / 1e9
+    per_launch = {}
+    for l in LAUNCHES:
+        def one(l=l):
+            for L in layers:
+                linear_small([L[n] for n in l], x[SHAPES_7B[l[0]][1]], y[l])
+        ms_l, gl = timed_graph(torch, one, reps=3)
+        del gl
+        per_launch["|".join(l)] = {"us": ms_l * 1e3 / len(layers), "bytes": algorithmic_bytes(l)}
+
+    out = {
+        "metric": "codebook GEMV HBM GB/s + us/layer @7B bs=1; prefill GEMM TFLOP/s @M=2048",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16xf16->f32 (bf16 activations in/out)", "data": "synthetic (seed 0, generated on device)",
+        "config": {"workload": "cfg2: one Qwen2.5-7B-shaped layer, 7 block linears, bs=1, d=8, K=65536, uint16 tags "
+                               "(2 bpw), fp16 row scales, bf16 x/y; 4 launches per layer (q|k|v, o, gate|up, down)",
+                   "layers_rotated": len(layers), "bytes_per_layer": layer_bytes, "tag_bytes_per_layer": tag_bytes},
+        "us_per_layer": ms_per_step * 1e3,
+        "tag_only_GBps": tag_bytes / (ms_per_step * 1e-3) / 1e9,
+        "per_launch": per_launch,
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<16,8,1,1,false> (gate|up launch, 2 x 18944x3584)",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "bytes_per_launch": gu_bytes, "us_per_launch": dur_us, "traffic": None},
+    }
+    if not args.no_prefill:
+        pf = prefill(torch, dev, layers[0])
+        out["prefill"] = {"M": 2048, "gate_18944x3584": pf["gate"], "down_3584x18944": pf["down"],
+                          "peak_tflops": MFMA_PEAK_TFLOPS,
+                          "frac_of_peak": min(pf["gate"]["tflops"], pf["down"]["tflops"]) / MFMA_PEAK_TFLOPS}
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(torch, layers[0], x)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -4,10 +4,10 @@
 
 namespace sq {
 
-int launch_gemv_b16d8(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
-int launch_gemv_b12d4(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
-int launch_gemv_b10d4(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
-int launch_gemv_b8d4(const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_gemv_b16d8(int, const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_gemv_b12d4(int, const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_gemv_b10d4(int, const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_gemv_b8d4(int, const GemvArgs&, int, int, int, int, size_t, hipStream_t);
 
 // xp[m, b, c] = fp16(x[b, perms[m, c]])
 __global__ __launch_bounds__(256) void permute_x_kernel(const uint16_t* __restrict__ x, int64_t ldx, int x_dtype,
@@ -45,36 +45,32 @@ static size_t xp_bytes(const sq_matrix& m, int B) {
 
 struct Plan { int TS, S, nwaves; };
 
-// Host mirror of gemv_cfg<>::REGS / LB.
-static int cfg_regs(int bits, int d, int S, int NB) {
-    const int ud = unit_dwords(bits), xh = ud * 32 / bits * d / 2;
-    return NB * S * xh + GEMV_PF * S * ud + 56;
+// Host mirror of gemv_cfg<>::XW / OK / LB.
+static int cfg_xw(int bits, int d, int S, int NB) {
+    const int ud = unit_dwords(bits);
+    return NB * S * (ud * 32 / bits * d / 2);
 }
-static int cfg_lb(int bits, int d, int S, int NB) { return cfg_regs(bits, d, S, NB) <= 256 ? 512 : 256; }
+static int cfg_lb(int bits, int d, int S, int NB) { return cfg_xw(bits, d, S, NB) < 64 ? 512 : 256; }
 
 // Team size / slots for U units per row: fewest idle lanes, then fewest slots.
 static Plan plan_for(int U, int bits, int d) {
     Plan best{0, 0, 0};
     double best_eff = -1.0;
-    const int cands[] = {16, 32, 64, 128, 192, 256, 320, 384, 448, 512};
+    const int cands[] = {16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 640, 768, 1024};
     const int slots[] = {1, 2, 3, 5};
     for (int ts : cands)
         for (int s : slots) {
             if (ts * s < U) continue;
-            if (cfg_regs(bits, d, s, 1) > 440) break;
+            if (cfg_xw(bits, d, s, 1) > 192) break;
             if (ts > cfg_lb(bits, d, s, 1)) break;
-            const double eff = (double)U / (ts * s) - 0.02 * (s - 1) - (ts > 64 ? 0.01 : 0.0);
+            const double eff = (double)U / (ts * s) - 0.02 * (s - 1) - (ts > 64 ? 0.05 : 0.0);   // barriers cost
             if (eff > best_eff + 1e-9) { best_eff = eff; best.TS = ts; best.S = s; }
             break;
         }
     if (best.TS == 0) return best;
-    const int lb = cfg_lb(bits, d, best.S, 1);
-    if (best.TS >= 64) {
-        const int wpr = best.TS / 64;
-        int rg = (lb / 64) / wpr;
-        if (rg < 1) rg = 1;
-        best.nwaves = wpr * rg;
-    } else best.nwaves = lb / 64;
+    // 4 waves per workgroup (several workgroups per CU) unless a row needs more waves than that
+    const int wpr = best.TS > 64 ? best.TS / 64 : 1;
+    best.nwaves = wpr * (4 / wpr > 0 ? 4 / wpr : 1);
     return best;
 }
 
@@ -90,7 +86,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
     if (small_workspace(mats, n, B) > ws_bytes)
         return fail(SQ_EWORKSPACE, "sq_linear_small: workspace %zu < %zu", ws_bytes, small_workspace(mats, n, B));
     const int cus = device_cus();
-    const bool x_ok = (ldx % 2 == 0) && (((uintptr_t)x & 3) == 0);
+    const bool x_ok = (B == 1 || ldx % 8 == 0) && (((uintptr_t)x & 15) == 0);   // 16-byte activation loads
     size_t ws_off = 0;
     int i = 0;
     while (i < n) {
@@ -142,15 +138,23 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
             const int left = B - b0;
             int nbt = left >= 4 ? 4 : left >= 2 ? 2 : 1;
             // fewer activation rows per pass when the registers or the workgroup width do not allow more
-            while (nbt > 1 && (cfg_regs(m0.bits, m0.d, pl.S, nbt) > 440 || cfg_lb(m0.bits, m0.d, pl.S, nbt) < wpr * 64)) nbt >>= 1;
+            while (nbt > 1 && (cfg_xw(m0.bits, m0.d, pl.S, nbt) > 192 || cfg_lb(m0.bits, m0.d, pl.S, nbt) < wpr * 64)) nbt >>= 1;
             const int lb = cfg_lb(m0.bits, m0.d, pl.S, nbt);
             int nwaves = pl.nwaves;
-            if (nwaves * 64 > lb) nwaves = (lb / 64) / wpr * wpr;
+            // a codebook that leaves room for one workgroup per CU: make that workgroup as wide as allowed
+            if (nwaves * 64 > lb || a.table_bytes > 80 * 1024) nwaves = (lb / 64) / wpr * wpr;
             const int ngrp = pl.TS > 64 ? nwaves / wpr : nwaves * (64 / pl.TS);
             const size_t smem = (size_t)a.table_bytes + (wpr > 1 ? (size_t)GEMV_PF * ngrp * wpr * nbt * sizeof(float) : 0);
             // persistent grid: workgroups per CU bounded by LDS and wave slots, split over the pieces by rows
-            int per_cu = smem > 80 * 1024 ? 1 : smem > 40 * 1024 ? 2 : smem > 20 * 1024 ? 4 : 8;
-            if (nwaves * per_cu > 16) per_cu = 16 / nwaves > 0 ? 16 / nwaves : 1;
+            int rc = SQ_EUNSUPPORTED;
+#define SQ_CASE(BI, DD) if (m0.bits == BI && m0.d == DD) rc = launch_gemv_b##BI##d##DD(OP, a, pl.S, nbt, GRID, nwaves * 64, smem, s)
+#define OP 1
+#define GRID 0
+            SQ_CASE(16, 8); SQ_CASE(12, 4); SQ_CASE(10, 4); SQ_CASE(8, 4);      // workgroups that fit on a CU
+#undef OP
+#undef GRID
+            if (rc < 1) return rc < 0 ? rc : fail(SQ_ELAUNCH, "sq_linear_small: kernel does not fit a CU");
+            const int per_cu = rc;
             const int64_t row_quant = (int64_t)ngrp * GEMV_PF;
             const int grid_target = cus * per_cu;
             int wg_begin = 0;
@@ -165,9 +169,12 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
                 wg_begin += cnt;
             }
             a.b0 = b0;
-            int rc = SQ_EUNSUPPORTED;
-#define SQ_CASE(BI, DD) if (m0.bits == BI && m0.d == DD) rc = launch_gemv_b##BI##d##DD(a, pl.S, nbt, wg_begin, nwaves * 64, smem, s)
+            rc = SQ_EUNSUPPORTED;
+#define OP 0
+#define GRID wg_begin
             SQ_CASE(16, 8); SQ_CASE(12, 4); SQ_CASE(10, 4); SQ_CASE(8, 4);
+#undef OP
+#undef GRID
 #undef SQ_CASE
             if (rc) return rc;
             b0 += nbt;

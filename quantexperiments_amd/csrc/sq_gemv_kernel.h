@@ -6,28 +6,33 @@
 // team owns units tl, tl + TS, ... (S slots) of EVERY row the team visits, so the activations that
 // multiply those units never change: they sit in registers as packed fp16 pairs for the whole
 // kernel (bf16 activations are converted once, exactly for every fp16-normal value).  The only
-// per-row traffic is the tag stream itself, read with one wide coalesced load per slot, plus
-// one gather per tag from the codebook, which is staged in LDS when it fits and read through
-// L1/L2 otherwise.  Products are v_dot2_f32_f16 (fp16 x fp16 pairs, fp32 accumulate); the team
-// sum is a cross-lane butterfly, and teams wider than a wave add their per-wave partials
-// through LDS once per row block.
+// per-row traffic is the tag stream itself, read with one wide coalesced load per slot and
+// prefetched one batch of rows ahead, plus one gather per tag from the codebook, which is
+// staged in LDS when it fits and read through L1/L2 otherwise.  Products are v_dot2_f32_f16
+// (fp16 x fp16 pairs, fp32 accumulate) with one accumulator per row in flight, so consecutive
+// dot instructions are independent.  The team sum is six DPP adds (no LDS traffic); teams wider
+// than a wave add their per-wave partials through LDS once per batch.
 //
-// Column orders: rows are visited in row_order (sorted by mask), a lane reloads its activation
-// registers from the pre-permuted copy xp[mask] only when the mask of its row changes.
+// Each team walks a contiguous range of row_order (rows sorted by column order), so the column
+// order changes at most M - 1 times per matrix; a batch whose rows do not all share the
+// current order takes a one-row-at-a-time path that reloads the activation registers from
+// the pre-permuted copy xp[order].
 #pragma once
+#include <mutex>
+#include <unordered_map>
 #include "sq_common.h"
 
 namespace sq {
 
 constexpr int GEMV_MAX_PIECES = 4;
-constexpr int GEMV_PF = 4;   // rows whose tag loads are issued before any of them is consumed
+constexpr int GEMV_PF = 2;   // rows per batch; two batches of tag loads are in flight per lane
 
 struct GemvPiece {
     sq_matrix m;
-    const uint16_t* xp;   // fp16 [M, B, C] pre-permuted activations (M > 1) or NULL
+    const uint16_t* xp;   // fp16 [M, B, C] pre-permuted activations (pieces with column orders) or NULL
     int U;                // units per row
     int wg_begin;         // first workgroup of this piece
-    int wg_count;
+    int wg_count;         // workgroups that share this piece's rows
 };
 
 struct GemvArgs {
@@ -74,7 +79,25 @@ __device__ __forceinline__ uint32_t unit_tag(const dwords<UD>& u, int t) {
     uint32_t v;
     if (s + BITS <= 32) v = u.v[w] >> s;
     else v = __builtin_amdgcn_alignbit(u.v[w + 1 < UD ? w + 1 : w], u.v[w], s);
-    return v & ((1u << BITS) - 1u);
+    return (s + BITS == 32) ? v : v & ((1u << BITS) - 1u);
+}
+
+// v + (v moved across lanes by a DPP pattern); lanes the pattern leaves out add zero
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false);
+    return v + __builtin_bit_cast(float, t);
+}
+
+// Sum over each team of `span` lanes (16, 32 or 64); valid in the LAST lane of every team.
+__device__ __forceinline__ float team_sum(float v, int span) {
+    v = dpp_add<0xB1, 0xf>(v);                     // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xf>(v);                     // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xf>(v);                    // row_half_mirror
+    v = dpp_add<0x140, 0xf>(v);                    // row_mirror: every lane holds its row-of-16 sum
+    if (span >= 32) v = dpp_add<0x142, 0xa>(v);    // row_bcast15 into rows 1 and 3
+    if (span >= 64) v = dpp_add<0x143, 0xc>(v);    // row_bcast31 into rows 2 and 3
+    return v;
 }
 
 // Register estimate of one instantiation -> workgroup size limit the compiler may assume.
@@ -82,22 +105,103 @@ template <int BITS, int D, int S, int NB> struct gemv_cfg {
     static constexpr int UD = unit_of<BITS>::UD;
     static constexpr int TPU = UD * 32 / BITS;
     static constexpr int XH = TPU * D / 2;
-    static constexpr int REGS = NB * S * XH + GEMV_PF * S * UD + 56;
-    static constexpr bool OK = REGS <= 440;
-    static constexpr int LB = REGS <= 256 ? 512 : 256;      // threads per workgroup the kernel is built for
+    static constexpr int XW = NB * S * XH;            // dwords of activations a lane keeps in registers
+    static constexpr bool OK = XW <= 192;
+    static constexpr int LB = XW < 64 ? 512 : 256;    // threads per workgroup it is built for (256 or 512 VGPRs per lane)
 };
 
 template <int D> struct cw_t;
 template <> struct cw_t<8> { typedef u32x4 type; };
 template <> struct cw_t<4> { typedef u32x2 type; };
 
+__device__ __forceinline__ void store_y(void* y, int y_dtype, int64_t o, float v) {
+    if (y_dtype == SQ_BF16) reinterpret_cast<uint16_t*>(y)[o] = f2bf(v);
+    else if (y_dtype == SQ_F16) reinterpret_cast<uint16_t*>(y)[o] = f2h(v);
+    else reinterpret_cast<float*>(y)[o] = v;
+}
+
+template <int BITS, int D, int S, int NB, bool LDS_TAB>
+struct GemvBody {
+    static constexpr int UD = unit_of<BITS>::UD;
+    static constexpr int TPU = UD * 32 / BITS;      // tags per unit
+    static constexpr int XH = TPU * D / 2;          // fp16 pairs of activation per slot
+    static constexpr int H = D / 2;                 // fp16 pairs per codeword
+    typedef typename cw_t<D>::type CW;
+
+    // activation registers of this lane for column order `rm` (16-byte loads; bf16 -> fp16 once)
+    static __device__ __forceinline__ void load_x(uint32_t (&xr)[NB][S][XH], const GemvArgs& a, const GemvPiece& P,
+                                                  int rm, int tl, int nb) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int s = 0; s < S; ++s) {
+                const int u = tl + s * a.TS;
+                const bool ok = b < nb && u < P.U;
+                const int c0 = u * (TPU * D);
+                const uint16_t* src = P.xp ? P.xp + ((int64_t)rm * a.B + a.b0 + b) * P.m.C + c0
+                                           : a.x + (int64_t)(a.b0 + b) * a.ldx + c0;
+                const bool cvt = !P.xp && a.x_dtype == SQ_BF16;
+#pragma unroll
+                for (int i = 0; i < XH; i += 4) {
+                    u32x4 v = {0u, 0u, 0u, 0u};
+                    if (ok) v = *reinterpret_cast<const u32x4*>(src + 2 * i);
+                    if (cvt) { v.x = bf2h_x2(v.x); v.y = bf2h_x2(v.y); v.z = bf2h_x2(v.z); v.w = bf2h_x2(v.w); }
+                    xr[b][s][i] = v.x; xr[b][s][i + 1] = v.y; xr[b][s][i + 2] = v.z; xr[b][s][i + 3] = v.w;
+                }
+            }
+    }
+
+    // NF rows at once: acc[f][b] = sum over this lane's units of <codeword, activations>.  A slot past the
+    // row's end holds zero tags and zero activations; its sum is dropped so that codeword 0 (possibly
+    // non-finite) never reaches rows that do not use it.
+    template <int NF>
+    static __device__ __forceinline__ void rows(float (&out)[NF][NB], const dwords<UD> (&tg)[NF][S],
+                                                const uint32_t (&boff)[NF], const uint32_t (&xr)[NB][S][XH],
+                                                const bool (&live)[S], const unsigned char* smem,
+                                                const unsigned char* table) {
+#pragma unroll
+        for (int f = 0; f < NF; ++f)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) out[f][b] = 0.f;
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            float acc[NF][NB];
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+#pragma unroll
+                for (int b = 0; b < NB; ++b) acc[f][b] = 0.f;
+#pragma unroll
+            for (int t = 0; t < TPU; ++t) {
+                CW cw[NF];
+#pragma unroll
+                for (int f = 0; f < NF; ++f) {
+                    const uint32_t tag = unit_tag<BITS, UD>(tg[f][s], t) + boff[f];
+                    if (LDS_TAB) cw[f] = *reinterpret_cast<const CW*>(smem + tag * (D * 2));
+                    else cw[f] = *reinterpret_cast<const CW*>(table + (size_t)tag * (D * 2));
+                }
+#pragma unroll
+                for (int h = 0; h < H; ++h)
+#pragma unroll
+                    for (int f = 0; f < NF; ++f) {
+                        const uint32_t cwh = cw[f][h];   // copy first: bit_cast straight from a vector element reads element 0
+                        const half2v c2 = __builtin_bit_cast(half2v, cwh);
+#pragma unroll
+                        for (int b = 0; b < NB; ++b)
+                            acc[f][b] = __builtin_amdgcn_fdot2(c2, __builtin_bit_cast(half2v, xr[b][s][t * H + h]), acc[f][b], false);
+                    }
+            }
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+#pragma unroll
+                for (int b = 0; b < NB; ++b) out[f][b] += live[s] ? acc[f][b] : 0.f;
+        }
+    }
+};
+
 template <int BITS, int D, int S, int NB, bool LDS_TAB>
 __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_kernel(GemvArgs a) {
-    constexpr int UD = unit_of<BITS>::UD;
-    constexpr int TPU = UD * 32 / BITS;      // tags per unit
-    constexpr int XH = TPU * D / 2;          // fp16 pairs of activation per slot
-    constexpr int H = D / 2;                 // fp16 pairs per codeword
-    typedef typename cw_t<D>::type CW;
+    typedef GemvBody<BITS, D, S, NB, LDS_TAB> K;
+    constexpr int UD = K::UD, XH = K::XH, PF = GEMV_PF;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     int pi = 0;
@@ -107,13 +211,13 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_kernel(Ge
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int TS = a.TS;
     const int wpr = TS > 64 ? TS >> 6 : 1;             // waves per row
-    const int rpw = TS < 64 ? 64 / TS : 1;             // rows per wave
+    const int span = TS < 64 ? TS : 64;                // lanes of one wave that share a row
     const int tl = TS > 64 ? (wave % wpr) * 64 + lane : lane & (TS - 1);
-    const int grp = TS > 64 ? wave / wpr : wave * rpw + lane / TS;   // row group of this lane
-    const int ngrp = TS > 64 ? nwaves / wpr : nwaves * rpw;
+    const int grp = TS > 64 ? wave / wpr : wave * (64 / TS) + lane / TS;   // team of this lane
+    const int ngrp = TS > 64 ? nwaves / wpr : nwaves * (64 / TS);
+    const bool writer = (lane & (span - 1)) == span - 1;                   // holds the team sum after team_sum()
 
-    // ---- codebook into LDS
-    float* part = reinterpret_cast<float*>(smem + a.table_bytes);      // [GEMV_PF * ngrp rows][wpr][NB] per-wave partial sums
+    float* part = reinterpret_cast<float*>(smem + a.table_bytes);          // [ngrp][PF][wpr][NB] per-wave partial sums
     if (LDS_TAB) {
         const u32x4* src = reinterpret_cast<const u32x4*>(m.table);
         u32x4* dst = reinterpret_cast<u32x4*>(smem);
@@ -121,181 +225,340 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_kernel(Ge
         __syncthreads();
     }
 
-    // ---- rows of this workgroup: positions [p0, p1) of row_order
+    // rows of this workgroup: positions [p0, p1) of row_order, a contiguous share per team
     const int wg = blockIdx.x - P.wg_begin;
     const int p0 = (int)((int64_t)m.R * wg / P.wg_count), p1 = (int)((int64_t)m.R * (wg + 1) / P.wg_count);
+    const int rpt = (p1 - p0 + ngrp - 1) / ngrp;                           // rows per team
+    const int q0 = p0 + grp * rpt, q1 = q0 + rpt < p1 ? q0 + rpt : p1;
+    const int nbatch = (rpt + PF - 1) / PF;                                // same trip count for every team
 
-    uint32_t xr[NB][S][XH];
-    int cur_mask = -1;
     const uint32_t* tags = reinterpret_cast<const uint32_t*>(m.tags);
     const int nb = a.B - a.b0 < NB ? a.B - a.b0 : NB;
-
-    for (int pbase = p0; pbase < p1; pbase += ngrp * GEMV_PF) {
-        dwords<UD> tg[GEMV_PF][S];
-        int rows[GEMV_PF];
+    bool live[S];
 #pragma unroll
-        for (int f = 0; f < GEMV_PF; ++f) {
-            const int pos = pbase + f * ngrp + grp;
-            rows[f] = pos < p1 ? (m.row_order ? m.row_order[pos] : pos) : -1;
+    for (int s = 0; s < S; ++s) live[s] = tl + s * TS < P.U;
+    uint32_t xr[NB][S][XH];
+    int cur_mask = m.row_mask ? -1 : 0;
+    if (!m.row_mask) K::load_x(xr, a, P, 0, tl, nb);
+
+    // a batch: PF consecutive rows of this team, their tags, codebook offsets and column orders
+    struct Batch { dwords<UD> tg[PF][S]; int row[PF]; uint32_t boff[PF]; int order[PF]; };
+    Batch cur, nxt;
+    auto fetch = [&](int q, Batch& bt) {
+#pragma unroll
+        for (int f = 0; f < PF; ++f) {
+            const int pos = q + f;
+            const int r = pos < q1 ? (m.row_order ? m.row_order[pos] : pos) : -1;
+            bt.row[f] = r;
+            bt.boff[f] = (r >= 0 && m.row_book) ? (uint32_t)m.row_book[r] << BITS : 0u;
+            bt.order[f] = (r >= 0 && m.row_mask) ? (int)m.row_mask[r] : 0;
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 const int u = tl + s * TS;
-                if (rows[f] >= 0 && u < P.U) tg[f][s] = load_unit<UD>(tags + (int64_t)rows[f] * m.W + u * UD);
+                if (r >= 0 && u < P.U) bt.tg[f][s] = load_unit<UD>(tags + (int64_t)r * m.W + u * UD);
                 else {
 #pragma unroll
-                    for (int i = 0; i < UD; ++i) tg[f][s].v[i] = 0u;
+                    for (int i = 0; i < UD; ++i) bt.tg[f][s].v[i] = 0u;
                 }
             }
         }
+    };
+    fetch(q0, cur);
+
+    for (int it = 0; it < nbatch; ++it) {
+        if (it + 1 < nbatch) fetch(q0 + (it + 1) * PF, nxt);
+        float acc[PF][NB];
 #pragma unroll
-        for (int f = 0; f < GEMV_PF; ++f) {
-            const int r = rows[f];
-            const int rm = (r >= 0 && m.row_mask) ? m.row_mask[r] : 0;
-            if (r >= 0 && rm != cur_mask) {          // (re)load the activation registers
-                cur_mask = rm;
+        for (int f = 0; f < PF; ++f)
 #pragma unroll
-                for (int b = 0; b < NB; ++b)
+            for (int b = 0; b < NB; ++b) acc[f][b] = 0.f;
+        // One pass per distinct column order among the batch's rows: a single pass unless the batch
+        // straddles an order boundary (at most M - 1 such batches per team walk).
+        uint32_t pending = 0;
 #pragma unroll
-                    for (int s = 0; s < S; ++s) {
-                        const int u = tl + s * TS;
-                        const bool ok = b < nb && u < P.U;
-                        const int c0 = u * (TPU * D);
-                        if (P.xp) {
-                            const uint32_t* src = reinterpret_cast<const uint32_t*>(
-                                P.xp + ((int64_t)rm * a.B + a.b0 + b) * m.C + c0);
+        for (int f = 0; f < PF; ++f) pending |= (cur.row[f] >= 0 ? 1u : 0u) << f;
+        while (pending) {
+            if (m.row_mask) {
+                int want = cur_mask;
 #pragma unroll
-                            for (int i = 0; i < XH; ++i) xr[b][s][i] = ok ? src[i] : 0u;
-                        } else {
-                            const uint32_t* src = reinterpret_cast<const uint32_t*>(a.x + (int64_t)(a.b0 + b) * a.ldx + c0);
-#pragma unroll
-                            for (int i = 0; i < XH; ++i) {
-                                const uint32_t v = ok ? src[i] : 0u;
-                                xr[b][s][i] = a.x_dtype == SQ_BF16 ? bf2h_x2(v) : v;
-                            }
-                        }
-                    }
+                for (int f = PF - 1; f >= 0; --f)
+                    if (pending >> f & 1u) want = cur.order[f];                 // order of the first pending row
+                if (want != cur_mask) { cur_mask = want; K::load_x(xr, a, P, want, tl, nb); }
             }
-            float acc[NB];
+            float tmp[PF][NB];
+            K::template rows<PF>(tmp, cur.tg, cur.boff, xr, live, smem, reinterpret_cast<const unsigned char*>(m.table));
 #pragma unroll
-            for (int b = 0; b < NB; ++b) acc[b] = 0.f;
-            const uint32_t boff = (r >= 0 && m.row_book) ? (uint32_t)m.row_book[r] << BITS : 0u;
+            for (int f = 0; f < PF; ++f)
+                if ((pending >> f & 1u) && cur.order[f] == cur_mask) {
 #pragma unroll
-            for (int s = 0; s < S; ++s) {
-                float sl[NB];        // this slot's sum; dropped for lanes past the row's end so that
-#pragma unroll                       // codeword 0 (what their zero tags gather) never reaches the result
-                for (int b = 0; b < NB; ++b) sl[b] = 0.f;
-#pragma unroll
-                for (int t = 0; t < TPU; ++t) {
-                    const uint32_t tag = unit_tag<BITS, UD>(tg[f][s], t) + boff;
-                    CW cw;
-                    if (LDS_TAB) cw = *reinterpret_cast<const CW*>(smem + tag * (D * 2));
-                    else cw = *reinterpret_cast<const CW*>(reinterpret_cast<const unsigned char*>(m.table) + (size_t)tag * (D * 2));
-#pragma unroll
-                    for (int h = 0; h < H; ++h) {
-                        const uint32_t cwh = cw[h];      // copy first: bit_cast straight from a vector element reads element 0
-                        const half2v c2 = __builtin_bit_cast(half2v, cwh);
-#pragma unroll
-                        for (int b = 0; b < NB; ++b)
-                            sl[b] = __builtin_amdgcn_fdot2(c2, __builtin_bit_cast(half2v, xr[b][s][t * H + h]), sl[b], false);
-                    }
+                    for (int b = 0; b < NB; ++b) acc[f][b] = tmp[f][b];
+                    pending &= ~(1u << f);
                 }
-                const bool live = tl + s * TS < P.U;
+        }
 #pragma unroll
-                for (int b = 0; b < NB; ++b) acc[b] += live ? sl[b] : 0.f;
-            }
-            // ---- team sum
-            const int span = TS < 64 ? TS : 64;
+        for (int f = 0; f < PF; ++f)
 #pragma unroll
-            for (int b = 0; b < NB; ++b)
-                for (int o = span >> 1; o > 0; o >>= 1) acc[b] += __shfl_xor(acc[b], o, 64);
-            if (wpr == 1) {
-                if ((lane & (span - 1)) == 0 && r >= 0) {
+            for (int b = 0; b < NB; ++b) acc[f][b] = team_sum(acc[f][b], span);
+        if (wpr == 1) {
+            if (writer) {
+#pragma unroll
+                for (int f = 0; f < PF; ++f) {
+                    const int r = cur.row[f];
+                    if (r < 0) continue;
                     const float sc = h2f(m.row_scale[r]);
-                    for (int b = 0; b < nb; ++b) {
-                        const int64_t o = (int64_t)(a.b0 + b) * a.ldy + m.y_off + r;
-                        const float v = acc[b] * sc;
-                        if (a.y_dtype == SQ_BF16) reinterpret_cast<uint16_t*>(a.y)[o] = f2bf(v);
-                        else if (a.y_dtype == SQ_F16) reinterpret_cast<uint16_t*>(a.y)[o] = f2h(v);
-                        else reinterpret_cast<float*>(a.y)[o] = v;
-                    }
+                    for (int b = 0; b < nb; ++b)
+                        store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, acc[f][b] * sc);
                 }
-            } else if (lane == 0) {
-                // part[(f * ngrp + grp) * wpr + wave % wpr][b]
-#pragma unroll
-                for (int b = 0; b < NB; ++b) part[(((f * ngrp + grp) * wpr) + wave % wpr) * NB + b] = acc[b];
             }
-        }
-        if (wpr > 1) {
+        } else {
+            if (lane == 63) {
+#pragma unroll
+                for (int f = 0; f < PF; ++f)
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) part[((grp * PF + f) * wpr + wave % wpr) * NB + b] = acc[f][b];
+            }
             __syncthreads();
-            for (int i = tid; i < GEMV_PF * ngrp * nb; i += blockDim.x) {
-                const int b = i % nb, q = i / nb;              // q = f * ngrp + grp
-                const int pos = pbase + q;
-                if (pos < p1) {
+            for (int i = tid; i < ngrp * PF * nb; i += blockDim.x) {
+                const int b = i % nb, q = i / nb;                           // q = team * PF + f
+                const int g = q / PF, f = q - g * PF;
+                const int pos = p0 + g * rpt + it * PF + f;
+                const int pend = p0 + (g + 1) * rpt < p1 ? p0 + (g + 1) * rpt : p1;
+                if (pos < pend) {
                     const int r = m.row_order ? m.row_order[pos] : pos;
                     float v = 0.f;
                     for (int w = 0; w < wpr; ++w) v += part[(q * wpr + w) * NB + b];
-                    v *= h2f(m.row_scale[r]);
-                    const int64_t o = (int64_t)(a.b0 + b) * a.ldy + m.y_off + r;
-                    if (a.y_dtype == SQ_BF16) reinterpret_cast<uint16_t*>(a.y)[o] = f2bf(v);
-                    else if (a.y_dtype == SQ_F16) reinterpret_cast<uint16_t*>(a.y)[o] = f2h(v);
-                    else reinterpret_cast<float*>(a.y)[o] = v;
+                    store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, v * h2f(m.row_scale[r]));
                 }
             }
             __syncthreads();
+        }
+        cur = nxt;
+    }
+}
+
+// Rows as wide as a wave or wider (TS = 64 * waves-per-row): the row a wave works on is uniform, so the
+// row index, its base address, codebook offset and column order live in scalar registers and the inner
+// loop is branch-free: lanes past the row's end re-read the last unit (their activations are zero and
+// their sums are dropped), batches past the team's last row re-read it and skip the store.
+template <int BITS, int D, int S, int NB, bool LDS_TAB>
+__global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_wave_kernel(GemvArgs a) {
+    typedef GemvBody<BITS, D, S, NB, LDS_TAB> K;
+    constexpr int UD = K::UD, XH = K::XH, PF = GEMV_PF;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = blockDim.x >> 6;
+    int pi = 0;
+    while (pi + 1 < a.n && (int)blockIdx.x >= a.p[pi + 1].wg_begin) ++pi;
+    const GemvPiece& P = a.p[pi];
+    const sq_matrix& m = P.m;
+    const int TS = a.TS, wpr = TS >> 6;
+    const int team = wave / wpr, wcol = wave - team * wpr, nteams = nwaves / wpr;
+    const int tl = wcol * 64 + lane;
+
+    float* part = reinterpret_cast<float*>(smem + a.table_bytes);          // [nteams][PF][wpr][NB] per-wave partial sums
+    if (LDS_TAB) {
+        const u32x4* src = reinterpret_cast<const u32x4*>(m.table);
+        u32x4* dst = reinterpret_cast<u32x4*>(smem);
+        for (int i = tid; i < a.table_bytes / 16; i += blockDim.x) dst[i] = src[i];
+        __syncthreads();
+    }
+
+    const int wg = blockIdx.x - P.wg_begin;
+    const int p0 = (int)((int64_t)m.R * wg / P.wg_count), p1 = (int)((int64_t)m.R * (wg + 1) / P.wg_count);
+    const int rpt = (p1 - p0 + nteams - 1) / nteams;                       // rows per team
+    const int q0 = p0 + team * rpt, q1 = q0 + rpt < p1 ? q0 + rpt : p1;
+    const int nbatch = (rpt + PF - 1) / PF;                                // same trip count for every team
+    const bool has = q0 < q1;
+
+    const uint32_t* tags = reinterpret_cast<const uint32_t*>(m.tags);
+    const unsigned char* table = reinterpret_cast<const unsigned char*>(m.table);
+    const int nb = a.B - a.b0 < NB ? a.B - a.b0 : NB;
+    bool live[S];
+    uint32_t uoff[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const int u = tl + s * TS;
+        live[s] = u < P.U;
+        uoff[s] = (uint32_t)(live[s] ? u : P.U - 1) * UD;
+    }
+    uint32_t xr[NB][S][XH];
+    int cur_order = m.row_mask ? -1 : 0;
+    if (!m.row_mask) K::load_x(xr, a, P, 0, tl, nb);
+
+    // tags of PF consecutive rows starting at position q (positions past the team's end repeat its last row)
+    auto fetch = [&](int q, dwords<UD> (&t)[PF][S], int (&row)[PF]) {
+#pragma unroll
+        for (int f = 0; f < PF; ++f) {
+            const int pos = q + f < q1 ? q + f : q1 - 1;
+            const int r = m.row_order ? m.row_order[pos] : pos;
+            row[f] = r;
+            const uint32_t* rp = tags + (size_t)r * m.W;
+#pragma unroll
+            for (int s = 0; s < S; ++s) t[f][s] = load_unit<UD>(rp + uoff[s]);
+        }
+    };
+
+    auto process = [&](int it, const dwords<UD> (&t)[PF][S], const int (&row)[PF]) {
+        float acc[PF][NB];
+        if (has) {
+            uint32_t boff[PF];
+#pragma unroll
+            for (int f = 0; f < PF; ++f) boff[f] = m.row_book ? (uint32_t)m.row_book[row[f]] << BITS : 0u;
+            bool same = true;
+            if (m.row_mask) {
+#pragma unroll
+                for (int f = 0; f < PF; ++f) same = same && (int)m.row_mask[row[f]] == cur_order;
+            }
+            if (same) {
+                K::template rows<PF>(acc, t, boff, xr, live, smem, table);
+            } else {
+                // the column order changes inside this batch (at most M - 1 times per team): row by row
+#pragma unroll
+                for (int f = 0; f < PF; ++f) {
+                    const int ord = m.row_mask[row[f]];
+                    if (ord != cur_order) { cur_order = ord; K::load_x(xr, a, P, ord, tl, nb); }
+                    float a1[1][NB];
+                    const dwords<UD> (&t1)[1][S] = reinterpret_cast<const dwords<UD> (&)[1][S]>(t[f]);
+                    const uint32_t b1[1] = {boff[f]};
+                    K::template rows<1>(a1, t1, b1, xr, live, smem, table);
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) acc[f][b] = a1[0][b];
+                }
+            }
+#pragma unroll
+            for (int f = 0; f < PF; ++f)
+#pragma unroll
+                for (int b = 0; b < NB; ++b) acc[f][b] = team_sum(acc[f][b], 64);
+        }
+        const int qb = q0 + it * PF;
+        if (wpr == 1) {
+            if (has && lane == 63) {
+#pragma unroll
+                for (int f = 0; f < PF; ++f) {
+                    if (qb + f >= q1) continue;
+                    const int r = row[f];
+                    const float sc = h2f(m.row_scale[r]);
+                    for (int b = 0; b < nb; ++b)
+                        store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, acc[f][b] * sc);
+                }
+            }
+        } else {
+            if (has && lane == 63) {
+#pragma unroll
+                for (int f = 0; f < PF; ++f)
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) part[((team * PF + f) * wpr + wcol) * NB + b] = acc[f][b];
+            }
+            __syncthreads();
+            for (int i = tid; i < nteams * PF * nb; i += blockDim.x) {
+                const int b = i % nb, q = i / nb;                           // q = team * PF + f
+                const int g = q / PF, f = q - g * PF;
+                const int pos = p0 + g * rpt + it * PF + f;
+                const int pend = p0 + (g + 1) * rpt < p1 ? p0 + (g + 1) * rpt : p1;
+                if (pos < pend) {
+                    const int r = m.row_order ? m.row_order[pos] : pos;
+                    float v = 0.f;
+                    for (int w = 0; w < wpr; ++w) v += part[(q * wpr + w) * NB + b];
+                    store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, v * h2f(m.row_scale[r]));
+                }
+            }
+            __syncthreads();
+        }
+    };
+
+    dwords<UD> tA[PF][S], tB[PF][S];
+    int rA[PF], rB[PF];
+    if (has) fetch(q0, tA, rA);
+    for (int it = 0; it < nbatch; it += 2) {                               // two batches per trip: A computes while B loads
+        if (has && it + 1 < nbatch) fetch(q0 + (it + 1) * PF, tB, rB);
+        process(it, tA, rA);
+        if (it + 1 < nbatch) {
+            if (has && it + 2 < nbatch) fetch(q0 + (it + 2) * PF, tA, rA);
+            process(it + 1, tB, rB);
         }
     }
 }
 
+// Workgroups of `threads` threads and `smem` bytes of LDS that fit on one CU (from the runtime's occupancy
+// calculator, i.e. from the registers the compiler really used); cached per instantiation.
+template <int BITS, int D, int S, int NB, bool LDS_TAB, bool WAVE>
+static inline int occupancy_of(int threads, size_t smem) {
+    static std::mutex mu;
+    static std::unordered_map<uint64_t, int> cache;
+    const uint64_t key = ((uint64_t)threads << 32) | (uint64_t)smem;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = cache.find(key);
+    if (it != cache.end()) return it->second;
+    void (*k)(GemvArgs) = WAVE ? gemv_wave_kernel<BITS, D, S, NB, LDS_TAB> : gemv_kernel<BITS, D, S, NB, LDS_TAB>;
+    if (smem > 64 * 1024) {      // allow the 160 KB of a gfx950 CU
+        (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipGetLastError();
+    }
+    // from the registers the compiler used: 512 VGPRs per SIMD lane in granules of 8, at most 8 waves per SIMD
+    hipFuncAttributes fa;
+    int n = 1;
+    if (hipFuncGetAttributes(&fa, (const void*)k) == hipSuccess && fa.numRegs > 0) {
+        int wps = 512 / ((fa.numRegs + 7) / 8 * 8);
+        if (wps > 8) wps = 8;
+        n = 4 * wps / (threads / 64);
+    } else {
+        (void)hipGetLastError();
+    }
+    if (smem && (size_t)n * smem > 160 * 1024) n = (int)(160 * 1024 / smem);
+    if (n < 1) n = 1;
+    cache[key] = n;
+    return n;
+}
+
+// op 0: launch; op 1: return the occupancy (workgroups per CU) for (threads, smem)
 template <int BITS, int D, int S, int NB>
-static inline int launch_inst(const GemvArgs& a, int grid, int threads, size_t smem, hipStream_t s) {
+static inline int launch_inst(int op, const GemvArgs& a, int grid, int threads, size_t smem, hipStream_t s) {
     if constexpr (!gemv_cfg<BITS, D, S, NB>::OK) {
         return fail(SQ_EUNSUPPORTED, "sq_linear_small: no kernel for bits %d d %d slots %d rows %d", BITS, D, S, NB);
     } else {
         if (threads > gemv_cfg<BITS, D, S, NB>::LB)
             return fail(SQ_ELAUNCH, "sq_linear_small: %d threads > %d", threads, gemv_cfg<BITS, D, S, NB>::LB);
-        if (a.table_bytes) {
-            auto k = gemv_kernel<BITS, D, S, NB, true>;
-            if (smem > 64 * 1024) {
-                static bool raised = false;
-                if (!raised) {
-                    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-                    (void)hipGetLastError();
-                    raised = true;
-                }
-            }
-            hipLaunchKernelGGL(k, dim3(grid), dim3(threads), smem, s, a);
-        } else {
-            hipLaunchKernelGGL((gemv_kernel<BITS, D, S, NB, false>), dim3(grid), dim3(threads), smem, s, a);
+        const bool wave = a.TS >= 64;
+        if (op == 1) {
+            if (wave) return a.table_bytes ? occupancy_of<BITS, D, S, NB, true, true>(threads, smem)
+                                           : occupancy_of<BITS, D, S, NB, false, true>(threads, smem);
+            return a.table_bytes ? occupancy_of<BITS, D, S, NB, true, false>(threads, smem)
+                                 : occupancy_of<BITS, D, S, NB, false, false>(threads, smem);
         }
+        void (*k)(GemvArgs);
+        if (wave) k = a.table_bytes ? gemv_wave_kernel<BITS, D, S, NB, true> : gemv_wave_kernel<BITS, D, S, NB, false>;
+        else k = a.table_bytes ? gemv_kernel<BITS, D, S, NB, true> : gemv_kernel<BITS, D, S, NB, false>;
+        hipLaunchKernelGGL(k, dim3(grid), dim3(threads), smem, s, a);
         return check_launch("sq_linear_small");
     }
 }
 
 template <int BITS, int D, int S>
-static inline int launch_nb(const GemvArgs& a, int nbt, int grid, int threads, size_t smem, hipStream_t s) {
+static inline int launch_nb(int op, const GemvArgs& a, int nbt, int grid, int threads, size_t smem, hipStream_t s) {
     switch (nbt) {
-        case 1: return launch_inst<BITS, D, S, 1>(a, grid, threads, smem, s);
-        case 2: return launch_inst<BITS, D, S, 2>(a, grid, threads, smem, s);
-        default: return launch_inst<BITS, D, S, 4>(a, grid, threads, smem, s);
+        case 1: return launch_inst<BITS, D, S, 1>(op, a, grid, threads, smem, s);
+        case 2: return launch_inst<BITS, D, S, 2>(op, a, grid, threads, smem, s);
+        default: return launch_inst<BITS, D, S, 4>(op, a, grid, threads, smem, s);
     }
 }
 
 template <int BITS, int D>
-static inline int launch_s(const GemvArgs& a, int S, int nbt, int grid, int threads, size_t smem, hipStream_t s) {
+static inline int launch_s(int op, const GemvArgs& a, int S, int nbt, int grid, int threads, size_t smem, hipStream_t s) {
     switch (S) {
-        case 1: return launch_nb<BITS, D, 1>(a, nbt, grid, threads, smem, s);
-        case 2: return launch_nb<BITS, D, 2>(a, nbt, grid, threads, smem, s);
-        case 3: return launch_nb<BITS, D, 3>(a, nbt, grid, threads, smem, s);
-        case 5: return launch_nb<BITS, D, 5>(a, nbt, grid, threads, smem, s);
+        case 1: return launch_nb<BITS, D, 1>(op, a, nbt, grid, threads, smem, s);
+        case 2: return launch_nb<BITS, D, 2>(op, a, nbt, grid, threads, smem, s);
+        case 3: return launch_nb<BITS, D, 3>(op, a, nbt, grid, threads, smem, s);
+        case 5: return launch_nb<BITS, D, 5>(op, a, nbt, grid, threads, smem, s);
     }
     return fail(SQ_EUNSUPPORTED, "sq_linear_small: slots %d", S);
 }
 
 // One translation unit per tag format instantiates its kernels behind a plain function.
-#define SQ_GEMV_FORMAT(BI, DD)                                                                              \
-    int launch_gemv_b##BI##d##DD(const GemvArgs& a, int S, int nbt, int grid, int threads, size_t smem,   \
-                                 hipStream_t s) {                                                          \
-        return launch_s<BI, DD>(a, S, nbt, grid, threads, smem, s);                                        \
+#define SQ_GEMV_FORMAT(BI, DD)                                                                                  \
+    int launch_gemv_b##BI##d##DD(int op, const GemvArgs& a, int S, int nbt, int grid, int threads, size_t smem, \
+                                 hipStream_t s) {                                                              \
+        return launch_s<BI, DD>(op, a, S, nbt, grid, threads, smem, s);                                        \
     }
 
 }  // namespace sq
