@@ -120,6 +120,26 @@ __device__ __forceinline__ void store_y(void* y, int y_dtype, int64_t o, float v
     else reinterpret_cast<float*>(y)[o] = v;
 }
 
+// Codebook into LDS, eight 16-byte loads in flight per thread before the first store.
+__device__ __forceinline__ void stage_table(const uint16_t* table, int bytes, unsigned char* smem) {
+    const u32x4* src = reinterpret_cast<const u32x4*>(table);
+    u32x4* dst = reinterpret_cast<u32x4*>(smem);
+    const int n = bytes / 16, tid = threadIdx.x, step = blockDim.x;
+    for (int i0 = tid; i0 < n; i0 += 8 * step) {
+        u32x4 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = i0 + k * step;
+            v[k] = src[i < n ? i : n - 1];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = i0 + k * step;
+            if (i < n) dst[i] = v[k];
+        }
+    }
+}
+
 template <int BITS, int D, int S, int NB, bool LDS_TAB>
 struct GemvBody {
     static constexpr int UD = unit_of<BITS>::UD;
@@ -135,18 +155,24 @@ struct GemvBody {
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int s = 0; s < S; ++s) {
+                // lanes past the row's end and activation rows past B load a valid address and keep zeros:
+                // no branch around the loads, so they all issue back to back
                 const int u = tl + s * a.TS;
                 const bool ok = b < nb && u < P.U;
-                const int c0 = u * (TPU * D);
-                const uint16_t* src = P.xp ? P.xp + ((int64_t)rm * a.B + a.b0 + b) * P.m.C + c0
-                                           : a.x + (int64_t)(a.b0 + b) * a.ldx + c0;
+                const int c0 = (u < P.U ? u : P.U - 1) * (TPU * D);
+                const int bb = a.b0 + (b < nb ? b : nb - 1);
+                const uint16_t* src = P.xp ? P.xp + ((int64_t)rm * a.B + bb) * P.m.C + c0
+                                           : a.x + (int64_t)bb * a.ldx + c0;
                 const bool cvt = !P.xp && a.x_dtype == SQ_BF16;
+                u32x4 v[XH / 4];
 #pragma unroll
-                for (int i = 0; i < XH; i += 4) {
-                    u32x4 v = {0u, 0u, 0u, 0u};
-                    if (ok) v = *reinterpret_cast<const u32x4*>(src + 2 * i);
-                    if (cvt) { v.x = bf2h_x2(v.x); v.y = bf2h_x2(v.y); v.z = bf2h_x2(v.z); v.w = bf2h_x2(v.w); }
-                    xr[b][s][i] = v.x; xr[b][s][i + 1] = v.y; xr[b][s][i + 2] = v.z; xr[b][s][i + 3] = v.w;
+                for (int i = 0; i < XH / 4; ++i) v[i] = *reinterpret_cast<const u32x4*>(src + 8 * i);
+#pragma unroll
+                for (int i = 0; i < XH / 4; ++i) {
+                    u32x4 w = v[i];
+                    if (cvt) { w.x = bf2h_x2(w.x); w.y = bf2h_x2(w.y); w.z = bf2h_x2(w.z); w.w = bf2h_x2(w.w); }
+                    xr[b][s][4 * i] = ok ? w.x : 0u; xr[b][s][4 * i + 1] = ok ? w.y : 0u;
+                    xr[b][s][4 * i + 2] = ok ? w.z : 0u; xr[b][s][4 * i + 3] = ok ? w.w : 0u;
                 }
             }
     }
@@ -219,9 +245,7 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_kernel(Ge
 
     float* part = reinterpret_cast<float*>(smem + a.table_bytes);          // [ngrp][PF][wpr][NB] per-wave partial sums
     if (LDS_TAB) {
-        const u32x4* src = reinterpret_cast<const u32x4*>(m.table);
-        u32x4* dst = reinterpret_cast<u32x4*>(smem);
-        for (int i = tid; i < a.table_bytes / 16; i += blockDim.x) dst[i] = src[i];
+        stage_table(m.table, a.table_bytes, smem);
         __syncthreads();
     }
 
@@ -242,7 +266,8 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_kernel(Ge
     if (!m.row_mask) K::load_x(xr, a, P, 0, tl, nb);
 
     // a batch: PF consecutive rows of this team, their tags, codebook offsets and column orders
-    struct Batch { dwords<UD> tg[PF][S]; int row[PF]; uint32_t boff[PF]; int order[PF]; };
+    // (everything a batch needs from memory is loaded here, so nothing waits behind the next batch's prefetch)
+    struct Batch { dwords<UD> tg[PF][S]; int row[PF]; uint32_t boff[PF]; int order[PF]; float scale[PF]; };
     Batch cur, nxt;
     auto fetch = [&](int q, Batch& bt) {
 #pragma unroll
@@ -252,6 +277,7 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_kernel(Ge
             bt.row[f] = r;
             bt.boff[f] = (r >= 0 && m.row_book) ? (uint32_t)m.row_book[r] << BITS : 0u;
             bt.order[f] = (r >= 0 && m.row_mask) ? (int)m.row_mask[r] : 0;
+            bt.scale[f] = r >= 0 ? h2f(m.row_scale[r]) : 0.f;
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 const int u = tl + s * TS;
@@ -305,7 +331,7 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_kernel(Ge
                 for (int f = 0; f < PF; ++f) {
                     const int r = cur.row[f];
                     if (r < 0) continue;
-                    const float sc = h2f(m.row_scale[r]);
+                    const float sc = cur.scale[f];
                     for (int b = 0; b < nb; ++b)
                         store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, acc[f][b] * sc);
                 }
@@ -357,12 +383,6 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_wave_kern
     const int tl = wcol * 64 + lane;
 
     float* part = reinterpret_cast<float*>(smem + a.table_bytes);          // [nteams][PF][wpr][NB] per-wave partial sums
-    if (LDS_TAB) {
-        const u32x4* src = reinterpret_cast<const u32x4*>(m.table);
-        u32x4* dst = reinterpret_cast<u32x4*>(smem);
-        for (int i = tid; i < a.table_bytes / 16; i += blockDim.x) dst[i] = src[i];
-        __syncthreads();
-    }
 
     const int wg = blockIdx.x - P.wg_begin;
     const int p0 = (int)((int64_t)m.R * wg / P.wg_count), p1 = (int)((int64_t)m.R * (wg + 1) / P.wg_count);
@@ -386,41 +406,54 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_wave_kern
     int cur_order = m.row_mask ? -1 : 0;
     if (!m.row_mask) K::load_x(xr, a, P, 0, tl, nb);
 
-    // tags of PF consecutive rows starting at position q (positions past the team's end repeat its last row)
-    auto fetch = [&](int q, dwords<UD> (&t)[PF][S], int (&row)[PF]) {
+    // Row metadata (row id, scale, codebook offset, column order) of 64 consecutive positions is held one
+    // position per lane and handed out with v_readlane, so the batch loop issues no global load besides the
+    // tag stream and never waits behind its own prefetch.  Positions past the team's end repeat its last row.
+    int cb = q0, mrow = 0, mord = 0;
+    float mscale = 0.f;
+    uint32_t mboff = 0u;
+    auto refill = [&](int base) {
+        cb = base;
+        const int pos = base + lane < q1 ? base + lane : q1 - 1;
+        mrow = m.row_order ? m.row_order[pos] : pos;
+        mscale = h2f(m.row_scale[mrow]);
+        mboff = m.row_book ? (uint32_t)m.row_book[mrow] << BITS : 0u;
+        mord = m.row_mask ? (int)m.row_mask[mrow] : 0;
+    };
+    struct Batch { dwords<UD> t[PF][S]; int row[PF]; float scale[PF]; uint32_t boff[PF]; int order[PF]; };
+    auto fetch = [&](int q, Batch& B) {
+        if (q + PF > cb + 64) refill(q);
 #pragma unroll
         for (int f = 0; f < PF; ++f) {
             const int pos = q + f < q1 ? q + f : q1 - 1;
-            const int r = m.row_order ? m.row_order[pos] : pos;
-            row[f] = r;
+            const int j = pos - cb;
+            const int r = __builtin_amdgcn_readlane(mrow, j);
+            B.row[f] = r;
+            B.scale[f] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mscale), j));
+            B.boff[f] = (uint32_t)__builtin_amdgcn_readlane((int)mboff, j);
+            B.order[f] = __builtin_amdgcn_readlane(mord, j);
             const uint32_t* rp = tags + (size_t)r * m.W;
 #pragma unroll
-            for (int s = 0; s < S; ++s) t[f][s] = load_unit<UD>(rp + uoff[s]);
+            for (int s = 0; s < S; ++s) B.t[f][s] = load_unit<UD>(rp + uoff[s]);
         }
     };
 
-    auto process = [&](int it, const dwords<UD> (&t)[PF][S], const int (&row)[PF]) {
+    auto process = [&](int it, const Batch& B) {
         float acc[PF][NB];
         if (has) {
-            uint32_t boff[PF];
-#pragma unroll
-            for (int f = 0; f < PF; ++f) boff[f] = m.row_book ? (uint32_t)m.row_book[row[f]] << BITS : 0u;
             bool same = true;
-            if (m.row_mask) {
 #pragma unroll
-                for (int f = 0; f < PF; ++f) same = same && (int)m.row_mask[row[f]] == cur_order;
-            }
+            for (int f = 0; f < PF; ++f) same = same && B.order[f] == cur_order;
             if (same) {
-                K::template rows<PF>(acc, t, boff, xr, live, smem, table);
+                K::template rows<PF>(acc, B.t, B.boff, xr, live, smem, table);
             } else {
                 // the column order changes inside this batch (at most M - 1 times per team): row by row
 #pragma unroll
                 for (int f = 0; f < PF; ++f) {
-                    const int ord = m.row_mask[row[f]];
-                    if (ord != cur_order) { cur_order = ord; K::load_x(xr, a, P, ord, tl, nb); }
+                    if (B.order[f] != cur_order) { cur_order = B.order[f]; K::load_x(xr, a, P, cur_order, tl, nb); }
                     float a1[1][NB];
-                    const dwords<UD> (&t1)[1][S] = reinterpret_cast<const dwords<UD> (&)[1][S]>(t[f]);
-                    const uint32_t b1[1] = {boff[f]};
+                    const dwords<UD> (&t1)[1][S] = reinterpret_cast<const dwords<UD> (&)[1][S]>(B.t[f]);
+                    const uint32_t b1[1] = {B.boff[f]};
                     K::template rows<1>(a1, t1, b1, xr, live, smem, table);
 #pragma unroll
                     for (int b = 0; b < NB; ++b) acc[f][b] = a1[0][b];
@@ -437,10 +470,8 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_wave_kern
 #pragma unroll
                 for (int f = 0; f < PF; ++f) {
                     if (qb + f >= q1) continue;
-                    const int r = row[f];
-                    const float sc = h2f(m.row_scale[r]);
                     for (int b = 0; b < nb; ++b)
-                        store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, acc[f][b] * sc);
+                        store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + B.row[f], acc[f][b] * B.scale[f]);
                 }
             }
         } else {
@@ -451,31 +482,37 @@ __global__ __launch_bounds__((gemv_cfg<BITS, D, S, NB>::LB)) void gemv_wave_kern
                     for (int b = 0; b < NB; ++b) part[((team * PF + f) * wpr + wcol) * NB + b] = acc[f][b];
             }
             __syncthreads();
-            for (int i = tid; i < nteams * PF * nb; i += blockDim.x) {
-                const int b = i % nb, q = i / nb;                           // q = team * PF + f
-                const int g = q / PF, f = q - g * PF;
-                const int pos = p0 + g * rpt + it * PF + f;
-                const int pend = p0 + (g + 1) * rpt < p1 ? p0 + (g + 1) * rpt : p1;
-                if (pos < pend) {
-                    const int r = m.row_order ? m.row_order[pos] : pos;
+            // the first wave of each team adds the team's per-wave partials (lane = f * NB + b)
+            if (has && wcol == 0 && lane < PF * NB) {
+                const int f = lane / NB, b = lane - f * NB;
+                if (qb + f < q1 && b < nb) {
                     float v = 0.f;
-                    for (int w = 0; w < wpr; ++w) v += part[(q * wpr + w) * NB + b];
-                    store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, v * h2f(m.row_scale[r]));
+                    for (int w = 0; w < wpr; ++w) v += part[((team * PF + f) * wpr + w) * NB + b];
+                    int r = B.row[0];
+                    float sc = B.scale[0];
+#pragma unroll
+                    for (int g = 1; g < PF; ++g)
+                        if (f == g) { r = B.row[g]; sc = B.scale[g]; }
+                    store_y(a.y, a.y_dtype, (int64_t)(a.b0 + b) * a.ldy + m.y_off + r, v * sc);
                 }
             }
             __syncthreads();
         }
     };
 
-    dwords<UD> tA[PF][S], tB[PF][S];
-    int rA[PF], rB[PF];
-    if (has) fetch(q0, tA, rA);
+    // start-up: metadata, activations and codebook are requested together and the first tag fetch follows
+    // as soon as the row ids are known, so the kernel pays two memory latencies before its first product
+    Batch bA, bB;
+    if (has) refill(q0);
+    if (LDS_TAB) stage_table(m.table, a.table_bytes, smem);
+    if (has) fetch(q0, bA);
+    if (LDS_TAB) __syncthreads();
     for (int it = 0; it < nbatch; it += 2) {                               // two batches per trip: A computes while B loads
-        if (has && it + 1 < nbatch) fetch(q0 + (it + 1) * PF, tB, rB);
-        process(it, tA, rA);
+        if (has && it + 1 < nbatch) fetch(q0 + (it + 1) * PF, bB);
+        process(it, bA);
         if (it + 1 < nbatch) {
-            if (has && it + 2 < nbatch) fetch(q0 + (it + 2) * PF, tA, rA);
-            process(it + 1, tB, rB);
+            if (has && it + 2 < nbatch) fetch(q0 + (it + 2) * PF, bA);
+            process(it + 1, bB);
         }
     }
 }
