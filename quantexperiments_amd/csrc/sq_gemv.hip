@@ -1,6 +1,6 @@
 // Host side of the decode-time product: picks the team geometry per shape, fuses stacked pieces
 // into one persistent launch, prepares permuted activations for pieces with column orders.
-#include "sq_gemv_kernel.h"
+#include "sq_rows_mfma.h"
 
 namespace sq {
 
@@ -8,6 +8,21 @@ int launch_gemv_b16d8(int, const GemvArgs&, int, int, int, int, size_t, hipStrea
 int launch_gemv_b12d4(int, const GemvArgs&, int, int, int, int, size_t, hipStream_t);
 int launch_gemv_b10d4(int, const GemvArgs&, int, int, int, int, size_t, hipStream_t);
 int launch_gemv_b8d4(int, const GemvArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_mma_b16d8(int, const MmaArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_mma_b12d4(int, const MmaArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_mma_b10d4(int, const MmaArgs&, int, int, int, int, size_t, hipStream_t);
+int launch_mma_b8d4(int, const MmaArgs&, int, int, int, int, size_t, hipStream_t);
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int ks, int B, int R,
+                                                            const uint16_t* __restrict__ row_scale, void* y, int64_t ldy,
+                                                            int y_off, int y_dtype) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= B * R) return;
+    const int b = i / R, r = i - b * R;
+    float v = 0.f;
+    for (int s = 0; s < ks; ++s) v += part[((int64_t)s * B + b) * R + r];
+    store_y(y, y_dtype, (int64_t)b * ldy + y_off + r, v * h2f(row_scale[r]));
+}
 
 // xp[m, b, c] = fp16(x[b, perms[m, c]])
 __global__ __launch_bounds__(256) void permute_x_kernel(const uint16_t* __restrict__ x, int64_t ldx, int x_dtype,
@@ -74,11 +89,102 @@ static Plan plan_for(int U, int bits, int d) {
     return best;
 }
 
+// ---- matrix-core path (pieces without column orders)
+struct MmaPlan { int RW, NT, KW, ks; };
+
+static bool mma_shape(const sq_matrix& m) { return fast_shape(m) && !m.perms; }
+
+// Rounds per wave, waves per workgroup and workgroup-level column slices that cover ceil(U / 4) rounds
+// with the fewest idle rounds (ties: more rounds per wave, i.e. fewer waves to add up).
+static MmaPlan mma_plan(const sq_matrix& m, int B) {
+    const int ud = unit_dwords(m.bits), tpu = ud * 32 / m.bits, spu = tpu / (8 / m.d);
+    const int rounds = (m.W / ud + 3) / 4, r1 = 32 / spu;
+    MmaPlan best{0, 0, 0, 0};
+    double best_cost = 1e30;
+    const int NT = B > 16 ? 2 : 1;
+    for (int rw = NT == 1 ? r1 : r1 / 2; rw >= 1 && rw >= r1 / 4; rw /= 2) {
+        const int need = (rounds + rw - 1) / rw;
+        const int ks = (need + 7) / 8, kw = (need + ks - 1) / ks;
+        const double cost = (double)rw * kw * ks / rounds + 0.03 * (ks - 1) + 0.002 * kw;
+        if (cost < best_cost - 1e-9) { best_cost = cost; best = MmaPlan{rw, NT, kw, ks}; }
+    }
+    return best;
+}
+
+static size_t mma_part_bytes(const sq_matrix& m, int B) {
+    const MmaPlan pl = mma_plan(m, B);
+    return pl.ks > 1 ? ((((size_t)pl.ks * B * m.R * 4) + 255) & ~(size_t)255) : 0;
+}
+
 size_t small_workspace(const sq_matrix* mats, int n, int B) {
     size_t tot = 0;
-    for (int i = 0; i < n; ++i)
-        if (mats[i].perms && fast_shape(mats[i])) tot += xp_bytes(mats[i], B);
+    for (int i = 0; i < n; ++i) {
+        if (mma_shape(mats[i])) tot += mma_part_bytes(mats[i], B);
+        else if (mats[i].perms && fast_shape(mats[i])) tot += xp_bytes(mats[i], B);
+    }
     return tot;
+}
+
+// Pieces [0, cnt) share format and row length: one persistent launch (+ one reduction per piece if ks > 1).
+static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                            int64_t ldy, int B, char* ws, size_t& ws_off, int cus, hipStream_t s) {
+    const sq_matrix& m0 = mats[0];
+    const MmaPlan pl = mma_plan(m0, B);
+    MmaArgs a;
+    a.n = cnt;
+    a.x = (const uint16_t*)x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.B = B; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+    a.U = m0.W / unit_dwords(m0.bits);
+    a.ks = pl.ks;
+    const size_t tab0 = (size_t)m0.G * ((size_t)1 << m0.bits) * m0.d * 2;
+    a.table_bytes = tab0 <= 128 * 1024 ? (int)tab0 : 0;
+    const int threads = pl.KW * 64;
+    const size_t smem = (size_t)a.table_bytes + 16 + (pl.KW > 1 ? (size_t)MMA_TT * pl.KW * 64 * pl.NT * 16 : 0);
+    int rc = SQ_EUNSUPPORTED;
+#define SQ_CASE(BI, DD) if (m0.bits == BI && m0.d == DD) rc = launch_mma_b##BI##d##DD(OP, a, pl.RW, pl.NT, GRID, threads, smem, s)
+#define OP 1
+#define GRID 0
+    SQ_CASE(16, 8); SQ_CASE(12, 4); SQ_CASE(10, 4); SQ_CASE(8, 4);
+#undef OP
+#undef GRID
+    if (rc < 1) return rc < 0 ? rc : fail(SQ_ELAUNCH, "sq_linear_small: kernel does not fit a CU");
+    const int slots = cus * rc;                                  // workgroups resident at once
+    int64_t rows_total = 0;
+    for (int k = 0; k < cnt; ++k) rows_total += mats[k].R;
+    int wg = 0;
+    for (int k = 0; k < cnt; ++k) {
+        MmaPiece& P = a.p[k];
+        P.m = mats[k];
+        P.part = nullptr;
+        if (pl.ks > 1) {
+            P.part = (float*)(ws + ws_off);
+            ws_off += mma_part_bytes(mats[k], B);
+        }
+        const int ntiles = (mats[k].R + 15) / 16;
+        int nshare = (int)((mats[k].R * (int64_t)slots / rows_total) / pl.ks);
+        if (nshare > ntiles) nshare = ntiles;
+        if (nshare < 1) nshare = 1;
+        P.wg_begin = wg;
+        P.wg_count = nshare * pl.ks;
+        wg += P.wg_count;
+    }
+    for (int k = cnt; k < GEMV_MAX_PIECES; ++k) a.p[k] = a.p[0];
+#define OP 0
+#define GRID wg
+    rc = SQ_EUNSUPPORTED;
+    SQ_CASE(16, 8); SQ_CASE(12, 4); SQ_CASE(10, 4); SQ_CASE(8, 4);
+#undef OP
+#undef GRID
+#undef SQ_CASE
+    if (rc) return rc;
+    if (pl.ks > 1)
+        for (int k = 0; k < cnt; ++k) {
+            const sq_matrix& mk = mats[k];
+            hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((B * mk.R + 255) / 256)), dim3(256), 0, s,
+                               a.p[k].part, pl.ks, B, mk.R, mk.row_scale, y, ldy, mk.y_off, y_dtype);
+            rc = check_launch("sq_linear_small(splitk_reduce)");
+            if (rc) return rc;
+        }
+    return SQ_OK;
 }
 
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
@@ -93,11 +199,22 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         const sq_matrix& m0 = mats[i];
         if (m0.R == 0) { ++i; continue; }
         const int ud = unit_dwords(m0.bits);
+        if (mma_shape(m0) && x_ok) {
+            int j = i + 1;
+            while (j < n && j - i < GEMV_MAX_PIECES && mma_shape(mats[j]) && mats[j].bits == m0.bits && mats[j].d == m0.d &&
+                   mats[j].W == m0.W && mats[j].G == m0.G && mats[j].R > 0)
+                ++j;
+            int rc = launch_mma_group(mats + i, j - i, x, x_dtype, ldx, y, y_dtype, ldy, B, (char*)ws, ws_off, cus, s);
+            if (rc) return rc;
+            i = j;
+            continue;
+        }
         const Plan pl = (fast_shape(m0) && x_ok) ? plan_for(m0.W / ud, m0.bits, m0.d) : Plan{0, 0, 0};
         if (pl.TS == 0) {
             int rc = launch_small_generic(mats + i, 1, x, x_dtype, ldx, y, y_dtype, ldy, B, s);
             if (rc) return rc;
-            if (m0.perms && fast_shape(m0)) ws_off += xp_bytes(m0, B);
+            if (mma_shape(m0)) ws_off += mma_part_bytes(m0, B);
+            else if (m0.perms && fast_shape(m0)) ws_off += xp_bytes(m0, B);
             ++i;
             continue;
         }

@@ -1,0 +1,339 @@
+// Decode-time codebook product on the matrix cores, B = 1..32 activation rows, for gfx950.
+//
+// v_mfma_f32_16x16x32_f16 multiplies a 16 x 32 tile of weights (A) by 32 x 16 activations (B):
+//   A: lane l supplies row l % 16, 8 consecutive k starting at 8 * (l / 16)
+//   B: lane l supplies activation row (token) l % 16, the same 8 k
+//   D: lane l holds token l % 16, weight rows 4 * (l / 16) .. + 3
+// Eight consecutive k of one weight row are exactly two d = 4 codewords or one d = 8 codeword, so a
+// lane builds its A operand by gathering raw fp16 codewords (from LDS when the codebook fits) with no
+// arithmetic at all, the sum over k happens inside the accumulator, and the cost of a tile does not
+// depend on how many of the 16 activation rows are real.  The row scale multiplies the fp32 result.
+//
+// Work split.  A wave owns a slice of the columns for its whole life, so its B operands (the
+// activations of that slice, converted bf16 -> fp16 once) are loaded once and stay in registers; it
+// walks over 16-row tiles, prefetching the next tile's tags while it multiplies the current one.
+// The tag stream is read in lane units (UD dwords = TPU whole tags = UK columns): in round n the four
+// lane groups g = 0..3 of a row read units 4n + g, one wide load each, and the round's SPU matrix
+// instructions consume the units chunk pair by chunk pair.  The KW waves of a workgroup split the
+// columns of a tile; their accumulators are added through LDS by one wave per tile (round robin, two
+// buffers, one barrier per tile).  Rows longer than KW * RW rounds are split over `ks` workgroups whose
+// partial sums go to a workspace and are added, in slice order, by splitk_reduce_kernel.
+#pragma once
+#include <mutex>
+#include <unordered_map>
+#include "sq_gemv_kernel.h"
+
+namespace sq {
+
+struct MmaPiece {
+    sq_matrix m;
+    float* part;          // ks > 1: fp32 [ks, B, R] unscaled partial sums of this piece
+    int wg_begin;         // first workgroup of this piece
+    int wg_count;         // nshare * ks workgroups
+};
+
+struct MmaArgs {
+    MmaPiece p[GEMV_MAX_PIECES];
+    int n;
+    const uint16_t* x;
+    int64_t ldx;
+    void* y;
+    int64_t ldy;
+    int B;
+    int x_dtype, y_dtype;
+    int U;                // lane units per row
+    int ks;               // workgroup-level column slices
+    int table_bytes;      // bytes of codebook staged in LDS (0 = read through cache)
+};
+
+constexpr int MMA_TT = 4;     // 16-row tiles multiplied between two workgroup barriers
+
+// Optional timeline of the first wave of every workgroup (debug builds define SQ_TRACE_POINT).
+#ifndef SQ_TRACE_POINT
+#define SQ_TRACE_POINT(k)
+#endif
+
+// two packed bf16 -> two packed fp16 (round toward zero: exact for every fp16-normal value)
+__device__ __forceinline__ uint32_t bf2h_pk(uint32_t v) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(__builtin_bit_cast(float, v << 16),
+                                                                  __builtin_bit_cast(float, v & 0xFFFF0000u)));
+}
+
+template <int BITS, int D, int RW, int NT, bool LDS_TAB>
+__global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
+    constexpr int UD = unit_of<BITS>::UD;
+    constexpr int TPU = UD * 32 / BITS;      // tags per lane unit
+    constexpr int CPS = 8 / D;               // codewords a lane feeds into one matrix instruction
+    constexpr int SPU = TPU / CPS;           // matrix instructions per round
+    constexpr int UK = TPU * D;              // columns per lane unit
+    constexpr int ESZ = D * 2;               // bytes per codeword
+    constexpr int TT = MMA_TT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, lg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), KW = blockDim.x >> 6;
+    int pi = 0;
+    while (pi + 1 < a.n && (int)blockIdx.x >= a.p[pi + 1].wg_begin) ++pi;
+    const MmaPiece& P = a.p[pi];
+    const sq_matrix& m = P.m;
+    const int w = blockIdx.x - P.wg_begin, slice = w % a.ks, share = w / a.ks, nshare = P.wg_count / a.ks;
+    const int ntiles = (m.R + 15) >> 4;
+    const int t0 = (int)((int64_t)ntiles * share / nshare), t1 = (int)((int64_t)ntiles * (share + 1) / nshare);
+    SQ_TRACE_POINT(0);
+
+    // LDS: [codebook][one all-zero codeword][reduction buffer: TT tiles x KW waves x 64 lanes x NT x 16 bytes]
+    const int zero_off = a.table_bytes;                                 // units past the row's end gather this entry
+    const uint32_t zero_idx = (uint32_t)(a.table_bytes / ESZ);
+    float4v* red = reinterpret_cast<float4v*>(smem + a.table_bytes + 16);
+
+    // ---- this wave's rounds
+    const int rbase = (slice * KW + wave) * RW;
+    bool live[RW];
+    bool lane_live = true;
+    uint32_t uoff[RW];
+    int ucol[RW];
+#pragma unroll
+    for (int n = 0; n < RW; ++n) {
+        const int u = 4 * (rbase + n) + lg;
+        live[n] = u < a.U;
+        lane_live = lane_live && live[n];
+        const int uc = live[n] ? u : a.U - 1;
+        uoff[n] = (uint32_t)uc * UD;
+        ucol[n] = uc * UK;
+    }
+    // Units past the row's end (only in waves that cover the tail of the columns) must contribute exact
+    // zeros even if codeword 0 is not finite: their tags are zeroed and their codebook offset points at the
+    // all-zero LDS entry (or, without LDS, their operand is zeroed).  Interior waves skip all of that.
+    const bool all_live = __builtin_amdgcn_readfirstlane(__all(lane_live) ? 1 : 0) != 0;
+    const uint32_t* tags = reinterpret_cast<const uint32_t*>(m.tags);
+    const unsigned char* table = reinterpret_cast<const unsigned char*>(m.table);
+
+    // ---- a tile's memory: tags of this lane's row, its codebook offset, the scales of its four output rows
+    struct Tile { dwords<UD> t[RW]; uint32_t boff; };
+    auto fetch = [&](int t, Tile& T, float (&sc)[4]) {
+        const int row0 = t << 4;
+        const int r = row0 + li < m.R ? row0 + li : m.R - 1;
+        T.boff = m.row_book ? (uint32_t)m.row_book[r] << BITS : 0u;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int ro = row0 + 4 * lg + v;
+            sc[v] = h2f(m.row_scale[ro < m.R ? ro : m.R - 1]);
+        }
+        const uint32_t* rp = tags + (size_t)r * m.W;
+#pragma unroll
+        for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(rp + uoff[n]);
+        if (!all_live) {
+#pragma unroll
+            for (int n = 0; n < RW; ++n)
+#pragma unroll
+                for (int i = 0; i < UD; ++i) T.t[n].v[i] = live[n] ? T.t[n].v[i] : 0u;
+        }
+    };
+
+    // ---- start-up: every load the first product needs is requested before anything waits: the first tile's
+    // tags, the activations of this wave's columns (raw), the codebook
+    Tile tA, tB;
+    float sc[TT + 1][4];                                      // [TT]: first tile of the next group, fetched early
+    if (t0 < t1) fetch(t0, tA, sc[0]);
+    u32x4 xraw[RW][SPU][NT];
+#pragma unroll
+    for (int n = 0; n < RW; ++n)
+#pragma unroll
+        for (int s = 0; s < SPU; ++s)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int tok = nt * 16 + li;
+                xraw[n][s][nt] = *reinterpret_cast<const u32x4*>(a.x + (int64_t)(tok < a.B ? tok : a.B - 1) * a.ldx + ucol[n] + 8 * s);
+            }
+    if (LDS_TAB) {
+        stage_table(m.table, a.table_bytes, smem);
+        if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0u;
+    }
+    // the B operands: this wave's activations as fp16, in registers for the whole kernel
+    half8v xb[RW][SPU][NT];
+#pragma unroll
+    for (int n = 0; n < RW; ++n)
+#pragma unroll
+        for (int s = 0; s < SPU; ++s)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                u32x4 v = xraw[n][s][nt];
+                if (a.x_dtype == SQ_BF16) { v.x = bf2h_pk(v.x); v.y = bf2h_pk(v.y); v.z = bf2h_pk(v.z); v.w = bf2h_pk(v.w); }
+                if (!(live[n] && nt * 16 + li < a.B)) v = u32x4{0u, 0u, 0u, 0u};
+                xb[n][s][nt] = __builtin_bit_cast(half8v, v);
+            }
+    SQ_TRACE_POINT(1);
+    if (LDS_TAB) __syncthreads();
+    SQ_TRACE_POINT(2);
+
+    // One tile: NS = RW * SPU matrix instructions.  The codeword gathers run PD instructions ahead of the
+    // matrix instruction that consumes them, so LDS latency overlaps the multiplies of earlier steps.
+    constexpr int NS = RW * SPU, PD = NS < 6 ? NS : 6;
+    auto multiply = [&](const Tile& cur, float4v (&acc)[NT]) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] = float4v{0.f, 0.f, 0.f, 0.f};
+        u32x4 av[NS];
+        auto gather = [&](int k) {
+            const int n = k / SPU, s = k - n * SPU;
+            const bool dead = !all_live && !live[n];
+            const uint32_t bo = ((LDS_TAB && dead) ? zero_idx : cur.boff) * ESZ;      // byte offset of the row's codebook
+            if (D == 8) {
+                const uint32_t tag = unit_tag<BITS, UD>(cur.t[n], s);
+                if (LDS_TAB) av[k] = *reinterpret_cast<const u32x4*>(smem + (tag * ESZ + bo));
+                else av[k] = *reinterpret_cast<const u32x4*>(table + ((size_t)tag * ESZ + bo));
+            } else {
+                const uint32_t g0 = unit_tag<BITS, UD>(cur.t[n], 2 * s);
+                const uint32_t g1 = unit_tag<BITS, UD>(cur.t[n], 2 * s + 1);
+                u32x2 c0, c1;
+                if (LDS_TAB) {
+                    c0 = *reinterpret_cast<const u32x2*>(smem + (g0 * ESZ + bo));
+                    c1 = *reinterpret_cast<const u32x2*>(smem + (g1 * ESZ + bo));
+                } else {
+                    c0 = *reinterpret_cast<const u32x2*>(table + ((size_t)g0 * ESZ + bo));
+                    c1 = *reinterpret_cast<const u32x2*>(table + ((size_t)g1 * ESZ + bo));
+                }
+                av[k] = u32x4{c0.x, c0.y, c1.x, c1.y};
+            }
+            if (!LDS_TAB && dead) av[k] = u32x4{0u, 0u, 0u, 0u};
+        };
+#pragma unroll
+        for (int k = 0; k < PD; ++k) gather(k);
+#pragma unroll
+        for (int k = 0; k < NS; ++k) {
+            if (k + PD < NS) gather(k + PD);
+            __builtin_amdgcn_sched_barrier(0);          // keep the gathers ahead of the multiply they are not for
+            const int n = k / SPU, s = k - n * SPU;
+            const half8v af = __builtin_bit_cast(half8v, av[k]);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, xb[n][s][nt], acc[nt], 0, 0, 0);
+        }
+    };
+
+    // ---- groups of TT tiles: multiply them one after the other (the next tile's tags load meanwhile), then
+    // add the KW waves' accumulators through LDS, each tile of the group by a different wave
+    for (int tg = t0, grp = 0; tg < t1; tg += TT, ++grp) {
+        float4v acc[TT][NT];
+        if (grp > 0) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sc[0][v] = sc[TT][v];
+        }
+#pragma unroll
+        for (int tt = 0; tt < TT; tt += 2) {
+            if (tg + tt < t1) {
+                if (tg + tt + 1 < t1) fetch(tg + tt + 1, tB, sc[tt + 1]);
+                multiply(tA, acc[tt]);
+            }
+            if (tg + tt + 1 < t1) {
+                if (tg + tt + 2 < t1) fetch(tg + tt + 2, tA, sc[tt + 2]);
+                multiply(tB, acc[tt + 1]);
+            }
+        }
+        SQ_TRACE_POINT(3 + 3 * (grp < 4 ? grp : 4));
+        if (KW > 1) {
+            if (grp > 0) __syncthreads();                     // the previous group's reducers are done reading
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) red[((tt * KW + wave) * 64 + lane) * NT + nt] = acc[tt][nt];
+            __syncthreads();
+        }
+        SQ_TRACE_POINT(4 + 3 * (grp < 4 ? grp : 4));
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+            const int t = tg + tt;
+            if (t >= t1) continue;
+            if (KW > 1 && wave != (tt + grp) % KW) continue;   // this tile's reducer
+            float4v tot[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                if (KW > 1) {
+                    float4v s4 = red[((tt * KW) * 64 + lane) * NT + nt];
+                    for (int k = 1; k < KW; ++k) {
+                        const float4v o = red[((tt * KW + k) * 64 + lane) * NT + nt];
+                        s4.x += o.x; s4.y += o.y; s4.z += o.z; s4.w += o.w;
+                    }
+                    tot[nt] = s4;
+                } else tot[nt] = acc[tt][nt];
+            }
+            const int row0 = t << 4;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int tok = nt * 16 + li;
+                if (tok >= a.B) continue;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int r = row0 + 4 * lg + v;
+                    if (r >= m.R) continue;
+                    if (a.ks > 1) P.part[((int64_t)slice * a.B + tok) * m.R + r] = tot[nt][v];
+                    else store_y(a.y, a.y_dtype, (int64_t)tok * a.ldy + m.y_off + r, tot[nt][v] * sc[tt][v]);
+                }
+            }
+        }
+        SQ_TRACE_POINT(5 + 3 * (grp < 4 ? grp : 4));
+    }
+    SQ_TRACE_POINT(19);
+}
+
+// y[b, y_off + r] = row_scale[r] * sum over column slices (in slice order) of part[s, b, r]
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int ks, int B, int R,
+                                                            const uint16_t* __restrict__ row_scale, void* y, int64_t ldy,
+                                                            int y_off, int y_dtype);
+
+// op 0: launch; op 1: workgroups of `threads` threads and `smem` bytes of LDS that fit on one CU
+template <int BITS, int D, int RW, int NT>
+static inline int mma_inst(int op, const MmaArgs& a, int grid, int threads, size_t smem, hipStream_t s) {
+    void (*k)(MmaArgs) = a.table_bytes ? rows_mfma_kernel<BITS, D, RW, NT, true> : rows_mfma_kernel<BITS, D, RW, NT, false>;
+    if (op == 1) {
+        static std::mutex mu;
+        static std::unordered_map<uint64_t, int> cache;
+        const uint64_t key = ((uint64_t)threads << 40) | ((uint64_t)(a.table_bytes != 0) << 39) | (uint64_t)smem;
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = cache.find(key);
+        if (it != cache.end()) return it->second;
+        if (smem > 64 * 1024) {      // allow the 160 KB of a gfx950 CU
+            (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipGetLastError();
+        }
+        hipFuncAttributes fa;
+        int n = 1;
+        if (hipFuncGetAttributes(&fa, (const void*)k) == hipSuccess && fa.numRegs > 0) {
+            int wps = 512 / ((fa.numRegs + 7) / 8 * 8);     // 512 VGPRs per SIMD lane, granules of 8
+            if (wps > 8) wps = 8;
+            n = 4 * wps / (threads / 64);
+        } else {
+            (void)hipGetLastError();
+        }
+        if (smem && (size_t)n * smem > 160 * 1024) n = (int)(160 * 1024 / smem);
+        if (n < 1) n = 1;
+        cache[key] = n;
+        return n;
+    }
+    hipLaunchKernelGGL(k, dim3(grid), dim3(threads), smem, s, a);
+    return check_launch("sq_linear_small(mfma)");
+}
+
+// (RW, NT) pairs built per format: RW * SPU * NT <= 32 activation operands (128 registers) per lane
+template <int BITS, int D>
+static inline int mma_dispatch(int op, const MmaArgs& a, int RW, int NT, int grid, int threads, size_t smem, hipStream_t s) {
+    constexpr int SPU = (unit_of<BITS>::UD * 32 / BITS) / (8 / D);
+    constexpr int R1 = 32 / SPU;          // most rounds per wave with 16 activation rows
+#define SQ_MMA(RW_, NT_) if (RW == RW_ && NT == NT_) return mma_inst<BITS, D, RW_, NT_>(op, a, grid, threads, smem, s)
+    SQ_MMA(R1, 1);
+    SQ_MMA(R1 / 2, 1);
+    SQ_MMA(R1 / 2, 2);
+    if constexpr (R1 >= 4) {
+        SQ_MMA(R1 / 4, 1);
+        SQ_MMA(R1 / 4, 2);
+    }
+#undef SQ_MMA
+    return fail(SQ_EUNSUPPORTED, "sq_linear_small: no matrix-core kernel for %d rounds, %d token tiles", RW, NT);
+}
+
+#define SQ_MMA_FORMAT(BI, DD)                                                                               \
+    int launch_mma_b##BI##d##DD(int op, const MmaArgs& a, int RW, int NT, int grid, int threads, size_t smem, \
+                                hipStream_t s) {                                                            \
+        return mma_dispatch<BI, DD>(op, a, RW, NT, grid, threads, smem, s);                                 \
+    }
+
+}  // namespace sq
