@@ -144,15 +144,26 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
 int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y,
                          int y_dtype, int64_t ldy, int B, hipStream_t s);
 
+bool gemm256_ok(int C, int64_t ldx, int64_t ldw, const void* x, const void* w);
+int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ldw, const uint16_t* row_scale, void* y,
+                   int y_dtype, int64_t ldy, int y_off, int T, int R, int C, hipStream_t s);
+int launch_bf16_to_f16(const uint16_t* x, int64_t ldx, int T, int C, uint16_t* out, hipStream_t s);
+
 static bool x_vec_ok(const void* x, int64_t ldx, int C) { return C % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x & 15) == 0; }
+// Activation rows from which the large-tile route (decode each piece once into the workspace as raw fp16
+// codewords, then the 256 x 256 tile GEMM with the row scale in its epilogue) replaces the fused 128 x 128
+// kernel, which re-gathers every codeword once per 128 activation rows.
+constexpr int GEMM256_MIN_T = 256;
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 static bool fused_ok(const sq_matrix& m) { return (m.d == 8 || m.d == 4) && !m.perms && ((uintptr_t)m.table & 15) == 0; }
 static size_t dense_bytes(const sq_matrix& m) { return (((size_t)m.R * m.C * 2) + 255) & ~(size_t)255; }
 
 size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
-    (void)T;
     size_t need = 0;
+    const bool big = T >= GEMM256_MIN_T && mats[0].C % 64 == 0;
     for (int i = 0; i < n; ++i)
-        if (!fused_ok(mats[i]) && dense_bytes(mats[i]) > need) need = dense_bytes(mats[i]);
+        if ((big || !fused_ok(mats[i])) && dense_bytes(mats[i]) > need) need = dense_bytes(mats[i]);
+    if (big) need += align256((size_t)T * mats[0].C * 2);       // fp16 copy of bf16 activations
     return need;
 }
 
@@ -168,6 +179,8 @@ int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, con
                       void* y, int y_dtype, int64_t ldy, int T, hipStream_t s) {
     if (!x_vec_ok(x, ldx, C) || !x_vec_ok(w, ldw, C))
         return fail(SQ_EUNSUPPORTED, "sq_gemm_dense: C, ldx, ldw must be multiples of 8 and pointers 16-byte aligned");
+    if (x_dtype == SQ_F16 && w_dtype == SQ_F16 && T >= GEMM256_MIN_T && gemm256_ok(C, ldx, ldw, x, w))
+        return launch_gemm256((const uint16_t*)x, ldx, (const uint16_t*)w, ldw, nullptr, y, y_dtype, ldy, 0, T, R, C, s);
     GemmArgs a{};
     a.m.R = R; a.m.C = C; a.m.y_off = 0;
     a.wd = (const uint16_t*)w; a.ldw = ldw;
@@ -191,6 +204,28 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
     }
     if (gemm_workspace(mats, n, T) > ws_bytes)
         return fail(SQ_EWORKSPACE, "sq_linear_gemm: workspace %zu < %zu", ws_bytes, gemm_workspace(mats, n, T));
+    if (T >= GEMM256_MIN_T && mats[0].C % 64 == 0) {
+        const int C = mats[0].C;
+        const uint16_t* xh = (const uint16_t*)x;
+        int64_t ldxh = ldx;
+        char* wd = (char*)ws;
+        if (x_dtype == SQ_BF16) {
+            int rc = launch_bf16_to_f16((const uint16_t*)x, ldx, T, C, (uint16_t*)ws, s);
+            if (rc) return rc;
+            xh = (const uint16_t*)ws;
+            ldxh = C;
+        }
+        wd += align256((size_t)T * C * 2);
+        for (int i = 0; i < n; ++i) {
+            const sq_matrix& m = mats[i];
+            if (m.R == 0) continue;
+            int rc = launch_dequant(m, wd, SQ_F16, C, 0, m.R, s, /*raw=*/true);
+            if (rc) return rc;
+            rc = launch_gemm256(xh, ldxh, (const uint16_t*)wd, C, m.row_scale, y, y_dtype, ldy, m.y_off, T, m.R, C, s);
+            if (rc) return rc;
+        }
+        return SQ_OK;
+    }
     for (int i = 0; i < n; ++i) {
         const sq_matrix& m = mats[i];
         if (m.R == 0) continue;

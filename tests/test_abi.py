@@ -70,6 +70,8 @@ def test_workspace_sizes_are_host_arithmetic():
     plain = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 8, 16, 1, 1, 32, 0)
     masked = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, 0x6000, 0x7000, None, 64, 512, 8, 16, 1, 16, 32, 0)
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 1, 0) == 0
-    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 0
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == 0
+    # from 256 activation rows on: raw fp16 codewords of the largest piece + an fp16 copy of the activations
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 64 * 512 * 2 + 2048 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == 16 * 2 * 512 * 2
-    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2048, 1) == 64 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == 64 * 512 * 2

@@ -175,6 +175,8 @@ def test_stacked_pieces_write_their_column_slices():
 GEMM = [  # R, C, d, bits, G, M, T
     (300, 1280, 4, 10, 4, 1, 33), (200, 1280, 4, 12, 1, 1, 100), (257, 512, 8, 16, 1, 1, 128), (130, 3584, 8, 16, 1, 1, 300),
     (96, 256, 4, 10, 4, 16, 70), (140, 5120, 8, 16, 1, 16, 129), (50, 96, 2, 5, 3, 1, 40), (64, 200, 4, 8, 1, 1, 35),
+    # 256 activation rows and more: the 256 x 256 tile route (ragged row / token counts, mixture books, column orders)
+    (300, 1280, 4, 10, 4, 1, 260), (140, 5120, 8, 16, 1, 16, 300), (513, 640, 4, 8, 1, 1, 256), (257, 3584, 8, 16, 1, 1, 511),
 ]
 
 
