@@ -42,6 +42,9 @@ typedef struct sq_matrix {
     const int32_t*  row_order;  /* optional [R]: row ids sorted by row_mask (stable); NULL = natural */
     int32_t R, C, d, bits, G, M, W;
     int32_t y_off;              /* first output column of this piece in the stacked Y */
+    const void*     stream;     /* optional: device copy of the buffer sq_stream_build wrote for `tags`; NULL = none */
+    int32_t stream_runs;        /* what sq_stream_runs returned for that buffer */
+    int32_t reserved;           /* 0 */
 } sq_matrix;
 
 /* Library / device identification.  sq_version: ABI version (major*100 + minor). */
@@ -84,8 +87,25 @@ int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C,
 
 /* Bytes of workspace sq_linear_small (which = 0) or sq_linear_gemm (which = 1) needs for these
  * pieces at `rows` activation rows; the caller grows its buffer before any graph capture
- * (the reference grows its buffers the same way: batched_runs.py:628-640, runs_gemm.py:396-404). */
+ * (the reference grows its buffers the same way: batched_runs.py:628-640, runs_gemm.py:396-404).
+ * A workspace must be 256-byte aligned and its first 4096 bytes must be ZERO when it is first handed
+ * to the library (they hold arrival counters that every call leaves at zero again); one workspace
+ * serves one stream at a time. */
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which);
+
+/* Load-time regrouping of a matrix' tags for codebooks that do not fit LDS (d = 8, K = 8192..65,536, one
+ * codebook, no column orders): the batch-1 product then gathers codewords from a 64 KB LDS slice instead of
+ * from L2.  HOST pointers: `tags_host` is the file's tag tensor in host memory, `out_host` receives
+ * sq_stream_bytes() bytes that the caller copies to the device (16-byte aligned) and names in
+ * sq_matrix.stream.  sq_stream_bytes returns 0 for formats the stream does not cover.  The tags tensor
+ * stays the source of truth (sq_dequant, B > 1 and the prefill GEMM read it); this plays the part of the
+ * reference's load-time run-length layout (reference shapequant/kernels/proto_runs.py:178-260
+ * build_runs / RunsLayout), with a layout chosen for LDS gathers rather than run-length grouping. */
+int32_t sq_stream_runs(int32_t R, int32_t C, int32_t d, int32_t bits, int32_t runs);
+size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                       int32_t runs);
+int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                    int32_t runs, void* out_host, size_t out_bytes);
 
 #ifdef __cplusplus
 }

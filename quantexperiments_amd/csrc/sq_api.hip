@@ -1,7 +1,7 @@
 // extern "C" surface of libsqhip.so: argument checks, error text, dispatch to the launchers.
 #include <stdarg.h>
 #include <stdio.h>
-#include "sq_common.h"
+#include "sq_stream.h"
 
 namespace sq {
 
@@ -73,7 +73,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 100; }
+int sq_version(void) { return 101; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -93,7 +93,9 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
     if (rc) return rc;
     if (B > SQ_SMALL_BMAX) return fail(SQ_EINVAL, "sq_linear_small: B %d > %d", B, SQ_SMALL_BMAX);
     if (B == 0 || n_mats == 0) return SQ_OK;
-    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, workspace, ws_bytes, (hipStream_t)stream);
+    const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
+    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
+                        has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
 }
 
 int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
@@ -101,7 +103,9 @@ int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_d
     int rc = check_xy("sq_linear_gemm", mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T);
     if (rc) return rc;
     if (T == 0 || n_mats == 0) return SQ_OK;
-    return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T, workspace, ws_bytes, (hipStream_t)stream);
+    const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
+    return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
+                       has_ws ? ws_bytes - SQ_WS_HEADER : 0, (hipStream_t)stream);
 }
 
 int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype, int64_t ldx,
@@ -117,7 +121,26 @@ int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C,
 
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which) {
     if (!mats || n_mats <= 0 || rows <= 0) return 0;
-    return which == 0 ? small_workspace(mats, n_mats, rows) : gemm_workspace(mats, n_mats, rows);
+    const size_t inner = which == 0 ? small_workspace(mats, n_mats, rows) : gemm_workspace(mats, n_mats, rows);
+    return inner ? inner + SQ_WS_HEADER : 0;
+}
+
+int32_t sq_stream_runs(int32_t R, int32_t C, int32_t d, int32_t bits, int32_t runs) {
+    if (d <= 0 || !stream_format_ok(R, C, d, bits)) return 0;
+    return stream_geom(R, C, d, bits, runs).runs;
+}
+
+size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t runs) {
+    if (!tags_host || d <= 0 || !stream_format_ok(R, C, d, bits) || (int64_t)W * 32 < (int64_t)(C / d) * bits) return 0;
+    return stream_bytes_host((const uint32_t*)tags_host, R, W, C, d, bits, runs);
+}
+
+int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t runs,
+                    void* out_host, size_t out_bytes) {
+    if (!tags_host || !out_host) return fail(SQ_EINVAL, "sq_stream_build: null pointer");
+    if (d <= 0 || !stream_format_ok(R, C, d, bits)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: d %d bits %d R %d not covered", d, bits, R);
+    if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_stream_build: W %d too small", W);
+    return stream_build_host((const uint32_t*)tags_host, R, W, C, d, bits, runs, (unsigned char*)out_host, out_bytes);
 }
 
 }  // extern "C"

@@ -46,6 +46,12 @@ template <> struct store_as<SQ_F32> { typedef float type; static __device__ __fo
 template <> struct store_as<SQ_F16> { typedef uint16_t type; static __device__ __forceinline__ uint16_t cvt(float f) { return f2h(f); } };
 template <> struct store_as<SQ_BF16> { typedef uint16_t type; static __device__ __forceinline__ uint16_t cvt(float f) { return f2bf(f); } };
 
+__device__ __forceinline__ void store_y(void* y, int y_dtype, int64_t o, float v) {
+    if (y_dtype == SQ_BF16) reinterpret_cast<uint16_t*>(y)[o] = f2bf(v);
+    else if (y_dtype == SQ_F16) reinterpret_cast<uint16_t*>(y)[o] = f2h(v);
+    else reinterpret_cast<float*>(y)[o] = v;
+}
+
 // Tag j of a row's little-endian bit stream (any width 1..16).  `W` bounds the second word.
 __device__ __forceinline__ uint32_t tag_at(const uint32_t* __restrict__ row, int W, int bits, int j) {
     const int p = j * bits, w = p >> 5, s = p & 31;
@@ -61,6 +67,11 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// A caller's workspace starts with SQ_WS_HEADER bytes of arrival counters that are zero whenever no call is
+// running (kernels that use them put them back to zero); the launchers get the part behind the header.
+constexpr size_t SQ_WS_HEADER = 4096;
+constexpr int SQ_WS_COUNTERS = 1024;
+
 // error plumbing shared by the launchers (defined in sq_api.hip)
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
@@ -69,7 +80,7 @@ int check_launch(const char* what);
 int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s,
                    bool raw = false);
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                 int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s);
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s);
 size_t small_workspace(const sq_matrix* mats, int n, int B);
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                 int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s);

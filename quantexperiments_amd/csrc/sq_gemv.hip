@@ -1,6 +1,7 @@
 // Host side of the decode-time product: picks the team geometry per shape, fuses stacked pieces
 // into one persistent launch, prepares permuted activations for pieces with column orders.
 #include "sq_rows_mfma.h"
+#include "sq_stream.h"
 
 namespace sq {
 
@@ -119,7 +120,8 @@ static size_t mma_part_bytes(const sq_matrix& m, int B) {
 size_t small_workspace(const sq_matrix* mats, int n, int B) {
     size_t tot = 0;
     for (int i = 0; i < n; ++i) {
-        if (mma_shape(mats[i])) tot += mma_part_bytes(mats[i], B);
+        if (B == 1 && stream_shape(mats[i])) tot += stream_part_bytes(mats[i]);
+        else if (mma_shape(mats[i])) tot += mma_part_bytes(mats[i], B);
         else if (mats[i].perms && fast_shape(mats[i])) tot += xp_bytes(mats[i], B);
     }
     return tot;
@@ -188,17 +190,26 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
 }
 
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                 int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s) {
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s) {
     if (small_workspace(mats, n, B) > ws_bytes)
         return fail(SQ_EWORKSPACE, "sq_linear_small: workspace %zu < %zu", ws_bytes, small_workspace(mats, n, B));
     const int cus = device_cus();
     const bool x_ok = (B == 1 || ldx % 8 == 0) && (((uintptr_t)x & 15) == 0);   // 16-byte activation loads
     size_t ws_off = 0;
+    int counters_used = 0;
     int i = 0;
     while (i < n) {
         const sq_matrix& m0 = mats[i];
         if (m0.R == 0) { ++i; continue; }
         const int ud = unit_dwords(m0.bits);
+        if (B == 1 && stream_shape(m0) && x_ok) {
+            int j = i + 1;
+            while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_shape(mats[j]) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
+            int rc = launch_stream_group(mats + i, j - i, x, x_dtype, y, y_dtype, (char*)ws, ws_off, counters, counters_used, cus, s);
+            if (rc) return rc;
+            i = j;
+            continue;
+        }
         if (mma_shape(m0) && x_ok) {
             int j = i + 1;
             while (j < n && j - i < GEMV_MAX_PIECES && mma_shape(mats[j]) && mats[j].bits == m0.bits && mats[j].d == m0.d &&
@@ -213,7 +224,8 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         if (pl.TS == 0) {
             int rc = launch_small_generic(mats + i, 1, x, x_dtype, ldx, y, y_dtype, ldy, B, s);
             if (rc) return rc;
-            if (mma_shape(m0)) ws_off += mma_part_bytes(m0, B);
+            if (B == 1 && stream_shape(m0)) ws_off += stream_part_bytes(m0);
+            else if (mma_shape(m0)) ws_off += mma_part_bytes(m0, B);
             else if (m0.perms && fast_shape(m0)) ws_off += xp_bytes(m0, B);
             ++i;
             continue;

@@ -114,12 +114,6 @@ template <int D> struct cw_t;
 template <> struct cw_t<8> { typedef u32x4 type; };
 template <> struct cw_t<4> { typedef u32x2 type; };
 
-__device__ __forceinline__ void store_y(void* y, int y_dtype, int64_t o, float v) {
-    if (y_dtype == SQ_BF16) reinterpret_cast<uint16_t*>(y)[o] = f2bf(v);
-    else if (y_dtype == SQ_F16) reinterpret_cast<uint16_t*>(y)[o] = f2h(v);
-    else reinterpret_cast<float*>(y)[o] = v;
-}
-
 // Codebook into LDS, eight 16-byte loads in flight per thread before the first store.
 __device__ __forceinline__ void stage_table(const uint16_t* table, int bytes, unsigned char* smem) {
     const u32x4* src = reinterpret_cast<const u32x4*>(table);

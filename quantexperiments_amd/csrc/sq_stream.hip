@@ -1,0 +1,400 @@
+// Bucketed tag stream: the batch-1 product for codebooks too large for LDS (K = 8192 .. 65,536 at d = 8).
+//
+// A 65,536 x 8 fp16 codebook is 1 MiB; gathering 16-byte codewords from it through L2 is what bounds the
+// row-major kernels.  Here the tags of a matrix are regrouped once, at load time, by the part of the
+// codebook they point into, so that every workgroup gathers from a 64 KB slice held in LDS:
+//
+//   bucket (kp, s)   column part kp (PC chunks of d columns each) x codebook slice s (tags s*4096 .. +4095)
+//   entry            24 bits: tag & 4095 | (chunk - kp * PC) << 12
+//   lane task        the entries of one row in one bucket (about C/d / (KP * NS) of them)
+//
+// Rows are cut into `runs` runs of GR * 64 consecutive rows, one workgroup per (bucket, run); the caller
+// picks `runs` so that the pieces it launches together make about two workgroups per CU.  Within a bucket the
+// rows of a run are sorted by entry count (descending, stable) and cut into groups of 64: one lane per row,
+// one wave per group.  A group is stored as steps of 64 x 12 bytes (4 entries per lane per step, lane-major,
+// so a wave reads 768 contiguous bytes per step) padded to the longest row of the group; sorting keeps that
+// padding near 10 percent.  A workgroup stages its slice and its part of x in LDS; each lane accumulates
+// dot(codeword, x chunk) over its entries in fp32 and writes one partial sum per (bucket, row).  The
+// workgroups of all buckets that cover the same run count themselves off on a counter in the workspace; the
+// last one to arrive adds the NS * KP partials of each row of the run in a fixed order (so results do not
+// depend on scheduling), applies the row scale and stores y.
+//
+// Stream buffer (one allocation, offsets follow from R and C/d alone):
+//   goff   uint32 [NV * NG + 1]   first step of every group, cumulative over buckets (NV = KP * NS buckets,
+//                                 NG = ceil(R / 64) groups per bucket, bucket v = kp * NS + s)
+//   slots  uint32 [NV * NG * 64]  row | count << 19 per lane; row 0x7FFFF marks a lane without a row;
+//                                 lanes 64 g .. 64 g + 63 of a bucket are group g, groups GR i .. GR i + GR - 1 run i
+//   steps  [total][64][3] uint32  entries
+#include <algorithm>
+#include <string.h>
+#include <thread>
+#include <vector>
+#include "sq_stream.h"
+
+namespace sq {
+
+StreamGeom stream_geom(int R, int C, int d, int bits, int runs) {
+    StreamGeom g;
+    g.U = C / d;
+    g.NS = 1 << (bits - STREAM_SLICE_BITS);
+    g.KP = (g.U + STREAM_PART_MAX - 1) / STREAM_PART_MAX;
+    g.PC = (g.U + g.KP - 1) / g.KP;
+    g.NV = g.NS * g.KP;
+    g.NG = (R + 63) / 64;
+    if (runs <= 0) runs = (STREAM_DEFAULT_WGS + g.NV / 2) / g.NV;
+    if (runs < 1) runs = 1;
+    if (runs > g.NG) runs = g.NG;
+    g.GR = (g.NG + runs - 1) / runs;
+    g.runs = (g.NG + g.GR - 1) / g.GR;
+    g.off_slots = (((size_t)g.NV * g.NG + 1) * 4 + 255) & ~(size_t)255;
+    g.off_steps = (g.off_slots + (size_t)g.NV * g.NG * 64 * 4 + 255) & ~(size_t)255;
+    return g;
+}
+
+bool stream_format_ok(int R, int C, int d, int bits) {
+    return d == 8 && bits > STREAM_SLICE_BITS && bits <= 16 && C % d == 0 && R > 0 && R < STREAM_NO_ROW;
+}
+
+static inline uint32_t host_tag(const uint32_t* row, int W, int bits, int j) {
+    const int64_t p = (int64_t)j * bits;
+    const int w = (int)(p >> 5), s = (int)(p & 31);
+    uint64_t v = row[w];
+    if (s + bits > 32 && w + 1 < W) v |= (uint64_t)row[w + 1] << 32;
+    return (uint32_t)(v >> s) & ((1u << bits) - 1u);
+}
+
+static void parallel_rows(int R, const std::function<void(int, int)>& fn) {
+    unsigned nt = std::thread::hardware_concurrency();
+    if (nt < 1) nt = 1;
+    if (nt > 16) nt = 16;
+    if ((unsigned)R < nt * 64) nt = 1;
+    if (nt == 1) { fn(0, R); return; }
+    std::vector<std::thread> th;
+    const int per = (R + (int)nt - 1) / (int)nt;
+    for (unsigned t = 0; t < nt; ++t) {
+        const int a = (int)t * per, b = std::min(R, a + per);
+        if (a < b) th.emplace_back(fn, a, b);
+    }
+    for (auto& t : th) t.join();
+}
+
+// counts[v * R + r] and, per bucket, the sorted row order with its group step counts
+struct StreamPlan {
+    StreamGeom g;
+    std::vector<uint16_t> cnt;       // [NV][R]
+    std::vector<uint32_t> pos;       // [NV][R]: position of row r in bucket v's sorted order
+    std::vector<uint32_t> goff;      // [NV * NG + 1]
+};
+
+static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs, StreamPlan& P) {
+    P.g = stream_geom(R, C, d, bits, runs);
+    const StreamGeom& g = P.g;
+    P.cnt.assign((size_t)g.NV * R, 0);
+    P.pos.assign((size_t)g.NV * R, 0);
+    P.goff.assign((size_t)g.NV * g.NG + 1, 0);
+    parallel_rows(R, [&](int a, int b) {
+        for (int r = a; r < b; ++r) {
+            const uint32_t* row = tags + (size_t)r * W;
+            for (int j = 0; j < g.U; ++j) {
+                const uint32_t t = host_tag(row, W, bits, j);
+                const int v = (j / g.PC) * g.NS + (int)(t >> STREAM_SLICE_BITS);
+                ++P.cnt[(size_t)v * R + r];
+            }
+        }
+    });
+    std::vector<uint32_t> steps((size_t)g.NV * g.NG);
+    parallel_rows(g.NV, [&](int a, int b) {
+        std::vector<uint32_t> order(R);
+        for (int v = a; v < b; ++v) {
+            const uint16_t* c = &P.cnt[(size_t)v * R];
+            for (int r = 0; r < R; ++r) order[r] = (uint32_t)r;
+            for (int r0 = 0; r0 < R; r0 += g.GR * 64)
+                std::stable_sort(order.begin() + r0, order.begin() + std::min(R, r0 + g.GR * 64),
+                                 [c](uint32_t x, uint32_t y) { return c[x] > c[y]; });
+            for (int k = 0; k < R; ++k) P.pos[(size_t)v * R + order[k]] = (uint32_t)k;
+            for (int gi = 0; gi < g.NG; ++gi) steps[(size_t)v * g.NG + gi] = (c[order[(size_t)gi * 64]] + 3u) / 4u;
+        }
+    });
+    uint64_t tot = 0;
+    for (size_t k = 0; k < steps.size(); ++k) { P.goff[k] = (uint32_t)tot; tot += steps[k]; }
+    P.goff[steps.size()] = (uint32_t)tot;
+    P.g.total_steps = tot;
+}
+
+size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs) {
+    StreamPlan P;
+    plan_stream(tags, R, W, C, d, bits, runs, P);
+    return P.g.off_steps + (size_t)P.g.total_steps * 768;
+}
+
+int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs, unsigned char* out,
+                      size_t bytes) {
+    StreamPlan P;
+    plan_stream(tags, R, W, C, d, bits, runs, P);
+    const StreamGeom& g = P.g;
+    const size_t need = g.off_steps + (size_t)g.total_steps * 768;
+    if (g.total_steps >= ((uint64_t)1 << 32)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: matrix too large");
+    if (bytes < need) return fail(SQ_EINVAL, "sq_stream_build: buffer %zu < %zu", bytes, need);
+    memset(out, 0, need);
+    memcpy(out, P.goff.data(), P.goff.size() * 4);
+    uint32_t* slots = (uint32_t*)(out + g.off_slots);
+    for (size_t k = 0; k < (size_t)g.NV * g.NG * 64; ++k) slots[k] = STREAM_NO_ROW;
+    unsigned char* steps = out + g.off_steps;
+    parallel_rows(R, [&](int a, int b) {
+        std::vector<uint32_t> q(g.NV);
+        for (int r = a; r < b; ++r) {
+            const uint32_t* row = tags + (size_t)r * W;
+            std::fill(q.begin(), q.end(), 0u);
+            for (int v = 0; v < g.NV; ++v) {
+                const uint32_t k = P.pos[(size_t)v * R + r];
+                slots[(size_t)v * g.NG * 64 + k] = (uint32_t)r | ((uint32_t)P.cnt[(size_t)v * R + r] << STREAM_ROW_BITS);
+            }
+            for (int j = 0; j < g.U; ++j) {
+                const uint32_t t = host_tag(row, W, bits, j);
+                const int kp = j / g.PC, v = kp * g.NS + (int)(t >> STREAM_SLICE_BITS);
+                const uint32_t k = P.pos[(size_t)v * R + r], n = q[v]++;
+                const uint32_t e = (t & ((1u << STREAM_SLICE_BITS) - 1u)) | ((uint32_t)(j - kp * g.PC) << STREAM_SLICE_BITS);
+                unsigned char* rec = steps + ((size_t)P.goff[(size_t)v * g.NG + (k >> 6)] + (n >> 2)) * 768 + (k & 63) * 12 +
+                                     (n & 3) * 3;
+                rec[0] = (unsigned char)e; rec[1] = (unsigned char)(e >> 8); rec[2] = (unsigned char)(e >> 16);
+            }
+        }
+    });
+    return SQ_OK;
+}
+
+// ---------------------------------------------------------------------------------------- device
+
+struct StreamPiece {
+    const unsigned char* stream;
+    const uint16_t* table;
+    const uint16_t* row_scale;
+    float* part;                      // [NV][R]
+    unsigned* counters;               // one per run; zero before the launch, zero after it
+    int R, U, NS, NV, PC, NG, GR, y_off;
+    uint32_t off_slots, off_steps;
+    int wg_begin, nwg;                // first workgroup of the piece; workgroups (= runs) per bucket
+};
+
+struct StreamArgs {
+    StreamPiece p[GEMV_MAX_PIECES_STREAM];
+    int n;
+    const uint16_t* x;
+    void* y;
+    int x_dtype, y_dtype;
+};
+
+constexpr int STREAM_X_OFF = 65536;   // x part follows the 64 KB slice in LDS
+constexpr int STREAM_PF = 4;          // steps fetched ahead
+constexpr int STREAM_NW = 8;          // waves per workgroup
+
+struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
+
+__global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
+    constexpr int NW = STREAM_NW;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int pi = 0;
+#pragma unroll
+    for (int k = 1; k < GEMV_MAX_PIECES_STREAM; ++k)
+        if (k < a.n && (int)blockIdx.x >= a.p[k].wg_begin) pi = k;
+    const StreamPiece& P = a.p[pi];
+    const int local = (int)blockIdx.x - P.wg_begin;
+    const int v = local / P.nwg, wi = local - v * P.nwg;
+    const int s = v % P.NS, kp = v / P.NS;
+    // this workgroup's run: groups g0 .. g1 - 1 of the bucket
+    const int g0 = wi * P.GR, g1 = min(P.NG, g0 + P.GR);
+
+    const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG;
+    const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + (size_t)v * P.NG * 64;
+    const unsigned char* steps = P.stream + P.off_steps + lane * 12;
+    float* part = P.part + (size_t)v * P.R;
+
+    // The groups of a run are sorted longest first; wave w takes the w-th of the first eight, the (7 - w)-th of
+    // the next eight and so on, which evens out the waves' shares.  The head of a group (its first step, its
+    // step count, the lane's row and count) is fetched one group ahead; the first one goes out before the
+    // staging loads.
+    auto group_of = [&](int k) { return g0 + k * NW + ((k & 1) ? NW - 1 - wave : wave); };
+    auto head = [&](int k) {
+        StreamHead h{0u, 0, STREAM_NO_ROW};
+        const int g = group_of(k);
+        if (g < g1) {
+            h.st0 = goff[g];
+            h.nst = (int)(goff[g + 1] - h.st0);
+            h.slot = slots[(size_t)g * 64 + lane];
+        }
+        return h;
+    };
+    StreamHead hn = head(0);
+    const int nk = (g1 - g0 + NW - 1) / NW;
+
+    // stage the codebook slice and this part of x (as fp16)
+    {
+        const u32x4* src = reinterpret_cast<const u32x4*>(P.table) + (size_t)s * (1 << STREAM_SLICE_BITS);
+        u32x4* dst = reinterpret_cast<u32x4*>(lds);
+        u32x4 t[(1 << STREAM_SLICE_BITS) / (NW * 64)];
+#pragma unroll
+        for (int k = 0; k < (1 << STREAM_SLICE_BITS) / (NW * 64); ++k) t[k] = src[tid + k * NW * 64];
+        const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
+        const u32x4* xs = reinterpret_cast<const u32x4*>(a.x) + c0;
+        u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_X_OFF);
+        for (int k = tid; k < nc; k += NW * 64) {
+            u32x4 q = xs[k];
+            if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
+            xd[k] = q;
+        }
+#pragma unroll
+        for (int k = 0; k < (1 << STREAM_SLICE_BITS) / (NW * 64); ++k) dst[tid + k * NW * 64] = t[k];
+    }
+    // first steps of the first group: in flight across the barrier
+    u32x3 nx[STREAM_PF];
+    {
+        const unsigned char* eb = steps + (size_t)hn.st0 * 768;
+#pragma unroll
+        for (int k = 0; k < STREAM_PF; ++k) {
+            nx[k] = u32x3{0u, 0u, 0u};
+            if (hn.nst > 0) nx[k] = *reinterpret_cast<const u32x3*>(eb + (size_t)min(k, hn.nst - 1) * 768);
+        }
+    }
+    __syncthreads();
+
+    for (int k = 0; k < nk; ++k) {
+        const StreamHead h = hn;
+        hn = k + 1 < nk ? head(k + 1) : StreamHead{0u, 0, STREAM_NO_ROW};
+        const int nst = h.nst;
+        const int cnt = (int)(h.slot >> STREAM_ROW_BITS);
+        const uint32_t row = h.slot & STREAM_NO_ROW;
+        const unsigned char* eb = steps + (size_t)h.st0 * 768;
+        float acc = 0.f;
+        for (int t0 = 0; t0 < nst; t0 += STREAM_PF) {
+            u32x3 cur[STREAM_PF];
+#pragma unroll
+            for (int q = 0; q < STREAM_PF; ++q) cur[q] = nx[q];
+            if (t0 + STREAM_PF < nst) {                         // wave-uniform
+#pragma unroll
+                for (int q = 0; q < STREAM_PF; ++q)
+                    nx[q] = *reinterpret_cast<const u32x3*>(eb + (size_t)min(t0 + STREAM_PF + q, nst - 1) * 768);
+            } else if (hn.nst > 0) {                            // the next group's first steps
+                const unsigned char* en = steps + (size_t)hn.st0 * 768;
+#pragma unroll
+                for (int q = 0; q < STREAM_PF; ++q)
+                    nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, hn.nst - 1) * 768);
+            }
+#pragma unroll
+            for (int q = 0; q < STREAM_PF; ++q) {
+                if (t0 + q >= nst) break;                       // wave-uniform
+                const uint32_t e[4] = {cur[q].x & 0xFFFFFFu, (cur[q].x >> 24) | ((cur[q].y & 0xFFFFu) << 8),
+                                       (cur[q].y >> 16) | ((cur[q].z & 0xFFu) << 16), cur[q].z >> 8};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t ta = (e[j] << 4) & 0xFFF0u;
+                    const uint32_t xa = ((e[j] >> 8) & 0xFFFF0u) | (uint32_t)STREAM_X_OFF;
+                    const u32x4 cw = *reinterpret_cast<const u32x4*>(lds + ta);
+                    const u32x4 xv = *reinterpret_cast<const u32x4*>(lds + xa);
+                    float dsum = 0.f;
+#pragma unroll
+                    for (int hh = 0; hh < 4; ++hh) {
+                        const uint32_t cwh = cw[hh], xvh = xv[hh];  // bit_cast straight from a vector element misreads it
+                        dsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, cwh), __builtin_bit_cast(half2v, xvh), dsum, false);
+                    }
+                    acc += ((t0 + q) * 4 + j < cnt) ? dsum : 0.f;
+                }
+            }
+        }
+        if (nst == 0 && hn.nst > 0) {                           // a group without steps fetched nothing for its successor
+            const unsigned char* en = steps + (size_t)hn.st0 * 768;
+#pragma unroll
+            for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, hn.nst - 1) * 768);
+        }
+        // device-scope store: written through to memory, so other XCDs' L2s never hold a stale copy and no
+        // cache-wide write-back is needed before the workgroup counts itself off
+        if (row != STREAM_NO_ROW) __hip_atomic_store(part + row, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // Count this workgroup off once all its partial sums have been acknowledged (the barrier waits for every
+    // wave's outstanding stores).  The workgroup that finds every other bucket's workgroup already counted
+    // reads all partial sums back with device-scope loads and finishes the rows.
+    unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_X_OFF + P.PC * 16);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned old = atomicAdd(P.counters + wi, 1u);
+        if (old == (unsigned)P.NV - 1u) P.counters[wi] = 0u;    // everyone has arrived: leave the counter as found
+        *flag = old;
+    }
+    __syncthreads();
+    if (*flag != (unsigned)P.NV - 1u) return;
+    const int r0 = g0 * 64, r1 = min(P.R, g1 * 64);
+    for (int r = r0 + tid; r < r1; r += NW * 64) {
+        float sum = 0.f;
+        for (int v0 = 0; v0 < P.NV; v0 += 16) {                 // NV is a multiple of the slice count, a power of two >= 2
+            float t[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                t[k] = v0 + k < P.NV ? __hip_atomic_load(P.part + (size_t)(v0 + k) * P.R + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) sum += t[k];
+        }
+        store_y(a.y, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
+    }
+}
+
+static int stream_launch(const StreamArgs& a, int grid, size_t smem, hipStream_t s) {
+    static bool raised = false;
+    if (!raised) {
+        (void)hipFuncSetAttribute((const void*)stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipGetLastError();
+        raised = true;
+    }
+    hipLaunchKernelGGL(stream_kernel, dim3((unsigned)grid), dim3(STREAM_NW * 64), smem, s, a);
+    return check_launch("sq_linear_small(stream)");
+}
+
+bool stream_shape(const sq_matrix& m) {
+    return m.stream && m.stream_runs > 0 && !m.perms && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
+           (((uintptr_t)m.table | (uintptr_t)m.stream) & 15) == 0;
+}
+
+size_t stream_part_bytes(const sq_matrix& m) {
+    const StreamGeom g = stream_geom(m.R, m.C, m.d, m.bits, m.stream_runs);
+    return (((size_t)g.NV * m.R * 4) + 255) & ~(size_t)255;
+}
+
+// Pieces [0, cnt) (same C): one launch.  `counters` is the zeroed head of the workspace.
+int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, void* y, int y_dtype, char* ws,
+                        size_t& ws_off, unsigned* counters, int& counters_used, int cus, hipStream_t s) {
+    StreamArgs a;
+    a.n = cnt;
+    a.x = (const uint16_t*)x;
+    a.y = y;
+    a.x_dtype = x_dtype;
+    a.y_dtype = y_dtype;
+    const StreamGeom g0 = stream_geom(mats[0].R, mats[0].C, mats[0].d, mats[0].bits, mats[0].stream_runs);
+    const size_t smem = (size_t)STREAM_X_OFF + (size_t)g0.PC * 16 + 16;
+    (void)cus;
+    int wg = 0;
+    for (int k = 0; k < cnt; ++k) {
+        const sq_matrix& m = mats[k];
+        const StreamGeom g = stream_geom(m.R, m.C, m.d, m.bits, m.stream_runs);
+        if (g.runs != m.stream_runs) return fail(SQ_EINVAL, "sq_linear_small: stream_runs %d is not what sq_stream_runs returns (%d)", m.stream_runs, g.runs);
+        StreamPiece& P = a.p[k];
+        P.stream = (const unsigned char*)m.stream;
+        P.table = m.table;
+        P.row_scale = m.row_scale;
+        P.part = (float*)(ws + ws_off);
+        ws_off += stream_part_bytes(m);
+        P.R = m.R; P.U = g.U; P.NS = g.NS; P.NV = g.NV; P.PC = g.PC; P.NG = g.NG; P.GR = g.GR; P.y_off = m.y_off;
+        P.off_slots = (uint32_t)g.off_slots; P.off_steps = (uint32_t)g.off_steps;
+        const int nwg = g.runs;
+        if (counters_used + nwg > SQ_WS_COUNTERS) return fail(SQ_EUNSUPPORTED, "sq_linear_small: too many row-block runs");
+        P.counters = counters + counters_used;
+        counters_used += nwg;
+        P.wg_begin = wg;
+        P.nwg = nwg;
+        wg += g.NV * nwg;
+    }
+    for (int k = cnt; k < GEMV_MAX_PIECES_STREAM; ++k) a.p[k] = a.p[0];
+    return stream_launch(a, wg, smem, s);
+}
+
+}  // namespace sq

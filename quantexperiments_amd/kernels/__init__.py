@@ -26,20 +26,23 @@ class _Workspace:
     bufs: dict = {}
 
     @classmethod
-    def get(cls, nbytes: int, dev) -> torch.Tensor:
-        key = str(dev)
+    def get(cls, nbytes: int, dev, kind: str = "kernels") -> torch.Tensor:
+        """kind "kernels": the buffer handed to the library (its first 4096 bytes are the library's counters
+        and stay zero between calls); any other kind names a separate buffer the caller may overwrite."""
+        key = (str(dev), kind)
         b = cls.bufs.get(key)
         if b is None or b.numel() < nbytes:
             if torch.cuda.is_current_stream_capturing():
                 raise RuntimeError("sqhip workspace must grow outside graph capture: run this shape once eagerly first")
-            b = cls.bufs[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+            b = cls.bufs[key] = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)   # counters start at zero
         return b
 
 
 class PackedLinear(torch.nn.Module):
     """A block linear run from packed tensors."""
 
-    def __init__(self, words, table, row_scale, row_book, row_mask, perms, K: int, d: int, bias=None):
+    def __init__(self, words, table, row_scale, row_book, row_mask, perms, K: int, d: int, bias=None,
+                 stream: bool = True):
         super().__init__()
         R, W = words.shape
         dev = words.device
@@ -77,6 +80,16 @@ class PackedLinear(torch.nn.Module):
             self.register_buffer("perms", None)
             self.register_buffer("row_order", None)
         self.bias = bias
+        # codebooks too large for LDS: regroup the tags by codebook slice once, for the batch-1 product
+        self.register_buffer("stream", None)
+        self.stream_runs = 0
+        if stream and not self.has_mask and self.G == 1 and table.numel() * 2 > 128 * 1024:
+            self.build_stream(0)
+
+    def build_stream(self, runs: int = 0) -> None:
+        """(Re)build the bucketed tag stream cut into `runs` row runs (0 = suited to a launch of this matrix
+        alone; prepare_stack picks the runs of pieces that are launched together)."""
+        self.stream, self.stream_runs = build_stream(self.words, self.C, self.d, self.bits, runs)
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -97,7 +110,7 @@ class PackedLinear(torch.nn.Module):
         p = lambda t: None if t is None else t.data_ptr()
         return SqMatrix(p(self.words), p(self.table), p(self.row_scale), p(self.row_book), p(self.row_mask),
                         p(self.perms), p(self.row_order), self.R, self.C, self.d, self.bits, self.G, self.M, self.W,
-                        y_off)
+                        y_off, p(self.stream), self.stream_runs if self.stream is not None else 0, 0)
 
     # ------------------------------------------------------------------ kernels
     def dense(self, dtype=torch.float32, out: torch.Tensor | None = None, rows: tuple | None = None) -> torch.Tensor:
@@ -140,6 +153,33 @@ class PackedLinear(torch.nn.Module):
     def stored_bytes(self) -> int:
         """Bytes the product must stream from HBM: tags + table + scales (as the reference counts)."""
         return sum(t.numel() * t.element_size() for t in (self.words, self.table, self.row_scale))
+
+
+def build_stream(words: torch.Tensor, C: int, d: int, bits: int, runs: int = 0):
+    """(stream, runs): the bucketed tag stream of one matrix (sq_stream_build) as a uint8 tensor on words'
+    device and the number of row runs it was cut into, or (None, 0) when the format is not covered.  The
+    regrouping itself is the library's host routine; the tags make one trip to host memory at load time."""
+    L = _lib.lib()
+    host = words.detach().to("cpu", torch.int32).contiguous()
+    R, W = host.shape
+    n = L.sq_stream_bytes(host.data_ptr(), R, W, C, d, bits, runs)
+    if n == 0:
+        return None, 0
+    out = torch.empty(n, dtype=torch.uint8)
+    _lib.check(L.sq_stream_build(host.data_ptr(), R, W, C, d, bits, runs, out.data_ptr(), n))
+    return out.to(words.device), L.sq_stream_runs(R, C, d, bits, runs)
+
+
+def prepare_stack(pieces, workgroups: int = 512) -> None:
+    """Cut the streams of pieces that are launched together so that the launch makes about `workgroups`
+    workgroups in total (two per CU on an MI355X), shared by rows.  Pieces without a stream are left alone."""
+    ps = [p for p in pieces if p.stream is not None]
+    rows = sum(p.R for p in ps)
+    for p in ps:
+        buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // 640)
+        runs = max(1, round(workgroups * p.R / rows / buckets))
+        if _lib.lib().sq_stream_runs(p.R, p.C, p.d, p.bits, runs) != p.stream_runs:
+            p.build_stream(runs)
 
 
 def _prep(pieces, x: torch.Tensor, y: torch.Tensor):

@@ -23,7 +23,7 @@ import re
 import torch
 
 from .. import _lib
-from ..kernels import PackedLinear, _Workspace, gemm_dense, linear_gemm, linear_small
+from ..kernels import PackedLinear, _Workspace, gemm_dense, linear_gemm, linear_small, prepare_stack
 
 BMAX = _lib.SMALL_BMAX
 
@@ -134,6 +134,8 @@ class PackedShards:
         self.cross = bmax            # M <= cross: small path, else the large-M path (tune() moves it)
         self.device = rls[0].device
         self.sq_name = ""            # set by the vLLM plugin (layer prefix)
+        if len(rls) > 1:
+            prepare_stack(self.rls)  # tag streams cut for a joint launch of these pieces
 
     @classmethod
     def from_packed(cls, pf, names: list, dev="cuda", **kw) -> "PackedShards":
@@ -147,7 +149,7 @@ class PackedShards:
     def nbytes(self) -> int:
         n = 0
         for rl in self.rls:
-            for t in (rl.words, rl.table, rl.row_scale, rl.row_book, rl.row_mask, rl.perms, rl.row_order):
+            for t in (rl.words, rl.table, rl.row_scale, rl.row_book, rl.row_mask, rl.perms, rl.row_order, rl.stream):
                 if t is not None:
                     n += t.numel() * t.element_size()
         return n
@@ -212,7 +214,7 @@ class PackedShards:
         rows = max(self.Rs)
         if self.large == "chunked":
             rows = min(rows, max(128, (self.chunk_bytes // (2 * self.C)) // 128 * 128))
-        scratch = _Workspace.get(rows * self.C * 2, x.device).view(torch.float16)
+        scratch = _Workspace.get(rows * self.C * 2, x.device, kind="dense").view(torch.float16)
         for rl, off in zip(self.rls, self.offs):
             for r0 in range(0, rl.R, rows):
                 r1 = min(rl.R, r0 + rows)

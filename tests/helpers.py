@@ -50,12 +50,12 @@ def synth(R, C, d, bits, G=1, M=1, seed=0, table_scale=0.5) -> Synth:
     return Synth(R, C, d, bits, G, M, tags, O.pack_bits(tags, bits), table, rs, rb, rm, perms)
 
 
-def to_device(s: Synth, dev="cuda"):
+def to_device(s: Synth, dev="cuda", stream=True):
     """PackedLinear on the GPU from a Synth."""
     from quantexperiments_amd.kernels import PackedLinear
     t = lambda a: None if a is None else torch.from_numpy(a).to(dev)
     return PackedLinear(t(s.words), t(s.table), t(s.row_scale), t(s.row_book), t(s.row_mask),
-                        torch.from_numpy(s.perms).to(dev), s.K, s.d)
+                        torch.from_numpy(s.perms).to(dev), s.K, s.d, stream=stream)
 
 
 def rand_x(B, C, dtype, seed=0, scale=1.0):

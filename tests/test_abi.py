@@ -26,13 +26,13 @@ def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     for name in _declared():
         assert getattr(L, name) is not None, name
-    assert L.sq_version() == 100
+    assert L.sq_version() == 101
 
 
 def test_struct_layout_matches_header():
-    # 7 pointers + 8 int32
-    assert ctypes.sizeof(_lib.SqMatrix) == 7 * 8 + 8 * 4
-    assert _lib.SqMatrix.R.offset == 56 and _lib.SqMatrix.y_off.offset == 56 + 28
+    # 7 pointers + 8 int32 + 1 pointer + 2 int32
+    assert ctypes.sizeof(_lib.SqMatrix) == 7 * 8 + 8 * 4 + 8 + 8
+    assert _lib.SqMatrix.R.offset == 56 and _lib.SqMatrix.y_off.offset == 56 + 28 and _lib.SqMatrix.stream.offset == 88
 
 
 def test_host_side_argument_checks():
@@ -72,6 +72,6 @@ def test_workspace_sizes_are_host_arithmetic():
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 1, 0) == 0
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == 0
     # from 256 activation rows on: raw fp16 codewords of the largest piece + an fp16 copy of the activations
-    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 64 * 512 * 2 + 2048 * 512 * 2
-    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == 16 * 2 * 512 * 2
-    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == 64 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 4096 + 64 * 512 * 2 + 2048 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == 4096 + 16 * 2 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == 4096 + 64 * 512 * 2

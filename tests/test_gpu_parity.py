@@ -158,10 +158,67 @@ def test_large_products_do_not_overflow():
     assert torch.isfinite(y).all() and rel_max_err(y.cpu().numpy(), ref) < 1e-5
 
 
+# ------------------------------------------------------------------ bucketed tag stream (codebooks beyond LDS, B = 1)
+STREAM = [  # R, C, bits
+    (70, 512, 16), (130, 5376, 16), (260, 3584, 16), (64, 1024, 15), (333, 2048, 14), (1, 8, 16), (65, 18944, 16),
+]
+
+
+@pytest.mark.parametrize("case", STREAM, ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_stream_gemv_matches_oracle_and_row_path(case, dtype):
+    from quantexperiments_amd.kernels import linear_small
+    R, C, bits = case
+    s = synth(R, C, 8, bits, seed=sum(case))
+    if R > 5:
+        s.tags[5] = 7                                   # a row whose tags all sit in one codebook slice
+        s.tags[4, ::2] = (1 << bits) - 1
+        s.words = O.pack_bits(s.tags, bits)
+    lin, plain = to_device(s), to_device(s, stream=False)
+    assert lin.stream is not None and plain.stream is None
+    x = rand_x(1, C, dtype, seed=R)
+    ref = _ref(s, x)
+    y32 = torch.full((1, R), 9.0, dtype=torch.float32, device="cuda")
+    linear_small([lin], x.cuda(), y32)
+    assert rel_max_err(y32.cpu().numpy(), ref) < TOL
+    yp = torch.empty(1, R, dtype=torch.float32, device="cuda")
+    linear_small([plain], x.cuda(), yp)
+    assert rel_max_err(y32.cpu().numpy(), yp.cpu().numpy().astype(np.float64)) < 1e-5
+    _check_lowp(lin.gemv(x.cuda()[0])[None], ref)
+    # the same buffers again: results do not depend on scheduling
+    y2 = torch.empty_like(y32)
+    linear_small([lin], x.cuda(), y2)
+    assert torch.equal(y2, y32)
+    # another cut into row runs: same sums up to the order of fp32 additions within a row
+    for runs in (1, 3):
+        lin.build_stream(runs)
+        linear_small([lin], x.cuda(), y2)
+        assert rel_max_err(y2.cpu().numpy(), y32.cpu().numpy().astype(np.float64)) < 1e-5
+
+
+def test_stream_padding_never_touches_the_codebook():
+    # codeword 0 of every slice is inf and no tag names it: padded stream entries (tag 0) must not leak into a sum
+    from quantexperiments_amd.kernels import linear_small
+    s = synth(100, 1024, 8, 16, seed=11)
+    s.tags[s.tags % 4096 == 0] += 1
+    s.words = O.pack_bits(s.tags, 16)
+    s.table[::4096] = np.float16(np.inf)
+    lin = to_device(s)
+    x = rand_x(1, s.C, torch.bfloat16, seed=3)
+    y = torch.empty(1, s.R, dtype=torch.float32, device="cuda")
+    linear_small([lin], x.cuda(), y)
+    tab = s.table.copy()
+    tab[::4096] = 0
+    ref = c_oracle.linear(_xf(x), O.decode_tensors(s.tags, tab, s.row_scale, None, None, s.perms, s.K))
+    assert torch.isfinite(y).all() and rel_max_err(y.cpu().numpy(), ref) < TOL
+
+
 def test_stacked_pieces_write_their_column_slices():
     from quantexperiments_amd.kernels import linear_small
+    from quantexperiments_amd.kernels import prepare_stack
     ss = [synth(R, 3584, 8, 16, seed=R) for R in (260, 70, 70)]
     lins = [to_device(s) for s in ss]
+    prepare_stack(lins)
     for B in (1, 4, 6):
         x = rand_x(B, 3584, torch.bfloat16, seed=B)
         y = torch.full((B, 400 + 16), 7.0, dtype=torch.float32, device="cuda")       # row stride wider than sum R

@@ -174,3 +174,89 @@ def test_neutral_defaults_and_registry():
     # the fake (meta) implementation gives the output shape without touching a kernel
     y = torch.ops.shapequant.linear(torch.empty(2, 3, 5, device="meta"), h)
     assert y.shape == (2, 3, 7) and y.device.type == "meta"
+
+
+# ---------------------------------------------------------------------------- bucketed tag stream (host builder)
+
+def _walk_stream(buf, R, C, d, bits, runs):
+    """Rebuild the [R, C/d] tag matrix from a stream buffer cut into `runs` row runs, checking its structure
+    on the way."""
+    U, NS = C // d, 1 << (bits - 12)
+    KP = -(-U // 640)
+    PC = -(-U // KP)
+    NV, NG = NS * KP, -(-R // 64)
+    RR = -(-NG // runs) * 64                                                  # rows per run
+    assert -(-NG * 64 // RR) == runs
+    off_slots = ((NV * NG + 1) * 4 + 255) & ~255
+    off_steps = (off_slots + NV * NG * 64 * 4 + 255) & ~255
+    goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
+    slots = np.frombuffer(buf, np.uint32, NV * NG * 64, off_slots).reshape(NV, NG * 64)
+    assert goff[0] == 0 and (np.diff(goff.astype(np.int64)) >= 0).all()
+    assert len(buf) == off_steps + int(goff[-1]) * 768
+    steps = np.frombuffer(buf, np.uint8, int(goff[-1]) * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.uint32)
+    ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
+    tags = np.full((R, U), -1, np.int64)
+    for v in range(NV):
+        kp, s = divmod(v, NS)
+        rows = slots[v] & 0x7FFFF
+        cnts = slots[v] >> 19
+        real = rows != 0x7FFFF
+        assert sorted(rows[real].tolist()) == list(range(R))                  # every row once per bucket
+        for r0 in range(0, NG * 64, RR):                                      # sorted by count within each run
+            blk = cnts[r0:r0 + RR][real[r0:r0 + RR]].astype(np.int64)
+            assert (np.diff(blk) <= 0).all()
+            assert sorted(rows[r0:r0 + RR][real[r0:r0 + RR]].tolist()) == list(range(r0, min(R, r0 + RR)))
+        for g in range(NG):
+            n = int(goff[v * NG + g + 1]) - int(goff[v * NG + g])
+            assert n == -(-int(cnts[g * 64]) // 4)                            # padded to the group's longest row
+            e = ent[int(goff[v * NG + g]):int(goff[v * NG + g + 1])]          # [n, 64, 4]
+            e = e.transpose(1, 0, 2).reshape(64, n * 4)
+            for lane in range(64):
+                k = g * 64 + lane
+                if not real[k]:
+                    assert (e[lane] == 0).all()
+                    continue
+                c = int(cnts[k])
+                assert (e[lane, c:] == 0).all()                               # padding is zero
+                chunk = (e[lane, :c] >> 12) + kp * PC
+                assert (np.diff(chunk.astype(np.int64)) > 0).all() and (chunk < min(U, (kp + 1) * PC)).all()
+                assert (tags[rows[k], chunk] == -1).all()
+                tags[rows[k], chunk] = (e[lane, :c] & 0xFFF) + (s << 12)
+    return tags
+
+
+@pytest.mark.parametrize("R,C,bits,runs", [(70, 512, 16, 0), (130, 5376, 16, 2), (64, 1024, 13, 5), (1, 8, 14, 0),
+                                            (1100, 256, 15, 4), (1100, 256, 15, 7)])
+def test_stream_builder_keeps_every_tag(R, C, bits, runs):
+    import ctypes
+    from quantexperiments_amd import _lib
+    from oracle import sq_oracle as O
+    L = _lib.lib()
+    rng = np.random.default_rng(R + C)
+    U = C // 8
+    tags = rng.integers(0, 1 << bits, (R, U))
+    if R > 3:
+        tags[3] = 5                                                           # one row entirely in slice 0
+    words = np.ascontiguousarray(O.pack_bits(tags, bits))
+    W = words.shape[1]
+    ptr = words.ctypes.data_as(ctypes.c_void_p)
+    n = L.sq_stream_bytes(ptr, R, W, C, 8, bits, runs)
+    assert n > 0
+    eff = L.sq_stream_runs(R, C, 8, bits, runs)
+    assert 1 <= eff <= -(-R // 64) and (runs == 0 or eff <= runs)
+    out = np.zeros(n, np.uint8)
+    assert L.sq_stream_build(ptr, R, W, C, 8, bits, runs, out.ctypes.data_as(ctypes.c_void_p), n) == 0
+    assert np.array_equal(_walk_stream(out.tobytes(), R, C, 8, bits, eff), tags)
+    assert L.sq_stream_build(ptr, R, W, C, 8, bits, runs, out.ctypes.data_as(ctypes.c_void_p), n - 1) == _lib.SQ_EINVAL
+
+
+def test_stream_builder_rejects_other_formats():
+    import ctypes
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    words = np.zeros((4, 16), np.int32)
+    ptr = words.ctypes.data_as(ctypes.c_void_p)
+    assert L.sq_stream_bytes(ptr, 4, 16, 128, 4, 16, 0) == 0                  # d = 4
+    assert L.sq_stream_bytes(ptr, 4, 16, 128, 8, 12, 0) == 0                  # codebook fits LDS: no stream
+    assert L.sq_stream_runs(4, 128, 8, 12, 0) == 0
+    assert L.sq_stream_build(ptr, 4, 16, 128, 8, 12, 0, ptr, 64) == _lib.SQ_EUNSUPPORTED
