@@ -8,6 +8,10 @@ the serving path runs it: 4 launches (q|k|v stacked, o, gate|up stacked, down) t
 Steps rotate over enough distinct layers (>= 4x the 256 MB last-level cache) that tags stream from
 HBM.  K steps are captured in one HIP graph and timed between device synchronisations.
 
+The batch-1 kernels read a load-time regrouping of the tags by codebook slice (about 3.5 bytes per
+tag in HBM instead of the file's 2), built by the library when a layer is loaded; value still counts
+the packed file's bytes, which is what the metric is quoted on.
+
 value = packed (algorithmic) bytes of a layer / time per layer, in GB/s.  The same JSON line
 carries us_per_layer, the roofline of the dominant kernel (gate|up launch, HIP events around graph
 replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s, and the CPU baseline (the
@@ -27,6 +31,9 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes one gate|up launch of stream_kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (37,815.7 KiB x 1.9998 read + 15,263.5 KiB x 1.0 written; scale factors from a 256 MiB copy in the same runs)
+GATE_UP_TRAFFIC_BYTES = 93_070_000
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16
 
 SHAPES_7B = {"q": (3584, 3584), "k": (512, 3584), "v": (512, 3584), "o": (3584, 3584),
@@ -46,8 +53,9 @@ def algorithmic_bytes(names, B=1):
 
 
 def make_layer(torch, dev, gen):
-    """One layer of PackedLinear pieces with seeded synthetic contents, generated on the device."""
-    from quantexperiments_amd.kernels import PackedLinear
+    """One layer of PackedLinear pieces with seeded synthetic contents, generated on the device; the pieces of
+    each launch get their load-time tag streams cut for that launch (as PackedShards does at load)."""
+    from quantexperiments_amd.kernels import PackedLinear, prepare_stack
     out = {}
     for nm, (R, C) in SHAPES_7B.items():
         W = (C // D) * BITS // 32
@@ -55,6 +63,8 @@ def make_layer(torch, dev, gen):
         table = torch.randn(1 << BITS, D, device=dev, generator=gen).to(torch.float16)
         rs = (torch.randn(R, device=dev, generator=gen) * 0.005 + 0.02).abs().to(torch.float16)
         out[nm] = PackedLinear(words, table, rs, None, None, torch.arange(C, device=dev)[None], 1 << BITS, D)
+    for l in LAUNCHES:
+        prepare_stack([out[n] for n in l])
     return out
 
 
@@ -117,6 +127,16 @@ def prefill(torch, dev, layer, steps=3):
     return res
 
 
+def copy_probe(torch, dev):
+    """Three 256 MiB device-to-device copies: a kernel of known HBM traffic to scale profiler counters by."""
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    return {"bytes_read": 256 << 20, "bytes_written": 256 << 20, "launches": 3}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -125,6 +145,11 @@ def main():
     ap.add_argument("--layers", type=int, default=28, help="distinct layers the steps rotate over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="run only the dominant launch (gate|up) and print only its roofline object: the command "
+                         "the rocprofv3 summaries under profiles/ are made with")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three 256 MiB device copies (a kernel of known traffic to scale rocprofv3 counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the one-GPU hot path; multi-GPU runs are not part of this build (use --gpus 1)")
@@ -145,6 +170,24 @@ def main():
         for l in LAUNCHES:
             linear_small([L[n] for n in l], x[SHAPES_7B[l[0]][1]], y[l])
 
+    gu = LAUNCHES[2]
+    if args.roofline_only:
+        def gate_up_only():
+            for L in layers:
+                linear_small([L[n] for n in gu], x[3584], y[gu])
+        ms, g2 = timed_graph(torch, gate_up_only)
+        del g2
+        dur_us = ms * 1e3 / len(layers)
+        out = {"roofline": {"bound": "hbm", "kernel": "sq::stream_kernel (gate|up launch, 2 x 18944x3584)",
+                            "achieved": algorithmic_bytes(gu) / (dur_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": algorithmic_bytes(gu) / (dur_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                            "bytes_per_launch": algorithmic_bytes(gu), "us_per_launch": dur_us, "traffic": GATE_UP_TRAFFIC_BYTES,
+                            "stream_bytes_per_launch": sum(layers[0][n].stream.numel() for n in gu)}}
+        if args.copy_probe:
+            out["copy_probe"] = copy_probe(torch, dev)
+        print(json.dumps(out))
+        return
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -164,7 +207,6 @@ def main():
     value = layer_bytes / (ms_per_step * 1e-3) / 1e9
 
     # dominant kernel: the gate|up launch alone, over all layers, HIP events around graph replays
-    gu = LAUNCHES[2]
 
     def gate_up_all():
         for L in layers:
@@ -194,10 +236,13 @@ def main():
         "us_per_layer": ms_per_step * 1e3,
         "tag_only_GBps": tag_bytes / (ms_per_step * 1e-3) / 1e9,
         "per_launch": per_launch,
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<16,8,1,1,false> (gate|up launch, 2 x 18944x3584)",
+        "roofline": {"bound": "hbm", "kernel": "sq::stream_kernel (gate|up launch, 2 x 18944x3584)",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "bytes_per_launch": gu_bytes, "us_per_launch": dur_us, "traffic": None},
+                     "bytes_per_launch": gu_bytes, "us_per_launch": dur_us, "traffic": GATE_UP_TRAFFIC_BYTES,
+                     "stream_bytes_per_launch": sum(layers[0][n].stream.numel() for n in gu)},
     }
+    if args.copy_probe:
+        out["copy_probe"] = copy_probe(torch, dev)
     if not args.no_prefill:
         pf = prefill(torch, dev, layers[0])
         out["prefill"] = {"M": 2048, "gate_18944x3584": pf["gate"], "down_3584x18944": pf["down"],

@@ -190,6 +190,11 @@ constexpr int STREAM_NW = 8;          // waves per workgroup
 
 struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
 
+// Optional per-wave timeline (debug builds define SQ_TRACE_POINT).
+#ifndef SQ_TRACE_POINT
+#define SQ_TRACE_POINT(k)
+#endif
+
 __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     constexpr int NW = STREAM_NW;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -202,65 +207,80 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     const int local = (int)blockIdx.x - P.wg_begin;
     const int v = local / P.nwg, wi = local - v * P.nwg;
     const int s = v % P.NS, kp = v / P.NS;
-    // this workgroup's run: groups g0 .. g1 - 1 of the bucket
-    const int g0 = wi * P.GR, g1 = min(P.NG, g0 + P.GR);
+    SQ_TRACE_POINT(0);
+    // this workgroup's run: groups g0 .. g0 + ng - 1 of the bucket
+    const int g0 = wi * P.GR, ng = min(P.NG, g0 + P.GR) - g0;
 
-    const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG;
-    const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + (size_t)v * P.NG * 64;
+    const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG + g0;
+    const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
     const unsigned char* steps = P.stream + P.off_steps + lane * 12;
     float* part = P.part + (size_t)v * P.R;
+    unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_X_OFF + P.PC * 16);   // [0] arrival result, [1] next group
 
-    // The groups of a run are sorted longest first; wave w takes the w-th of the first eight, the (7 - w)-th of
-    // the next eight and so on, which evens out the waves' shares.  The head of a group (its first step, its
-    // step count, the lane's row and count) is fetched one group ahead; the first one goes out before the
-    // staging loads.
-    auto group_of = [&](int k) { return g0 + k * NW + ((k & 1) ? NW - 1 - wave : wave); };
+    // The groups of a run are sorted longest first.  Wave w starts with group w, then group 15 - w; after
+    // that every wave draws the next unclaimed group from a counter in LDS, so all waves stay busy to the end.
+    // The head of a group (its first step, its step count, the lane's row and count) is fetched one group
+    // ahead; the first one goes out before the staging loads.
     auto head = [&](int k) {
         StreamHead h{0u, 0, STREAM_NO_ROW};
-        const int g = group_of(k);
-        if (g < g1) {
-            h.st0 = goff[g];
-            h.nst = (int)(goff[g + 1] - h.st0);
-            h.slot = slots[(size_t)g * 64 + lane];
+        if (k < ng) {
+            h.st0 = goff[k];
+            h.nst = (int)(goff[k + 1] - h.st0);
+            h.slot = slots[(size_t)k * 64 + lane];
         }
         return h;
     };
-    StreamHead hn = head(0);
-    const int nk = (g1 - g0 + NW - 1) / NW;
+    auto first_steps = [&](const StreamHead& h, u32x3* nx) {
+        if (h.nst > 0) {                                        // wave-uniform
+            const unsigned char* en = steps + (size_t)h.st0 * 768;
+#pragma unroll
+            for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, h.nst - 1) * 768);
+        }
+    };
+    int kcur = wave, knext = 2 * NW - 1 - wave;
+    StreamHead hn = head(kcur);
+    u32x3 nx[STREAM_PF];
+#pragma unroll
+    for (int q = 0; q < STREAM_PF; ++q) nx[q] = u32x3{0u, 0u, 0u};
 
-    // stage the codebook slice and this part of x (as fp16)
+    // stage the codebook slice and this part of x (as fp16); the first group's steps are requested before the
+    // LDS stores wait for the staging loads
     {
         const u32x4* src = reinterpret_cast<const u32x4*>(P.table) + (size_t)s * (1 << STREAM_SLICE_BITS);
         u32x4* dst = reinterpret_cast<u32x4*>(lds);
-        u32x4 t[(1 << STREAM_SLICE_BITS) / (NW * 64)];
+        constexpr int NT = (1 << STREAM_SLICE_BITS) / (NW * 64);
+        u32x4 t[NT], xq[2];
 #pragma unroll
-        for (int k = 0; k < (1 << STREAM_SLICE_BITS) / (NW * 64); ++k) t[k] = src[tid + k * NW * 64];
+        for (int k = 0; k < NT; ++k) t[k] = src[tid + k * NW * 64];
         const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
         const u32x4* xs = reinterpret_cast<const u32x4*>(a.x) + c0;
         u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_X_OFF);
-        for (int k = tid; k < nc; k += NW * 64) {
-            u32x4 q = xs[k];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) xq[k] = xs[min(tid + k * NW * 64, nc - 1)];      // PC <= 640 < 2 * 512
+        first_steps(hn, nx);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            u32x4 q = xq[k];
             if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
-            xd[k] = q;
+            if (tid + k * NW * 64 < nc) xd[tid + k * NW * 64] = q;
         }
 #pragma unroll
-        for (int k = 0; k < (1 << STREAM_SLICE_BITS) / (NW * 64); ++k) dst[tid + k * NW * 64] = t[k];
-    }
-    // first steps of the first group: in flight across the barrier
-    u32x3 nx[STREAM_PF];
-    {
-        const unsigned char* eb = steps + (size_t)hn.st0 * 768;
-#pragma unroll
-        for (int k = 0; k < STREAM_PF; ++k) {
-            nx[k] = u32x3{0u, 0u, 0u};
-            if (hn.nst > 0) nx[k] = *reinterpret_cast<const u32x3*>(eb + (size_t)min(k, hn.nst - 1) * 768);
-        }
+        for (int k = 0; k < NT; ++k) dst[tid + k * NW * 64] = t[k];
+        if (tid == 0) flag[1] = 2 * NW;
     }
     __syncthreads();
+    SQ_TRACE_POINT(1);
 
-    for (int k = 0; k < nk; ++k) {
+    while (kcur < ng) {
         const StreamHead h = hn;
-        hn = k + 1 < nk ? head(k + 1) : StreamHead{0u, 0, STREAM_NO_ROW};
+        hn = head(knext);
+        int kafter = ng;
+        if (knext < ng) {
+            unsigned tk = 0;
+            if (lane == 0) tk = __hip_atomic_fetch_add(flag + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            kafter = (int)__builtin_amdgcn_readfirstlane(tk);
+        }
         const int nst = h.nst;
         const int cnt = (int)(h.slot >> STREAM_ROW_BITS);
         const uint32_t row = h.slot & STREAM_NO_ROW;
@@ -274,11 +294,8 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
                 for (int q = 0; q < STREAM_PF; ++q)
                     nx[q] = *reinterpret_cast<const u32x3*>(eb + (size_t)min(t0 + STREAM_PF + q, nst - 1) * 768);
-            } else if (hn.nst > 0) {                            // the next group's first steps
-                const unsigned char* en = steps + (size_t)hn.st0 * 768;
-#pragma unroll
-                for (int q = 0; q < STREAM_PF; ++q)
-                    nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, hn.nst - 1) * 768);
+            } else {
+                first_steps(hn, nx);                            // the next group's first steps
             }
 #pragma unroll
             for (int q = 0; q < STREAM_PF; ++q) {
@@ -301,42 +318,70 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                 }
             }
         }
-        if (nst == 0 && hn.nst > 0) {                           // a group without steps fetched nothing for its successor
-            const unsigned char* en = steps + (size_t)hn.st0 * 768;
-#pragma unroll
-            for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, hn.nst - 1) * 768);
-        }
+        if (nst == 0) first_steps(hn, nx);                      // a group without steps fetched nothing for its successor
         // device-scope store: written through to memory, so other XCDs' L2s never hold a stale copy and no
         // cache-wide write-back is needed before the workgroup counts itself off
         if (row != STREAM_NO_ROW) __hip_atomic_store(part + row, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        kcur = knext;
+        knext = kafter;
     }
 
     // Count this workgroup off once all its partial sums have been acknowledged (the barrier waits for every
     // wave's outstanding stores).  The workgroup that finds every other bucket's workgroup already counted
     // reads all partial sums back with device-scope loads and finishes the rows.
-    unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_X_OFF + P.PC * 16);
+    SQ_TRACE_POINT(2);
     __builtin_amdgcn_s_waitcnt(0);
+    SQ_TRACE_POINT(3);
     __syncthreads();
+    SQ_TRACE_POINT(4);
     if (tid == 0) {
         const unsigned old = atomicAdd(P.counters + wi, 1u);
         if (old == (unsigned)P.NV - 1u) P.counters[wi] = 0u;    // everyone has arrived: leave the counter as found
-        *flag = old;
+        flag[0] = old;
     }
     __syncthreads();
-    if (*flag != (unsigned)P.NV - 1u) return;
-    const int r0 = g0 * 64, r1 = min(P.R, g1 * 64);
-    for (int r = r0 + tid; r < r1; r += NW * 64) {
-        float sum = 0.f;
-        for (int v0 = 0; v0 < P.NV; v0 += 16) {                 // NV is a multiple of the slice count, a power of two >= 2
-            float t[16];
+    SQ_TRACE_POINT(5);
+    if (flag[0] != (unsigned)P.NV - 1u) return;
+    // 64 partial sums in flight per thread: four rows at a time when a row has 16 buckets, else one row's
+    // buckets 64 at a time; a row's partials are always added in bucket order
+    const int r0 = g0 * 64, r1 = min(P.R, (g0 + ng) * 64);
+    const float* pp = P.part;
+    if (P.NV <= 16) {
+        for (int rb = r0 + tid; rb < r1; rb += 4 * NW * 64) {
+            float t[4][16];
 #pragma unroll
-            for (int k = 0; k < 16; ++k)
-                t[k] = v0 + k < P.NV ? __hip_atomic_load(P.part + (size_t)(v0 + k) * P.R + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+            for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int k = 0; k < 16; ++k) sum += t[k];
+                for (int k = 0; k < 16; ++k) {
+                    const int r = rb + q * NW * 64;
+                    t[q][k] = (r < r1 && k < P.NV)
+                                  ? __hip_atomic_load(pp + (size_t)k * P.R + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+                }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int r = rb + q * NW * 64;
+                float sum = 0.f;
+#pragma unroll
+                for (int k = 0; k < 16; ++k) sum += t[q][k];
+                if (r < r1) store_y(a.y, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
+            }
         }
-        store_y(a.y, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
+    } else {
+        for (int r = r0 + tid; r < r1; r += NW * 64) {
+            float sum = 0.f;
+            for (int v0 = 0; v0 < P.NV; v0 += 64) {
+                float t[64];
+#pragma unroll
+                for (int k = 0; k < 64; ++k)
+                    t[k] = v0 + k < P.NV
+                               ? __hip_atomic_load(pp + (size_t)(v0 + k) * P.R + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+#pragma unroll
+                for (int k = 0; k < 64; ++k) sum += t[k];
+            }
+            store_y(a.y, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
+        }
     }
+    SQ_TRACE_POINT(6);
 }
 
 static int stream_launch(const StreamArgs& a, int grid, size_t smem, hipStream_t s) {
@@ -370,7 +415,7 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     a.x_dtype = x_dtype;
     a.y_dtype = y_dtype;
     const StreamGeom g0 = stream_geom(mats[0].R, mats[0].C, mats[0].d, mats[0].bits, mats[0].stream_runs);
-    const size_t smem = (size_t)STREAM_X_OFF + (size_t)g0.PC * 16 + 16;
+    const size_t smem = (size_t)STREAM_X_OFF + (size_t)g0.PC * 16 + 16;      // slice, x part, two words of flags
     (void)cus;
     int wg = 0;
     for (int k = 0; k < cnt; ++k) {
