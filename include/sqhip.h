@@ -43,8 +43,8 @@ typedef struct sq_matrix {
     int32_t R, C, d, bits, G, M, W;
     int32_t y_off;              /* first output column of this piece in the stacked Y */
     const void*     stream;     /* optional: device copy of the buffer sq_stream_build wrote for `tags`; NULL = none */
-    int32_t stream_runs;        /* what sq_stream_runs returned for that buffer */
-    int32_t reserved;           /* 0 */
+    int32_t stream_runs;        /* runs_out of sq_stream_build for that buffer */
+    int32_t stream_groups;      /* groups_out of sq_stream_build for that buffer */
 } sq_matrix;
 
 /* Library / device identification.  sq_version: ABI version (major*100 + minor). */
@@ -94,18 +94,24 @@ int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C,
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which);
 
 /* Load-time regrouping of a matrix' tags for codebooks that do not fit LDS (d = 8, K = 8192..65,536, one
- * codebook, no column orders): the batch-1 product then gathers codewords from a 64 KB LDS slice instead of
- * from L2.  HOST pointers: `tags_host` is the file's tag tensor in host memory, `out_host` receives
- * sq_stream_bytes() bytes that the caller copies to the device (16-byte aligned) and names in
- * sq_matrix.stream.  sq_stream_bytes returns 0 for formats the stream does not cover.  The tags tensor
- * stays the source of truth (sq_dequant, B > 1 and the prefill GEMM read it); this plays the part of the
- * reference's load-time run-length layout (reference shapequant/kernels/proto_runs.py:178-260
- * build_runs / RunsLayout), with a layout chosen for LDS gathers rather than run-length grouping. */
-int32_t sq_stream_runs(int32_t R, int32_t C, int32_t d, int32_t bits, int32_t runs);
+ * codebook): the batch-1 product then gathers codewords from a 64 KB LDS slice instead of from L2.
+ * HOST pointers: `tags_host` is the file's tag tensor in host memory, `row_mask_host` the file's row_mask
+ * (NULL when the matrix has one column order), `out_host` receives sq_stream_bytes() bytes that the caller
+ * copies to the device (16-byte aligned) and names in sq_matrix.stream, together with *runs_out and
+ * *groups_out in sq_matrix.stream_runs / stream_groups.  sq_stream_bytes returns 0 for formats the stream does
+ * not cover.  `runs` asks for that many row runs; each run becomes 2^(bits - 12) * ceil(C / 5120) workgroups
+ * of the batch-1 launch, so pick it to give the pieces launched together about two workgroups per CU in
+ * total (0 = a good value for a matrix launched alone); rows with different column orders never share a run,
+ * so *runs_out can exceed the request.  A matrix with column orders must be given to sq_linear_small with
+ * the same row_mask and with perms on the device.  The tags tensor stays the source of truth (sq_dequant,
+ * B > 1 and the prefill GEMM read it); this plays the part of the reference's load-time layouts (reference
+ * shapequant/kernels/proto_runs.py:295-349 pack_lane_major / RunsLinear, batched_runs.py:213-373 tile_words),
+ * with a layout chosen for LDS gathers. */
 size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
-                       int32_t runs);
+                       const uint8_t* row_mask_host, int32_t runs);
 int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
-                    int32_t runs, void* out_host, size_t out_bytes);
+                    const uint8_t* row_mask_host, int32_t runs, void* out_host, size_t out_bytes,
+                    int32_t* runs_out, int32_t* groups_out);
 
 #ifdef __cplusplus
 }

@@ -24,7 +24,7 @@ class SqMatrix(ctypes.Structure):
                 ("row_order", ctypes.c_void_p),
                 ("R", ctypes.c_int32), ("C", ctypes.c_int32), ("d", ctypes.c_int32), ("bits", ctypes.c_int32),
                 ("G", ctypes.c_int32), ("M", ctypes.c_int32), ("W", ctypes.c_int32), ("y_off", ctypes.c_int32),
-                ("stream", ctypes.c_void_p), ("stream_runs", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("stream", ctypes.c_void_p), ("stream_runs", ctypes.c_int32), ("stream_groups", ctypes.c_int32)]
 
 
 class SqError(RuntimeError):
@@ -55,11 +55,10 @@ def lib() -> ctypes.CDLL:
         L.sq_gemm_dense.argtypes = [vp, ctypes.c_int, i64, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp]
         L.sq_workspace_bytes.argtypes = [mp, i32, i32, ctypes.c_int]
         L.sq_workspace_bytes.restype = sz
-        L.sq_stream_runs.argtypes = [i32, i32, i32, i32, i32]
-        L.sq_stream_runs.restype = i32
-        L.sq_stream_bytes.argtypes = [vp, i32, i32, i32, i32, i32, i32]
+        ip = ctypes.POINTER(ctypes.c_int32)
+        L.sq_stream_bytes.argtypes = [vp, i32, i32, i32, i32, i32, vp, i32]
         L.sq_stream_bytes.restype = sz
-        L.sq_stream_build.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, sz]
+        L.sq_stream_build.argtypes = [vp, i32, i32, i32, i32, i32, vp, i32, vp, sz, ip, ip]
         L.sq_stream_build.restype = ctypes.c_int
         for f in (L.sq_dequant, L.sq_linear_small, L.sq_linear_gemm, L.sq_gemm_dense):
             f.restype = ctypes.c_int
@@ -68,7 +67,7 @@ def lib() -> ctypes.CDLL:
 
 
 EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
-           "sq_workspace_bytes", "sq_stream_runs", "sq_stream_bytes", "sq_stream_build")
+           "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build")
 
 
 def check(rc: int) -> None:

@@ -125,22 +125,20 @@ size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, i
     return inner ? inner + SQ_WS_HEADER : 0;
 }
 
-int32_t sq_stream_runs(int32_t R, int32_t C, int32_t d, int32_t bits, int32_t runs) {
-    if (d <= 0 || !stream_format_ok(R, C, d, bits)) return 0;
-    return stream_geom(R, C, d, bits, runs).runs;
-}
-
-size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t runs) {
+size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                       const uint8_t* row_mask_host, int32_t runs) {
     if (!tags_host || d <= 0 || !stream_format_ok(R, C, d, bits) || (int64_t)W * 32 < (int64_t)(C / d) * bits) return 0;
-    return stream_bytes_host((const uint32_t*)tags_host, R, W, C, d, bits, runs);
+    return stream_bytes_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs);
 }
 
-int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t runs,
-                    void* out_host, size_t out_bytes) {
-    if (!tags_host || !out_host) return fail(SQ_EINVAL, "sq_stream_build: null pointer");
+int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                    const uint8_t* row_mask_host, int32_t runs, void* out_host, size_t out_bytes, int32_t* runs_out,
+                    int32_t* groups_out) {
+    if (!tags_host || !out_host || !runs_out || !groups_out) return fail(SQ_EINVAL, "sq_stream_build: null pointer");
     if (d <= 0 || !stream_format_ok(R, C, d, bits)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: d %d bits %d R %d not covered", d, bits, R);
     if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_stream_build: W %d too small", W);
-    return stream_build_host((const uint32_t*)tags_host, R, W, C, d, bits, runs, (unsigned char*)out_host, out_bytes);
+    return stream_build_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs, (unsigned char*)out_host,
+                             out_bytes, runs_out, groups_out);
 }
 
 }  // extern "C"

@@ -15,15 +15,16 @@ constexpr int STREAM_DEFAULT_WGS = 512;      // workgroups a matrix launched alo
 
 struct StreamGeom {
     int U, NS, KP, PC, NV, NG;               // chunks per row, slices, column parts, chunks per part, buckets, groups
-    int GR, runs;                            // groups per run of rows, runs
-    size_t off_slots, off_steps;             // byte offsets inside the stream buffer
+    int runs;
+    size_t off_slots, off_runs, off_rows, off_steps;   // byte offsets inside the stream buffer
     uint64_t total_steps;                    // filled by the builder only
 };
 
-StreamGeom stream_geom(int R, int C, int d, int bits, int runs);
+StreamGeom stream_geom(int C, int d, int bits, int groups, int runs);
 bool stream_format_ok(int R, int C, int d, int bits);
-size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs);
-int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs, unsigned char* out, size_t bytes);
+size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs);
+int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
+                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out);
 bool stream_shape(const sq_matrix& m);
 size_t stream_part_bytes(const sq_matrix& m);
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, void* y, int y_dtype, char* ws,

@@ -8,22 +8,27 @@
 //   entry            24 bits: tag & 4095 | (chunk - kp * PC) << 12
 //   lane task        the entries of one row in one bucket (about C/d / (KP * NS) of them)
 //
-// Rows are cut into `runs` runs of GR * 64 consecutive rows, one workgroup per (bucket, run); the caller
-// picks `runs` so that the pieces it launches together make about two workgroups per CU.  Within a bucket the
-// rows of a run are sorted by entry count (descending, stable) and cut into groups of 64: one lane per row,
-// one wave per group.  A group is stored as steps of 64 x 12 bytes (4 entries per lane per step, lane-major,
-// so a wave reads 768 contiguous bytes per step) padded to the longest row of the group; sorting keeps that
-// padding near 10 percent.  A workgroup stages its slice and its part of x in LDS; each lane accumulates
-// dot(codeword, x chunk) over its entries in fp32 and writes one partial sum per (bucket, row).  The
-// workgroups of all buckets that cover the same run count themselves off on a counter in the workspace; the
-// last one to arrive adds the NS * KP partials of each row of the run in a fixed order (so results do not
-// depend on scheduling), applies the row scale and stores y.
+// Rows are first ordered by column order (row_mask, stable), so that consecutive rows share one; each column
+// order's rows are cut into groups of 64 (the last group of an order may be short) and into runs of at most GR
+// groups, one workgroup per (bucket, run); the caller picks the number of runs so that the pieces it launches
+// together make about two workgroups per CU.  Within a bucket the rows of a run are sorted by entry count
+// (descending, stable): one lane per row, one wave per group.  A group is stored as steps of 64 x 12 bytes
+// (4 entries per lane per step, lane-major, so a wave reads 768 contiguous bytes per step) padded to the longest
+// row of the group; sorting keeps that padding near 10 percent.  A workgroup stages its slice and its part of x
+// (gathered through the run's column order, if any) in LDS; each lane accumulates dot(codeword, x chunk) over
+// its entries in fp32 and writes one partial sum per (bucket, row).  The workgroups of all buckets that cover
+// the same run count themselves off on a counter in the workspace; the last one to arrive adds the NS * KP
+// partials of each row of the run in a fixed order (so results do not depend on scheduling), applies the row
+// scale and stores y.
 //
-// Stream buffer (one allocation, offsets follow from R and C/d alone):
+// Stream buffer (one allocation; offsets follow from C/d, the tag width, the group and run counts):
 //   goff   uint32 [NV * NG + 1]   first step of every group, cumulative over buckets (NV = KP * NS buckets,
-//                                 NG = ceil(R / 64) groups per bucket, bucket v = kp * NS + s)
-//   slots  uint32 [NV * NG * 64]  row | count << 19 per lane; row 0x7FFFF marks a lane without a row;
-//                                 lanes 64 g .. 64 g + 63 of a bucket are group g, groups GR i .. GR i + GR - 1 run i
+//                                 NG groups per bucket, bucket v = kp * NS + s)
+//   slots  uint32 [NV * NG * 64]  place | count << 19 per lane; place = the row's index in `rows` (below),
+//                                 0x7FFFF marks a lane without a row; lanes 64 g .. 64 g + 63 of a bucket are group g
+//   runs   int32 [runs][4]        first group, group count, column order, 0
+//   rows   uint32 [NG * 64]       the rows ordered by column order, 64 per group (0x7FFFF where a group is short):
+//                                 places 64 g0 .. 64 (g0 + ng) - 1 are a run's rows, and partial sums are indexed by place
 //   steps  [total][64][3] uint32  entries
 #include <algorithm>
 #include <string.h>
@@ -33,26 +38,26 @@
 
 namespace sq {
 
-StreamGeom stream_geom(int R, int C, int d, int bits, int runs) {
+StreamGeom stream_geom(int C, int d, int bits, int groups, int runs) {
     StreamGeom g;
     g.U = C / d;
     g.NS = 1 << (bits - STREAM_SLICE_BITS);
     g.KP = (g.U + STREAM_PART_MAX - 1) / STREAM_PART_MAX;
     g.PC = (g.U + g.KP - 1) / g.KP;
     g.NV = g.NS * g.KP;
-    g.NG = (R + 63) / 64;
-    if (runs <= 0) runs = (STREAM_DEFAULT_WGS + g.NV / 2) / g.NV;
-    if (runs < 1) runs = 1;
-    if (runs > g.NG) runs = g.NG;
-    g.GR = (g.NG + runs - 1) / runs;
-    g.runs = (g.NG + g.GR - 1) / g.GR;
+    g.NG = groups;
+    g.runs = runs;
     g.off_slots = (((size_t)g.NV * g.NG + 1) * 4 + 255) & ~(size_t)255;
-    g.off_steps = (g.off_slots + (size_t)g.NV * g.NG * 64 * 4 + 255) & ~(size_t)255;
+    g.off_runs = (g.off_slots + (size_t)g.NV * g.NG * 64 * 4 + 255) & ~(size_t)255;
+    g.off_rows = (g.off_runs + (size_t)runs * 16 + 255) & ~(size_t)255;
+    g.off_steps = (g.off_rows + (size_t)g.NG * 64 * 4 + 255) & ~(size_t)255;
+    g.total_steps = 0;
     return g;
 }
 
+// (R + 64 * 256 bounds the places: every column order can leave one group short)
 bool stream_format_ok(int R, int C, int d, int bits) {
-    return d == 8 && bits > STREAM_SLICE_BITS && bits <= 16 && C % d == 0 && R > 0 && R < STREAM_NO_ROW;
+    return d == 8 && bits > STREAM_SLICE_BITS && bits <= 16 && C % d == 0 && R > 0 && R + 64 * 256 < (int)STREAM_NO_ROW;
 }
 
 static inline uint32_t host_tag(const uint32_t* row, int W, int bits, int j) {
@@ -78,16 +83,55 @@ static void parallel_rows(int R, const std::function<void(int, int)>& fn) {
     for (auto& t : th) t.join();
 }
 
-// counts[v * R + r] and, per bucket, the sorted row order with its group step counts
+struct StreamRun { int32_t g0, ng, order, zero; };
+
 struct StreamPlan {
     StreamGeom g;
+    std::vector<StreamRun> runs;
+    std::vector<uint32_t> base;      // [NG * 64]: rows ordered by column order, STREAM_NO_ROW where a group is short
     std::vector<uint16_t> cnt;       // [NV][R]
-    std::vector<uint32_t> pos;       // [NV][R]: position of row r in bucket v's sorted order
+    std::vector<uint32_t> pos;       // [NV][R]: lane position (group * 64 + lane) of row r in bucket v
     std::vector<uint32_t> goff;      // [NV * NG + 1]
 };
 
-static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs, StreamPlan& P) {
-    P.g = stream_geom(R, C, d, bits, runs);
+static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
+                        StreamPlan& P) {
+    // rows by column order, groups and runs
+    std::vector<uint32_t> order(R);
+    for (int r = 0; r < R; ++r) order[r] = (uint32_t)r;
+    if (row_mask)
+        std::stable_sort(order.begin(), order.end(), [row_mask](uint32_t a, uint32_t b) { return row_mask[a] < row_mask[b]; });
+    StreamGeom g0 = stream_geom(C, d, bits, 0, 0);
+    if (runs <= 0) runs = (STREAM_DEFAULT_WGS + g0.NV / 2) / g0.NV;
+    if (runs < 1) runs = 1;
+    // groups per column order; GR = the fewest groups per run that keep the run count within the request (or
+    // at one run per column order when there are more orders than that)
+    std::vector<int> first, ngm;
+    for (int a = 0; a < R;) {
+        int b = a;
+        const int m = row_mask ? row_mask[order[a]] : 0;
+        while (b < R && (row_mask ? row_mask[order[b]] : 0) == m) ++b;
+        first.push_back(a);
+        ngm.push_back((b - a + 63) / 64);
+        a = b;
+    }
+    first.push_back(R);
+    int GR = 1;
+    for (;; ++GR) {
+        int64_t n = 0;
+        bool whole = true;
+        for (int q : ngm) { n += (q + GR - 1) / GR; whole = whole && q <= GR; }
+        if (n <= runs || whole) break;
+    }
+    P.runs.clear();
+    P.base.clear();
+    for (size_t i = 0; i < ngm.size(); ++i) {
+        const int a = first[i], b = first[i + 1], gbase = (int)(P.base.size() / 64);
+        const int m = row_mask ? row_mask[order[a]] : 0;
+        for (int k = 0; k < ngm[i] * 64; ++k) P.base.push_back(a + k < b ? order[a + k] : STREAM_NO_ROW);
+        for (int q = 0; q < ngm[i]; q += GR) P.runs.push_back(StreamRun{gbase + q, std::min(GR, ngm[i] - q), m, 0});
+    }
+    P.g = stream_geom(C, d, bits, (int)(P.base.size() / 64), (int)P.runs.size());
     const StreamGeom& g = P.g;
     P.cnt.assign((size_t)g.NV * R, 0);
     P.pos.assign((size_t)g.NV * R, 0);
@@ -102,17 +146,20 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
             }
         }
     });
-    std::vector<uint32_t> steps((size_t)g.NV * g.NG);
+    std::vector<uint32_t> steps((size_t)g.NV * g.NG, 0);
     parallel_rows(g.NV, [&](int a, int b) {
-        std::vector<uint32_t> order(R);
+        std::vector<uint32_t> rows;
         for (int v = a; v < b; ++v) {
             const uint16_t* c = &P.cnt[(size_t)v * R];
-            for (int r = 0; r < R; ++r) order[r] = (uint32_t)r;
-            for (int r0 = 0; r0 < R; r0 += g.GR * 64)
-                std::stable_sort(order.begin() + r0, order.begin() + std::min(R, r0 + g.GR * 64),
-                                 [c](uint32_t x, uint32_t y) { return c[x] > c[y]; });
-            for (int k = 0; k < R; ++k) P.pos[(size_t)v * R + order[k]] = (uint32_t)k;
-            for (int gi = 0; gi < g.NG; ++gi) steps[(size_t)v * g.NG + gi] = (c[order[(size_t)gi * 64]] + 3u) / 4u;
+            for (const StreamRun& run : P.runs) {
+                rows.clear();
+                for (int k = run.g0 * 64; k < (run.g0 + run.ng) * 64; ++k)
+                    if (P.base[k] != STREAM_NO_ROW) rows.push_back(P.base[k]);
+                std::stable_sort(rows.begin(), rows.end(), [c](uint32_t x, uint32_t y) { return c[x] > c[y]; });
+                for (size_t k = 0; k < rows.size(); ++k) P.pos[(size_t)v * R + rows[k]] = (uint32_t)(run.g0 * 64 + k);
+                for (size_t k = 0; k < rows.size(); k += 64)
+                    steps[(size_t)v * g.NG + run.g0 + k / 64] = (c[rows[k]] + 3u) / 4u;
+            }
         }
     });
     uint64_t tot = 0;
@@ -121,22 +168,27 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     P.g.total_steps = tot;
 }
 
-size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs) {
+size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs) {
     StreamPlan P;
-    plan_stream(tags, R, W, C, d, bits, runs, P);
+    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P);
     return P.g.off_steps + (size_t)P.g.total_steps * 768;
 }
 
-int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, int runs, unsigned char* out,
-                      size_t bytes) {
+int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
+                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out) {
     StreamPlan P;
-    plan_stream(tags, R, W, C, d, bits, runs, P);
+    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P);
     const StreamGeom& g = P.g;
     const size_t need = g.off_steps + (size_t)g.total_steps * 768;
     if (g.total_steps >= ((uint64_t)1 << 32)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: matrix too large");
     if (bytes < need) return fail(SQ_EINVAL, "sq_stream_build: buffer %zu < %zu", bytes, need);
     memset(out, 0, need);
     memcpy(out, P.goff.data(), P.goff.size() * 4);
+    memcpy(out + g.off_runs, P.runs.data(), P.runs.size() * sizeof(StreamRun));
+    memcpy(out + g.off_rows, P.base.data(), P.base.size() * 4);
+    std::vector<uint32_t> place(R);
+    for (size_t k = 0; k < P.base.size(); ++k)
+        if (P.base[k] != STREAM_NO_ROW) place[P.base[k]] = (uint32_t)k;
     uint32_t* slots = (uint32_t*)(out + g.off_slots);
     for (size_t k = 0; k < (size_t)g.NV * g.NG * 64; ++k) slots[k] = STREAM_NO_ROW;
     unsigned char* steps = out + g.off_steps;
@@ -147,7 +199,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             std::fill(q.begin(), q.end(), 0u);
             for (int v = 0; v < g.NV; ++v) {
                 const uint32_t k = P.pos[(size_t)v * R + r];
-                slots[(size_t)v * g.NG * 64 + k] = (uint32_t)r | ((uint32_t)P.cnt[(size_t)v * R + r] << STREAM_ROW_BITS);
+                slots[(size_t)v * g.NG * 64 + k] = place[r] | ((uint32_t)P.cnt[(size_t)v * R + r] << STREAM_ROW_BITS);
             }
             for (int j = 0; j < g.U; ++j) {
                 const uint32_t t = host_tag(row, W, bits, j);
@@ -160,6 +212,8 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             }
         }
     });
+    if (runs_out) *runs_out = g.runs;
+    if (groups_out) *groups_out = g.NG;
     return SQ_OK;
 }
 
@@ -169,10 +223,11 @@ struct StreamPiece {
     const unsigned char* stream;
     const uint16_t* table;
     const uint16_t* row_scale;
-    float* part;                      // [NV][R]
+    float* part;                      // [NV][NG * 64], indexed by place
     unsigned* counters;               // one per run; zero before the launch, zero after it
-    int R, U, NS, NV, PC, NG, GR, y_off;
-    uint32_t off_slots, off_steps;
+    const int32_t* perms;             // [M, C] column orders or NULL
+    int R, C, U, NS, NV, PC, NG, y_off;
+    uint32_t off_slots, off_runs, off_rows, off_steps;
     int wg_begin, nwg;                // first workgroup of the piece; workgroups (= runs) per bucket
 };
 
@@ -208,13 +263,16 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     const int v = local / P.nwg, wi = local - v * P.nwg;
     const int s = v % P.NS, kp = v / P.NS;
     SQ_TRACE_POINT(0);
-    // this workgroup's run: groups g0 .. g0 + ng - 1 of the bucket
-    const int g0 = wi * P.GR, ng = min(P.NG, g0 + P.GR) - g0;
+    // this workgroup's run: groups g0 .. g0 + ng - 1 of the bucket, all of one column order
+    // (without column orders every run but the last has ceil(NG / runs) groups: no need to wait for the table)
+    const int32_t* run = reinterpret_cast<const int32_t*>(P.stream + P.off_runs) + wi * 4;
+    const int gr = (P.NG + P.nwg - 1) / P.nwg;
+    const int g0 = P.perms ? run[0] : wi * gr, ng = P.perms ? run[1] : min(gr, P.NG - g0);
 
     const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG + g0;
     const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
     const unsigned char* steps = P.stream + P.off_steps + lane * 12;
-    float* part = P.part + (size_t)v * P.R;
+    float* part = P.part + (size_t)v * P.NG * 64;
     unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_X_OFF + P.PC * 16);   // [0] arrival result, [1] next group
 
     // The groups of a run are sorted longest first.  Wave w starts with group w, then group 15 - w; after
@@ -255,8 +313,21 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
         const u32x4* xs = reinterpret_cast<const u32x4*>(a.x) + c0;
         u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_X_OFF);
+        if (P.perms == nullptr) {
 #pragma unroll
-        for (int k = 0; k < 2; ++k) xq[k] = xs[min(tid + k * NW * 64, nc - 1)];      // PC <= 640 < 2 * 512
+            for (int k = 0; k < 2; ++k) xq[k] = xs[min(tid + k * NW * 64, nc - 1)];  // PC <= 640 < 2 * 512
+        } else {
+            // chunk j of a row with column order m multiplies x[perm_m[8 j .. 8 j + 7]]
+            const int32_t* pm = P.perms + (size_t)run[2] * P.C + (size_t)c0 * 8;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const int32_t* pk = pm + (size_t)min(tid + k * NW * 64, nc - 1) * 8;
+                const u32x4 i0 = *reinterpret_cast<const u32x4*>(pk), i1 = *reinterpret_cast<const u32x4*>(pk + 4);
+                const uint32_t e0 = a.x[i0.x], e1 = a.x[i0.y], e2 = a.x[i0.z], e3 = a.x[i0.w];
+                const uint32_t e4 = a.x[i1.x], e5 = a.x[i1.y], e6 = a.x[i1.z], e7 = a.x[i1.w];
+                xq[k] = u32x4{e0 | (e1 << 16), e2 | (e3 << 16), e4 | (e5 << 16), e6 | (e7 << 16)};
+            }
+        }
         first_steps(hn, nx);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -344,37 +415,45 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     if (flag[0] != (unsigned)P.NV - 1u) return;
     // 64 partial sums in flight per thread: four rows at a time when a row has 16 buckets, else one row's
     // buckets 64 at a time; a row's partials are always added in bucket order
-    const int r0 = g0 * 64, r1 = min(P.R, (g0 + ng) * 64);
-    const float* pp = P.part;
+    // places 64 g0 .. 64 (g0 + ng) - 1: consecutive partial sums; `rows` says which row each place is
+    const uint32_t* rows0 = reinterpret_cast<const uint32_t*>(P.stream + P.off_rows) + (size_t)g0 * 64;
+    const int nl = ng * 64;
+    const size_t np = (size_t)P.NG * 64;
+    const float* pp = P.part + (size_t)g0 * 64;
     if (P.NV <= 16) {
-        for (int rb = r0 + tid; rb < r1; rb += 4 * NW * 64) {
+        for (int ib = tid; ib < nl; ib += 4 * NW * 64) {
             float t[4][16];
+            uint32_t rr[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = ib + q * NW * 64;
+                rr[q] = i >= nl ? STREAM_NO_ROW : P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
-                for (int k = 0; k < 16; ++k) {
-                    const int r = rb + q * NW * 64;
-                    t[q][k] = (r < r1 && k < P.NV)
-                                  ? __hip_atomic_load(pp + (size_t)k * P.R + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
-                }
+                for (int k = 0; k < 16; ++k)
+                    t[q][k] = (ib + q * NW * 64 < nl && k < P.NV)
+                                  ? __hip_atomic_load(pp + (size_t)k * np + ib + q * NW * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int r = rb + q * NW * 64;
                 float sum = 0.f;
 #pragma unroll
                 for (int k = 0; k < 16; ++k) sum += t[q][k];
-                if (r < r1) store_y(a.y, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
+                if (rr[q] != STREAM_NO_ROW) store_y(a.y, a.y_dtype, (int64_t)P.y_off + rr[q], sum * h2f(P.row_scale[rr[q]]));
             }
         }
     } else {
-        for (int r = r0 + tid; r < r1; r += NW * 64) {
+        for (int i = tid; i < nl; i += NW * 64) {
+            const uint32_t r = P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
+            if (r == STREAM_NO_ROW) continue;
             float sum = 0.f;
             for (int v0 = 0; v0 < P.NV; v0 += 64) {
                 float t[64];
 #pragma unroll
                 for (int k = 0; k < 64; ++k)
                     t[k] = v0 + k < P.NV
-                               ? __hip_atomic_load(pp + (size_t)(v0 + k) * P.R + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+                               ? __hip_atomic_load(pp + (size_t)(v0 + k) * np + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
 #pragma unroll
                 for (int k = 0; k < 64; ++k) sum += t[k];
             }
@@ -396,13 +475,13 @@ static int stream_launch(const StreamArgs& a, int grid, size_t smem, hipStream_t
 }
 
 bool stream_shape(const sq_matrix& m) {
-    return m.stream && m.stream_runs > 0 && !m.perms && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
-           (((uintptr_t)m.table | (uintptr_t)m.stream) & 15) == 0;
+    return m.stream && m.stream_runs > 0 && m.stream_groups > 0 && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
+           (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0;
 }
 
 size_t stream_part_bytes(const sq_matrix& m) {
-    const StreamGeom g = stream_geom(m.R, m.C, m.d, m.bits, m.stream_runs);
-    return (((size_t)g.NV * m.R * 4) + 255) & ~(size_t)255;
+    const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, m.stream_runs);
+    return (((size_t)g.NV * g.NG * 64 * 4) + 255) & ~(size_t)255;
 }
 
 // Pieces [0, cnt) (same C): one launch.  `counters` is the zeroed head of the workspace.
@@ -414,22 +493,25 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     a.y = y;
     a.x_dtype = x_dtype;
     a.y_dtype = y_dtype;
-    const StreamGeom g0 = stream_geom(mats[0].R, mats[0].C, mats[0].d, mats[0].bits, mats[0].stream_runs);
+    const StreamGeom g0 = stream_geom(mats[0].C, mats[0].d, mats[0].bits, mats[0].stream_groups, mats[0].stream_runs);
     const size_t smem = (size_t)STREAM_X_OFF + (size_t)g0.PC * 16 + 16;      // slice, x part, two words of flags
     (void)cus;
     int wg = 0;
     for (int k = 0; k < cnt; ++k) {
         const sq_matrix& m = mats[k];
-        const StreamGeom g = stream_geom(m.R, m.C, m.d, m.bits, m.stream_runs);
-        if (g.runs != m.stream_runs) return fail(SQ_EINVAL, "sq_linear_small: stream_runs %d is not what sq_stream_runs returns (%d)", m.stream_runs, g.runs);
+        const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, m.stream_runs);
+        if (m.stream_groups < (m.R + 63) / 64 || m.stream_runs > m.stream_groups)
+            return fail(SQ_EINVAL, "sq_linear_small: stream_runs %d / stream_groups %d do not fit %d rows", m.stream_runs, m.stream_groups, m.R);
         StreamPiece& P = a.p[k];
         P.stream = (const unsigned char*)m.stream;
         P.table = m.table;
         P.row_scale = m.row_scale;
         P.part = (float*)(ws + ws_off);
         ws_off += stream_part_bytes(m);
-        P.R = m.R; P.U = g.U; P.NS = g.NS; P.NV = g.NV; P.PC = g.PC; P.NG = g.NG; P.GR = g.GR; P.y_off = m.y_off;
-        P.off_slots = (uint32_t)g.off_slots; P.off_steps = (uint32_t)g.off_steps;
+        P.perms = m.perms;
+        P.R = m.R; P.C = m.C; P.U = g.U; P.NS = g.NS; P.NV = g.NV; P.PC = g.PC; P.NG = g.NG; P.y_off = m.y_off;
+        P.off_slots = (uint32_t)g.off_slots; P.off_runs = (uint32_t)g.off_runs; P.off_rows = (uint32_t)g.off_rows;
+        P.off_steps = (uint32_t)g.off_steps;
         const int nwg = g.runs;
         if (counters_used + nwg > SQ_WS_COUNTERS) return fail(SQ_EUNSUPPORTED, "sq_linear_small: too many row-block runs");
         P.counters = counters + counters_used;

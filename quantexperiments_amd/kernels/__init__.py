@@ -82,14 +82,17 @@ class PackedLinear(torch.nn.Module):
         self.bias = bias
         # codebooks too large for LDS: regroup the tags by codebook slice once, for the batch-1 product
         self.register_buffer("stream", None)
-        self.stream_runs = 0
-        if stream and not self.has_mask and self.G == 1 and table.numel() * 2 > 128 * 1024:
+        self.stream_runs = self.stream_groups = 0
+        self.stream_asked = None
+        if stream and self.G == 1 and table.numel() * 2 > 128 * 1024:
             self.build_stream(0)
 
     def build_stream(self, runs: int = 0) -> None:
-        """(Re)build the bucketed tag stream cut into `runs` row runs (0 = suited to a launch of this matrix
-        alone; prepare_stack picks the runs of pieces that are launched together)."""
-        self.stream, self.stream_runs = build_stream(self.words, self.C, self.d, self.bits, runs)
+        """(Re)build the bucketed tag stream cut into about `runs` row runs (0 = suited to a launch of this
+        matrix alone; prepare_stack picks the runs of pieces that are launched together)."""
+        self.stream, self.stream_runs, self.stream_groups = build_stream(
+            self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs)
+        self.stream_asked = runs
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -110,7 +113,8 @@ class PackedLinear(torch.nn.Module):
         p = lambda t: None if t is None else t.data_ptr()
         return SqMatrix(p(self.words), p(self.table), p(self.row_scale), p(self.row_book), p(self.row_mask),
                         p(self.perms), p(self.row_order), self.R, self.C, self.d, self.bits, self.G, self.M, self.W,
-                        y_off, p(self.stream), self.stream_runs if self.stream is not None else 0, 0)
+                        y_off, p(self.stream), self.stream_runs if self.stream is not None else 0,
+                        self.stream_groups if self.stream is not None else 0)
 
     # ------------------------------------------------------------------ kernels
     def dense(self, dtype=torch.float32, out: torch.Tensor | None = None, rows: tuple | None = None) -> torch.Tensor:
@@ -155,19 +159,24 @@ class PackedLinear(torch.nn.Module):
         return sum(t.numel() * t.element_size() for t in (self.words, self.table, self.row_scale))
 
 
-def build_stream(words: torch.Tensor, C: int, d: int, bits: int, runs: int = 0):
-    """(stream, runs): the bucketed tag stream of one matrix (sq_stream_build) as a uint8 tensor on words'
-    device and the number of row runs it was cut into, or (None, 0) when the format is not covered.  The
-    regrouping itself is the library's host routine; the tags make one trip to host memory at load time."""
+def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, runs: int = 0):
+    """(stream, runs, groups): the bucketed tag stream of one matrix (sq_stream_build) as a uint8 tensor on
+    words' device with the run and group counts the library cut it into, or (None, 0, 0) when the format is not
+    covered.  The regrouping itself is the library's host routine; the tags make one trip to host memory at
+    load time."""
     L = _lib.lib()
     host = words.detach().to("cpu", torch.int32).contiguous()
+    mask = None if row_mask is None else row_mask.detach().to("cpu", torch.uint8).contiguous()
+    mp = None if mask is None else mask.data_ptr()
     R, W = host.shape
-    n = L.sq_stream_bytes(host.data_ptr(), R, W, C, d, bits, runs)
+    n = L.sq_stream_bytes(host.data_ptr(), R, W, C, d, bits, mp, runs)
     if n == 0:
-        return None, 0
+        return None, 0, 0
     out = torch.empty(n, dtype=torch.uint8)
-    _lib.check(L.sq_stream_build(host.data_ptr(), R, W, C, d, bits, runs, out.data_ptr(), n))
-    return out.to(words.device), L.sq_stream_runs(R, C, d, bits, runs)
+    r, g = ctypes.c_int32(0), ctypes.c_int32(0)
+    _lib.check(L.sq_stream_build(host.data_ptr(), R, W, C, d, bits, mp, runs, out.data_ptr(), n, ctypes.byref(r),
+                                 ctypes.byref(g)))
+    return out.to(words.device), r.value, g.value
 
 
 def prepare_stack(pieces, workgroups: int = 512) -> None:
@@ -178,7 +187,7 @@ def prepare_stack(pieces, workgroups: int = 512) -> None:
     for p in ps:
         buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // 640)
         runs = max(1, round(workgroups * p.R / rows / buckets))
-        if _lib.lib().sq_stream_runs(p.R, p.C, p.d, p.bits, runs) != p.stream_runs:
+        if runs != p.stream_asked and not (len(ps) == 1 and p.stream_asked == 0):
             p.build_stream(runs)
 
 

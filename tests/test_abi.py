@@ -32,7 +32,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layout_matches_header():
     # 7 pointers + 8 int32 + 1 pointer + 2 int32
     assert ctypes.sizeof(_lib.SqMatrix) == 7 * 8 + 8 * 4 + 8 + 8
-    assert _lib.SqMatrix.R.offset == 56 and _lib.SqMatrix.y_off.offset == 56 + 28 and _lib.SqMatrix.stream.offset == 88
+    assert _lib.SqMatrix.R.offset == 56 and _lib.SqMatrix.y_off.offset == 56 + 28 and _lib.SqMatrix.stream.offset == 88 and _lib.SqMatrix.stream_groups.offset == 100
 
 
 def test_host_side_argument_checks():

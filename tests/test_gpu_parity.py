@@ -159,8 +159,9 @@ def test_large_products_do_not_overflow():
 
 
 # ------------------------------------------------------------------ bucketed tag stream (codebooks beyond LDS, B = 1)
-STREAM = [  # R, C, bits
-    (70, 512, 16), (130, 5376, 16), (260, 3584, 16), (64, 1024, 15), (333, 2048, 14), (1, 8, 16), (65, 18944, 16),
+STREAM = [  # R, C, bits, M
+    (70, 512, 16, 1), (130, 5376, 16, 1), (260, 3584, 16, 1), (64, 1024, 15, 1), (333, 2048, 14, 1), (1, 8, 16, 1),
+    (65, 18944, 16, 1), (300, 5120, 16, 16), (33, 640, 16, 8), (700, 1024, 14, 3), (40, 17408, 16, 16),
 ]
 
 
@@ -168,8 +169,8 @@ STREAM = [  # R, C, bits
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
 def test_stream_gemv_matches_oracle_and_row_path(case, dtype):
     from quantexperiments_amd.kernels import linear_small
-    R, C, bits = case
-    s = synth(R, C, 8, bits, seed=sum(case))
+    R, C, bits, M = case
+    s = synth(R, C, 8, bits, 1, M, seed=sum(case))
     if R > 5:
         s.tags[5] = 7                                   # a row whose tags all sit in one codebook slice
         s.tags[4, ::2] = (1 << bits) - 1

@@ -178,34 +178,68 @@ def test_neutral_defaults_and_registry():
 
 # ---------------------------------------------------------------------------- bucketed tag stream (host builder)
 
-def _walk_stream(buf, R, C, d, bits, runs):
-    """Rebuild the [R, C/d] tag matrix from a stream buffer cut into `runs` row runs, checking its structure
-    on the way."""
+def _build_stream(words, R, C, bits, row_mask, runs):
+    import ctypes
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    W = words.shape[1]
+    ptr = words.ctypes.data_as(ctypes.c_void_p)
+    mp = None if row_mask is None else row_mask.ctypes.data_as(ctypes.c_void_p)
+    n = L.sq_stream_bytes(ptr, R, W, C, 8, bits, mp, runs)
+    assert n > 0
+    out = np.zeros(n, np.uint8)
+    r, g = ctypes.c_int32(0), ctypes.c_int32(0)
+    args = (ptr, R, W, C, 8, bits, mp, runs, out.ctypes.data_as(ctypes.c_void_p))
+    assert L.sq_stream_build(*args, n, ctypes.byref(r), ctypes.byref(g)) == 0
+    assert L.sq_stream_build(*args, n - 1, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EINVAL
+    return out.tobytes(), r.value, g.value
+
+
+def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
+    """Rebuild the [R, C/d] tag matrix from a stream buffer, checking its structure on the way."""
     U, NS = C // d, 1 << (bits - 12)
     KP = -(-U // 640)
     PC = -(-U // KP)
-    NV, NG = NS * KP, -(-R // 64)
-    RR = -(-NG // runs) * 64                                                  # rows per run
-    assert -(-NG * 64 // RR) == runs
+    NV = NS * KP
     off_slots = ((NV * NG + 1) * 4 + 255) & ~255
-    off_steps = (off_slots + NV * NG * 64 * 4 + 255) & ~255
+    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
+    off_rows = (off_runs + runs * 16 + 255) & ~255
+    off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
     goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
     slots = np.frombuffer(buf, np.uint32, NV * NG * 64, off_slots).reshape(NV, NG * 64)
+    rt = np.frombuffer(buf, np.int32, runs * 4, off_runs).reshape(runs, 4)
+    base = np.frombuffer(buf, np.uint32, NG * 64, off_rows)                   # place -> row
+    assert sorted(base[base != 0x7FFFF].tolist()) == list(range(R))
+    if row_mask is None:
+        assert (base[:R] == np.arange(R)).all()
     assert goff[0] == 0 and (np.diff(goff.astype(np.int64)) >= 0).all()
     assert len(buf) == off_steps + int(goff[-1]) * 768
+    # runs tile the groups in order; every run has one column order
+    assert rt[0, 0] == 0 and (rt[1:, 0] == rt[:-1, 0] + rt[:-1, 1]).all() and rt[-1, 0] + rt[-1, 1] == NG
+    assert (rt[:, 1] >= 1).all() and (rt[:, 3] == 0).all() and (np.diff(rt[:, 2]) >= 0).all()
     steps = np.frombuffer(buf, np.uint8, int(goff[-1]) * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.uint32)
     ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
     tags = np.full((R, U), -1, np.int64)
+    run_rows = None
     for v in range(NV):
         kp, s = divmod(v, NS)
-        rows = slots[v] & 0x7FFFF
+        places = slots[v] & 0x7FFFF
         cnts = slots[v] >> 19
-        real = rows != 0x7FFFF
+        real = places != 0x7FFFF
+        rows = np.where(real, base[np.where(real, places, 0)], 0x7FFFF)
+        assert (rows[real] != 0x7FFFF).all()
         assert sorted(rows[real].tolist()) == list(range(R))                  # every row once per bucket
-        for r0 in range(0, NG * 64, RR):                                      # sorted by count within each run
-            blk = cnts[r0:r0 + RR][real[r0:r0 + RR]].astype(np.int64)
-            assert (np.diff(blk) <= 0).all()
-            assert sorted(rows[r0:r0 + RR][real[r0:r0 + RR]].tolist()) == list(range(r0, min(R, r0 + RR)))
+        sets = []
+        for g0, ng, order, _ in rt:                                           # sorted by count within each run
+            sl = slice(g0 * 64, (g0 + ng) * 64)
+            assert (np.diff(cnts[sl][real[sl]].astype(np.int64)) <= 0).all()
+            assert real[sl][:int(real[sl].sum())].all()                       # rows first, empty lanes last
+            sets.append(frozenset(rows[sl][real[sl]].tolist()))
+            assert ((places[sl][real[sl]] >= g0 * 64) & (places[sl][real[sl]] < (g0 + ng) * 64)).all()
+            if row_mask is not None:
+                assert (row_mask[rows[sl][real[sl]]] == order).all()
+        run_rows = run_rows or sets
+        assert sets == run_rows                                               # the same rows in every bucket's run
         for g in range(NG):
             n = int(goff[v * NG + g + 1]) - int(goff[v * NG + g])
             assert n == -(-int(cnts[g * 64]) // 4)                            # padded to the group's longest row
@@ -225,29 +259,20 @@ def _walk_stream(buf, R, C, d, bits, runs):
     return tags
 
 
-@pytest.mark.parametrize("R,C,bits,runs", [(70, 512, 16, 0), (130, 5376, 16, 2), (64, 1024, 13, 5), (1, 8, 14, 0),
-                                            (1100, 256, 15, 4), (1100, 256, 15, 7)])
-def test_stream_builder_keeps_every_tag(R, C, bits, runs):
-    import ctypes
-    from quantexperiments_amd import _lib
-    from oracle import sq_oracle as O
-    L = _lib.lib()
-    rng = np.random.default_rng(R + C)
+@pytest.mark.parametrize("R,C,bits,runs,M", [(70, 512, 16, 0, 1), (130, 5376, 16, 2, 1), (64, 1024, 13, 5, 1), (1, 8, 14, 0, 1),
+                                              (1100, 256, 15, 4, 1), (1100, 256, 15, 7, 1), (300, 512, 16, 3, 4),
+                                              (1000, 256, 14, 2, 16), (5, 64, 16, 0, 3)])
+def test_stream_builder_keeps_every_tag(R, C, bits, runs, M):
+    rng = np.random.default_rng(R + C + M)
     U = C // 8
     tags = rng.integers(0, 1 << bits, (R, U))
     if R > 3:
         tags[3] = 5                                                           # one row entirely in slice 0
+    row_mask = rng.integers(0, M, R).astype(np.uint8) if M > 1 else None
     words = np.ascontiguousarray(O.pack_bits(tags, bits))
-    W = words.shape[1]
-    ptr = words.ctypes.data_as(ctypes.c_void_p)
-    n = L.sq_stream_bytes(ptr, R, W, C, 8, bits, runs)
-    assert n > 0
-    eff = L.sq_stream_runs(R, C, 8, bits, runs)
-    assert 1 <= eff <= -(-R // 64) and (runs == 0 or eff <= runs)
-    out = np.zeros(n, np.uint8)
-    assert L.sq_stream_build(ptr, R, W, C, 8, bits, runs, out.ctypes.data_as(ctypes.c_void_p), n) == 0
-    assert np.array_equal(_walk_stream(out.tobytes(), R, C, 8, bits, eff), tags)
-    assert L.sq_stream_build(ptr, R, W, C, 8, bits, runs, out.ctypes.data_as(ctypes.c_void_p), n - 1) == _lib.SQ_EINVAL
+    buf, eff, NG = _build_stream(words, R, C, bits, row_mask, runs)
+    assert NG >= -(-R // 64) and 1 <= eff <= NG
+    assert np.array_equal(_walk_stream(buf, R, C, 8, bits, eff, NG, row_mask), tags)
 
 
 def test_stream_builder_rejects_other_formats():
@@ -256,7 +281,7 @@ def test_stream_builder_rejects_other_formats():
     L = _lib.lib()
     words = np.zeros((4, 16), np.int32)
     ptr = words.ctypes.data_as(ctypes.c_void_p)
-    assert L.sq_stream_bytes(ptr, 4, 16, 128, 4, 16, 0) == 0                  # d = 4
-    assert L.sq_stream_bytes(ptr, 4, 16, 128, 8, 12, 0) == 0                  # codebook fits LDS: no stream
-    assert L.sq_stream_runs(4, 128, 8, 12, 0) == 0
-    assert L.sq_stream_build(ptr, 4, 16, 128, 8, 12, 0, ptr, 64) == _lib.SQ_EUNSUPPORTED
+    r, g = ctypes.c_int32(0), ctypes.c_int32(0)
+    assert L.sq_stream_bytes(ptr, 4, 16, 128, 4, 16, None, 0) == 0            # d = 4
+    assert L.sq_stream_bytes(ptr, 4, 16, 128, 8, 12, None, 0) == 0            # codebook fits LDS: no stream
+    assert L.sq_stream_build(ptr, 4, 16, 128, 8, 12, None, 0, ptr, 64, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EUNSUPPORTED
