@@ -1,11 +1,22 @@
 // Large-tile fp16 GEMM for prefill: Y[T, R] = X[T, C] . W[R, C]^T, fp32 accumulate, optional row scale.
 //
-// Workgroup tile 256 tokens x 256 weight rows x 64 columns, 4 waves in 2 x 2, each wave a 128 x 128
-// tile of sixteen v_mfma_f32_32x32x16_f16 accumulators (256 accumulator registers per lane).  Both
-// operands are K-contiguous fp16 in memory; a column tile of each (256 x 64 halves = 32 KB) is copied
-// from global memory straight into LDS, double buffered (128 KB), one barrier per column tile.  LDS rows
-// are 128 bytes; the 16-byte piece c of row r is stored at slot c ^ ((r >> 1) & 7), which makes the operand
-// reads (16 lanes = 16 rows x one piece per cycle) conflict free.
+// Workgroup tile 256 tokens x 256 weight rows, 8 waves in 2 x 4, each wave a 128 x 64 tile of eight
+// v_mfma_f32_32x32x16_f16 accumulators (128 accumulator registers per lane), so two waves share a SIMD and
+// one issues matrix instructions while the other waits at a barrier.  Both operands are K-contiguous fp16 in
+// memory.  The K loop moves in slabs of 64 columns; a slab of ONE operand (256 rows x 128 bytes = 32 KB, whole
+// 128-byte lines: half-line requests get 10.5 TB/s out of L2 over the chip, whole lines 15.2 TB/s, and a
+// 256 x 256 tile needs about 10 TB/s at the clock the matrix cores sustain) is copied from global memory
+// straight into LDS (global_load_lds_dwordx4: no staging registers) into a ring of five 32 KB slots: X_s, W_s,
+// X_s+1, W_s+1, X_s+2 are resident or on their way while slab s is multiplied.  A CU accepts one such copy
+// instruction per 16 clocks, so a wave that issues its eight copies of a slab back to back stalls for hundreds
+// of clocks and its matrix instructions with it: the copies are issued one at a time between matrix
+// instructions.  Waits are counted: at the one barrier per slab a wave waits for its own copies of slab s + 1
+// only (s_waitcnt vmcnt(4) leaves the four younger X_s+2 copies in flight).  Operand fragments are read one
+// 16-column step ahead of the matrix instructions that use them.
+//
+// LDS rows are 128 bytes; the 16-byte piece c of row r is stored at slot c ^ ((r >> 1) & 7).  A ds_read_b128
+// serves 16 lanes per clock from 64 banks (256 bytes); 16 consecutive rows of one piece then fall on 16
+// different 16-byte bank groups ((r & 1) * 8 + slot), so the operand reads are conflict free.
 //
 // Operand layout of v_mfma_f32_32x32x16_f16, lane l: A row / B column l % 32, k = 8 * (l / 32) .. + 7;
 // D[v], v = 0..15: row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32.  Rows of D are tokens, columns
@@ -14,7 +25,8 @@
 
 namespace sq {
 
-constexpr int G_BM = 256, G_BN = 256, G_BK = 64;
+constexpr int G_BM = 256, G_BN = 256, G_BK = 64, G_WAVES = 8;
+constexpr int G_SLOTS = 5, G_SLOT_BYTES = 256 * G_BK * 2;        // 5 x 32 KB = all 160 KB of LDS
 
 struct Gemm256Args {
     const uint16_t* x;        // fp16 [T, C], row stride ldx
@@ -26,43 +38,44 @@ struct Gemm256Args {
     int tiles_t, tiles_r;     // token / weight-row tiles (for the workgroup -> tile mapping)
 };
 
-__device__ __forceinline__ int swz(int r, int c) { return c ^ ((r >> 1) & 7); }
+// s_waitcnt immediate that waits until at most n vector-memory operations are outstanding and leaves the
+// other counters alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
-__global__ __launch_bounds__(256) void gemm256_kernel(Gemm256Args a) {
+__global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    // [2 buffers][X tile 32 KB | W tile 32 KB]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // consecutive tiles walk the token tiles of one weight tile, so a weight tile is fetched from HBM once and
-    // its re-reads hit L2 while the (small) activation matrix stays resident
     // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so workgroup i of the launch
     // takes tile (i % 8) * (n / 8) + i / 8: every XCD then works on one contiguous run of tiles and a weight
     // tile is fetched by one L2 only.  The grid is padded to a multiple of 8; surplus workgroups leave.
     const int per_xcd = gridDim.x >> 3;
     const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
     if (tile >= a.tiles_t * a.tiles_r) return;
+    // consecutive tiles walk the token tiles of one weight tile, so a weight tile is fetched from HBM once and
+    // its re-reads hit L2 while the (small) activation matrix stays resident
     const int bt = tile % a.tiles_t, br = tile / a.tiles_t;
     const int t0 = bt * G_BM, r0 = br * G_BN;
-    const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+    const int wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
 
-    float16v acc[4][4];
+    float16v acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // Staging goes straight from global memory into LDS (global_load_lds_dwordx4: no staging registers, no
-    // LDS store instructions).  One such load fills 1 KB = 8 LDS rows in lane order, so lane s lands in LDS
-    // row s >> 3, slot s & 7 of its chunk, and therefore fetches the piece that the swizzle puts there:
-    // piece (s & 7) ^ f(row).  A tile is 32 chunks; wave w fills chunks 8 w .. 8 w + 7 of both operands.
-    // Global addresses are a uniform base (advanced per column tile) plus per-lane 32-bit element offsets
-    // computed once; rows past the matrix edge re-read the last row (their outputs are never stored).
+    // Copies.  One global_load_lds_dwordx4 fills 1 KB = 8 LDS rows in lane order, so lane s lands in row
+    // s >> 3, slot s & 7 of its block and therefore fetches the piece the swizzle puts there.  Wave w copies
+    // rows 32 w .. 32 w + 31 of an operand slab: 4 instructions.  Global addresses are a uniform base (advanced
+    // per slab) plus per-lane 32-bit element offsets computed once; rows past the matrix edge re-read the last
+    // row (their outputs are never stored).  Half h = 2 s is X of slab s, h = 2 s + 1 is W of slab s; half h
+    // lives in ring slot h % 5.
     const int lrow = lane >> 3, slot = lane & 7;
-    uint32_t xo[8], wo[8];
+    uint32_t xo[4], wo[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int row = (wave * 8 + j) * 8 + lrow;
+    for (int j = 0; j < 4; ++j) {
+        const int row = wave * 32 + j * 8 + lrow;
         const int c = slot ^ ((row >> 1) & 7);
         const int t = t0 + row < a.T ? row : a.T - 1 - t0;
         const int r = r0 + row < a.R ? row : a.R - 1 - r0;
@@ -73,61 +86,101 @@ __global__ __launch_bounds__(256) void gemm256_kernel(Gemm256Args a) {
     const uint16_t* wt = a.w + (int64_t)r0 * a.ldw;
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    auto stage = [&](int k0, int buf) {
-        const uint16_t* xk = xt + k0;
-        const uint16_t* wk = wt + k0;
-        unsigned char* dx = smem + buf * 65536 + wave * 8192;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            __builtin_amdgcn_global_load_lds((gptr_t)(xk + xo[j]), (lptr_t)(dx + j * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(wk + wo[j]), (lptr_t)(dx + 32768 + j * 1024), 16, 0, 0);
-        }
+    auto copy_x = [&](int s, int j) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(xt + s * G_BK + xo[j]),
+                                         (lptr_t)(smem + ((2 * s) % G_SLOTS) * G_SLOT_BYTES + wave * 4096 + j * 1024), 16, 0, 0);
+    };
+    auto copy_w = [&](int s, int j) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(wt + s * G_BK + wo[j]),
+                                         (lptr_t)(smem + ((2 * s + 1) % G_SLOTS) * G_SLOT_BYTES + wave * 4096 + j * 1024), 16, 0, 0);
     };
 
-    // Operand fragments.  The swizzle term depends only on row mod 16 and the rows a lane reads differ by
-    // multiples of 32, so one base offset per operand plus compile-time multiples of 32 rows (4096 bytes)
-    // covers them all; the column step kk only flips bits 5-6 of the offset (kk << 5).
-    half8v fa[4][4], fb[4][4];
-    const int frow = lane & 31, fhalf = lane >> 5;
-    const uint32_t fa_off = (uint32_t)((wm + frow) * 128 + swz(frow, fhalf) * 16);
-    const uint32_t fb_off = (uint32_t)((wn + frow) * 128 + swz(frow, fhalf) * 16 + 32768);
-    auto load_frags = [&](const unsigned char* buf, int kk) {
-        const unsigned char* pa = buf + (fa_off ^ (uint32_t)(kk << 5));
-        const unsigned char* pb = buf + (fb_off ^ (uint32_t)(kk << 5));
+    // Fragments.  A lane reads row (lane & 31) + 32 i of its wave's rows, piece 2 kk + (lane >> 5); the swizzle
+    // term depends on the row modulo 16 only and the column step kk only flips bits 5-6 of the offset, so one
+    // offset per operand plus compile-time multiples of 32 rows (4096 bytes) covers all reads of a slab.
+    half8v fa[2][4], fb[2][2];
+    const int frow = lane & 31, fhalf = lane >> 5, fsw = (frow >> 1) & 7;
+    const uint32_t fa_off = (uint32_t)((wm + frow) * 128 + ((fhalf ^ fsw) << 4));
+    const uint32_t fb_off = (uint32_t)((wn + frow) * 128 + ((fhalf ^ fsw) << 4));
+    auto load_frags = [&](int s, int kk, int set) {
+        const unsigned char* pa = smem + ((2 * s) % G_SLOTS) * G_SLOT_BYTES + (fa_off ^ (uint32_t)(kk << 5));
+        const unsigned char* pb = smem + ((2 * s + 1) % G_SLOTS) * G_SLOT_BYTES + (fb_off ^ (uint32_t)(kk << 5));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) fa[kk][i] = *reinterpret_cast<const half8v*>(pa + i * 4096);
+        for (int i = 0; i < 4; ++i) fa[set][i] = *reinterpret_cast<const half8v*>(pa + i * 4096);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) fb[kk][j] = *reinterpret_cast<const half8v*>(pb + j * 4096);
+        for (int j = 0; j < 2; ++j) fb[set][j] = *reinterpret_cast<const half8v*>(pb + j * 4096);
     };
-    auto multiply = [&](int kk) {
+    auto mma_row = [&](int set, int i) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
     };
+#ifndef SQ_SB
+#define SQ_SB() __builtin_amdgcn_sched_barrier(0)
+#endif
 
-    // Column-tile loop: read all of this tile's fragments (the matrix instructions start as the first ones
-    // arrive), then start the next tile's transfer into the other buffer, then multiply.  No LDS read follows
-    // the transfer inside an iteration, so nothing waits for it before the barrier at the end.
     const int nk = a.C / G_BK;
-    stage(0, 0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const unsigned char* buf = smem + (kt & 1) * 65536;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) load_frags(buf, kk);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt + 1 < nk) stage((kt + 1) * G_BK, (kt + 1) & 1);
-        __builtin_amdgcn_sched_barrier(0);
+    for (int j = 0; j < 4; ++j) copy_x(0, j);
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) multiply(kk);
-        __syncthreads();
+    for (int j = 0; j < 4; ++j) copy_w(0, j);
+    if (nk > 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) copy_x(1, j);
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+    } else {
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
     }
+    __builtin_amdgcn_s_barrier();
+    load_frags(0, 0, 0);
+    for (int s = 0; s < nk; ++s) {
+        // Each 16-column step starts with two matrix instructions (the wait in front of them covers only
+        // fragment reads issued a whole step earlier), then requests the next step's fragments, then finishes
+        // its matrix instructions with this slab's share of copies in between.
+        const bool more1 = s + 1 < nk, more2 = s + 2 < nk;
+        // step 0: W of slab s + 1 goes out first (it is needed at the end of this slab)
+        mma_row(0, 0); SQ_SB();
+        load_frags(s, 1, 1); SQ_SB();
+        mma_row(0, 1); SQ_SB();
+        if (more1) { copy_w(s + 1, 0); copy_w(s + 1, 1); } SQ_SB();
+        mma_row(0, 2); SQ_SB();
+        if (more1) copy_w(s + 1, 2); SQ_SB();
+        mma_row(0, 3); SQ_SB();
+        if (more1) copy_w(s + 1, 3); SQ_SB();
+        // steps 1 and 2: X of slab s + 2
+        mma_row(1, 0); SQ_SB();
+        load_frags(s, 2, 0); SQ_SB();
+        mma_row(1, 1); SQ_SB();
+        if (more2) copy_x(s + 2, 0); SQ_SB();
+        mma_row(1, 2); SQ_SB();
+        if (more2) copy_x(s + 2, 1); SQ_SB();
+        mma_row(1, 3); SQ_SB();
+        mma_row(0, 0); SQ_SB();
+        load_frags(s, 3, 1); SQ_SB();
+        mma_row(0, 1); SQ_SB();
+        if (more2) copy_x(s + 2, 2); SQ_SB();
+        mma_row(0, 2); SQ_SB();
+        if (more2) copy_x(s + 2, 3); SQ_SB();
+        mma_row(0, 3); SQ_SB();
+        // step 3: this wave's copies of slab s + 1 are waited for (the four X copies of slab s + 2 stay in
+        // flight), then the barrier: everybody's copies of slab s + 1 have landed and everybody has read slab s
+        // to the end, so its two slots can take W of slab s + 2 and X of slab s + 3 during the next slab
+        mma_row(1, 0); SQ_SB();
+        if (more1) {
+            if (more2) __builtin_amdgcn_s_waitcnt(vmcnt_only(4)); else __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+            SQ_SB();
+            __builtin_amdgcn_s_barrier();
+            SQ_SB();
+            load_frags(s + 1, 0, 0);
+        }
+        SQ_SB();
+        mma_row(1, 1); mma_row(1, 2); mma_row(1, 3); SQ_SB();
+    }
+#undef SQ_SB
 
     // epilogue
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 2; ++j) {
         const int r = r0 + wn + j * 32 + (lane & 31);
         if (r >= a.R) continue;
         const float sc_r = a.row_scale ? h2f(a.row_scale[r]) : 1.f;
@@ -158,7 +211,7 @@ __global__ __launch_bounds__(256) void bf16_to_f16_kernel(const uint16_t* __rest
 }
 
 bool gemm256_ok(int C, int64_t ldx, int64_t ldw, const void* x, const void* w) {
-    return C % G_BK == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
+    return C % 64 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
 }
 
 // x and w fp16.  row_scale may be NULL.
@@ -176,7 +229,7 @@ int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ld
     a.tiles_t = (T + G_BM - 1) / G_BM;
     a.tiles_r = (R + G_BN - 1) / G_BN;
     const unsigned grid = (unsigned)((a.tiles_t * a.tiles_r + 7) / 8 * 8);
-    hipLaunchKernelGGL(gemm256_kernel, dim3(grid), dim3(256), 131072, s, a);
+    hipLaunchKernelGGL(gemm256_kernel, dim3(grid), dim3(G_WAVES * 64), G_SLOTS * G_SLOT_BYTES, s, a);
     return check_launch("sq_linear_gemm(gemm256)");
 }
 
