@@ -11,6 +11,7 @@
 //   A: row l % 32, k = 8 * (l / 32) .. + 7        (tokens)
 //   B: col l % 32, k = 8 * (l / 32) .. + 7        (weight rows)
 //   D[v], v = 0..15: row 8 * (v / 4) + 4 * (l / 32) + v % 4, col l % 32
+#include <algorithm>
 #include "sq_common.h"
 
 namespace sq {
@@ -145,8 +146,11 @@ int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtyp
                          int y_dtype, int64_t ldy, int B, hipStream_t s);
 
 bool gemm256_ok(int C, int64_t ldx, int64_t ldw, const void* x, const void* w);
+int gemm256_ksplit(int T, int R, int C, int cus);
+size_t gemm256_part_bytes(int T, int R, int C, int cus);
+int device_cus();
 int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ldw, const uint16_t* row_scale, void* y,
-                   int y_dtype, int64_t ldy, int y_off, int T, int R, int C, hipStream_t s);
+                   int y_dtype, int64_t ldy, int y_off, int T, int R, int C, float* part, int cus, hipStream_t s);
 int launch_bf16_to_f16(const uint16_t* x, int64_t ldx, int T, int C, uint16_t* out, hipStream_t s);
 
 static bool x_vec_ok(const void* x, int64_t ldx, int C) { return C % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x & 15) == 0; }
@@ -163,7 +167,12 @@ size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
     const bool big = T >= GEMM256_MIN_T && mats[0].C % 64 == 0;
     for (int i = 0; i < n; ++i)
         if ((big || !fused_ok(mats[i])) && dense_bytes(mats[i]) > need) need = dense_bytes(mats[i]);
-    if (big) need += align256((size_t)T * mats[0].C * 2);       // fp16 copy of bf16 activations
+    if (big) {
+        need += align256((size_t)T * mats[0].C * 2);            // fp16 copy of bf16 activations
+        size_t part = 0;                                        // fp32 partial products of a K split
+        for (int i = 0; i < n; ++i) part = std::max(part, gemm256_part_bytes(T, mats[i].R, mats[i].C, device_cus()));
+        need += part;
+    }
     return need;
 }
 
@@ -180,7 +189,7 @@ int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, con
     if (!x_vec_ok(x, ldx, C) || !x_vec_ok(w, ldw, C))
         return fail(SQ_EUNSUPPORTED, "sq_gemm_dense: C, ldx, ldw must be multiples of 8 and pointers 16-byte aligned");
     if (x_dtype == SQ_F16 && w_dtype == SQ_F16 && T >= GEMM256_MIN_T && gemm256_ok(C, ldx, ldw, x, w))
-        return launch_gemm256((const uint16_t*)x, ldx, (const uint16_t*)w, ldw, nullptr, y, y_dtype, ldy, 0, T, R, C, s);
+        return launch_gemm256((const uint16_t*)x, ldx, (const uint16_t*)w, ldw, nullptr, y, y_dtype, ldy, 0, T, R, C, nullptr, 0, s);
     GemmArgs a{};
     a.m.R = R; a.m.C = C; a.m.y_off = 0;
     a.wd = (const uint16_t*)w; a.ldw = ldw;
@@ -216,12 +225,17 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
             ldxh = C;
         }
         wd += align256((size_t)T * C * 2);
+        size_t dense = 0;
+        for (int i = 0; i < n; ++i) dense = std::max(dense, dense_bytes(mats[i]));
+        float* part = (float*)(wd + dense);
+        const int cus = device_cus();
         for (int i = 0; i < n; ++i) {
             const sq_matrix& m = mats[i];
             if (m.R == 0) continue;
             int rc = launch_dequant(m, wd, SQ_F16, C, 0, m.R, s, /*raw=*/true);
             if (rc) return rc;
-            rc = launch_gemm256(xh, ldxh, (const uint16_t*)wd, C, m.row_scale, y, y_dtype, ldy, m.y_off, T, m.R, C, s);
+            rc = launch_gemm256(xh, ldxh, (const uint16_t*)wd, C, m.row_scale, y, y_dtype, ldy, m.y_off, T, m.R, C,
+                                gemm256_part_bytes(T, m.R, C, cus) ? part : nullptr, cus, s);
             if (rc) return rc;
         }
         return SQ_OK;

@@ -36,6 +36,8 @@ struct Gemm256Args {
     int64_t ldx, ldw, ldy;
     int T, R, C, y_off, y_dtype;
     int tiles_t, tiles_r;     // token / weight-row tiles (for the workgroup -> tile mapping)
+    int ks;                   // K split: workgroup (tile, kz) multiplies slabs [kz nk / ks, (kz + 1) nk / ks)
+    float* part;              // ks > 1: fp32 partial products [ks][T][R], unscaled
 };
 
 // s_waitcnt immediate that waits until at most n vector-memory operations are outstanding and leaves the
@@ -50,10 +52,12 @@ __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
     // tile is fetched by one L2 only.  The grid is padded to a multiple of 8; surplus workgroups leave.
     const int per_xcd = gridDim.x >> 3;
     const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    if (tile >= a.tiles_t * a.tiles_r) return;
+    const int ntiles = a.tiles_t * a.tiles_r;
+    if (tile >= ntiles * a.ks) return;
+    const int kz = tile / ntiles;
     // consecutive tiles walk the token tiles of one weight tile, so a weight tile is fetched from HBM once and
     // its re-reads hit L2 while the (small) activation matrix stays resident
-    const int bt = tile % a.tiles_t, br = tile / a.tiles_t;
+    const int bt = (tile % ntiles) % a.tiles_t, br = (tile % ntiles) / a.tiles_t;
     const int t0 = bt * G_BM, r0 = br * G_BN;
     const int wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
 
@@ -82,8 +86,10 @@ __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
         xo[j] = (uint32_t)(t * (int)a.ldx + c * 8);
         wo[j] = (uint32_t)(r * (int)a.ldw + c * 8);
     }
-    const uint16_t* xt = a.x + (int64_t)t0 * a.ldx;
-    const uint16_t* wt = a.w + (int64_t)r0 * a.ldw;
+    const int nk_all = a.C / G_BK, k_begin = (int)((int64_t)kz * nk_all / a.ks);
+    const int nk = (int)((int64_t)(kz + 1) * nk_all / a.ks) - k_begin;
+    const uint16_t* xt = a.x + (int64_t)t0 * a.ldx + (int64_t)k_begin * G_BK;
+    const uint16_t* wt = a.w + (int64_t)r0 * a.ldw + (int64_t)k_begin * G_BK;
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
     auto copy_x = [&](int s, int j) {
@@ -119,7 +125,6 @@ __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
 #define SQ_SB() __builtin_amdgcn_sched_barrier(0)
 #endif
 
-    const int nk = a.C / G_BK;
 #pragma unroll
     for (int j = 0; j < 4; ++j) copy_x(0, j);
 #pragma unroll
@@ -190,6 +195,10 @@ __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
             for (int v = 0; v < 16; ++v) {
                 const int t = t0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 if (t >= a.T) continue;
+                if (a.ks > 1) {
+                    a.part[((int64_t)kz * a.T + t) * a.R + r] = acc[i][j][v];
+                    continue;
+                }
                 const float val = acc[i][j][v] * sc_r;
                 const int64_t o = (int64_t)t * a.ldy + a.y_off + r;
                 if (a.y_dtype == SQ_BF16) reinterpret_cast<uint16_t*>(a.y)[o] = f2bf(val);
@@ -210,13 +219,41 @@ __global__ __launch_bounds__(256) void bf16_to_f16_kernel(const uint16_t* __rest
     *reinterpret_cast<u32x4*>(out + i) = v;
 }
 
+// y[t, y_off + r] = row_scale[r] * sum over kz of part[kz][t][r]
+__global__ __launch_bounds__(256) void gemm256_reduce_kernel(const float* __restrict__ part, int ks, int T, int R,
+                                                             const uint16_t* __restrict__ row_scale, void* y, int64_t ldy,
+                                                             int y_off, int y_dtype) {
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= (int64_t)T * R) return;                            // R % 4 == 0 (checked by the launcher)
+    const int t = (int)(i / R), r = (int)(i - (int64_t)t * R);
+    float4v sum = *reinterpret_cast<const float4v*>(part + i);
+    for (int kz = 1; kz < ks; ++kz) sum += *reinterpret_cast<const float4v*>(part + (int64_t)kz * T * R + i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        store_y(y, y_dtype, (int64_t)t * ldy + y_off + r + e, sum[e] * (row_scale ? h2f(row_scale[r + e]) : 1.f));
+}
+
+// K split for shapes with too few tiles to fill the chip (e.g. 2048 x 3584 outputs = 112 tiles on 256 CUs)
+int gemm256_ksplit(int T, int R, int C, int cus) {
+    const int tiles = ((T + G_BM - 1) / G_BM) * ((R + G_BN - 1) / G_BN);
+    int ks = cus / tiles;
+    if (ks > 4) ks = 4;
+    while (ks > 1 && (C / G_BK) / ks < 16) --ks;                // keep at least 16 slabs per workgroup
+    return (ks < 1 || R % 4) ? 1 : ks;
+}
+
+size_t gemm256_part_bytes(int T, int R, int C, int cus) {
+    const int ks = gemm256_ksplit(T, R, C, cus);
+    return ks > 1 ? ((size_t)ks * T * R * 4 + 255) & ~(size_t)255 : 0;
+}
+
 bool gemm256_ok(int C, int64_t ldx, int64_t ldw, const void* x, const void* w) {
     return C % 64 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
 }
 
-// x and w fp16.  row_scale may be NULL.
+// x and w fp16.  row_scale may be NULL.  `part` (gemm256_part_bytes) enables the K split; NULL = no split.
 int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ldw, const uint16_t* row_scale, void* y,
-                   int y_dtype, int64_t ldy, int y_off, int T, int R, int C, hipStream_t s) {
+                   int y_dtype, int64_t ldy, int y_off, int T, int R, int C, float* part, int cus, hipStream_t s) {
     static bool raised = false;
     if (!raised) {
         (void)hipFuncSetAttribute((const void*)gemm256_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -228,9 +265,16 @@ int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ld
     a.T = T; a.R = R; a.C = C; a.y_off = y_off; a.y_dtype = y_dtype;
     a.tiles_t = (T + G_BM - 1) / G_BM;
     a.tiles_r = (R + G_BN - 1) / G_BN;
-    const unsigned grid = (unsigned)((a.tiles_t * a.tiles_r + 7) / 8 * 8);
+    a.ks = part ? gemm256_ksplit(T, R, C, cus) : 1;
+    a.part = part;
+    const unsigned grid = (unsigned)((a.tiles_t * a.tiles_r * a.ks + 7) / 8 * 8);
     hipLaunchKernelGGL(gemm256_kernel, dim3(grid), dim3(G_WAVES * 64), G_SLOTS * G_SLOT_BYTES, s, a);
-    return check_launch("sq_linear_gemm(gemm256)");
+    int rc = check_launch("sq_linear_gemm(gemm256)");
+    if (rc || a.ks == 1) return rc;
+    const int64_t n4 = (int64_t)T * R / 4;
+    hipLaunchKernelGGL(gemm256_reduce_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, part, a.ks, T, R, row_scale, y,
+                       ldy, y_off, y_dtype);
+    return check_launch("sq_linear_gemm(gemm256 reduce)");
 }
 
 int launch_bf16_to_f16(const uint16_t* x, int64_t ldx, int T, int C, uint16_t* out, hipStream_t s) {

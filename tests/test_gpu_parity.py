@@ -235,6 +235,8 @@ GEMM = [  # R, C, d, bits, G, M, T
     (96, 256, 4, 10, 4, 16, 70), (140, 5120, 8, 16, 1, 16, 129), (50, 96, 2, 5, 3, 1, 40), (64, 200, 4, 8, 1, 1, 35),
     # 256 activation rows and more: the 256 x 256 tile route (ragged row / token counts, mixture books, column orders)
     (300, 1280, 4, 10, 4, 1, 260), (140, 5120, 8, 16, 1, 16, 300), (513, 640, 4, 8, 1, 1, 256), (257, 3584, 8, 16, 1, 1, 511),
+    # few tiles, long rows: K split over 3 and 4 workgroups with fp32 partial products
+    (260, 3584, 8, 16, 1, 1, 511), (512, 4096, 8, 14, 1, 1, 256),
 ]
 
 
