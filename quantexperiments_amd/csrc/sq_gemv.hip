@@ -90,6 +90,15 @@ static Plan plan_for(int U, int bits, int d) {
     return best;
 }
 
+// The tag-stream kernel multiplies one activation row.  It is also the fastest route for two rows of a large
+// matrix (two passes beat the L2-gather kernel from about 32 M weights: measured 58.7 against 84.4 us for two
+// 18944 x 3584 pieces, 25.3 against 14.0 us for one 3584 x 3584) and for any B <= 32 of a piece with column
+// orders (the alternative there is the VALU kernel): the launcher then runs it once per activation row.
+static bool stream_rows(const sq_matrix& m, int B) {
+    if (!stream_shape(m)) return false;
+    return B == 1 || m.perms != nullptr || (B == 2 && (int64_t)m.R * m.C >= (int64_t)32 << 20);
+}
+
 // ---- matrix-core path (pieces without column orders)
 struct MmaPlan { int RW, NT, KW, ks; };
 
@@ -120,7 +129,7 @@ static size_t mma_part_bytes(const sq_matrix& m, int B) {
 size_t small_workspace(const sq_matrix* mats, int n, int B) {
     size_t tot = 0;
     for (int i = 0; i < n; ++i) {
-        if (B == 1 && stream_shape(mats[i])) tot += stream_part_bytes(mats[i]);
+        if (stream_rows(mats[i], B)) tot += stream_part_bytes(mats[i]);
         else if (mma_shape(mats[i])) tot += mma_part_bytes(mats[i], B);
         else if (mats[i].perms && fast_shape(mats[i])) tot += xp_bytes(mats[i], B);
     }
@@ -202,11 +211,19 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         const sq_matrix& m0 = mats[i];
         if (m0.R == 0) { ++i; continue; }
         const int ud = unit_dwords(m0.bits);
-        if (B == 1 && stream_shape(m0) && x_ok) {
+        if (stream_rows(m0, B) && x_ok) {
             int j = i + 1;
-            while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_shape(mats[j]) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
-            int rc = launch_stream_group(mats + i, j - i, x, x_dtype, y, y_dtype, (char*)ws, ws_off, counters, counters_used, cus, s);
-            if (rc) return rc;
+            while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_rows(mats[j], B) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
+            const size_t ws0 = ws_off, ysz = y_dtype == SQ_F32 ? 4 : 2;
+            const int c0 = counters_used;
+            for (int b = 0; b < B; ++b) {                       // same partial sums and counters for every row: one stream
+                ws_off = ws0;
+                counters_used = c0;
+                int rc = launch_stream_group(mats + i, j - i, (const char*)x + (size_t)b * ldx * 2, x_dtype,
+                                             (char*)y + (size_t)b * ldy * ysz, y_dtype, (char*)ws, ws_off, counters,
+                                             counters_used, cus, s);
+                if (rc) return rc;
+            }
             i = j;
             continue;
         }
@@ -224,7 +241,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         if (pl.TS == 0) {
             int rc = launch_small_generic(mats + i, 1, x, x_dtype, ldx, y, y_dtype, ldy, B, s);
             if (rc) return rc;
-            if (B == 1 && stream_shape(m0)) ws_off += stream_part_bytes(m0);
+            if (stream_rows(m0, B)) ws_off += stream_part_bytes(m0);
             else if (mma_shape(m0)) ws_off += mma_part_bytes(m0, B);
             else if (m0.perms && fast_shape(m0)) ws_off += xp_bytes(m0, B);
             ++i;
