@@ -90,13 +90,14 @@ static Plan plan_for(int U, int bits, int d) {
     return best;
 }
 
-// The tag-stream kernel multiplies one activation row.  It is also the fastest route for two rows of a large
-// matrix (two passes beat the L2-gather kernel from about 32 M weights: measured 58.7 against 84.4 us for two
-// 18944 x 3584 pieces, 25.3 against 14.0 us for one 3584 x 3584) and for any B <= 32 of a piece with column
-// orders (the alternative there is the VALU kernel): the launcher then runs it once per activation row.
+// The tag-stream kernel multiplies up to 8 activation rows per pass (every codeword gathered once, one x gather
+// per row).  With column orders (where the alternative is the VALU kernel) it is used for any B <= 32.  Without,
+// it wins over the matrix-core kernel's single L2 gather per tag for up to 4 rows of a large matrix (measured on
+// the two 18944 x 3584 pieces: 49 / 73 / 119 us at B = 2 / 4 / 8 against 85 us; on one 3584 x 3584: 21 / 26 us
+// against 14 us).
 static bool stream_rows(const sq_matrix& m, int B) {
     if (!stream_shape(m)) return false;
-    return B == 1 || m.perms != nullptr || (B == 2 && (int64_t)m.R * m.C >= (int64_t)32 << 20);
+    return B == 1 || m.perms != nullptr || (B <= 4 && (int64_t)m.R * m.C >= (int64_t)32 << 20);
 }
 
 // ---- matrix-core path (pieces without column orders)
@@ -129,7 +130,7 @@ static size_t mma_part_bytes(const sq_matrix& m, int B) {
 size_t small_workspace(const sq_matrix* mats, int n, int B) {
     size_t tot = 0;
     for (int i = 0; i < n; ++i) {
-        if (stream_rows(mats[i], B)) tot += stream_part_bytes(mats[i]);
+        if (stream_rows(mats[i], B)) tot += stream_part_bytes(mats[i], B);
         else if (mma_shape(mats[i])) tot += mma_part_bytes(mats[i], B);
         else if (mats[i].perms && fast_shape(mats[i])) tot += xp_bytes(mats[i], B);
     }
@@ -216,14 +217,17 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
             while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_rows(mats[j], B) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
             const size_t ws0 = ws_off, ysz = y_dtype == SQ_F32 ? 4 : 2;
             const int c0 = counters_used;
-            for (int b = 0; b < B; ++b) {                       // same partial sums and counters for every row: one stream
+            size_t ws_end = ws0;
+            for (int b0 = 0; b0 < B; b0 += 8) {                 // same partial sums and counters for every pass: one stream
                 ws_off = ws0;
                 counters_used = c0;
-                int rc = launch_stream_group(mats + i, j - i, (const char*)x + (size_t)b * ldx * 2, x_dtype,
-                                             (char*)y + (size_t)b * ldy * ysz, y_dtype, (char*)ws, ws_off, counters,
-                                             counters_used, cus, s);
+                int rc = launch_stream_group(mats + i, j - i, (const char*)x + (size_t)b0 * ldx * 2, x_dtype, ldx,
+                                             (char*)y + (size_t)b0 * ldy * ysz, y_dtype, ldy, B - b0 < 8 ? B - b0 : 8, B,
+                                             (char*)ws, ws_off, counters, counters_used, s);
                 if (rc) return rc;
+                ws_end = ws_off;
             }
+            ws_off = ws_end;
             i = j;
             continue;
         }
@@ -241,7 +245,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         if (pl.TS == 0) {
             int rc = launch_small_generic(mats + i, 1, x, x_dtype, ldx, y, y_dtype, ldy, B, s);
             if (rc) return rc;
-            if (stream_rows(m0, B)) ws_off += stream_part_bytes(m0);
+            if (stream_rows(m0, B)) ws_off += stream_part_bytes(m0, B);
             else if (mma_shape(m0)) ws_off += mma_part_bytes(m0, B);
             else if (m0.perms && fast_shape(m0)) ws_off += xp_bytes(m0, B);
             ++i;

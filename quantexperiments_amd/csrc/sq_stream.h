@@ -26,8 +26,9 @@ size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int b
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                       unsigned char* out, size_t bytes, int* runs_out, int* groups_out);
 bool stream_shape(const sq_matrix& m);
-size_t stream_part_bytes(const sq_matrix& m);
-int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, void* y, int y_dtype, char* ws,
-                        size_t& ws_off, unsigned* counters, int& counters_used, int cus, hipStream_t s);
+size_t stream_part_bytes(const sq_matrix& m, int B);
+int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                        int64_t ldy, int nb, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
+                        hipStream_t s);
 
 }  // namespace sq

@@ -223,7 +223,7 @@ struct StreamPiece {
     const unsigned char* stream;
     const uint16_t* table;
     const uint16_t* row_scale;
-    float* part;                      // [NV][NG * 64], indexed by place
+    float* part;                      // [NV][NB][NG * 64], indexed by place
     unsigned* counters;               // one per run; zero before the launch, zero after it
     const int32_t* perms;             // [M, C] column orders or NULL
     int R, C, U, NS, NV, PC, NG, y_off;
@@ -234,14 +234,16 @@ struct StreamPiece {
 struct StreamArgs {
     StreamPiece p[GEMV_MAX_PIECES_STREAM];
     int n;
-    const uint16_t* x;
-    void* y;
+    const uint16_t* x;                // activation row b0
+    void* y;                          // output row b0
+    int64_t ldx, ldy;
+    int nb;                           // activation rows of this pass (<= NB)
     int x_dtype, y_dtype;
 };
 
-constexpr int STREAM_X_OFF = 65536;   // x part follows the 64 KB slice in LDS
+constexpr int STREAM_TAB = 65536;     // the codebook slice
+constexpr int STREAM_XS = STREAM_PART_MAX * 16;   // LDS bytes of one activation row's part of x
 constexpr int STREAM_PF = 4;          // steps fetched ahead
-constexpr int STREAM_NW = 8;          // waves per workgroup
 
 struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
 
@@ -250,8 +252,10 @@ struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
 #define SQ_TRACE_POINT(k)
 #endif
 
-__global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
-    constexpr int NW = STREAM_NW;
+// NB activation rows per pass (every entry's codeword is gathered once and multiplied with NB x chunks), NW waves.
+// LDS: [codebook slice 64 KB][NB x parts of 10 KB][two words of flags].
+template <int NB, int NW>
+__global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int pi = 0;
@@ -272,10 +276,11 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG + g0;
     const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
     const unsigned char* steps = P.stream + P.off_steps + lane * 12;
-    float* part = P.part + (size_t)v * P.NG * 64;
-    unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_X_OFF + P.PC * 16);   // [0] arrival result, [1] next group
+    const size_t np = (size_t)P.NG * 64;
+    float* part = P.part + (size_t)v * NB * np;
+    unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_TAB + NB * STREAM_XS);   // [0] arrival result, [1] next group
 
-    // The groups of a run are sorted longest first.  Wave w starts with group w, then group 15 - w; after
+    // The groups of a run are sorted longest first.  Wave w starts with group w, then group 2 NW - 1 - w; after
     // that every wave draws the next unclaimed group from a counter in LDS, so all waves stay busy to the end.
     // The head of a group (its first step, its step count, the lane's row and count) is fetched one group
     // ahead; the first one goes out before the staging loads.
@@ -301,40 +306,48 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
     for (int q = 0; q < STREAM_PF; ++q) nx[q] = u32x3{0u, 0u, 0u};
 
-    // stage the codebook slice and this part of x (as fp16); the first group's steps are requested before the
-    // LDS stores wait for the staging loads
+    // stage the codebook slice and this part of the NB activation rows (as fp16); the first group's steps are
+    // requested before the LDS stores wait for the staging loads
     {
         const u32x4* src = reinterpret_cast<const u32x4*>(P.table) + (size_t)s * (1 << STREAM_SLICE_BITS);
         u32x4* dst = reinterpret_cast<u32x4*>(lds);
         constexpr int NT = (1 << STREAM_SLICE_BITS) / (NW * 64);
-        u32x4 t[NT], xq[2];
+        constexpr int NX = (STREAM_PART_MAX + NW * 64 - 1) / (NW * 64);              // x chunks per thread and row
+        u32x4 t[NT], xq[NB][NX];
 #pragma unroll
         for (int k = 0; k < NT; ++k) t[k] = src[tid + k * NW * 64];
         const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
-        const u32x4* xs = reinterpret_cast<const u32x4*>(a.x) + c0;
-        u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_X_OFF);
-        if (P.perms == nullptr) {
 #pragma unroll
-            for (int k = 0; k < 2; ++k) xq[k] = xs[min(tid + k * NW * 64, nc - 1)];  // PC <= 640 < 2 * 512
-        } else {
-            // chunk j of a row with column order m multiplies x[perm_m[8 j .. 8 j + 7]]
-            const int32_t* pm = P.perms + (size_t)run[2] * P.C + (size_t)c0 * 8;
+        for (int b = 0; b < NB; ++b) {
+            const uint16_t* xr = a.x + (int64_t)min(b, a.nb - 1) * a.ldx;
+            if (P.perms == nullptr) {
+                const u32x4* xs = reinterpret_cast<const u32x4*>(xr) + c0;
 #pragma unroll
-            for (int k = 0; k < 2; ++k) {
-                const int32_t* pk = pm + (size_t)min(tid + k * NW * 64, nc - 1) * 8;
-                const u32x4 i0 = *reinterpret_cast<const u32x4*>(pk), i1 = *reinterpret_cast<const u32x4*>(pk + 4);
-                const uint32_t e0 = a.x[i0.x], e1 = a.x[i0.y], e2 = a.x[i0.z], e3 = a.x[i0.w];
-                const uint32_t e4 = a.x[i1.x], e5 = a.x[i1.y], e6 = a.x[i1.z], e7 = a.x[i1.w];
-                xq[k] = u32x4{e0 | (e1 << 16), e2 | (e3 << 16), e4 | (e5 << 16), e6 | (e7 << 16)};
+                for (int k = 0; k < NX; ++k) xq[b][k] = xs[min(tid + k * NW * 64, nc - 1)];
+            } else {
+                // chunk j of a row with column order m multiplies x[perm_m[8 j .. 8 j + 7]]
+                const int32_t* pm = P.perms + (size_t)run[2] * P.C + (size_t)c0 * 8;
+#pragma unroll
+                for (int k = 0; k < NX; ++k) {
+                    const int32_t* pk = pm + (size_t)min(tid + k * NW * 64, nc - 1) * 8;
+                    const u32x4 i0 = *reinterpret_cast<const u32x4*>(pk), i1 = *reinterpret_cast<const u32x4*>(pk + 4);
+                    const uint32_t e0 = xr[i0.x], e1 = xr[i0.y], e2 = xr[i0.z], e3 = xr[i0.w];
+                    const uint32_t e4 = xr[i1.x], e5 = xr[i1.y], e6 = xr[i1.z], e7 = xr[i1.w];
+                    xq[b][k] = u32x4{e0 | (e1 << 16), e2 | (e3 << 16), e4 | (e5 << 16), e6 | (e7 << 16)};
+                }
             }
         }
         first_steps(hn, nx);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            u32x4 q = xq[k];
-            if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
-            if (tid + k * NW * 64 < nc) xd[tid + k * NW * 64] = q;
+        for (int b = 0; b < NB; ++b) {
+            u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_TAB + b * STREAM_XS);
+#pragma unroll
+            for (int k = 0; k < NX; ++k) {
+                u32x4 q = xq[b][k];
+                if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
+                if (tid + k * NW * 64 < nc) xd[tid + k * NW * 64] = q;
+            }
         }
 #pragma unroll
         for (int k = 0; k < NT; ++k) dst[tid + k * NW * 64] = t[k];
@@ -356,7 +369,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         const int cnt = (int)(h.slot >> STREAM_ROW_BITS);
         const uint32_t row = h.slot & STREAM_NO_ROW;
         const unsigned char* eb = steps + (size_t)h.st0 * 768;
-        float acc = 0.f;
+        float acc[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[b] = 0.f;
         for (int t0 = 0; t0 < nst; t0 += STREAM_PF) {
             u32x3 cur[STREAM_PF];
 #pragma unroll
@@ -376,23 +391,30 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t ta = (e[j] << 4) & 0xFFF0u;
-                    const uint32_t xa = ((e[j] >> 8) & 0xFFFF0u) | (uint32_t)STREAM_X_OFF;
+                    const uint32_t xa = ((e[j] >> 8) & 0xFFFF0u) | (uint32_t)STREAM_TAB;
                     const u32x4 cw = *reinterpret_cast<const u32x4*>(lds + ta);
-                    const u32x4 xv = *reinterpret_cast<const u32x4*>(lds + xa);
-                    float dsum = 0.f;
+                    const bool valid = (t0 + q) * 4 + j < cnt;
 #pragma unroll
-                    for (int hh = 0; hh < 4; ++hh) {
-                        const uint32_t cwh = cw[hh], xvh = xv[hh];  // bit_cast straight from a vector element misreads it
-                        dsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, cwh), __builtin_bit_cast(half2v, xvh), dsum, false);
+                    for (int b = 0; b < NB; ++b) {
+                        const u32x4 xv = *reinterpret_cast<const u32x4*>(lds + xa + b * STREAM_XS);
+                        float dsum = 0.f;
+#pragma unroll
+                        for (int hh = 0; hh < 4; ++hh) {
+                            const uint32_t cwh = cw[hh], xvh = xv[hh];  // bit_cast straight from a vector element misreads it
+                            dsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, cwh), __builtin_bit_cast(half2v, xvh), dsum, false);
+                        }
+                        acc[b] += valid ? dsum : 0.f;
                     }
-                    acc += ((t0 + q) * 4 + j < cnt) ? dsum : 0.f;
                 }
             }
         }
         if (nst == 0) first_steps(hn, nx);                      // a group without steps fetched nothing for its successor
-        // device-scope store: written through to memory, so other XCDs' L2s never hold a stale copy and no
+        // device-scope stores: written through to memory, so other XCDs' L2s never hold a stale copy and no
         // cache-wide write-back is needed before the workgroup counts itself off
-        if (row != STREAM_NO_ROW) __hip_atomic_store(part + row, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (row != STREAM_NO_ROW) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) __hip_atomic_store(part + b * np + row, acc[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         kcur = knext;
         knext = kafter;
     }
@@ -413,64 +435,77 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     __syncthreads();
     SQ_TRACE_POINT(5);
     if (flag[0] != (unsigned)P.NV - 1u) return;
-    // 64 partial sums in flight per thread: four rows at a time when a row has 16 buckets, else one row's
-    // buckets 64 at a time; a row's partials are always added in bucket order
-    // places 64 g0 .. 64 (g0 + ng) - 1: consecutive partial sums; `rows` says which row each place is
+    // places 64 g0 .. 64 (g0 + ng) - 1: consecutive partial sums; `rows` says which row each place is.  An item
+    // is one (activation row, place); 64 partial sums are in flight per thread: four items at a time when a row
+    // has 16 buckets, else one item's buckets 64 at a time; a row's partials are always added in bucket order
     const uint32_t* rows0 = reinterpret_cast<const uint32_t*>(P.stream + P.off_rows) + (size_t)g0 * 64;
-    const int nl = ng * 64;
-    const size_t np = (size_t)P.NG * 64;
+    const int nl = ng * 64, items = nl * a.nb;
     const float* pp = P.part + (size_t)g0 * 64;
+    const size_t ysz = a.y_dtype == SQ_F32 ? 4 : 2;
+    auto row_of = [&](int i) -> uint32_t {
+        return P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
+    };
     if (P.NV <= 16) {
-        for (int ib = tid; ib < nl; ib += 4 * NW * 64) {
+        for (int ib = tid; ib < items; ib += 4 * NW * 64) {
             float t[4][16];
             uint32_t rr[4];
+            int bb[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int i = ib + q * NW * 64;
-                rr[q] = i >= nl ? STREAM_NO_ROW : P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
+                const int it = ib + q * NW * 64;
+                bb[q] = it < items ? it / nl : 0;
+                rr[q] = it < items ? row_of(it - bb[q] * nl) : STREAM_NO_ROW;
             }
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
+            for (int q = 0; q < 4; ++q) {
+                const int it = ib + q * NW * 64;
+                const uint32_t off = (uint32_t)(bb[q] * (int)np + (it - bb[q] * nl));  // uniform base + 32-bit lane offset
 #pragma unroll
                 for (int k = 0; k < 16; ++k)
-                    t[q][k] = (ib + q * NW * 64 < nl && k < P.NV)
-                                  ? __hip_atomic_load(pp + (size_t)k * np + ib + q * NW * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+                    t[q][k] = (it < items && k < P.NV)
+                                  ? __hip_atomic_load(pp + (size_t)k * NB * np + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 float sum = 0.f;
 #pragma unroll
                 for (int k = 0; k < 16; ++k) sum += t[q][k];
-                if (rr[q] != STREAM_NO_ROW) store_y(a.y, a.y_dtype, (int64_t)P.y_off + rr[q], sum * h2f(P.row_scale[rr[q]]));
+                if (rr[q] != STREAM_NO_ROW)
+                    store_y((char*)a.y + (size_t)bb[q] * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + rr[q], sum * h2f(P.row_scale[rr[q]]));
             }
         }
     } else {
-        for (int i = tid; i < nl; i += NW * 64) {
-            const uint32_t r = P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
+        for (int it = tid; it < items; it += NW * 64) {
+            const int b = it / nl, i = it - b * nl;
+            const uint32_t r = row_of(i);
             if (r == STREAM_NO_ROW) continue;
+            const uint32_t off = (uint32_t)(b * (int)np + i);
             float sum = 0.f;
             for (int v0 = 0; v0 < P.NV; v0 += 64) {
                 float t[64];
 #pragma unroll
                 for (int k = 0; k < 64; ++k)
                     t[k] = v0 + k < P.NV
-                               ? __hip_atomic_load(pp + (size_t)(v0 + k) * np + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+                               ? __hip_atomic_load(pp + (size_t)(v0 + k) * NB * np + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
 #pragma unroll
                 for (int k = 0; k < 64; ++k) sum += t[k];
             }
-            store_y(a.y, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
+            store_y((char*)a.y + (size_t)b * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
         }
     }
     SQ_TRACE_POINT(6);
 }
 
-static int stream_launch(const StreamArgs& a, int grid, size_t smem, hipStream_t s) {
+template <int NB, int NW>
+static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
     static bool raised = false;
     if (!raised) {
-        (void)hipFuncSetAttribute((const void*)stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         (void)hipGetLastError();
         raised = true;
     }
-    hipLaunchKernelGGL(stream_kernel, dim3((unsigned)grid), dim3(STREAM_NW * 64), smem, s, a);
+    const size_t smem = (size_t)STREAM_TAB + (size_t)NB * STREAM_XS + 16;
+    hipLaunchKernelGGL((stream_kernel<NB, NW>), dim3((unsigned)grid), dim3(NW * 64), smem, s, a);
     return check_launch("sq_linear_small(stream)");
 }
 
@@ -479,23 +514,28 @@ bool stream_shape(const sq_matrix& m) {
            (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0;
 }
 
-size_t stream_part_bytes(const sq_matrix& m) {
+// rows of one pass: 1, 2, 4 or 8
+int stream_pass_rows(int B) { return B > 4 ? 8 : B > 2 ? 4 : B > 1 ? 2 : 1; }
+
+size_t stream_part_bytes(const sq_matrix& m, int B) {
     const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, m.stream_runs);
-    return (((size_t)g.NV * g.NG * 64 * 4) + 255) & ~(size_t)255;
+    return (((size_t)g.NV * stream_pass_rows(B) * g.NG * 64 * 4) + 255) & ~(size_t)255;
 }
 
-// Pieces [0, cnt) (same C): one launch.  `counters` is the zeroed head of the workspace.
-int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, void* y, int y_dtype, char* ws,
-                        size_t& ws_off, unsigned* counters, int& counters_used, int cus, hipStream_t s) {
+// Pieces [0, cnt) (same C), activation rows b0 .. b0 + nb - 1 (nb <= 8): one launch.  `counters` is the zeroed head
+// of the workspace.
+int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                        int64_t ldy, int nb, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
+                        hipStream_t s) {
     StreamArgs a;
     a.n = cnt;
     a.x = (const uint16_t*)x;
     a.y = y;
+    a.ldx = ldx;
+    a.ldy = ldy;
+    a.nb = nb;
     a.x_dtype = x_dtype;
     a.y_dtype = y_dtype;
-    const StreamGeom g0 = stream_geom(mats[0].C, mats[0].d, mats[0].bits, mats[0].stream_groups, mats[0].stream_runs);
-    const size_t smem = (size_t)STREAM_X_OFF + (size_t)g0.PC * 16 + 16;      // slice, x part, two words of flags
-    (void)cus;
     int wg = 0;
     for (int k = 0; k < cnt; ++k) {
         const sq_matrix& m = mats[k];
@@ -507,7 +547,7 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         P.table = m.table;
         P.row_scale = m.row_scale;
         P.part = (float*)(ws + ws_off);
-        ws_off += stream_part_bytes(m);
+        ws_off += stream_part_bytes(m, B);
         P.perms = m.perms;
         P.R = m.R; P.C = m.C; P.U = g.U; P.NS = g.NS; P.NV = g.NV; P.PC = g.PC; P.NG = g.NG; P.y_off = m.y_off;
         P.off_slots = (uint32_t)g.off_slots; P.off_runs = (uint32_t)g.off_runs; P.off_rows = (uint32_t)g.off_rows;
@@ -521,7 +561,12 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         wg += g.NV * nwg;
     }
     for (int k = cnt; k < GEMV_MAX_PIECES_STREAM; ++k) a.p[k] = a.p[0];
-    return stream_launch(a, wg, smem, s);
+    switch (stream_pass_rows(nb)) {
+        case 1: return stream_launch<1, 8>(a, wg, s);           // 74 KB of LDS: two workgroups of 8 waves per CU
+        case 2: return stream_launch<2, 16>(a, wg, s);          // from here one workgroup of 16 waves per CU
+        case 4: return stream_launch<4, 16>(a, wg, s);
+        default: return stream_launch<8, 16>(a, wg, s);
+    }
 }
 
 }  // namespace sq

@@ -190,17 +190,17 @@ def test_stream_gemv_matches_oracle_and_row_path(case, dtype):
     y2 = torch.empty_like(y32)
     linear_small([lin], x.cuda(), y2)
     assert torch.equal(y2, y32)
-    # a few activation rows: with column orders the launcher runs the stream kernel once per row, and each row
-    # must then equal its own batch-1 result bit for bit
-    for B in (2, 5):
+    # several activation rows per pass (1, 2, 4 or 8; more passes beyond 8 rows with column orders): every row
+    # must equal its own batch-1 result bit for bit, since its sums are formed in the same order
+    for B in (2, 3, 5, 8) + ((11,) if M > 1 else ()):
         xb = rand_x(B, C, dtype, seed=R + B)
         yb = torch.full((B, R + 3), 5.0, dtype=torch.float32, device="cuda")
         linear_small([lin], xb.cuda(), yb[:, :R])
         assert rel_max_err(yb[:, :R].cpu().numpy(), _ref(s, xb)) < TOL and (yb[:, R:] == 5.0).all()
-        if M > 1:
+        if M > 1:                                       # (without column orders small matrices take the matrix-core kernel)
             for b in range(B):
                 linear_small([lin], xb[b:b + 1].cuda(), y2)
-                assert torch.equal(y2[0], yb[b, :R])
+                assert torch.equal(y2[0], yb[b, :R]), (B, b)
     # another cut into row runs: same sums up to the order of fp32 additions within a row
     for runs in (1, 3):
         lin.build_stream(runs)
@@ -382,6 +382,15 @@ def test_full_size_gemv_against_c_oracle(shape):
     y = torch.empty(1, R, dtype=torch.float32, device="cuda")
     linear_small([lin], x.cuda(), y)
     assert rel_max_err(y.cpu().numpy(), ref) < TOL
+    if lin.stream is not None:
+        # three activation rows in one pass of the tag-stream kernel: each row bit-identical to its batch-1 result
+        x3 = rand_x(3, C, torch.bfloat16, seed=7)
+        y3 = torch.empty(3, R, dtype=torch.float32, device="cuda")
+        linear_small([lin], x3.cuda(), y3)
+        assert rel_max_err(y3.cpu().numpy(), c_oracle.linear(_xf(x3), w)) < TOL
+        for b in range(3):
+            linear_small([lin], x3[b:b + 1].cuda(), y)
+            assert torch.equal(y[0], y3[b])
     # decoded matrix checksum: bit-exact against the C decode over all 68M / 26M weights
     assert torch.equal(lin.dense(torch.float32).cpu(), torch.from_numpy(w))
 
