@@ -146,7 +146,6 @@ int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtyp
                          int y_dtype, int64_t ldy, int B, hipStream_t s);
 
 bool gemm256_ok(int C, int64_t ldx, int64_t ldw, const void* x, const void* w);
-int gemm256_ksplit(int T, int R, int C, int cus);
 size_t gemm256_part_bytes(int T, int R, int C, int cus);
 int device_cus();
 int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ldw, const uint16_t* row_scale, void* y,

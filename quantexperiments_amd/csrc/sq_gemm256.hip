@@ -36,8 +36,12 @@ struct Gemm256Args {
     int64_t ldx, ldw, ldy;
     int T, R, C, y_off, y_dtype;
     int tiles_t, tiles_r;     // token / weight-row tiles (for the workgroup -> tile mapping)
-    int ks;                   // K split: workgroup (tile, kz) multiplies slabs [kz nk / ks, (kz + 1) nk / ks)
-    float* part;              // ks > 1: fp32 partial products [ks][T][R], unscaled
+    // The last round of tiles rarely fills the chip (592 tiles on 256 CUs: 2 full rounds and 80 tiles).  Tiles
+    // [0, main_tiles) are multiplied whole; each of the remaining tail tiles is split over kt workgroups, each
+    // taking the slabs [kz nk / kt, (kz + 1) nk / kt) and leaving an unscaled fp32 partial tile in
+    // part[(tail tile * kt + kz)][256][256] for gemm256_reduce_kernel.
+    int main_tiles, kt;
+    float* part;
 };
 
 // s_waitcnt immediate that waits until at most n vector-memory operations are outstanding and leaves the
@@ -47,17 +51,26 @@ constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) 
 __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so workgroup i of the launch
-    // takes tile (i % 8) * (n / 8) + i / 8: every XCD then works on one contiguous run of tiles and a weight
-    // tile is fetched by one L2 only.  The grid is padded to a multiple of 8; surplus workgroups leave.
-    const int per_xcd = gridDim.x >> 3;
-    const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so XCD x = blockIdx % 8 takes one
+    // contiguous run of whole tiles (a weight tile is then fetched by one L2 only) and, after those, one
+    // contiguous run of tail parts.  The grid is padded; surplus workgroups leave.
     const int ntiles = a.tiles_t * a.tiles_r;
-    if (tile >= ntiles * a.ks) return;
-    const int kz = tile / ntiles;
+    const int xcd = (int)(blockIdx.x & 7), jx = (int)(blockIdx.x >> 3);
+    const int main_per = (a.main_tiles + 7) >> 3, parts = (ntiles - a.main_tiles) * a.kt, parts_per = (parts + 7) >> 3;
+    int tile, kz = 0, nparts = 1;
+    if (jx < main_per) {
+        tile = xcd * main_per + jx;
+        if (tile >= a.main_tiles) return;
+    } else {
+        const int pidx = xcd * parts_per + (jx - main_per);
+        if (pidx >= parts) return;
+        tile = a.main_tiles + pidx / a.kt;
+        kz = pidx - (pidx / a.kt) * a.kt;
+        nparts = a.kt;
+    }
     // consecutive tiles walk the token tiles of one weight tile, so a weight tile is fetched from HBM once and
     // its re-reads hit L2 while the (small) activation matrix stays resident
-    const int bt = (tile % ntiles) % a.tiles_t, br = (tile % ntiles) / a.tiles_t;
+    const int bt = tile % a.tiles_t, br = tile / a.tiles_t;
     const int t0 = bt * G_BM, r0 = br * G_BN;
     const int wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
 
@@ -86,8 +99,8 @@ __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
         xo[j] = (uint32_t)(t * (int)a.ldx + c * 8);
         wo[j] = (uint32_t)(r * (int)a.ldw + c * 8);
     }
-    const int nk_all = a.C / G_BK, k_begin = (int)((int64_t)kz * nk_all / a.ks);
-    const int nk = (int)((int64_t)(kz + 1) * nk_all / a.ks) - k_begin;
+    const int nk_all = a.C / G_BK, k_begin = (int)((int64_t)kz * nk_all / nparts);
+    const int nk = (int)((int64_t)(kz + 1) * nk_all / nparts) - k_begin;
     const uint16_t* xt = a.x + (int64_t)t0 * a.ldx + (int64_t)k_begin * G_BK;
     const uint16_t* wt = a.w + (int64_t)r0 * a.ldw + (int64_t)k_begin * G_BK;
     typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -195,8 +208,8 @@ __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
             for (int v = 0; v < 16; ++v) {
                 const int t = t0 + wm + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 if (t >= a.T) continue;
-                if (a.ks > 1) {
-                    a.part[((int64_t)kz * a.T + t) * a.R + r] = acc[i][j][v];
+                if (nparts > 1) {
+                    a.part[((int64_t)(tile - a.main_tiles) * a.kt + kz) * (G_BM * G_BN) + (t - t0) * G_BN + (r - r0)] = acc[i][j][v];
                     continue;
                 }
                 const float val = acc[i][j][v] * sc_r;
@@ -219,39 +232,48 @@ __global__ __launch_bounds__(256) void bf16_to_f16_kernel(const uint16_t* __rest
     *reinterpret_cast<u32x4*>(out + i) = v;
 }
 
-// y[t, y_off + r] = row_scale[r] * sum over kz of part[kz][t][r]
-__global__ __launch_bounds__(256) void gemm256_reduce_kernel(const float* __restrict__ part, int ks, int T, int R,
-                                                             const uint16_t* __restrict__ row_scale, void* y, int64_t ldy,
-                                                             int y_off, int y_dtype) {
-    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
-    if (i >= (int64_t)T * R) return;                            // R % 4 == 0 (checked by the launcher)
-    const int t = (int)(i / R), r = (int)(i - (int64_t)t * R);
-    float4v sum = *reinterpret_cast<const float4v*>(part + i);
-    for (int kz = 1; kz < ks; ++kz) sum += *reinterpret_cast<const float4v*>(part + (int64_t)kz * T * R + i);
+// tail tiles: y[t, y_off + r] = row_scale[r] * sum over kz of part[(tail tile * kt + kz)][t - t0][r - r0]
+__global__ __launch_bounds__(256) void gemm256_reduce_kernel(const float* __restrict__ part, int main_tiles, int kt, int tiles_t,
+                                                             int T, int R, const uint16_t* __restrict__ row_scale, void* y,
+                                                             int64_t ldy, int y_off, int y_dtype) {
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;      // element of a tail tile, 4 per thread
+    const int tail = (int)(i / (G_BM * G_BN)), e = (int)(i - (int64_t)tail * (G_BM * G_BN));
+    const int tile = main_tiles + tail, t = (tile % tiles_t) * G_BM + e / G_BN, r = (tile / tiles_t) * G_BN + e % G_BN;
+    if (t >= T) return;
+    const float* p = part + (int64_t)tail * kt * (G_BM * G_BN) + e;
+    float4v sum = *reinterpret_cast<const float4v*>(p);
+    for (int kz = 1; kz < kt; ++kz) sum += *reinterpret_cast<const float4v*>(p + (int64_t)kz * (G_BM * G_BN));
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-        store_y(y, y_dtype, (int64_t)t * ldy + y_off + r + e, sum[e] * (row_scale ? h2f(row_scale[r + e]) : 1.f));
+    for (int q = 0; q < 4; ++q)
+        if (r + q < R) store_y(y, y_dtype, (int64_t)t * ldy + y_off + r + q, sum[q] * (row_scale ? h2f(row_scale[r + q]) : 1.f));
 }
 
-// K split for shapes with too few tiles to fill the chip (e.g. 2048 x 3584 outputs = 112 tiles on 256 CUs)
-int gemm256_ksplit(int T, int R, int C, int cus) {
+// How the tiles of a T x R output are dealt to `cus` CUs: whole rounds of whole tiles, and the tiles of the last,
+// partial round split over kt workgroups each (kt = 1: no split) while a part keeps at least 16 slabs.
+struct Gemm256Plan { int main_tiles, tail_tiles, kt; };
+static Gemm256Plan gemm256_plan(int T, int R, int C, int cus) {
     const int tiles = ((T + G_BM - 1) / G_BM) * ((R + G_BN - 1) / G_BN);
-    int ks = cus / tiles;
-    if (ks > 4) ks = 4;
-    while (ks > 1 && (C / G_BK) / ks < 16) --ks;                // keep at least 16 slabs per workgroup
-    return (ks < 1 || R % 4) ? 1 : ks;
+    Gemm256Plan p{tiles, 0, 1};
+    if (cus < 8) return p;
+    const int main = tiles / cus * cus, tail = tiles - main;          // cus is a multiple of 8 on this hardware
+    if (tail == 0 || main % 8) return p;
+    int kt = cus / tail;
+    if (kt > 4) kt = 4;
+    while (kt > 1 && (C / G_BK) / kt < 16) --kt;
+    if (kt < 2) return p;
+    return Gemm256Plan{main, tail, kt};
 }
 
 size_t gemm256_part_bytes(int T, int R, int C, int cus) {
-    const int ks = gemm256_ksplit(T, R, C, cus);
-    return ks > 1 ? ((size_t)ks * T * R * 4 + 255) & ~(size_t)255 : 0;
+    const Gemm256Plan p = gemm256_plan(T, R, C, cus);
+    return ((size_t)p.tail_tiles * p.kt * G_BM * G_BN * 4 + 255) & ~(size_t)255;
 }
 
 bool gemm256_ok(int C, int64_t ldx, int64_t ldw, const void* x, const void* w) {
     return C % 64 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0;
 }
 
-// x and w fp16.  row_scale may be NULL.  `part` (gemm256_part_bytes) enables the K split; NULL = no split.
+// x and w fp16.  row_scale may be NULL.  `part` (gemm256_part_bytes) enables the split of the last round; NULL = no split.
 int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ldw, const uint16_t* row_scale, void* y,
                    int y_dtype, int64_t ldy, int y_off, int T, int R, int C, float* part, int cus, hipStream_t s) {
     static bool raised = false;
@@ -265,15 +287,17 @@ int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ld
     a.T = T; a.R = R; a.C = C; a.y_off = y_off; a.y_dtype = y_dtype;
     a.tiles_t = (T + G_BM - 1) / G_BM;
     a.tiles_r = (R + G_BN - 1) / G_BN;
-    a.ks = part ? gemm256_ksplit(T, R, C, cus) : 1;
+    const Gemm256Plan pl = part ? gemm256_plan(T, R, C, cus) : Gemm256Plan{a.tiles_t * a.tiles_r, 0, 1};
+    a.main_tiles = pl.main_tiles;
+    a.kt = pl.kt;
     a.part = part;
-    const unsigned grid = (unsigned)((a.tiles_t * a.tiles_r * a.ks + 7) / 8 * 8);
+    const unsigned grid = (unsigned)(8 * ((pl.main_tiles + 7) / 8 + (pl.tail_tiles * pl.kt + 7) / 8));
     hipLaunchKernelGGL(gemm256_kernel, dim3(grid), dim3(G_WAVES * 64), G_SLOTS * G_SLOT_BYTES, s, a);
     int rc = check_launch("sq_linear_gemm(gemm256)");
-    if (rc || a.ks == 1) return rc;
-    const int64_t n4 = (int64_t)T * R / 4;
-    hipLaunchKernelGGL(gemm256_reduce_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, part, a.ks, T, R, row_scale, y,
-                       ldy, y_off, y_dtype);
+    if (rc || pl.tail_tiles == 0) return rc;
+    const int64_t n4 = (int64_t)pl.tail_tiles * G_BM * G_BN / 4;
+    hipLaunchKernelGGL(gemm256_reduce_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, part, pl.main_tiles, pl.kt,
+                       a.tiles_t, T, R, row_scale, y, ldy, y_off, y_dtype);
     return check_launch("sq_linear_gemm(gemm256 reduce)");
 }
 
