@@ -413,3 +413,35 @@ def test_full_size_gemm_rows_against_gemv():
     w = s.decode()
     ref = c_oracle.linear(x[toks].float().cpu().numpy(), w)
     assert rel_max_err(y[toks].cpu().numpy(), ref) < TOL
+
+
+# ------------------------------------------------------------------ randomized sweep over the large-codebook paths
+def test_random_large_codebook_shapes_match_oracle():
+    """40 seeded random matrices with d = 8 and 14..16-bit tags: row counts around the 64-row group and run
+    boundaries, column counts around the 640-chunk part boundary, 1..6 column orders (some of them unused by any
+    row), random run cuts and 1..9 activation rows, stacked in pairs."""
+    from quantexperiments_amd.kernels import linear_small, prepare_stack
+    rng = np.random.default_rng(2024)
+    for it in range(20):
+        C = int(rng.choice([8, 64, 512, 640 * 8, 648 * 8, 1288 * 8, 3584]))
+        bits = int(rng.choice([14, 15, 16]))
+        pair, refs = [], []
+        B = int(rng.integers(1, 10))
+        x = rand_x(B, C, torch.bfloat16, seed=it)
+        for k in range(2):
+            R = int(rng.choice([1, 63, 64, 65, 130, 257, 700]))
+            M = int(rng.choice([1, 1, 2, 6]))
+            s = synth(R, C, 8, bits, 1, M, seed=100 * it + k)
+            if M > 2 and R > 3:
+                s.row_mask[:] = np.where(s.row_mask == 1, 3, s.row_mask)        # order 1 has no rows
+            lin = to_device(s)
+            assert lin.stream is not None
+            lin.build_stream(int(rng.integers(0, 9)))
+            pair.append(lin)
+            refs.append(_ref(s, x))
+        if it % 2:
+            prepare_stack(pair)
+        y = torch.full((B, pair[0].R + pair[1].R), 3.0, dtype=torch.float32, device="cuda")
+        linear_small(pair, x.cuda(), y)
+        ref = np.concatenate(refs, axis=1)
+        assert rel_max_err(y.cpu().numpy(), ref) < TOL, (it, C, bits, B, [p.R for p in pair], [p.M for p in pair])
