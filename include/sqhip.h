@@ -94,7 +94,8 @@ int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C,
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which);
 
 /* Load-time regrouping of a matrix' tags for codebooks that do not fit LDS (d = 8, K = 8192..65,536, one
- * codebook): the batch-1 product then gathers codewords from a 64 KB LDS slice instead of from L2.
+ * codebook): the decode-time product (batch 1, up to 4 rows of large matrices, any B <= 32 with column
+ * orders) then gathers codewords from a 64 KB LDS slice instead of from L2.
  * HOST pointers: `tags_host` is the file's tag tensor in host memory, `row_mask_host` the file's row_mask
  * (NULL when the matrix has one column order), `out_host` receives sq_stream_bytes() bytes that the caller
  * copies to the device (16-byte aligned) and names in sq_matrix.stream, together with *runs_out and
