@@ -114,6 +114,38 @@ int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, i
                     const uint8_t* row_mask_host, int32_t runs, void* out_host, size_t out_bytes,
                     int32_t* runs_out, int32_t* groups_out);
 
+/* ---- The packed file's block-32 side formats (reference shapequant/packed.py:30-40): the 8-bit output head
+ * `aux.lm_head` (q int8 [V, C], scale fp16 [V, C/32], w = q * scale of the row's 32-column block) and the 4-bit
+ * embedding `aux.embed` (q uint8 [V, C/2] with column 2k in the low and 2k+1 in the high nibble of byte k, each
+ * storing n + 8 for n in -8..7, scale fp16 [V, C/32]).  q, scale, x, y, out, ids, workspace: DEVICE pointers (q
+ * and scale of sq_q4_embed may also be pinned host memory, which the GPU reads over the bus: the reference's
+ * host = True embedding, shapequant/vllm_ext/core.py:605-616).  q 16-byte aligned, C a multiple of 32.
+ *
+ * sq_q8_linear: Y[b, v] = sum_c X[b, c] * w[v, c] for B activation rows, fp32 accumulation with the block scale
+ * applied to each block's fp32 sum (the reference kernel's arithmetic, shapequant/kernels/batched_runs.py:376-440).
+ * B <= SQ_SMALL_BMAX streams q once per 4 activation rows and needs no workspace; it replaces gemv_q8_batched /
+ * gemv_q8_tile (reference shapequant/kernels/batched_runs.py:826-861, called from vllm_ext/core.py:575-583) and
+ * proto_formats.gemv_q8 (shapequant/kernels/proto_formats.py:474-482); it reads the file's natural layout, so
+ * there is no counterpart of the reference's tile-major copy.  B > SQ_SMALL_BMAX decodes row chunks to fp16 in
+ * the workspace (scale folded in, one rounding) and multiplies them with the tile GEMM, as the reference's chunked
+ * route does (vllm_ext/core.py:584-591); sq_q8_workspace_bytes gives the size (0 for B <= SQ_SMALL_BMAX), with the
+ * same rules as sq_workspace_bytes.  x_dtype / y_dtype as in sq_linear_small. */
+int sq_q8_linear(const int8_t* q, const uint16_t* scale, int32_t V, int32_t C, const void* x, int x_dtype, int64_t ldx,
+                 void* y, int y_dtype, int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream);
+size_t sq_q8_workspace_bytes(int32_t V, int32_t C, int32_t B);
+
+/* Dense rows [r0, r1) of the 8-bit matrix into out[(r - r0) * ld_out + c]: SQ_F32 is the exact product, SQ_F16 /
+ * SQ_BF16 round it once.  Replaces Q8Head._rows (reference shapequant/vllm_ext/core.py:548-555) and
+ * packed.q8_rows (shapequant/packed.py:155-158). */
+int sq_q8_dequant(const int8_t* q, const uint16_t* scale, int32_t V, int32_t C, void* out, int out_dtype, int64_t ld_out,
+                  int32_t r0, int32_t r1, void* stream);
+
+/* Rows ids[0..n_ids) (int64) of the 4-bit embedding into out[i * ld_out + c], same rounding rule as above; an id
+ * outside [0, V) gives a row of zeros.  Replaces q4_embed (reference shapequant/vllm_ext/core.py:594-602) and
+ * packed.q4_embed_rows (shapequant/packed.py:148-152). */
+int sq_q4_embed(const uint8_t* q, const uint16_t* scale, int32_t V, int32_t C, const int64_t* ids, int64_t n_ids, void* out,
+                int out_dtype, int64_t ld_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -17,6 +17,10 @@ multi-threaded baseline), the arithmetic of the reference's CPU path:
   linear / linear_input_form shapequant/kernels/gemv.py:1-17 (y = x . W^T; masks as input gathers)
   round_fp16 / round_bf16    shapequant/kernels/cuda_dequant.py:13, batched_runs.py:873-881
   storage_bits               tests/test_packed.py:52-56 (reference test formula)
+  q4_embed_pack / q4_embed_rows   shapequant/packed.py:134-152    4-bit block-32 embedding
+  q8_pack                    shapequant/kernels/proto_formats.py:464-471   8-bit block-32 head
+  q8_rows                    shapequant/packed.py:155-158
+  q8_linear                  shapequant/kernels/batched_runs.py:376-440 (per-block sum times block scale)
 
 Pinning status (what fixes each function besides this file's own formula):
   pack_bits/unpack_bits  known-answer layout vectors of the reference's tests, closed forms for
@@ -28,6 +32,12 @@ Pinning status (what fixes each function besides this file's own formula):
                          (tests/golden/seeded_perms.json); perm_crc also by zlib on hand-built bytes.
   linear                 float64 brute force; equivalence of weight-side scatter and input-side gather.
   layer_seed             closed form with zlib.crc32.
+  q4_embed_pack/q8_pack  hand-computed known-answer blocks (integer-valued weights whose scale is exactly 1
+                         or 1/2, ties that must round to even, the all-zero block, clamping at -8 / -127),
+                         a pure-Python nibble/byte walk of the stored bytes, and the error bound |w - w'| <=
+                         scale/2 that any correct round-to-nearest block quantizer meets.
+  q4_embed_rows/q8_rows  the same known-answer blocks decoded back, pure-Python loops on small inputs.
+  q8_linear              float64 dense product of q8_rows (the two must agree to fp32 rounding).
 """
 
 from __future__ import annotations
@@ -246,3 +256,59 @@ def torch_cpu_layer(words, table, row_scale, row_mask, perms, bits: int, x_bf16)
     y = (x_bf16.float().reshape(-1, C) @ w.T).to(torch.bfloat16)
     t2 = time.perf_counter()
     return y, t1 - t0, t2 - t1
+
+
+# ----------------------------------------------------------------------------- block-32 side formats
+
+def _block_quant(w, top: int, lo: int):
+    """Blocks of 32 columns: scale = fp16(fp32(max|w|, at least 1e-8) / top) (1 where that underflows to 0),
+    n = clamp(round_half_even(w / scale), lo, top), all in fp32 like the reference's torch code."""
+    w = np.asarray(w, dtype=np.float32)
+    V, C = w.shape
+    if C % 32:
+        raise ValueError(f"C={C} is not a multiple of 32")
+    b = w.reshape(V, C // 32, 32)
+    amax = np.maximum(np.abs(b).max(-1), np.float32(1e-8))
+    s = (amax / np.float32(top)).astype(np.float32).astype(np.float16)
+    s = np.where(s == 0, np.float16(1), s)
+    n = np.clip(np.rint(b / s.astype(np.float32)[..., None]), lo, top)
+    return n, s
+
+
+def q4_embed_pack(w):
+    """w [V, C] -> (q uint8 [V, C/2], scale fp16 [V, C/32]): column 2k in the low nibble of byte k, 2k+1 in the
+    high nibble, each nibble n + 8."""
+    n, s = _block_quant(w, 7, -8)
+    u = (n + 8).astype(np.uint8).reshape(n.shape[0], -1, 2)
+    return (u[..., 0] | (u[..., 1] << np.uint8(4))).astype(np.uint8), s
+
+
+def q4_embed_rows(q, sc, ids) -> np.ndarray:
+    """fp32 [len(ids), C]: ((nibble) - 8) * scale of the block."""
+    ids = np.asarray(ids).reshape(-1)
+    b = np.asarray(q)[ids]
+    n = np.stack([b & 15, b >> 4], -1).reshape(b.shape[0], -1).astype(np.float32) - np.float32(8)
+    return (n.reshape(b.shape[0], -1, 32) * np.asarray(sc)[ids].astype(np.float32)[..., None]).reshape(b.shape[0], -1)
+
+
+def q8_pack(w):
+    """w [V, C] -> (q int8 [V, C], scale fp16 [V, C/32], dequantized fp32 [V, C])."""
+    n, s = _block_quant(w, 127, -127)
+    shape = np.asarray(w).shape
+    return n.reshape(shape).astype(np.int8), s, (n * s.astype(np.float32)[..., None]).reshape(shape).astype(np.float32)
+
+
+def q8_rows(q, sc, s: int = 0, e: int | None = None) -> np.ndarray:
+    """fp32 rows s:e: q * scale of the block (exact: 8-bit integer times fp16)."""
+    b = np.asarray(q)[s:e].astype(np.float32)
+    return (b.reshape(b.shape[0], -1, 32) * np.asarray(sc)[s:e].astype(np.float32)[..., None]).reshape(b.shape[0], -1)
+
+
+def q8_linear(x, q, sc, acc=np.float64) -> np.ndarray:
+    """y[b, v] = sum over blocks of scale[v, blk] * (sum over the block's 32 columns of x[b, c] * q[v, c]),
+    the order the reference kernel uses; float64 by default."""
+    x = np.atleast_2d(np.asarray(x, dtype=np.float32)).astype(acc)
+    q = np.asarray(q).astype(acc)
+    V, C = q.shape
+    part = np.einsum("bkc,vkc->bvk", x.reshape(x.shape[0], C // 32, 32), q.reshape(V, C // 32, 32))
+    return (part * np.asarray(sc).astype(acc)[None]).sum(-1)

@@ -60,14 +60,21 @@ def lib() -> ctypes.CDLL:
         L.sq_stream_bytes.restype = sz
         L.sq_stream_build.argtypes = [vp, i32, i32, i32, i32, i32, vp, i32, vp, sz, ip, ip]
         L.sq_stream_build.restype = ctypes.c_int
-        for f in (L.sq_dequant, L.sq_linear_small, L.sq_linear_gemm, L.sq_gemm_dense):
+        L.sq_q8_linear.argtypes = [vp, vp, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
+        L.sq_q8_workspace_bytes.argtypes = [i32, i32, i32]
+        L.sq_q8_workspace_bytes.restype = sz
+        L.sq_q8_dequant.argtypes = [vp, vp, i32, i32, vp, ctypes.c_int, i64, i32, i32, vp]
+        L.sq_q4_embed.argtypes = [vp, vp, i32, i32, vp, i64, vp, ctypes.c_int, i64, vp]
+        for f in (L.sq_dequant, L.sq_linear_small, L.sq_linear_gemm, L.sq_gemm_dense, L.sq_q8_linear, L.sq_q8_dequant,
+                  L.sq_q4_embed):
             f.restype = ctypes.c_int
         _lib = L
     return _lib
 
 
 EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
-           "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build")
+           "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build", "sq_q8_linear", "sq_q8_workspace_bytes",
+           "sq_q8_dequant", "sq_q4_embed")
 
 
 def check(rc: int) -> None:

@@ -73,7 +73,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 101; }
+int sq_version(void) { return 102; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -139,6 +139,59 @@ int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, i
     if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_stream_build: W %d too small", W);
     return stream_build_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs, (unsigned char*)out_host,
                              out_bytes, runs_out, groups_out);
+}
+
+static int check_q8(const char* who, const void* q, const void* scale, int32_t V, int32_t C) {
+    if (V < 0 || C <= 0 || C % 32) return fail(SQ_EINVAL, "%s: V %d C %d (C must be a positive multiple of 32)", who, V, C);
+    if (V > 0 && (!q || !scale)) return fail(SQ_EINVAL, "%s: null q / scale", who);
+    if (((uintptr_t)q & 15) || ((uintptr_t)scale & 1)) return fail(SQ_EINVAL, "%s: q must be 16-byte aligned, scale 2-byte", who);
+    return SQ_OK;
+}
+
+int sq_q8_linear(const int8_t* q, const uint16_t* scale, int32_t V, int32_t C, const void* x, int x_dtype, int64_t ldx,
+                 void* y, int y_dtype, int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream) {
+    int rc = check_q8("sq_q8_linear", q, scale, V, C);
+    if (rc) return rc;
+    if (B < 0) return fail(SQ_EINVAL, "sq_q8_linear: %d activation rows", B);
+    if (x_dtype != SQ_F16 && x_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_q8_linear: x_dtype %d", x_dtype);
+    if (y_dtype != SQ_F16 && y_dtype != SQ_BF16 && y_dtype != SQ_F32) return fail(SQ_EINVAL, "sq_q8_linear: y_dtype %d", y_dtype);
+    if (y_dtype != SQ_F32 && y_dtype != x_dtype) return fail(SQ_EINVAL, "sq_q8_linear: y_dtype %d != x_dtype %d", y_dtype, x_dtype);
+    if (B == 0 || V == 0) return SQ_OK;
+    if (!x || !y) return fail(SQ_EINVAL, "sq_q8_linear: null x / y");
+    if (B > 1 && (ldx < C || ldy < V)) return fail(SQ_EINVAL, "sq_q8_linear: ldx %lld / ldy %lld too small", (long long)ldx, (long long)ldy);
+    if (B <= SQ_SMALL_BMAX) return launch_q8_small(q, scale, V, C, x, x_dtype, ldx, y, y_dtype, ldy, B, (hipStream_t)stream);
+    const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
+    return launch_q8_large(q, scale, V, C, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
+                           has_ws ? ws_bytes - SQ_WS_HEADER : 0, (hipStream_t)stream);
+}
+
+size_t sq_q8_workspace_bytes(int32_t V, int32_t C, int32_t B) {
+    if (C <= 0 || C % 32) return 0;
+    const size_t inner = q8_workspace(V, C, B);
+    return inner ? inner + SQ_WS_HEADER : 0;
+}
+
+int sq_q8_dequant(const int8_t* q, const uint16_t* scale, int32_t V, int32_t C, void* out, int out_dtype, int64_t ld_out,
+                  int32_t r0, int32_t r1, void* stream) {
+    int rc = check_q8("sq_q8_dequant", q, scale, V, C);
+    if (rc) return rc;
+    if (out_dtype != SQ_F16 && out_dtype != SQ_BF16 && out_dtype != SQ_F32) return fail(SQ_EINVAL, "sq_q8_dequant: out_dtype %d", out_dtype);
+    if (r0 < 0 || r1 < r0 || r1 > V) return fail(SQ_EINVAL, "sq_q8_dequant: rows [%d, %d) outside [0, %d)", r0, r1, V);
+    if (r1 == r0) return SQ_OK;
+    if (!out || ld_out < C) return fail(SQ_EINVAL, "sq_q8_dequant: out %p ld_out %lld", out, (long long)ld_out);
+    return launch_q8_dequant(q, scale, C, out, out_dtype, ld_out, r0, r1, (hipStream_t)stream);
+}
+
+int sq_q4_embed(const uint8_t* q, const uint16_t* scale, int32_t V, int32_t C, const int64_t* ids, int64_t n_ids, void* out,
+                int out_dtype, int64_t ld_out, void* stream) {
+    int rc = check_q8("sq_q4_embed", q, scale, V, C);
+    if (rc) return rc;
+    if (out_dtype != SQ_F16 && out_dtype != SQ_BF16 && out_dtype != SQ_F32) return fail(SQ_EINVAL, "sq_q4_embed: out_dtype %d", out_dtype);
+    if (n_ids < 0) return fail(SQ_EINVAL, "sq_q4_embed: %lld ids", (long long)n_ids);
+    if (n_ids == 0) return SQ_OK;
+    if (!ids || !out || ld_out < C) return fail(SQ_EINVAL, "sq_q4_embed: ids %p out %p ld_out %lld", (const void*)ids, out, (long long)ld_out);
+    if ((uintptr_t)ids & 7) return fail(SQ_EINVAL, "sq_q4_embed: ids must be 8-byte aligned");
+    return launch_q4_embed(q, scale, V, C, ids, n_ids, out, out_dtype, ld_out, (hipStream_t)stream);
 }
 
 }  // extern "C"

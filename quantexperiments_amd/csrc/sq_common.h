@@ -75,6 +75,7 @@ constexpr int SQ_WS_COUNTERS = 1024;
 // error plumbing shared by the launchers (defined in sq_api.hip)
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
+int device_cus();       // compute units of the current device (cached)
 
 // launchers implemented in the kernel translation units
 int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s,
@@ -87,5 +88,16 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
 size_t gemm_workspace(const sq_matrix* mats, int n, int T);
 int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, const void* x, int x_dtype, int64_t ldx,
                       void* y, int y_dtype, int64_t ldy, int T, hipStream_t s);
+
+// the block-32 side formats (8-bit output head, 4-bit embedding)
+int launch_q8_small(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
+                    int y_dtype, int64_t ldy, int B, hipStream_t s);
+size_t q8_workspace(int V, int C, int T);
+int launch_q8_large(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
+                    int y_dtype, int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s);
+int launch_q8_dequant(const int8_t* q, const uint16_t* sc, int C, void* out, int out_dtype, int64_t ld_out, int r0, int r1,
+                      hipStream_t s);
+int launch_q4_embed(const uint8_t* q, const uint16_t* sc, int V, int C, const int64_t* ids, int64_t n_ids, void* out,
+                    int out_dtype, int64_t ld_out, hipStream_t s);
 
 }  // namespace sq

@@ -147,7 +147,6 @@ int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtyp
 
 bool gemm256_ok(int C, int64_t ldx, int64_t ldw, const void* x, const void* w);
 size_t gemm256_part_bytes(int T, int R, int C, int cus);
-int device_cus();
 int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ldw, const uint16_t* row_scale, void* y,
                    int y_dtype, int64_t ldy, int y_off, int T, int R, int C, float* part, int cus, hipStream_t s);
 int launch_bf16_to_f16(const uint16_t* x, int64_t ldx, int T, int C, uint16_t* out, hipStream_t s);
@@ -257,6 +256,72 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
             a.wd = (const uint16_t*)ws; a.ldw = m.C; a.w_dtype = SQ_F16;
             rc = run(a, 8, true, s);
         }
+        if (rc) return rc;
+    }
+    return SQ_OK;
+}
+
+// ---- the 8-bit block-32 head above SQ_SMALL_BMAX activation rows: row chunks decoded to fp16 (scale folded
+// in, one rounding, as the reference's chunked route does: shapequant/vllm_ext/core.py:548-555, 587-591) and
+// multiplied by the dense tile GEMM.  A chunk is as large as Q8_CHUNK_BYTES of fp16 allows so that one GEMM
+// launch has enough tiles for the whole chip.
+constexpr size_t Q8_CHUNK_BYTES = (size_t)256 << 20;
+
+static int q8_chunk_rows(int V, int C) {
+    int64_t rows = (int64_t)(Q8_CHUNK_BYTES / ((size_t)C * 2)) / 256 * 256;
+    if (rows < 256) rows = 256;
+    return rows < V ? (int)rows : V;
+}
+
+static bool q8_big(int T, int C) { return T >= GEMM256_MIN_T && C % 64 == 0; }
+
+size_t q8_workspace(int V, int C, int T) {
+    if (T <= SQ_SMALL_BMAX || V <= 0) return 0;
+    const int chunk = q8_chunk_rows(V, C);
+    size_t need = align256((size_t)chunk * C * 2);
+    if (q8_big(T, C)) {
+        const int last = V % chunk;                             // the split of a launch depends on its tile count
+        const size_t part = std::max(gemm256_part_bytes(T, chunk, C, device_cus()),
+                                     last ? gemm256_part_bytes(T, last, C, device_cus()) : (size_t)0);
+        need += align256((size_t)T * C * 2) + part;
+    }
+    return need;
+}
+
+int launch_q8_large(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
+                    int y_dtype, int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (q8_workspace(V, C, T) > ws_bytes)
+        return fail(SQ_EWORKSPACE, "sq_q8_linear: workspace %zu < %zu", ws_bytes, q8_workspace(V, C, T));
+    if (!x_vec_ok(x, ldx, C))
+        return fail(SQ_EUNSUPPORTED, "sq_q8_linear: more than %d rows need ldx %% 8 == 0 and 16-byte aligned x", SQ_SMALL_BMAX);
+    const int chunk = q8_chunk_rows(V, C);
+    const size_t ys = y_dtype == SQ_F32 ? 4 : 2;
+    char* wd = (char*)ws;
+    const bool big = q8_big(T, C);
+    const uint16_t* xh = (const uint16_t*)x;
+    int64_t ldxh = ldx;
+    float* part = nullptr;
+    const int cus = device_cus();
+    if (big) {
+        if (x_dtype == SQ_BF16) {
+            int rc = launch_bf16_to_f16((const uint16_t*)x, ldx, T, C, (uint16_t*)ws, s);
+            if (rc) return rc;
+            xh = (const uint16_t*)ws;
+            ldxh = C;
+        }
+        wd += align256((size_t)T * C * 2);
+        part = (float*)(wd + align256((size_t)chunk * C * 2));
+    }
+    for (int r0 = 0; r0 < V; r0 += chunk) {
+        const int r1 = r0 + chunk < V ? r0 + chunk : V;
+        int rc = launch_q8_dequant(q, sc, C, wd, SQ_F16, C, r0, r1, s);
+        if (rc) return rc;
+        void* yc = (char*)y + (size_t)r0 * ys;
+        if (big && gemm256_ok(C, ldxh, C, xh, wd))
+            rc = launch_gemm256(xh, ldxh, (const uint16_t*)wd, C, nullptr, yc, y_dtype, ldy, 0, T, r1 - r0, C,
+                                gemm256_part_bytes(T, r1 - r0, C, cus) ? part : nullptr, cus, s);
+        else
+            rc = launch_gemm_dense(wd, SQ_F16, C, r1 - r0, C, x, x_dtype, ldx, yc, y_dtype, ldy, T, s);
         if (rc) return rc;
     }
     return SQ_OK;

@@ -42,7 +42,6 @@ __global__ __launch_bounds__(256) void permute_x_kernel(const uint16_t* __restri
 
 int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y,
                          int y_dtype, int64_t ldy, int B, hipStream_t s);
-int device_cus();
 
 static int unit_dwords(int bits) { return bits == 12 ? 3 : bits == 10 ? 5 : 4; }
 

@@ -243,3 +243,63 @@ def gemm_dense(w: torch.Tensor, x: torch.Tensor, y: torch.Tensor) -> torch.Tenso
                                             _lib.DTYPES[x.dtype], x.stride(0), y.data_ptr(), _lib.DTYPES[y.dtype],
                                             y.stride(0), x.shape[0], _lib.stream_ptr(dev)))
     return y
+
+
+# ------------------------------------------------------------------ block-32 side formats (8-bit head, 4-bit embedding)
+
+def _q_check(q: torch.Tensor, sc: torch.Tensor, per_byte: int, qdtype: torch.dtype, who: str):
+    if q.dim() != 2 or q.dtype != qdtype or not q.is_contiguous() or not sc.is_contiguous():
+        raise ValueError(f"{who}: q must be a contiguous {qdtype} matrix")
+    V, C = q.shape[0], q.shape[1] * per_byte
+    if C % 32 or sc.dtype != torch.float16 or sc.shape != (V, C // 32):
+        raise ValueError(f"{who}: q {tuple(q.shape)}, scale {tuple(sc.shape)} {sc.dtype}")
+    return V, C
+
+
+def q8_linear(q: torch.Tensor, sc: torch.Tensor, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """y[:, :V] = x . w^T for the 8-bit block-32 matrix (q int8 [V, C], sc fp16 [V, C/32]); x [B, C]
+    fp16 / bf16, y [B, >= V] in x's dtype or fp32 (sq_q8_linear)."""
+    V, C = _q_check(q, sc, 1, torch.int8, "q8_linear")
+    if x.dim() != 2 or x.shape[1] != C or x.stride(1) != 1 or y.stride(1) != 1 or y.shape[0] != x.shape[0] or y.shape[1] < V:
+        raise ValueError(f"q8_linear: x {tuple(x.shape)}, y {tuple(y.shape)} for a [{V}, {C}] matrix")
+    dev = q.device
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        need = L.sq_q8_workspace_bytes(V, C, x.shape[0])
+        ws = _Workspace.get(need, dev) if need else None
+        _lib.check(L.sq_q8_linear(q.data_ptr(), sc.data_ptr(), V, C, x.data_ptr(), _lib.DTYPES[x.dtype], x.stride(0),
+                                  y.data_ptr(), _lib.DTYPES[y.dtype], y.stride(0), x.shape[0],
+                                  None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(),
+                                  _lib.stream_ptr(dev)))
+    return y
+
+
+def q8_dense(q: torch.Tensor, sc: torch.Tensor, r0: int, r1: int, dtype: torch.dtype = torch.float32,
+             out: torch.Tensor | None = None) -> torch.Tensor:
+    """Rows [r0, r1) of the 8-bit matrix as dense values (sq_q8_dequant); `out`: a flat buffer to decode into."""
+    V, C = _q_check(q, sc, 1, torch.int8, "q8_dense")
+    dev = q.device
+    n = r1 - r0
+    o = torch.empty(n, C, dtype=dtype, device=dev) if out is None else out[:n * C].view(n, C)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().sq_q8_dequant(q.data_ptr(), sc.data_ptr(), V, C, o.data_ptr(), _lib.DTYPES[o.dtype], C, r0, r1,
+                                            _lib.stream_ptr(dev)))
+    return o
+
+
+def q4_rows(q: torch.Tensor, sc: torch.Tensor, ids: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Rows `ids` (1-D, on the GPU) of the 4-bit block-32 embedding (q uint8 [V, C/2], sc fp16 [V, C/32]) as
+    [len(ids), C] in dtype (sq_q4_embed).  q / sc may be pinned host tensors; the output lives where ids do."""
+    V, C = _q_check(q, sc, 2, torch.uint8, "q4_rows")
+    dev = ids.device
+    if dev.type != "cuda":
+        raise ValueError("q4_rows: ids must be on the GPU")
+    for t in (q, sc):
+        if t.device != dev and not (t.device.type == "cpu" and t.is_pinned()):
+            raise ValueError("q4_rows: q / scale must be on the ids' device or in pinned host memory")
+    ids = ids.to(torch.int64).contiguous()
+    out = torch.empty(ids.shape[0], C, dtype=dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().sq_q4_embed(q.data_ptr(), sc.data_ptr(), V, C, ids.data_ptr(), ids.shape[0], out.data_ptr(),
+                                          _lib.DTYPES[dtype], C, _lib.stream_ptr(dev)))
+    return out

@@ -10,8 +10,18 @@ Per matrix `name` ([R, C] weight, d-wide chunks, G codebooks of K entries, M col
   {name}.row_book   uint8 [R]       only if G > 1
   {name}.row_mask   uint8 [R]       only if M > 1
 
-File metadata: "summary" and "matrices" (JSON strings; "aux" is passed through untouched).
+File metadata: "summary" and "matrices" (JSON strings).
 Column orders are regenerated from each matrix's seed and checked against its CRC.
+
+Optional aux section (metadata key "aux"; reference shapequant/packed.py:30-40), which makes a
+file self-contained:
+
+  aux.embed.q        uint8 [V, C/2]   4-bit embedding, blocks of 32 columns: n = clamp(round(w/s), -8, 7),
+                                      byte k = (n[2k] + 8) | (n[2k+1] + 8) << 4
+  aux.embed.scale    fp16  [V, C/32]  s = fp16(amax / 7); an all-zero block stores s = 1
+  aux.lm_head.q      int8  [V, C]     8-bit head: n = clamp(round(w/s), -127, 127)
+  aux.lm_head.scale  fp16  [V, C/32]  s = fp16(amax / 127)
+  aux.dense.<name>   every other parameter under its HF name, as stored
 
 This module is host logic (bit packing, file I/O, validation).  Decoding a matrix to a dense
 weight runs on the GPU through libsqhip.so; there is no CPU decode here.
@@ -143,9 +153,86 @@ def pack_matrix(fit, *, d: int, K: int, G: int, M: int, seed: int) -> tuple[dict
     return t, meta
 
 
+def _block_quant(w: torch.Tensor, top: int, lo: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Blocks of 32 columns of w [V, C] -> (integers in [lo, top] as float [V, C/32, 32], fp16 scale
+    [V, C/32]): scale = fp16(max|w| / top) per block, an underflowed scale replaced by 1."""
+    V, C = w.shape
+    if C % 32:
+        raise ValueError(f"C={C} is not a multiple of 32")
+    blocks = w.float().reshape(V, C // 32, 32)
+    s = (blocks.abs().amax(-1).clamp_min(1e-8) / float(top)).to(torch.float16)
+    s = torch.where(s == 0, torch.ones_like(s), s)
+    n = torch.round(blocks / s.float()[..., None]).clamp_(lo, top)
+    return n, s
+
+
+def q4_embed_pack(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """w [V, C] -> (q uint8 [V, C/2], scale fp16 [V, C/32]), the aux.embed tensors
+    (reference shapequant/packed.py:134-146)."""
+    V, C = w.shape
+    q = torch.empty(V, C // 2, dtype=torch.uint8, device=w.device)
+    sc = torch.empty(V, C // 32, dtype=torch.float16, device=w.device)
+    for r0 in range(0, V, 8192):                      # row slabs bound the float temporaries
+        n, s = _block_quant(w[r0:r0 + 8192], 7, -8)
+        u = (n + 8).to(torch.uint8).reshape(n.shape[0], C // 2, 2)
+        q[r0:r0 + 8192] = u[..., 0] | (u[..., 1] << 4)
+        sc[r0:r0 + 8192] = s
+    return q, sc
+
+
+def q8_pack(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """w [V, C] -> (q int8 [V, C], scale fp16 [V, C/32], the dequantized fp32 matrix), the
+    aux.lm_head tensors (reference shapequant/kernels/proto_formats.py:464-471)."""
+    n, s = _block_quant(w, 127, -127)
+    return n.reshape(w.shape).to(torch.int8), s, (n * s.float()[..., None]).reshape(w.shape)
+
+
+def q4_embed_rows(q: torch.Tensor, sc: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """fp32 [len(ids), C] rows of the 4-bit embedding, decoded on the GPU that holds q
+    (reference shapequant/packed.py:148-152)."""
+    from .kernels import q4_rows
+    return q4_rows(q, sc, ids.reshape(-1), torch.float32)
+
+
+def q8_rows(q: torch.Tensor, sc: torch.Tensor, s: int = 0, e: int | None = None) -> torch.Tensor:
+    """fp32 rows s:e of the 8-bit matrix, decoded on the GPU that holds q
+    (reference shapequant/packed.py:155-158)."""
+    from .kernels import q8_dense
+    s, e, _ = slice(s, e).indices(q.shape[0])
+    return q8_dense(q, sc, s, max(s, e), torch.float32)
+
+
+def aux_from_model(model, block_names) -> tuple[dict, dict]:
+    """The aux section of an HF causal LM: 4-bit embedding, 8-bit head and every parameter that is
+    neither of those nor one of the packed block linears `block_names`
+    (reference shapequant/packed.py:162-177)."""
+    E = model.model.embed_tokens.weight.detach()
+    H = model.lm_head.weight.detach()
+    eq, es = q4_embed_pack(E)
+    hq, hs, _ = q8_pack(H.float().cpu())
+    left_out = {f"{n}.weight" for n in block_names} | {"lm_head.weight", "model.embed_tokens.weight"}
+    t = {"aux.embed.q": eq.cpu(), "aux.embed.scale": es.cpu(), "aux.lm_head.q": hq, "aux.lm_head.scale": hs}
+    dense = []
+    for n, p in model.named_parameters():
+        if n not in left_out:
+            t[f"aux.dense.{n}"] = p.detach().cpu().contiguous()
+            dense.append(n)
+    meta = {"embed": "q4_b32", "lm_head": "q8_b32", "dense": sorted(dense), "config": model.config.to_dict(),
+            "vocab": E.shape[0], "hidden": E.shape[1],
+            "tied": bool(getattr(model.config, "tie_word_embeddings", False))}
+    return t, meta
+
+
+def aux_bits(meta: dict) -> dict:
+    """Storage bits of the aux embedding (4 + 16/32 per weight) and head (8 + 16/32)
+    (reference shapequant/packed.py:180-183)."""
+    n = meta["vocab"] * meta["hidden"]
+    return {"embed": n * 4.5, "lm_head": n * 8.5}
+
+
 def save(path, packed: dict, *, base_model: str, extra: dict | None = None, aux: tuple | None = None) -> dict:
     """Write {name: (tensors, meta)} to one safetensors file; returns the summary
-    (reference shapequant/packed.py:186-214).  `aux` = (tensors, meta) is stored as given."""
+    (reference shapequant/packed.py:186-214).  `aux` = (tensors, meta) from aux_from_model."""
     from safetensors.torch import save_file
     tensors, metas = {}, {}
     for name, (t, m) in packed.items():
@@ -161,6 +248,10 @@ def save(path, packed: dict, *, base_model: str, extra: dict | None = None, aux:
         at, am = aux
         tensors.update(at)
         md["aux"] = json.dumps(am, default=str)
+        dense = [v for k, v in at.items() if k.startswith("aux.dense.")]
+        ab = aux_bits(am)
+        all_bits = bits + ab["embed"] + ab["lm_head"] + sum(v.numel() * v.element_size() * 8 for v in dense)
+        summary["bpw_all"] = all_bits / (numel + 2 * am["vocab"] * am["hidden"] + sum(v.numel() for v in dense))
         summary["aux"] = True
     md["summary"] = json.dumps(summary)
     Path(path).parent.mkdir(parents=True, exist_ok=True)

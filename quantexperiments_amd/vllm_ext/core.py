@@ -23,7 +23,8 @@ import re
 import torch
 
 from .. import _lib
-from ..kernels import PackedLinear, _Workspace, gemm_dense, linear_gemm, linear_small, prepare_stack
+from ..kernels import (PackedLinear, _Workspace, gemm_dense, linear_gemm, linear_small, prepare_stack, q4_rows, q8_dense,
+                       q8_linear)
 
 BMAX = _lib.SMALL_BMAX
 
@@ -223,9 +224,110 @@ class PackedShards:
         return y
 
 
+class Q8Head:
+    """The packed file's 8-bit block-32 lm_head (aux.lm_head: q int8 [V, C], scale fp16 [V, C/32]) as
+    Y [M, R] = X [M, C] . W^T with R >= V: vLLM pads the vocabulary and the padded logits are 0
+    (reference shapequant/vllm_ext/core.py:489-591, same constructor, attributes and forward / R interface
+    as PackedShards, so it runs through the shapequant::linear op).
+
+      M <= small_max: sq_q8_linear streams the int8 rows once per four activation rows, straight into y;
+      M >  small_max: row chunks decoded to fp16 and multiplied by the tile GEMM (sq_q8_linear's second route).
+
+    The kernels read the file's natural layout at full cache-line width, so no tile-major copy is made:
+    `tiled` and `chunk_rows` are accepted for the reference's callers and change nothing but `dense()`'s slabs.
+
+    keep (int64 [V], ascending): the rows q / sc hold are these token ids of an R-row head (a pruned head);
+    forward scatters them into [M, R] and every other id gets -inf."""
+
+    def __init__(self, q: torch.Tensor, sc: torch.Tensor, R: int | None = None, small_max: int = 32,
+                 chunk_rows: int = 8192, tiled: bool | None = None, keep: torch.Tensor | None = None):
+        self.V, self.C = q.shape
+        self.keep = None
+        if keep is not None:
+            if keep.shape != (self.V,) or R is None or int(keep.max()) >= R:
+                raise ValueError(f"q8 head: keep {tuple(keep.shape)} for {self.V} rows, R {R}")
+            self.keep = keep.to(device=q.device, dtype=torch.int64).contiguous()
+        if self.C % 32 or sc.shape != (self.V, self.C // 32):
+            raise ValueError(f"q8 head: q {tuple(q.shape)}, scale {tuple(sc.shape)}")
+        if q.device.type != "cuda":
+            raise ValueError("Q8Head holds device tensors: pass cuda tensors")
+        self.R = self.V if R is None else R
+        if self.R < self.V:
+            raise ValueError(f"q8 head has {self.V} rows, layer wants {self.R}")
+        self.small_max = min(small_max, BMAX)
+        self.tiled = False
+        self.chunk_rows = chunk_rows
+        self.q, self.sc = q.contiguous(), sc.contiguous()
+
+    def nbytes(self) -> int:
+        return self.q.numel() + self.sc.numel() * 2
+
+    def _rows(self, s: int, e: int, out: torch.Tensor | None = None) -> torch.Tensor:
+        """fp16 rows s:e (block scale folded in, one rounding)."""
+        return q8_dense(self.q, self.sc, s, e, torch.float16, out=out)
+
+    def dense(self) -> torch.Tensor:
+        """fp16 [V, C] (testing)."""
+        return torch.cat([self._rows(s, min(self.V, s + self.chunk_rows))
+                          for s in range(0, self.V, self.chunk_rows)])
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        shp = x.shape
+        if shp[-1] != self.C:
+            raise ValueError(f"input size {shp[-1]} != {self.C}")
+        x2 = x.reshape(-1, self.C)
+        xin = x2 if x2.dtype in (torch.float16, torch.bfloat16) else x2.to(torch.float16)
+        if xin.stride(1) != 1 or xin.stride(0) % 8 or xin.data_ptr() % 16:
+            xin = xin.contiguous()
+        M = xin.shape[0]
+        if self.keep is not None:
+            yk = self._logits(xin, torch.empty(M, self.V, dtype=xin.dtype, device=xin.device), M)
+            y = torch.full((M, self.R), float("-inf"), dtype=x.dtype, device=xin.device)
+            y.index_copy_(1, self.keep, yk.to(x.dtype))
+            return y.view(*shp[:-1], self.R)
+        y = torch.empty(M, self.R, dtype=xin.dtype, device=xin.device)
+        if self.R > self.V:
+            y[:, self.V:] = 0
+        return self._logits(xin, y, M).to(x.dtype).view(*shp[:-1], self.R)
+
+    def _logits(self, x: torch.Tensor, y: torch.Tensor, M: int) -> torch.Tensor:
+        """Rows 0..V-1 of the head into y[:, :V] (y: [M, >= V] in x's dtype); returns y."""
+        if M == 0:
+            return y
+        if M <= self.small_max or M > BMAX:
+            return q8_linear(self.q, self.sc, x, y)
+        for m0 in range(0, M, self.small_max):          # a caller that lowered small_max below the kernel's limit
+            q8_linear(self.q, self.sc, x[m0:m0 + self.small_max], y[m0:m0 + self.small_max])
+        return y
+
+
+def q4_embed(q: torch.Tensor, sc: torch.Tensor, ids: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Rows `ids` (any shape) of the packed file's 4-bit block-32 embedding (aux.embed), [*ids, C] in dtype:
+    one gather kernel on torch's current stream (sq_q4_embed), HIP-graph capturable
+    (reference shapequant/vllm_ext/core.py:594-602)."""
+    return q4_rows(q, sc, ids.reshape(-1), dtype).view(*ids.shape, q.shape[1] * 2)
+
+
+class Q4Embedding:
+    """The 4-bit embedding behind the shapequant::embed op (an integer handle, like the linears, so that
+    model build / load / torch.compile never see its tensors; reference shapequant/vllm_ext/core.py:605-622).
+
+    host: q / sc are CPU tensors kept in pinned host memory; the gather kernel reads the looked-up rows over
+    the bus, so the table costs no HBM."""
+
+    def __init__(self, q: torch.Tensor, sc: torch.Tensor, dtype: torch.dtype, host: bool = False):
+        self.dtype, self.C, self.host = dtype, q.shape[1] * 2, host
+        if host:
+            q, sc = q.contiguous().pin_memory(), sc.contiguous().pin_memory()
+        self.q, self.sc = q, sc
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        return q4_embed(self.q, self.sc, ids, self.dtype)
+
+
 # ------------------------------------------------------------------ torch custom op
 
-_REGISTRY: list = []
+_REGISTRY: list = []        # PackedShards | Q8Head | Q4Embedding
 
 
 def register(ps) -> int:
@@ -248,3 +350,14 @@ def linear_op(x: torch.Tensor, handle: int) -> torch.Tensor:
 @linear_op.register_fake
 def _(x: torch.Tensor, handle: int) -> torch.Tensor:
     return x.new_empty(*x.shape[:-1], _REGISTRY[handle].R)
+
+
+@torch.library.custom_op("shapequant::embed", mutates_args=())
+def embed_op(ids: torch.Tensor, handle: int) -> torch.Tensor:
+    return _REGISTRY[handle].forward(ids)
+
+
+@embed_op.register_fake
+def _(ids: torch.Tensor, handle: int) -> torch.Tensor:
+    e = _REGISTRY[handle]
+    return torch.empty(*ids.shape, e.C, dtype=e.dtype, device=ids.device)

@@ -15,7 +15,7 @@ ROOT = Path(__file__).resolve().parents[1]
 def _declared():
     text = (ROOT / "include" / "sqhip.h").read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(sq_[a-z_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(sq_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_and_loader_agree():
@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     for name in _declared():
         assert getattr(L, name) is not None, name
-    assert L.sq_version() == 101
+    assert L.sq_version() == 102
 
 
 def test_struct_layout_matches_header():
@@ -75,3 +75,33 @@ def test_workspace_sizes_are_host_arithmetic():
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 4096 + 64 * 512 * 2 + 2048 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == 4096 + 16 * 2 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == 4096 + 64 * 512 * 2
+
+
+def test_block32_entry_points_check_arguments_on_the_host():
+    L = _lib.lib()
+    bf, f32 = _lib.SQ_BF16, _lib.SQ_F32
+    q, sc, x, y = 0x10000, 0x20000, 0x30000, 0x40000
+    assert L.sq_q8_linear(q, sc, 64, 48, x, bf, 48, y, bf, 64, 1, None, 0, None) == _lib.SQ_EINVAL      # C % 32
+    assert b"multiple of 32" in L.sq_last_error()
+    assert L.sq_q8_linear(q + 4, sc, 64, 64, x, bf, 64, y, bf, 64, 1, None, 0, None) == _lib.SQ_EINVAL  # q alignment
+    assert L.sq_q8_linear(None, sc, 64, 64, x, bf, 64, y, bf, 64, 1, None, 0, None) == _lib.SQ_EINVAL
+    assert L.sq_q8_linear(q, sc, 64, 64, x, f32, 64, y, f32, 64, 1, None, 0, None) == _lib.SQ_EINVAL    # x dtype
+    assert L.sq_q8_linear(q, sc, 64, 64, x, bf, 64, y, _lib.SQ_F16, 64, 1, None, 0, None) == _lib.SQ_EINVAL
+    assert L.sq_q8_linear(q, sc, 64, 64, x, bf, 32, y, bf, 64, 2, None, 0, None) == _lib.SQ_EINVAL      # ldx < C
+    assert L.sq_q8_linear(q, sc, 64, 64, x, bf, 64, y, bf, 63, 2, None, 0, None) == _lib.SQ_EINVAL      # ldy < V
+    assert L.sq_q8_linear(q, sc, 64, 64, x, bf, 64, y, bf, 64, 0, None, 0, None) == _lib.SQ_OK          # no rows
+    assert L.sq_q8_linear(q, sc, 0, 64, x, bf, 64, y, bf, 64, 4, None, 0, None) == _lib.SQ_OK           # no weights
+    # more than 32 activation rows need the workspace sq_q8_workspace_bytes names
+    assert L.sq_q8_linear(q, sc, 64, 64, x, bf, 64, y, bf, 64, 40, None, 0, None) == _lib.SQ_EWORKSPACE
+    assert L.sq_q8_workspace_bytes(64, 64, 32) == 0
+    assert L.sq_q8_workspace_bytes(64, 64, 40) == 4096 + 64 * 64 * 2
+    assert L.sq_q8_workspace_bytes(64, 48, 40) == 0
+    assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 64, 3, 65, None) == _lib.SQ_EINVAL                    # rows outside
+    assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 32, 0, 4, None) == _lib.SQ_EINVAL                     # ld_out < C
+    assert L.sq_q8_dequant(q, sc, 64, 64, y, 7, 64, 0, 4, None) == _lib.SQ_EINVAL
+    assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 64, 5, 5, None) == _lib.SQ_OK
+    assert L.sq_q4_embed(q, sc, 64, 64, x, -1, y, bf, 64, None) == _lib.SQ_EINVAL
+    assert L.sq_q4_embed(q, sc, 64, 64, x + 4, 3, y, bf, 64, None) == _lib.SQ_EINVAL                    # ids alignment
+    assert L.sq_q4_embed(q, sc, 64, 64, None, 3, y, bf, 64, None) == _lib.SQ_EINVAL
+    assert L.sq_q4_embed(q, sc, 64, 64, x, 3, y, bf, 48, None) == _lib.SQ_EINVAL                        # ld_out < C
+    assert L.sq_q4_embed(q, sc, 64, 64, x, 0, y, bf, 64, None) == _lib.SQ_OK

@@ -173,3 +173,121 @@ def test_baseline_byte_counts():
     shapes = [(3584, 3584)] * 2 + [(512, 3584)] * 2 + [(18944, 3584)] * 2 + [(3584, 18944)]
     assert sum(R * O.words_per_row(C // 8, 16) * 4 for R, C in shapes) == 58_261_504
     assert sum(R * O.words_per_row(C // 4, 12) * 4 for R, C in shapes) == 87_392_256
+
+
+# ------------------------------------------------------------------ block-32 side formats (4-bit embedding, 8-bit head)
+def _q4_known_block():
+    """32 integer weights whose largest magnitude is 7: the scale is exactly 1 and every weight is its own
+    level.  Columns 0..15 = -7..7 then 0, columns 16..31 the same backwards."""
+    a = list(range(-7, 8)) + [0]
+    return np.array([a + a[::-1]], dtype=np.float32)
+
+
+def test_q4_pack_known_answer_bytes():
+    w = _q4_known_block()
+    q, s = O.q4_embed_pack(w)
+    assert q.dtype == np.uint8 and q.shape == (1, 16) and s.dtype == np.float16 and s.shape == (1, 1)
+    assert float(s[0, 0]) == 1.0
+    # byte k = (w[2k] + 8) | (w[2k+1] + 8) << 4, written out by hand for the first half
+    assert q[0, :8].tolist() == [0x21, 0x43, 0x65, 0x87, 0xA9, 0xCB, 0xED, 0x8F]
+    assert q[0, 8:].tolist() == [0xF8, 0xDE, 0xBC, 0x9A, 0x78, 0x56, 0x34, 0x12]
+    assert np.array_equal(O.q4_embed_rows(q, s, [0]), w)
+
+
+def test_q4_pack_scale_halves_ties_and_clamp():
+    # largest magnitude 3.5 -> scale 0.5 exactly; w / s = 2.5 and 3.5 are ties: to even -> 2 and 4;
+    # -3.5 / 0.5 = -7; a block whose positive peak sets the scale clamps its negative twin side at -8
+    w = np.zeros((2, 32), np.float32)
+    w[0, :4] = [1.25, 1.75, -3.5, 0.25]          # levels 2.5 -> 2, 3.5 -> 4, -7, 0.5 -> 0
+    w[1, :3] = [7.0, -9.0, -7.6]                 # amax 9 -> s = fp16(9/7); -9/s = -7 exactly; see below
+    q, s = O.q4_embed_pack(w)
+    assert float(s[0, 0]) == 0.5
+    assert [(int(q[0, 0]) & 15) - 8, (int(q[0, 0]) >> 4) - 8, (int(q[0, 1]) & 15) - 8, (int(q[0, 1]) >> 4) - 8] == [2, 4, -7, 0]
+    s1 = float(np.float16(np.float32(9.0) / np.float32(7.0)))
+    assert float(s[1, 0]) == s1
+    lv = [round(7.0 / s1), round(-9.0 / s1), round(-7.6 / s1)]
+    assert [(int(q[1, 0]) & 15) - 8, (int(q[1, 0]) >> 4) - 8, (int(q[1, 1]) & 15) - 8] == lv
+    # the level -8 is reachable only through the clamp's lower side: fp16 rounding of the scale can push
+    # |w| / s just past 7.5
+    w2 = np.zeros((1, 32), np.float32)
+    w2[0, 0] = -1.0
+    q2, s2 = O.q4_embed_pack(w2)
+    want = max(-8, min(7, round(-1.0 / float(s2[0, 0]))))
+    assert (int(q2[0, 0]) & 15) - 8 == want and int(q2[0, 0]) >> 4 == 8
+
+
+def test_q4_and_q8_all_zero_block_stores_scale_one():
+    z = np.zeros((1, 64), np.float32)
+    z[0, 40] = 3.0
+    q, s = O.q4_embed_pack(z)
+    assert float(s[0, 0]) == 1.0 and q[0, :16].tolist() == [0x88] * 16
+    q8, s8, deq = O.q8_pack(z)
+    assert float(s8[0, 0]) == 1.0 and not q8[0, :32].any() and float(deq[0, 40]) == pytest.approx(3.0, rel=1e-3)
+
+
+def test_q8_pack_known_answer():
+    w = np.zeros((1, 64), np.float32)
+    w[0, :32] = np.arange(-16, 16) * 8.0          # peak 128 -> not 127: scale = fp16(128/127)
+    w[0, 32:] = np.arange(96, 128)                # peak 127 -> scale exactly 1, levels are the weights
+    q, s, deq = O.q8_pack(w)
+    assert q.dtype == np.int8 and s.dtype == np.float16 and deq.dtype == np.float32
+    assert float(s[0, 1]) == 1.0 and q[0, 32:].tolist() == list(range(96, 128))
+    s0 = float(np.float16(np.float32(128.0) / np.float32(127.0)))
+    assert float(s[0, 0]) == s0
+    assert q[0, :32].tolist() == [max(-127, min(127, round(v / s0))) for v in w[0, :32].tolist()]
+    assert np.array_equal(deq, O.q8_rows(q, s))
+    assert np.array_equal(O.q8_rows(q, s)[0, 32:], w[0, 32:])
+
+
+@pytest.mark.parametrize("which", ["q4", "q8"])
+def test_block_quant_python_walk_and_error_bound(which):
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((6, 96)) * rng.uniform(0.01, 3.0, (6, 1))).astype(np.float32)
+    if which == "q4":
+        q, s = O.q4_embed_pack(w)
+        rows = O.q4_embed_rows(q, s, np.arange(6))
+        level = lambda r, c: ((int(q[r, c // 2]) >> (4 * (c % 2))) & 15) - 8
+    else:
+        q, s, _ = O.q8_pack(w)
+        rows = O.q8_rows(q, s)
+        level = lambda r, c: int(q[r, c])
+    for r in range(6):
+        for c in range(96):
+            sc = float(s[r, c // 32])
+            assert float(rows[r, c]) == level(r, c) * sc                      # exact: small integer times fp16
+            assert abs(float(rows[r, c]) - float(w[r, c])) <= sc * 0.5 * (1 + 1e-3) or which == "q4" and level(r, c) == 7
+    # rows in any order, with repeats
+    if which == "q4":
+        ids = np.array([5, 0, 5, 2])
+        assert np.array_equal(O.q4_embed_rows(q, s, ids), rows[ids])
+    else:
+        assert np.array_equal(O.q8_rows(q, s, 2, 5), rows[2:5])
+
+
+def test_q8_linear_is_the_dense_product():
+    rng = np.random.default_rng(9)
+    w = rng.standard_normal((40, 128)).astype(np.float32)
+    q, s, deq = O.q8_pack(w)
+    x = rng.standard_normal((3, 128)).astype(np.float32)
+    a, b = O.q8_linear(x, q, s), O.linear(x, deq)
+    assert np.allclose(a, b, rtol=1e-12, atol=1e-12)
+    # and stays close to the unquantized product: 8 bits per weight is a ~0.4 % perturbation
+    full = O.linear(x, w)
+    assert np.abs(a - full).max() <= 0.02 * np.abs(full).max()
+
+
+def test_host_packers_agree_with_oracle():
+    # the shipped torch packers (host-side format writers) against the numpy restatement, bit for bit
+    from quantexperiments_amd import packed as P
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn(50, 160, generator=g) * torch.rand(50, 1, generator=g) * 4
+    w[7, 32:64] = 0
+    q, s = P.q4_embed_pack(w)
+    oq, os_ = O.q4_embed_pack(w.numpy())
+    assert np.array_equal(q.numpy(), oq) and np.array_equal(s.numpy(), os_)
+    q, s, deq = P.q8_pack(w)
+    oq, os_, odeq = O.q8_pack(w.numpy())
+    assert np.array_equal(q.numpy(), oq) and np.array_equal(s.numpy(), os_) and np.array_equal(deq.numpy(), odeq)
+    with pytest.raises(ValueError):
+        P.q8_pack(torch.zeros(2, 40))
+    assert P.aux_bits({"vocab": 10, "hidden": 64}) == {"embed": 640 * 4.5, "lm_head": 640 * 8.5}
