@@ -144,7 +144,7 @@ int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, i
 static int check_q8(const char* who, const void* q, const void* scale, int32_t V, int32_t C) {
     if (V < 0 || C <= 0 || C % 32) return fail(SQ_EINVAL, "%s: V %d C %d (C must be a positive multiple of 32)", who, V, C);
     if (V > 0 && (!q || !scale)) return fail(SQ_EINVAL, "%s: null q / scale", who);
-    if (((uintptr_t)q & 15) || ((uintptr_t)scale & 1)) return fail(SQ_EINVAL, "%s: q must be 16-byte aligned, scale 2-byte", who);
+    if (((uintptr_t)q & 15) || ((uintptr_t)scale & 15)) return fail(SQ_EINVAL, "%s: q and scale must be 16-byte aligned", who);
     return SQ_OK;
 }
 
@@ -159,15 +159,18 @@ int sq_q8_linear(const int8_t* q, const uint16_t* scale, int32_t V, int32_t C, c
     if (B == 0 || V == 0) return SQ_OK;
     if (!x || !y) return fail(SQ_EINVAL, "sq_q8_linear: null x / y");
     if (B > 1 && (ldx < C || ldy < V)) return fail(SQ_EINVAL, "sq_q8_linear: ldx %lld / ldy %lld too small", (long long)ldx, (long long)ldy);
-    if (B <= SQ_SMALL_BMAX) return launch_q8_small(q, scale, V, C, x, x_dtype, ldx, y, y_dtype, ldy, B, (hipStream_t)stream);
     const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
+    if (q8_mid(C, B))
+        return launch_q8_mid(q, scale, V, C, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
+                             has_ws ? ws_bytes - SQ_WS_HEADER : 0, (hipStream_t)stream);
+    if (B <= SQ_SMALL_BMAX) return launch_q8_small(q, scale, V, C, x, x_dtype, ldx, y, y_dtype, ldy, B, (hipStream_t)stream);
     return launch_q8_large(q, scale, V, C, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
                            has_ws ? ws_bytes - SQ_WS_HEADER : 0, (hipStream_t)stream);
 }
 
 size_t sq_q8_workspace_bytes(int32_t V, int32_t C, int32_t B) {
     if (C <= 0 || C % 32) return 0;
-    const size_t inner = q8_workspace(V, C, B);
+    const size_t inner = q8_mid(C, B) ? q8_mid_workspace(C, B) : q8_workspace(V, C, B);
     return inner ? inner + SQ_WS_HEADER : 0;
 }
 

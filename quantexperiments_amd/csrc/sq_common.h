@@ -92,6 +92,10 @@ int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, con
 // the block-32 side formats (8-bit output head, 4-bit embedding)
 int launch_q8_small(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
                     int y_dtype, int64_t ldy, int B, hipStream_t s);
+bool q8_mid(int C, int B);                  // 5 .. 128 activation rows on MFMA passes of 32
+size_t q8_mid_workspace(int C, int B);
+int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
+                  int y_dtype, int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s);
 size_t q8_workspace(int V, int C, int T);
 int launch_q8_large(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
                     int y_dtype, int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s);

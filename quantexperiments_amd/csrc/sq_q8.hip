@@ -181,6 +181,157 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_kernel(Q8Args a) {
     }
 }
 
+// ---- 5 .. Q8_MFMA_MAX_ROWS activation rows: fp16 MFMA, 32 activation rows per pass.
+// v_mfma_f32_32x32x16_f16 operand layout, lane l: A row / B column l % 32, k = 8 * (l / 32) .. + 7; result register
+// jj of lane l is D[(jj / 4) * 8 + (l / 32) * 4 + jj % 4][l % 32].  Weights are the A operand, loaded straight into
+// registers: a wave owns 32 rows, and per step of 128 columns lane (r, h) takes 16 bytes of row r at column
+// 128 s + 32 j + 16 h for j = 0..3, issued back to back, so the two lanes of a row consume a whole 128-byte line
+// while it is in flight.  Each 16-byte piece feeds two MFMAs; the k index of MFMA m of piece j is column
+// 128 s + 32 j + 16 h + 8 m + e, and the activations (B operand) are read with the same mapping from LDS, where
+// the workgroup keeps the current 256-column chunk of the fp16 activations (global_load_lds, double buffered).
+// What bounds this kernel is latency, not arithmetic: one wave alone moves 5 GB/s, so the design is many small
+// waves (one 32-row block each, <= 128 registers: 16 waves per CU) with four steps of loads in flight each.
+// The block scale is folded into the fp16 weight (one rounding, as the reference's tile kernel does,
+// shapequant/kernels/batched_runs.py:442-447): all 8 weights a lane feeds to one MFMA sit in one block.
+constexpr int Q8_MFMA_MAX_ROWS = 128;           // up to here passes of 32 beat decode + tile GEMM
+constexpr int Q8_XC = 256;                      // columns of x per LDS chunk (2 steps)
+constexpr int Q8_RING = 4;                      // steps of weight loads in flight per wave
+
+// x [B, C] (fp16 or bf16, any stride) -> fp16 [B, C] contiguous.
+__global__ __launch_bounds__(256) void q8_x_kernel(const uint16_t* __restrict__ x, int64_t ldx, int B, int C, int x_dtype,
+                                                   uint16_t* __restrict__ out) {
+    const int64_t n = (int64_t)B * C;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int b = (int)(i / C), c = (int)(i - (int64_t)b * C);
+        const uint16_t v = x[b * ldx + c];
+        out[i] = x_dtype == SQ_BF16 ? __builtin_bit_cast(uint16_t, bf2h(v)) : v;
+    }
+}
+
+struct Q8MfmaArgs {
+    const int8_t* q;
+    const uint16_t* sc;
+    const uint16_t* xh;     // fp16 [B, C], 16-byte aligned
+    void* y;
+    int64_t ldy;
+    int V, C, B, y_dtype, tasks;
+};
+
+constexpr int q8_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }   // wait on vmcnt only
+
+__global__ __launch_bounds__(256, 3) void q8_mfma_kernel(Q8MfmaArgs a) {
+    // x chunk in LDS: [32 activation rows][32 pieces of 16 bytes], piece p of row n stored in slot p ^ (n & 15),
+    // so the 16 lanes of a ds_read_b128 (16 different rows, same piece) hit 16 different bank groups
+    __shared__ __attribute__((aligned(16))) unsigned char xs[2][32 * Q8_XC * 2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int task_raw = blockIdx.x * 4 + wave;
+    const bool active = task_raw < a.tasks;                 // idle waves still copy x and meet the barriers
+    const int task = active ? task_raw : a.tasks - 1;
+    const int r = lane & 31, h = lane >> 5;
+    const int C = a.C, nblk = C >> 5, nsteps = C >> 7;      // C % 256 == 0: an even number of 128-column steps
+    const int nchunks = nsteps >> 1;
+    const int row = min(task * 32 + r, a.V - 1);
+    const int8_t* wp = a.q + (int64_t)row * C + h * 16;
+    const char* sp = (const char*)(a.sc + (int64_t)row * nblk);
+
+    // x copies: one instruction moves 1 KB = two activation rows of the chunk; wave w brings rows 8 w .. 8 w + 7.
+    // The lane that lands in slot (lane & 31) of its row fetches the piece the swizzle puts there.
+    typedef const __attribute__((address_space(1))) void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    uint32_t xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int rowx = wave * 8 + 2 * i + h;
+        const int piece = (lane & 31) ^ (rowx & 15);
+        xsrc[i] = (uint32_t)(min(rowx, a.B - 1) * C + piece * 8);         // halves
+    }
+    auto copy_x = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(a.xh + c * Q8_XC + xsrc[i]),
+                                             (lptr_t)(&xs[c & 1][(wave * 8 + 2 * i) * (Q8_XC * 2)]), 16, 0, 0);
+    };
+    const uint32_t xrow = (uint32_t)r * (Q8_XC * 2), xsw = (uint32_t)(r & 15);
+
+    float16v acc;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) acc[k] = 0.f;
+
+    u32x4 wr[Q8_RING][4];
+    u32x2 sr[Q8_RING];
+    copy_x(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int p = 0; p < Q8_RING; ++p) {
+        const int sp_ = p < nsteps ? p : nsteps - 1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wr[p][j] = *reinterpret_cast<const u32x4*>(wp + sp_ * 128 + j * 32);
+        sr[p] = *reinterpret_cast<const u32x2*>(sp + sp_ * 8);
+    }
+    for (int c0 = 0; c0 < nchunks; c0 += 2) {
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const int c = c0 + cc;
+            if (c < nchunks) {
+                // chunk c was requested one chunk ago, before the 10 loads of that chunk's two refills; the
+                // first chunk (prologue) and the last one (no refills left) wait for everything
+                if (c == 0 || c == nchunks - 1) __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
+                else __builtin_amdgcn_s_waitcnt(q8_vmcnt(10));
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                if (c + 1 < nchunks) copy_x(c + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                const unsigned char* xc = &xs[cc][0] + xrow;
+#pragma unroll
+                for (int sl = 0; sl < 2; ++sl) {
+                    const int slot = cc * 2 + sl;
+                    const int s = c * 2 + sl;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t spair = sr[slot][j >> 1];
+                        const uint16_t sbits = (j & 1) ? (uint16_t)(spair >> 16) : (uint16_t)(spair & 0xFFFFu);
+                        const half_t sh = __builtin_bit_cast(half_t, sbits);
+                        const half2v s2 = {sh, sh};
+                        half2v p[8];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const uint32_t wk = wr[slot][j][k];
+                            i8x4_to_h2(wk, p[2 * k], p[2 * k + 1]);
+                        }
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) p[k] = p[k] * s2;
+                        half8v a0, a1;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            a0[2 * k] = p[k][0]; a0[2 * k + 1] = p[k][1];
+                            a1[2 * k] = p[4 + k][0]; a1[2 * k + 1] = p[4 + k][1];
+                        }
+                        // pieces sl * 16 + j * 4 + h * 2 + m of this lane's activation row
+                        const uint32_t p0 = (uint32_t)(sl * 16 + j * 4 + h * 2);
+                        const half8v x0 = *reinterpret_cast<const half8v*>(xc + ((p0 ^ xsw) << 4));
+                        const half8v x1 = *reinterpret_cast<const half8v*>(xc + (((p0 + 1) ^ xsw) << 4));
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, x0, acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, x1, acc, 0, 0, 0);
+                    }
+                    // the slot is free: refill it Q8_RING steps ahead
+                    if (s + Q8_RING < nsteps) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            wr[slot][j] = *reinterpret_cast<const u32x4*>(wp + (s + Q8_RING) * 128 + j * 32);
+                        sr[slot] = *reinterpret_cast<const u32x2*>(sp + (s + Q8_RING) * 8);
+                    }
+                }
+            }
+        }
+    }
+    if (!active || r >= a.B) return;
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj) {
+        const int orow = task * 32 + (jj >> 2) * 8 + h * 4 + (jj & 3);
+        if (orow < a.V) store_y(a.y, a.y_dtype, (int64_t)r * a.ldy + orow, acc[jj]);
+    }
+}
+
 // Rows [r0, r1) as dense values, one 16-byte load (16 weights, half a block) per thread.
 template <int DT>
 __global__ __launch_bounds__(256) void q8_dequant_kernel(const int8_t* __restrict__ q, const uint16_t* __restrict__ sc,
@@ -240,6 +391,40 @@ static int q8_pass_rows(int B, int C) {
     int nb = B > 2 ? 4 : B > 1 ? 2 : 1;
     while (nb > 1 && nb * C > Q8_LDS_HALVES) nb >>= 1;
     return nb;
+}
+
+// The MFMA passes need C % 256 == 0 (whole 256-column chunks of x) and 32 activation rows of C halves within
+// 32-bit offsets.
+static bool q8_mfma_ok(int C) { return C % 256 == 0 && (int64_t)C * 32 < ((int64_t)1 << 31); }
+
+int q8_mid_rows() { return Q8_MFMA_MAX_ROWS; }
+
+bool q8_mid(int C, int B) { return B > 4 && B <= Q8_MFMA_MAX_ROWS && q8_mfma_ok(C); }
+
+size_t q8_mid_workspace(int C, int B) { return q8_mid(C, B) ? (((size_t)B * C * 2) + 255) & ~(size_t)255 : 0; }
+
+int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
+                  int y_dtype, int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (ws_bytes < q8_mid_workspace(C, B)) return fail(SQ_EWORKSPACE, "sq_q8_linear: workspace %zu < %zu", ws_bytes, q8_mid_workspace(C, B));
+    const size_t ys = y_dtype == SQ_F32 ? 4 : 2;
+    const int64_t n = (int64_t)B * C;
+    const int64_t want = (n + 255) / 256;
+    hipLaunchKernelGGL(q8_x_kernel, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, s, (const uint16_t*)x, ldx, B, C,
+                       x_dtype, (uint16_t*)ws);
+    int rc = check_launch("q8_x_kernel");
+    if (rc) return rc;
+    const int tasks = (V + 31) / 32;
+    for (int b0 = 0; b0 < B; b0 += 32) {
+        Q8MfmaArgs a{};
+        a.q = q; a.sc = sc;
+        a.xh = (const uint16_t*)ws + (int64_t)b0 * C;
+        a.y = (char*)y + (size_t)b0 * ldy * ys;
+        a.ldy = ldy; a.V = V; a.C = C; a.B = B - b0 < 32 ? B - b0 : 32; a.y_dtype = y_dtype; a.tasks = tasks;
+        hipLaunchKernelGGL(q8_mfma_kernel, dim3((unsigned)((tasks + 3) / 4)), dim3(256), 0, s, a);
+        rc = check_launch("q8_mfma_kernel");
+        if (rc) return rc;
+    }
+    return SQ_OK;
 }
 
 int launch_q8_small(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,

@@ -96,6 +96,12 @@ def test_block32_entry_points_check_arguments_on_the_host():
     assert L.sq_q8_workspace_bytes(64, 64, 32) == 0
     assert L.sq_q8_workspace_bytes(64, 64, 40) == 4096 + 64 * 64 * 2
     assert L.sq_q8_workspace_bytes(64, 48, 40) == 0
+    # 5 .. 128 rows with C % 256 == 0: an fp16 copy of the activations
+    assert L.sq_q8_workspace_bytes(64, 256, 4) == 0
+    assert L.sq_q8_workspace_bytes(64, 256, 8) == 4096 + 8 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 128) == 4096 + 128 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 129) == 4096 + 64 * 256 * 2
+    assert L.sq_q8_linear(q, sc, 64, 256, x, bf, 256, y, bf, 64, 8, None, 0, None) == _lib.SQ_EWORKSPACE
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 64, 3, 65, None) == _lib.SQ_EINVAL                    # rows outside
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 32, 0, 4, None) == _lib.SQ_EINVAL                     # ld_out < C
     assert L.sq_q8_dequant(q, sc, 64, 64, y, 7, 64, 0, 4, None) == _lib.SQ_EINVAL
