@@ -14,8 +14,9 @@ the packed file's bytes, which is what the metric is quoted on.
 
 value = packed (algorithmic) bytes of a layer / time per layer, in GB/s.  The same JSON line
 carries us_per_layer, the roofline of the dominant kernel (gate|up launch, HIP events around graph
-replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s, and the CPU baseline (the
-reference's CPU route, oracle port, on the host cores).
+replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s, the 8-bit block-32 output head
+(152,064 x 3,584) at a few decode batch sizes, and the CPU baseline (the reference's CPU route, oracle
+port, on the host cores).
 """
 
 from __future__ import annotations
@@ -127,6 +128,28 @@ def prefill(torch, dev, layer, steps=3):
     return res
 
 
+def lm_head(torch, dev, rows=(1, 4, 8, 32), reps=3):
+    """The 7B model's 8-bit block-32 output head (152,064 x 3,584 int8 + fp16 block scales = 579 MB, more than
+    twice the last-level cache): microseconds and weight bytes per second for a few decode batch sizes."""
+    from quantexperiments_amd.kernels import q8_linear
+    V, C = 152064, 3584
+    g = torch.Generator(device=dev).manual_seed(1)
+    q = torch.randint(-127, 128, (V, C), dtype=torch.int8, device=dev, generator=g)
+    sc = (torch.rand(V, C // 32, device=dev, generator=g) * 0.002 + 0.0005).to(torch.float16)
+    nbytes = q.numel() + sc.numel() * 2
+    res = {"shape": [V, C], "bytes": nbytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    for B in rows:
+        x = torch.randn(B, C, device=dev, generator=g).to(torch.bfloat16)
+        y = torch.empty(B, V, device=dev, dtype=torch.bfloat16)
+        q8_linear(q, sc, x, y)                   # grows the workspace outside capture
+        ms, gr = timed_graph(torch, lambda: [q8_linear(q, sc, x, y) for _ in range(5)], reps=reps)
+        del gr
+        ms /= 5
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        res[f"B{B}"] = {"us": ms * 1e3, "achieved": gbs, "frac": gbs / HBM_PEAK_GBS}
+    return res
+
+
 def copy_probe(torch, dev):
     """Three 256 MiB device-to-device copies: a kernel of known HBM traffic to scale profiler counters by."""
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -148,6 +171,10 @@ def main():
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant launch (gate|up) and print only its roofline object: the command "
                          "the rocprofv3 summaries under profiles/ are made with")
+    ap.add_argument("--no-head", action="store_true", help="skip the 8-bit lm_head GEMV")
+    ap.add_argument("--head-only", action="store_true",
+                    help="run only the 8-bit lm_head GEMV and print only its object (the command its rocprofv3 "
+                         "summary under profiles/ is made with)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic to scale rocprofv3 counters by)")
     args = ap.parse_args()
@@ -160,6 +187,9 @@ def main():
         sys.exit("bench.py needs an MI355X (no CPU fallback)")
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.head_only:
+        print(json.dumps({"lm_head": lm_head(torch, dev)}))
+        return
     gen = torch.Generator(device=dev).manual_seed(0)
     layers = [make_layer(torch, dev, gen) for _ in range(args.layers)]
     x = {C: torch.randn(1, C, device=dev, generator=gen).to(torch.bfloat16) for C in (3584, 18944)}
@@ -249,6 +279,9 @@ def main():
         out["prefill"] = {"M": 2048, "gate_18944x3584": pf["gate"], "down_3584x18944": pf["down"],
                           "peak_tflops": MFMA_PEAK_TFLOPS,
                           "frac_of_peak": min(pf["gate"]["tflops"], pf["down"]["tflops"]) / MFMA_PEAK_TFLOPS}
+    if not args.no_head:
+        del layers[1:]                           # the head needs 0.6 GB; the rotated layers are no longer used
+        out["lm_head_q8"] = lm_head(torch, dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, layers[0], x)
     print(json.dumps(out))

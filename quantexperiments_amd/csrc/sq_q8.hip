@@ -189,13 +189,15 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_kernel(Q8Args a) {
 // while it is in flight.  Each 16-byte piece feeds two MFMAs; the k index of MFMA m of piece j is column
 // 128 s + 32 j + 16 h + 8 m + e, and the activations (B operand) are read with the same mapping from LDS, where
 // the workgroup keeps the current 256-column chunk of the fp16 activations (global_load_lds, double buffered).
-// What bounds this kernel is latency, not arithmetic: one wave alone moves 5 GB/s, so the design is many small
-// waves (one 32-row block each, <= 128 registers: 16 waves per CU) with four steps of loads in flight each.
+// One wave alone moves only 5 GB/s (latency), so the design is many small waves: one 32-row block each, <= 128
+// registers, 16 waves per CU, two steps of loads in flight each.  What is left between this kernel (4 TB/s) and
+// the 4-row kernel (5.7 TB/s) is the address pattern the MFMA operand layout forces on direct loads: the 16
+// lanes of a quarter wave always belong to 16 different weight rows, i.e. 16 cache lines per quarter wave.
 // The block scale is folded into the fp16 weight (one rounding, as the reference's tile kernel does,
 // shapequant/kernels/batched_runs.py:442-447): all 8 weights a lane feeds to one MFMA sit in one block.
 constexpr int Q8_MFMA_MAX_ROWS = 128;           // up to here passes of 32 beat decode + tile GEMM
 constexpr int Q8_XC = 256;                      // columns of x per LDS chunk (2 steps)
-constexpr int Q8_RING = 4;                      // steps of weight loads in flight per wave
+constexpr int Q8_RING = 2;                      // steps of weight loads in flight per wave (2 or 4; measured equal)
 
 // x [B, C] (fp16 or bf16, any stride) -> fp16 [B, C] contiguous.
 __global__ __launch_bounds__(256) void q8_x_kernel(const uint16_t* __restrict__ x, int64_t ldx, int B, int C, int x_dtype,
@@ -211,15 +213,17 @@ __global__ __launch_bounds__(256) void q8_x_kernel(const uint16_t* __restrict__ 
 struct Q8MfmaArgs {
     const int8_t* q;
     const uint16_t* sc;
-    const uint16_t* xh;     // fp16 [B, C], 16-byte aligned
+    const uint16_t* xh;     // fp16 [B, ldxh], rows 16-byte aligned
     void* y;
     int64_t ldy;
+    int ldxh;
     int V, C, B, y_dtype, tasks;
 };
 
 constexpr int q8_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }   // wait on vmcnt only
 
-__global__ __launch_bounds__(256, 3) void q8_mfma_kernel(Q8MfmaArgs a) {
+template <int RING>
+__global__ __launch_bounds__(256, RING == 2 ? 4 : 3) void q8_mfma_kernel(Q8MfmaArgs a) {
     // x chunk in LDS: [32 activation rows][32 pieces of 16 bytes], piece p of row n stored in slot p ^ (n & 15),
     // so the 16 lanes of a ds_read_b128 (16 different rows, same piece) hit 16 different bank groups
     __shared__ __attribute__((aligned(16))) unsigned char xs[2][32 * Q8_XC * 2];
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(256, 3) void q8_mfma_kernel(Q8MfmaArgs a) {
     for (int i = 0; i < 4; ++i) {
         const int rowx = wave * 8 + 2 * i + h;
         const int piece = (lane & 31) ^ (rowx & 15);
-        xsrc[i] = (uint32_t)(min(rowx, a.B - 1) * C + piece * 8);         // halves
+        xsrc[i] = (uint32_t)(min(rowx, a.B - 1) * a.ldxh + piece * 8);    // halves
     }
     auto copy_x = [&](int c) {
 #pragma unroll
@@ -257,12 +261,12 @@ __global__ __launch_bounds__(256, 3) void q8_mfma_kernel(Q8MfmaArgs a) {
 #pragma unroll
     for (int k = 0; k < 16; ++k) acc[k] = 0.f;
 
-    u32x4 wr[Q8_RING][4];
-    u32x2 sr[Q8_RING];
+    u32x4 wr[RING][4];
+    u32x2 sr[RING];
     copy_x(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int p = 0; p < Q8_RING; ++p) {
+    for (int p = 0; p < RING; ++p) {
         const int sp_ = p < nsteps ? p : nsteps - 1;
 #pragma unroll
         for (int j = 0; j < 4; ++j) wr[p][j] = *reinterpret_cast<const u32x4*>(wp + sp_ * 128 + j * 32);
@@ -284,7 +288,7 @@ __global__ __launch_bounds__(256, 3) void q8_mfma_kernel(Q8MfmaArgs a) {
                 const unsigned char* xc = &xs[cc][0] + xrow;
 #pragma unroll
                 for (int sl = 0; sl < 2; ++sl) {
-                    const int slot = cc * 2 + sl;
+                    const int slot = (cc * 2 + sl) % RING;
                     const int s = c * 2 + sl;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
@@ -313,12 +317,12 @@ __global__ __launch_bounds__(256, 3) void q8_mfma_kernel(Q8MfmaArgs a) {
                         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, x0, acc, 0, 0, 0);
                         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, x1, acc, 0, 0, 0);
                     }
-                    // the slot is free: refill it Q8_RING steps ahead
-                    if (s + Q8_RING < nsteps) {
+                    // the slot is free: refill it RING steps ahead
+                    if (s + RING < nsteps) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
-                            wr[slot][j] = *reinterpret_cast<const u32x4*>(wp + (s + Q8_RING) * 128 + j * 32);
-                        sr[slot] = *reinterpret_cast<const u32x2*>(sp + (s + Q8_RING) * 8);
+                            wr[slot][j] = *reinterpret_cast<const u32x4*>(wp + (s + RING) * 128 + j * 32);
+                        sr[slot] = *reinterpret_cast<const u32x2*>(sp + (s + RING) * 8);
                     }
                 }
             }
@@ -407,20 +411,30 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
                   int y_dtype, int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s) {
     if (ws_bytes < q8_mid_workspace(C, B)) return fail(SQ_EWORKSPACE, "sq_q8_linear: workspace %zu < %zu", ws_bytes, q8_mid_workspace(C, B));
     const size_t ys = y_dtype == SQ_F32 ? 4 : 2;
-    const int64_t n = (int64_t)B * C;
-    const int64_t want = (n + 255) / 256;
-    hipLaunchKernelGGL(q8_x_kernel, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, s, (const uint16_t*)x, ldx, B, C,
-                       x_dtype, (uint16_t*)ws);
-    int rc = check_launch("q8_x_kernel");
-    if (rc) return rc;
+    // fp16 activations with 16-byte aligned rows are copied to LDS from where they are; anything else goes through
+    // an fp16 copy in the workspace first
+    const uint16_t* xh = (const uint16_t*)x;
+    int64_t ldxh = ldx;
+    int rc;
+    if (x_dtype != SQ_F16 || ((uintptr_t)x & 15) || ldx % 8 || ldx * 32 >= ((int64_t)1 << 31)) {
+        const int64_t n = (int64_t)B * C;
+        const int64_t want = (n + 255) / 256;
+        hipLaunchKernelGGL(q8_x_kernel, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, s, (const uint16_t*)x, ldx, B,
+                           C, x_dtype, (uint16_t*)ws);
+        rc = check_launch("q8_x_kernel");
+        if (rc) return rc;
+        xh = (const uint16_t*)ws;
+        ldxh = C;
+    }
     const int tasks = (V + 31) / 32;
     for (int b0 = 0; b0 < B; b0 += 32) {
         Q8MfmaArgs a{};
         a.q = q; a.sc = sc;
-        a.xh = (const uint16_t*)ws + (int64_t)b0 * C;
+        a.xh = xh + (int64_t)b0 * ldxh;
+        a.ldxh = (int)ldxh;
         a.y = (char*)y + (size_t)b0 * ldy * ys;
         a.ldy = ldy; a.V = V; a.C = C; a.B = B - b0 < 32 ? B - b0 : 32; a.y_dtype = y_dtype; a.tasks = tasks;
-        hipLaunchKernelGGL(q8_mfma_kernel, dim3((unsigned)((tasks + 3) / 4)), dim3(256), 0, s, a);
+        hipLaunchKernelGGL(q8_mfma_kernel<Q8_RING>, dim3((unsigned)((tasks + 3) / 4)), dim3(256), 0, s, a);
         rc = check_launch("q8_mfma_kernel");
         if (rc) return rc;
     }
