@@ -51,11 +51,75 @@ __global__ __launch_bounds__(256) void dequant_kernel(sq_matrix m, typename stor
     }
 }
 
+// Matrices with column orders: scattering 2-byte values straight to HBM costs 4x the plain decode, so a
+// workgroup decodes one row at a time into LDS at its permuted positions (ds_write of one element each, the
+// order read as whole 16/32-byte pieces) and then writes the row out in 16-byte pieces.
+template <int DT, int D>   // D = 8 or 4
+__global__ __launch_bounds__(256) void dequant_rows_lds_kernel(sq_matrix m, typename store_as<DT>::type* __restrict__ out,
+                                                               int64_t ld_out, int r0, int r1, int raw, int vec_out) {
+    typedef typename store_as<DT>::type T;
+    extern __shared__ __attribute__((aligned(16))) unsigned char row_smem[];
+    T* row_lds = reinterpret_cast<T*>(row_smem);
+    const int C = m.C, nch = C / D, tid = threadIdx.x;
+    constexpr int V = 16 / (int)sizeof(T);              // elements per 16-byte store
+    for (int r = r0 + blockIdx.x; r < r1; r += gridDim.x) {
+        const uint32_t* row = reinterpret_cast<const uint32_t*>(m.tags) + (int64_t)r * m.W;
+        const uint32_t boff = m.row_book ? (uint32_t)m.row_book[r] << m.bits : 0u;
+        const float s = raw ? 1.f : h2f(m.row_scale[r]);
+        const int32_t* pm = m.perms + (int64_t)(m.row_mask ? m.row_mask[r] : 0) * C;
+        for (int j = tid; j < nch; j += 256) {
+            const uint32_t tag = tag_at(row, m.W, m.bits, j) + boff;
+            const uint16_t* cw = m.table + (int64_t)tag * D;
+            uint32_t v[D / 2];
+            int32_t p[D];
+            if (D == 8) {
+                const u32x4 t = *reinterpret_cast<const u32x4*>(cw);
+                v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+                const u32x4 p0 = *reinterpret_cast<const u32x4*>(pm + j * 8), p1 = *reinterpret_cast<const u32x4*>(pm + j * 8 + 4);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) { p[k] = (int32_t)p0[k]; p[4 + k] = (int32_t)p1[k]; }
+            } else {
+                const u32x2 t = *reinterpret_cast<const u32x2*>(cw);
+                v[0] = t[0]; v[1] = t[1];
+                const u32x4 p0 = *reinterpret_cast<const u32x4*>(pm + j * 4);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[k] = (int32_t)p0[k];
+            }
+#pragma unroll
+            for (int k = 0; k < D / 2; ++k) {
+                row_lds[p[2 * k]] = store_as<DT>::cvt(h2f((uint16_t)(v[k] & 0xFFFFu)) * s);
+                row_lds[p[2 * k + 1]] = store_as<DT>::cvt(h2f((uint16_t)(v[k] >> 16)) * s);
+            }
+        }
+        __syncthreads();
+        T* o = out + (int64_t)(r - r0) * ld_out;
+        if (vec_out) {
+            for (int c = tid * V; c < C; c += 256 * V)
+                *reinterpret_cast<u32x4*>(o + c) = *reinterpret_cast<const u32x4*>(row_lds + c);
+        } else {
+            for (int c = tid; c < C; c += 256) o[c] = row_lds[c];
+        }
+        __syncthreads();
+    }
+}
+
 template <int DT>
 static int launch_dt(const sq_matrix& m, void* out, int64_t ld_out, int r0, int r1, hipStream_t s, int raw) {
     typedef typename store_as<DT>::type T;
     const int64_t n = (int64_t)(r1 - r0) * (m.C / m.d);
     if (n == 0) return SQ_OK;
+    const size_t row_bytes = (size_t)m.C * sizeof(T);
+    if (m.perms && (m.d == 8 || m.d == 4) && row_bytes <= 65536 && ((uintptr_t)m.perms & 15) == 0 && ((uintptr_t)m.table & 15) == 0 &&
+        m.C % 4 == 0) {
+        constexpr int V = 16 / (int)sizeof(T);
+        const int vec_out = ((uintptr_t)out & 15) == 0 && ld_out % V == 0 && m.C % V == 0;
+        const int per_cu = (int)(131072 / row_bytes) < 8 ? (int)(131072 / row_bytes) : 8;       // workgroups that share a CU's LDS
+        const int want = device_cus() * (per_cu < 1 ? 1 : per_cu);
+        const unsigned rgrid = (unsigned)(r1 - r0 < want ? r1 - r0 : want);
+        if (m.d == 8) hipLaunchKernelGGL((dequant_rows_lds_kernel<DT, 8>), dim3(rgrid), dim3(256), row_bytes, s, m, (T*)out, ld_out, r0, r1, raw, vec_out);
+        else hipLaunchKernelGGL((dequant_rows_lds_kernel<DT, 4>), dim3(rgrid), dim3(256), row_bytes, s, m, (T*)out, ld_out, r0, r1, raw, vec_out);
+        return check_launch("sq_dequant");
+    }
     const unsigned grid = (unsigned)((n + 255) / 256);
     if (m.d == 8) hipLaunchKernelGGL((dequant_kernel<DT, 8>), dim3(grid), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw);
     else if (m.d == 4) hipLaunchKernelGGL((dequant_kernel<DT, 4>), dim3(grid), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw);

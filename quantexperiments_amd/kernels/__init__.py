@@ -260,6 +260,8 @@ def q8_linear(q: torch.Tensor, sc: torch.Tensor, x: torch.Tensor, y: torch.Tenso
     """y[:, :V] = x . w^T for the 8-bit block-32 matrix (q int8 [V, C], sc fp16 [V, C/32]); x [B, C]
     fp16 / bf16, y [B, >= V] in x's dtype or fp32 (sq_q8_linear)."""
     V, C = _q_check(q, sc, 1, torch.int8, "q8_linear")
+    if q.device.type != "cuda" or x.device != q.device or y.device != q.device or sc.device != q.device:
+        raise ValueError("q8_linear: q, scale, x and y must be on one GPU (there is no CPU path)")
     if x.dim() != 2 or x.shape[1] != C or x.stride(1) != 1 or y.stride(1) != 1 or y.shape[0] != x.shape[0] or y.shape[1] < V:
         raise ValueError(f"q8_linear: x {tuple(x.shape)}, y {tuple(y.shape)} for a [{V}, {C}] matrix")
     dev = q.device
@@ -279,6 +281,8 @@ def q8_dense(q: torch.Tensor, sc: torch.Tensor, r0: int, r1: int, dtype: torch.d
     """Rows [r0, r1) of the 8-bit matrix as dense values (sq_q8_dequant); `out`: a flat buffer to decode into."""
     V, C = _q_check(q, sc, 1, torch.int8, "q8_dense")
     dev = q.device
+    if dev.type != "cuda" or sc.device != dev:
+        raise ValueError("q8_dense: q and scale must be on the GPU (there is no CPU path)")
     n = r1 - r0
     o = torch.empty(n, C, dtype=dtype, device=dev) if out is None else out[:n * C].view(n, C)
     with torch.cuda.device(dev):

@@ -50,6 +50,28 @@ def test_dequant_is_bit_exact(case):
     assert np.array_equal(lin.dense(torch.bfloat16).float().cpu().numpy(), O.round_bf16(ref))
 
 
+@pytest.mark.parametrize("case", [(70, 5120, 8, 16, 1, 16), (300, 1024, 4, 12, 4, 16), (9, 17408, 8, 16, 1, 3), (40, 36, 4, 6, 1, 2)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_dequant_with_column_orders_rows_through_lds(case):
+    # matrices with column orders are decoded row by row through LDS; row ranges, every dtype, an output
+    # that is not 16-byte aligned, a row (17408 fp32 = 68 KB) too long for LDS, and more rows than workgroups
+    import ctypes
+    from quantexperiments_amd import _lib
+    s = synth(*case, seed=sum(case))
+    lin = to_device(s)
+    ref = s.decode()
+    R, C = case[0], case[1]
+    assert torch.equal(lin.dense(torch.float32).cpu(), torch.from_numpy(ref))
+    assert np.array_equal(lin.dense(torch.float16).float().cpu().numpy(), O.round_fp16(ref))
+    assert np.array_equal(lin.dense(torch.bfloat16, rows=(3, R - 2)).float().cpu().numpy(), O.round_bf16(ref[3:R - 2]))
+    buf = torch.full((R * (C + 3) + 8,), float("nan"), dtype=torch.float16, device="cuda")
+    m = lin.descriptor()
+    _lib.check(_lib.lib().sq_dequant(ctypes.byref(m), buf.data_ptr() + 2, _lib.SQ_F16, C + 3, 1, R, _lib.stream_ptr(buf.device)))
+    got = buf[1:1 + (R - 1) * (C + 3)].view(R - 1, C + 3)
+    assert np.array_equal(got[:, :C].float().cpu().numpy(), O.round_fp16(ref[1:]))
+    assert torch.isnan(got[:, C:]).all() and torch.isnan(buf[0])
+
+
 def test_dequant_row_ranges_and_shared_buffer():
     s = synth(50, 128, 4, 8, seed=1)
     lin = to_device(s)

@@ -285,3 +285,56 @@ def test_stream_builder_rejects_other_formats():
     assert L.sq_stream_bytes(ptr, 4, 16, 128, 4, 16, None, 0) == 0            # d = 4
     assert L.sq_stream_bytes(ptr, 4, 16, 128, 8, 12, None, 0) == 0            # codebook fits LDS: no stream
     assert L.sq_stream_build(ptr, 4, 16, 128, 8, 12, None, 0, ptr, 64, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EUNSUPPORTED
+
+
+class _TinyLM(torch.nn.Module):
+    """The attributes aux_from_model reads off an HF causal LM."""
+
+    class _Cfg:
+        tie_word_embeddings = False
+
+        def to_dict(self):
+            return {"hidden_size": 64, "vocab_size": 40}
+
+    def __init__(self):
+        super().__init__()
+        g = torch.Generator().manual_seed(8)
+        self.model = torch.nn.Module()
+        self.model.embed_tokens = torch.nn.Embedding(40, 64)
+        self.model.norm = torch.nn.LayerNorm(64)
+        self.model.layers = torch.nn.ModuleList([torch.nn.Module()])
+        self.model.layers[0].mlp = torch.nn.Module()
+        self.model.layers[0].mlp.up_proj = torch.nn.Linear(64, 24, bias=True)
+        self.lm_head = torch.nn.Linear(64, 40, bias=False)
+        self.config = self._Cfg()
+        with torch.no_grad():
+            for p in self.parameters():
+                p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+
+
+def test_aux_section_round_trip(tmp_path):
+    # reference shapequant/packed.py:162-214: embedding as q4, head as q8, everything else but the packed block
+    # linears' weights stored as is; the summary counts all of it
+    s, t, meta, _, _ = _file(tmp_path)
+    lm = _TinyLM()
+    name = "model.layers.0.mlp.up_proj"
+    at, am = packed.aux_from_model(lm, [name])
+    assert am["embed"] == "q4_b32" and am["lm_head"] == "q8_b32" and am["vocab"] == 40 and am["hidden"] == 64 and not am["tied"]
+    assert am["dense"] == sorted(["model.norm.weight", "model.norm.bias", f"{name}.bias"])
+    eq, es = O.q4_embed_pack(lm.model.embed_tokens.weight.detach().numpy())
+    hq, hs, _ = O.q8_pack(lm.lm_head.weight.detach().numpy())
+    assert np.array_equal(at["aux.embed.q"].numpy(), eq) and np.array_equal(at["aux.embed.scale"].numpy(), es)
+    assert np.array_equal(at["aux.lm_head.q"].numpy(), hq) and np.array_equal(at["aux.lm_head.scale"].numpy(), hs)
+    path = tmp_path / "aux.safetensors"
+    summary = packed.save(path, {name: (t, meta)}, base_model="test/base", aux=(at, am))
+    dense_numel = 64 + 64 + 24
+    want = (meta["bits"] + 40 * 64 * 4.5 + 40 * 64 * 8.5 + dense_numel * 32) / (s.R * s.C + 2 * 40 * 64 + dense_numel)
+    assert summary["aux"] is True and abs(summary["bpw_all"] - want) < 1e-12
+    pf = packed.PackedFile(path)
+    assert pf.aux == am and pf.summary["aux"] is True
+    assert np.array_equal(pf.aux_tensor("lm_head.q").numpy(), hq) and pf.aux_tensor("lm_head.q").dtype == torch.int8
+    assert np.array_equal(pf.aux_tensor("embed.q").numpy(), eq) and pf.aux_tensor("embed.scale").dtype == torch.float16
+    assert torch.equal(pf.aux_tensor("dense.model.norm.weight"), lm.model.norm.weight.detach())
+    assert packed.PackedFile(_file(tmp_path)[4]).aux is None          # files without the section still load
+    with pytest.raises(ValueError):                                   # the decoders are GPU kernels
+        packed.q8_rows(torch.from_numpy(hq), torch.from_numpy(hs))
