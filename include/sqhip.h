@@ -107,7 +107,14 @@ size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, i
  * the same row_mask and with perms on the device.  The tags tensor stays the source of truth (sq_dequant,
  * B > 1 and the prefill GEMM read it); this plays the part of the reference's load-time layouts (reference
  * shapequant/kernels/proto_runs.py:295-349 pack_lane_major / RunsLinear, batched_runs.py:213-373 tile_words),
- * with a layout chosen for LDS gathers. */
+ * with a layout chosen for LDS gathers.
+ *
+ * The same two calls serve the formats whose codebook lives in LDS (d = 4 with 8-, 10- or 12-bit tags, one column
+ * order, rows of whole 128/160/96-bit units): for them the buffer is a tile-major copy of the tags (the units of
+ * each 16-row tile stored unit by unit, as large as the tags rounded up to 16 rows) that lets the decode-time
+ * kernel read with fully coalesced loads; `runs` is ignored, *runs_out = *groups_out = 0, and the caller passes
+ * the device copy in sq_matrix.stream with stream_runs = stream_groups = 0.  It is optional like the slice
+ * stream (the reference keeps such a copy too: shapequant/kernels/batched_runs.py tile_words). */
 size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
                        const uint8_t* row_mask_host, int32_t runs);
 int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,

@@ -127,7 +127,8 @@ size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, i
 
 size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
                        const uint8_t* row_mask_host, int32_t runs) {
-    if (!tags_host || d <= 0 || !stream_format_ok(R, C, d, bits) || (int64_t)W * 32 < (int64_t)(C / d) * bits) return 0;
+    if (!tags_host || d <= 0 || (int64_t)W * 32 < (int64_t)(C / d) * bits) return 0;
+    if (!stream_format_ok(R, C, d, bits)) return !row_mask_host && tiled_format_ok(R, W, C, d, bits) ? tiled_bytes(R, W) : 0;
     return stream_bytes_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs);
 }
 
@@ -135,6 +136,13 @@ int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, i
                     const uint8_t* row_mask_host, int32_t runs, void* out_host, size_t out_bytes, int32_t* runs_out,
                     int32_t* groups_out) {
     if (!tags_host || !out_host || !runs_out || !groups_out) return fail(SQ_EINVAL, "sq_stream_build: null pointer");
+    if (d > 0 && !stream_format_ok(R, C, d, bits) && !row_mask_host && tiled_format_ok(R, W, C, d, bits)) {
+        if (out_bytes < tiled_bytes(R, W)) return fail(SQ_EINVAL, "sq_stream_build: out_bytes %zu < %zu", out_bytes, tiled_bytes(R, W));
+        tiled_build((const uint32_t*)tags_host, R, W, bits, (uint32_t*)out_host);
+        *runs_out = 0;
+        *groups_out = 0;
+        return SQ_OK;
+    }
     if (d <= 0 || !stream_format_ok(R, C, d, bits)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: d %d bits %d R %d not covered", d, bits, R);
     if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_stream_build: W %d too small", W);
     return stream_build_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs, (unsigned char*)out_host,

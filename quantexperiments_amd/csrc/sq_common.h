@@ -89,6 +89,11 @@ size_t gemm_workspace(const sq_matrix* mats, int n, int T);
 int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, const void* x, int x_dtype, int64_t ldx,
                       void* y, int y_dtype, int64_t ldy, int T, hipStream_t s);
 
+// tile-major copy of the tags for the matrix-core decode kernel (host routines, sq_gemv.hip)
+bool tiled_format_ok(int R, int W, int C, int d, int bits);
+size_t tiled_bytes(int R, int W);
+void tiled_build(const uint32_t* tags, int R, int W, int bits, uint32_t* out);
+
 // the block-32 side formats (8-bit output head, 4-bit embedding)
 int launch_q8_small(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
                     int y_dtype, int64_t ldy, int B, hipStream_t s);

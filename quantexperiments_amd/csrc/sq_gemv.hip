@@ -54,6 +54,30 @@ static bool fast_shape(const sq_matrix& m) {
     return true;
 }
 
+// ---- tile-major copy of the tags for the matrix-core decode kernel (d = 4 formats, whose codebooks live in
+// LDS and which have no slice stream).  In the file's row-major layout the 16 lanes of a quarter wave read 16
+// different rows, 48 bytes each; in the copy the units of a 16-row tile are stored unit by unit,
+//     tiled[((t * U + u) * 16 + i) * UD + w] = tags[(16 t + i) * W + u * UD + w]      (rows past R: zeros)
+// so the same 16 lanes read 16 * UD consecutive dwords and a wave load covers one contiguous piece.
+bool tiled_format_ok(int R, int W, int C, int d, int bits) {
+    if (!(d == 4 && (bits == 12 || bits == 10 || bits == 8))) return false;
+    if (R <= 0 || C % d || W % unit_dwords(bits)) return false;
+    return (int64_t)(C / d) * bits == (int64_t)W * 32;
+}
+
+size_t tiled_bytes(int R, int W) { return (size_t)((R + 15) / 16) * 16 * W * 4; }
+
+void tiled_build(const uint32_t* tags, int R, int W, int bits, uint32_t* out) {
+    const int ud = unit_dwords(bits), U = W / ud, ntiles = (R + 15) / 16;
+    for (int t = 0; t < ntiles; ++t)
+        for (int u = 0; u < U; ++u)
+            for (int i = 0; i < 16; ++i) {
+                uint32_t* dst = out + (((size_t)t * U + u) * 16 + i) * ud;
+                const int r = t * 16 + i;
+                for (int w = 0; w < ud; ++w) dst[w] = r < R ? tags[(size_t)r * W + u * ud + w] : 0u;
+            }
+}
+
 static size_t xp_bytes(const sq_matrix& m, int B) {
     return (((size_t)(m.M > 1 ? m.M : 1) * B * m.C * 2) + 255) & ~(size_t)255;
 }
@@ -104,6 +128,12 @@ struct MmaPlan { int RW, NT, KW, ks; };
 
 static bool mma_shape(const sq_matrix& m) { return fast_shape(m) && !m.perms; }
 
+// bytes of codebook the matrix-core kernel stages in LDS (0: gathers go through the cache)
+static size_t mma_table_bytes(const sq_matrix& m) {
+    const size_t tab = (size_t)m.G * ((size_t)1 << m.bits) * m.d * 2;
+    return tab <= 128 * 1024 ? tab : 0;
+}
+
 // Rounds per wave, waves per workgroup and workgroup-level column slices that cover ceil(U / 4) rounds
 // with the fewest idle rounds (ties: more rounds per wave, i.e. fewer waves to add up).
 static MmaPlan mma_plan(const sq_matrix& m, int B) {
@@ -112,9 +142,17 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
     MmaPlan best{0, 0, 0, 0};
     double best_cost = 1e30;
     const int NT = B > 16 ? 2 : 1;
+    // waves per workgroup: 8, or as many as leave room in the CU's 160 KB of LDS for their reduction buffers
+    // next to a codebook that is staged there (4 books of 4096 d = 4 entries fill 128 KB)
+    const size_t tab = mma_table_bytes(m);
+    int max_kw = 8;
+    if (tab) {
+        const size_t room = 160 * 1024 - tab - 16, per_wave = (size_t)MMA_TT * 64 * NT * 16;
+        if (room / per_wave < 8) max_kw = (int)(room / per_wave);
+    }
     for (int rw = NT == 1 ? r1 : r1 / 2; rw >= 1 && rw >= r1 / 4; rw /= 2) {
         const int need = (rounds + rw - 1) / rw;
-        const int ks = (need + 7) / 8, kw = (need + ks - 1) / ks;
+        const int ks = (need + max_kw - 1) / max_kw, kw = (need + ks - 1) / ks;
         const double cost = (double)rw * kw * ks / rounds + 0.03 * (ks - 1) + 0.002 * kw;
         if (cost < best_cost - 1e-9) { best_cost = cost; best = MmaPlan{rw, NT, kw, ks}; }
     }
@@ -146,8 +184,7 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
     a.x = (const uint16_t*)x; a.ldx = ldx; a.y = y; a.ldy = ldy; a.B = B; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
     a.U = m0.W / unit_dwords(m0.bits);
     a.ks = pl.ks;
-    const size_t tab0 = (size_t)m0.G * ((size_t)1 << m0.bits) * m0.d * 2;
-    a.table_bytes = tab0 <= 128 * 1024 ? (int)tab0 : 0;
+    a.table_bytes = (int)mma_table_bytes(m0);
     const int threads = pl.KW * 64;
     const size_t smem = (size_t)a.table_bytes + 16 + (pl.KW > 1 ? (size_t)MMA_TT * pl.KW * 64 * pl.NT * 16 : 0);
     int rc = SQ_EUNSUPPORTED;
@@ -165,6 +202,9 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
     for (int k = 0; k < cnt; ++k) {
         MmaPiece& P = a.p[k];
         P.m = mats[k];
+        const sq_matrix& mk = mats[k];
+        P.tiled = mk.stream && !mk.perms && tiled_format_ok(mk.R, mk.W, mk.C, mk.d, mk.bits) && ((uintptr_t)mk.stream & 15) == 0
+                      ? (const uint32_t*)mk.stream : nullptr;
         P.part = nullptr;
         if (pl.ks > 1) {
             P.part = (float*)(ws + ws_off);

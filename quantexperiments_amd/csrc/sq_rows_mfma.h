@@ -27,6 +27,7 @@ namespace sq {
 
 struct MmaPiece {
     sq_matrix m;
+    const uint32_t* tiled; // tile-major copy of the tags (sq_matrix.stream of a d = 4 format) or NULL
     float* part;          // ks > 1: fp32 [ks, B, R] unscaled partial sums of this piece
     int wg_begin;         // first workgroup of this piece
     int wg_count;         // nshare * ks workgroups
@@ -119,9 +120,15 @@ __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
             const int ro = row0 + 4 * lg + v;
             sc[v] = h2f(m.row_scale[ro < m.R ? ro : m.R - 1]);
         }
-        const uint32_t* rp = tags + (size_t)r * m.W;
+        if (P.tiled) {           // unit u of the tile's 16 rows: 16 * UD consecutive dwords
+            const uint32_t* tp = P.tiled + ((size_t)t * a.U * 16 + li) * UD;
 #pragma unroll
-        for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(rp + uoff[n]);
+            for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(tp + (size_t)uoff[n] * 16);
+        } else {
+            const uint32_t* rp = tags + (size_t)r * m.W;
+#pragma unroll
+            for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(rp + uoff[n]);
+        }
         if (!all_live) {
 #pragma unroll
             for (int n = 0; n < RW; ++n)

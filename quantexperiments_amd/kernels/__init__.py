@@ -84,8 +84,14 @@ class PackedLinear(torch.nn.Module):
         self.register_buffer("stream", None)
         self.stream_runs = self.stream_groups = 0
         self.stream_asked = None
+        self.stream_tiled = False
         if stream and self.G == 1 and table.numel() * 2 > 128 * 1024:
             self.build_stream(0)
+        elif stream and not self.has_mask and d == 4 and table.numel() * 2 <= 128 * 1024:
+            # codebooks that live in LDS (d = 4): a tile-major copy of the tags, which the decode-time kernel
+            # reads with fully coalesced loads (same call; the library picks the layout by format)
+            self.build_stream(0)
+            self.stream_tiled = self.stream is not None
 
     def build_stream(self, runs: int = 0) -> None:
         """(Re)build the bucketed tag stream cut into about `runs` row runs (0 = suited to a launch of this
@@ -182,7 +188,7 @@ def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, 
 def prepare_stack(pieces, workgroups: int = 512) -> None:
     """Cut the streams of pieces that are launched together so that the launch makes about `workgroups`
     workgroups in total (two per CU on an MI355X), shared by rows.  Pieces without a stream are left alone."""
-    ps = [p for p in pieces if p.stream is not None]
+    ps = [p for p in pieces if p.stream is not None and not p.stream_tiled]
     rows = sum(p.R for p in ps)
     for p in ps:
         buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // 640)

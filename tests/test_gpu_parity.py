@@ -72,6 +72,27 @@ def test_dequant_with_column_orders_rows_through_lds(case):
     assert torch.isnan(got[:, C:]).all() and torch.isnan(buf[0])
 
 
+@pytest.mark.parametrize("case", [(70, 384, 4, 12, 1), (200, 3584, 4, 12, 4), (33, 640, 4, 10, 1), (50, 256, 4, 8, 2)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_tile_major_tags_give_identical_products(case):
+    # d = 4 matrices carry a tile-major copy of their tags for the decode-time kernel: same arithmetic in the
+    # same order as from the file layout, so the results are bit-identical
+    from quantexperiments_amd.kernels import linear_small
+    R, C, d, bits, G = case
+    s = synth(R, C, d, bits, G=G, seed=sum(case))
+    with_copy, plain = to_device(s), to_device(s, stream=False)
+    assert with_copy.stream is not None and with_copy.stream_tiled and plain.stream is None
+    assert with_copy.stream.numel() == -(-R // 16) * 16 * with_copy.W * 4
+    for B in (1, 5, 16, 32):
+        x = rand_x(B, C, torch.bfloat16, seed=B).cuda()
+        ya = torch.empty(B, R, dtype=torch.float32, device="cuda")
+        yb = torch.empty_like(ya)
+        linear_small([with_copy], x, ya)
+        linear_small([plain], x, yb)
+        assert torch.equal(ya, yb)
+        assert rel_max_err(ya.cpu().numpy(), _ref(s, x.cpu())) < TOL
+
+
 def test_dequant_row_ranges_and_shared_buffer():
     s = synth(50, 128, 4, 8, seed=1)
     lin = to_device(s)

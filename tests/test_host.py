@@ -287,6 +287,40 @@ def test_stream_builder_rejects_other_formats():
     assert L.sq_stream_build(ptr, 4, 16, 128, 8, 12, None, 0, ptr, 64, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EUNSUPPORTED
 
 
+@pytest.mark.parametrize("R,C,bits", [(70, 384, 12), (16, 128, 8), (33, 640, 10), (1, 32, 12)])
+def test_tile_major_copy_of_d4_tags(R, C, bits):
+    # d = 4 formats get a tile-major copy instead of a slice stream:
+    # tiled[((t * U + u) * 16 + i) * UD + w] = tags[(16 t + i) * W + u * UD + w], rows past R zero
+    import ctypes
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(R + bits)
+    tags = rng.integers(0, 1 << bits, (R, C // 4))
+    words = np.ascontiguousarray(O.pack_bits(tags, bits))
+    W = words.shape[1]
+    ud = {12: 3, 10: 5, 8: 4}[bits]
+    assert W % ud == 0
+    ptr = words.ctypes.data_as(ctypes.c_void_p)
+    nt = -(-R // 16)
+    n = L.sq_stream_bytes(ptr, R, W, C, 4, bits, None, 0)
+    assert n == nt * 16 * W * 4
+    out = np.full(n // 4, -1, np.int32)
+    r, g = ctypes.c_int32(7), ctypes.c_int32(7)
+    assert L.sq_stream_build(ptr, R, W, C, 4, bits, None, 0, out.ctypes.data_as(ctypes.c_void_p), n, ctypes.byref(r), ctypes.byref(g)) == 0
+    assert r.value == 0 and g.value == 0
+    padded = np.zeros((nt * 16, W), np.int32)
+    padded[:R] = words
+    want = padded.reshape(nt, 16, W // ud, ud).transpose(0, 2, 1, 3).reshape(-1)
+    assert np.array_equal(out, want)
+    assert L.sq_stream_build(ptr, R, W, C, 4, bits, None, 0, out.ctypes.data_as(ctypes.c_void_p), n - 4, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EINVAL
+    mask = np.zeros(R, np.uint8)                                             # column orders: no copy
+    assert L.sq_stream_bytes(ptr, R, W, C, 4, bits, mask.ctypes.data_as(ctypes.c_void_p), 0) == 0
+    if bits == 12 and C % 12 == 0:                                           # rows that are not whole units
+        w2 = np.ascontiguousarray(O.pack_bits(tags[:, :C // 4 - 8], bits))
+        if w2.shape[1] % 3:
+            assert L.sq_stream_bytes(w2.ctypes.data_as(ctypes.c_void_p), R, w2.shape[1], C - 32, 4, bits, None, 0) == 0
+
+
 class _TinyLM(torch.nn.Module):
     """The attributes aux_from_model reads off an HF causal LM."""
 
