@@ -401,8 +401,6 @@ static int q8_pass_rows(int B, int C) {
 // 32-bit offsets.
 static bool q8_mfma_ok(int C) { return C % 256 == 0 && (int64_t)C * 32 < ((int64_t)1 << 31); }
 
-int q8_mid_rows() { return Q8_MFMA_MAX_ROWS; }
-
 bool q8_mid(int C, int B) { return B > 4 && B <= Q8_MFMA_MAX_ROWS && q8_mfma_ok(C); }
 
 size_t q8_mid_workspace(int C, int B) { return q8_mid(C, B) ? (((size_t)B * C * 2) + 255) & ~(size_t)255 : 0; }
