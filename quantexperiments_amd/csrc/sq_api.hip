@@ -105,7 +105,7 @@ int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_d
     if (T == 0 || n_mats == 0) return SQ_OK;
     const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
     return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
-                       has_ws ? ws_bytes - SQ_WS_HEADER : 0, (hipStream_t)stream);
+                       has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
 }
 
 int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype, int64_t ldx,

@@ -84,7 +84,10 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
                  int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s);
 size_t small_workspace(const sq_matrix* mats, int n, int B);
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s);
+                int64_t ldy, int T, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s);
+// most activation rows for which passes of SQ_SMALL_BMAX rows through the decode-time kernel beat decode + GEMM
+// for these pieces (0: never)
+int small_pass_limit(const sq_matrix* mats, int n);
 size_t gemm_workspace(const sq_matrix* mats, int n, int T);
 int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, const void* x, int x_dtype, int64_t ldx,
                       void* y, int y_dtype, int64_t ldy, int T, hipStream_t s);

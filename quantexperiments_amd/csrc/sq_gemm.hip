@@ -154,13 +154,21 @@ int launch_bf16_to_f16(const uint16_t* x, int64_t ldx, int T, int C, uint16_t* o
 static bool x_vec_ok(const void* x, int64_t ldx, int C) { return C % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x & 15) == 0; }
 // Activation rows from which the large-tile route (decode each piece once into the workspace as raw fp16
 // codewords, then the 256 x 256 tile GEMM with the row scale in its epilogue) replaces the fused 128 x 128
-// kernel, which re-gathers every codeword once per 128 activation rows.
-constexpr int GEMM256_MIN_T = 256;
+// kernel, which re-gathers every codeword once per 128 activation rows.  It also wins below 256 rows (7B layer,
+// 64 rows: 0.60 ms against 1.90 ms on the fused kernel, whose grid is then a few dozen workgroups), so it is
+// used from the first row count sq_linear_small does not take.
+constexpr int GEMM256_MIN_T = SQ_SMALL_BMAX + 1;
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 static bool fused_ok(const sq_matrix& m) { return (m.d == 8 || m.d == 4) && !m.perms && ((uintptr_t)m.table & 15) == 0; }
 static size_t dense_bytes(const sq_matrix& m) { return (((size_t)m.R * m.C * 2) + 255) & ~(size_t)255; }
 
 size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
+    if (T > SQ_SMALL_BMAX && T <= small_pass_limit(mats, n)) {
+        // full passes and the last, shorter one may run different kernels with different needs
+        const size_t full = small_workspace(mats, n, SQ_SMALL_BMAX);
+        const size_t last = T % SQ_SMALL_BMAX ? small_workspace(mats, n, T % SQ_SMALL_BMAX) : 0;
+        return std::max(full, last);
+    }
     size_t need = 0;
     const bool big = T >= GEMM256_MIN_T && mats[0].C % 64 == 0;
     for (int i = 0; i < n; ++i)
@@ -197,7 +205,19 @@ int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, con
 }
 
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                int64_t ldy, int T, void* ws, size_t ws_bytes, hipStream_t s) {
+                int64_t ldy, int T, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s) {
+    if (T > SQ_SMALL_BMAX && T <= small_pass_limit(mats, n) && x_vec_ok(x, ldx, mats[0].C)) {
+        // a few passes of the decode-time kernel read the packed tags a few times; decoding to fp16 first
+        // (below) writes and reads 8 to 16 times as many bytes once
+        const size_t ys = y_dtype == SQ_F32 ? 4 : 2;
+        for (int t = 0; t < T; t += SQ_SMALL_BMAX) {
+            const int nb = T - t < SQ_SMALL_BMAX ? T - t : SQ_SMALL_BMAX;
+            int rc = launch_small(mats, n, (const char*)x + (size_t)t * ldx * 2, x_dtype, ldx, (char*)y + (size_t)t * ldy * ys,
+                                  y_dtype, ldy, nb, ws, ws_bytes, counters, s);
+            if (rc) return rc;
+        }
+        return SQ_OK;
+    }
     if (!x_vec_ok(x, ldx, mats[0].C)) {
         // odd strides: the any-shape kernel, SQ_SMALL_BMAX activation rows at a time
         for (int t = 0; t < T; t += SQ_SMALL_BMAX) {

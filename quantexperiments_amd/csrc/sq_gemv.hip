@@ -159,6 +159,17 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
     return best;
 }
 
+// Passes of 32 rows through the matrix-core decode kernel against decode + tile GEMM (7B layer): 104 us per pass
+// against 600-640 us when the codebook sits in LDS (d = 4), 201 us per pass when its gathers go to L2.
+int small_pass_limit(const sq_matrix* mats, int n) {
+    int limit = 160;
+    for (int i = 0; i < n; ++i) {
+        if (!mma_shape(mats[i])) return 0;
+        if (!mma_table_bytes(mats[i])) limit = 64;
+    }
+    return n > 0 ? limit : 0;
+}
+
 static size_t mma_part_bytes(const sq_matrix& m, int B) {
     const MmaPlan pl = mma_plan(m, B);
     return pl.ks > 1 ? ((((size_t)pl.ks * B * m.R * 4) + 255) & ~(size_t)255) : 0;

@@ -70,11 +70,16 @@ def test_workspace_sizes_are_host_arithmetic():
     plain = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 8, 16, 1, 1, 32, 0)
     masked = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, 0x6000, 0x7000, None, 64, 512, 8, 16, 1, 16, 32, 0)
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 1, 0) == 0
-    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == 0
-    # from 256 activation rows on: raw fp16 codewords of the largest piece + an fp16 copy of the activations
+    # 33 .. 64 rows of a matrix the matrix-core decode kernel takes: passes of 32 rows, its workspace (none here)
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 64, 1) == 0
+    lds = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 4, 12, 1, 1, 48, 0)
+    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 160, 1) == 0          # codebook in LDS: up to 160 rows
+    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 161, 1) == 4096 + 64 * 512 * 2 + 161 * 512 * 2
+    # beyond: raw fp16 codewords of the largest piece + an fp16 copy of the activations
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == 4096 + 64 * 512 * 2 + 100 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 4096 + 64 * 512 * 2 + 2048 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == 4096 + 16 * 2 * 512 * 2
-    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == 4096 + 64 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == 4096 + 64 * 512 * 2 + 100 * 512 * 2
 
 
 def test_block32_entry_points_check_arguments_on_the_host():
@@ -94,13 +99,13 @@ def test_block32_entry_points_check_arguments_on_the_host():
     # more than 32 activation rows need the workspace sq_q8_workspace_bytes names
     assert L.sq_q8_linear(q, sc, 64, 64, x, bf, 64, y, bf, 64, 40, None, 0, None) == _lib.SQ_EWORKSPACE
     assert L.sq_q8_workspace_bytes(64, 64, 32) == 0
-    assert L.sq_q8_workspace_bytes(64, 64, 40) == 4096 + 64 * 64 * 2
+    assert L.sq_q8_workspace_bytes(64, 64, 40) == 4096 + 64 * 64 * 2 + 40 * 64 * 2      # decoded rows + fp16 x
     assert L.sq_q8_workspace_bytes(64, 48, 40) == 0
     # 5 .. 128 rows with C % 256 == 0: an fp16 copy of the activations
     assert L.sq_q8_workspace_bytes(64, 256, 4) == 0
     assert L.sq_q8_workspace_bytes(64, 256, 8) == 4096 + 8 * 256 * 2
     assert L.sq_q8_workspace_bytes(64, 256, 128) == 4096 + 128 * 256 * 2
-    assert L.sq_q8_workspace_bytes(64, 256, 129) == 4096 + 64 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 129) == 4096 + 64 * 256 * 2 + 129 * 256 * 2
     assert L.sq_q8_linear(q, sc, 64, 256, x, bf, 256, y, bf, 64, 8, None, 0, None) == _lib.SQ_EWORKSPACE
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 64, 3, 65, None) == _lib.SQ_EINVAL                    # rows outside
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 32, 0, 4, None) == _lib.SQ_EINVAL                     # ld_out < C
