@@ -65,7 +65,9 @@ int sq_dequant(const sq_matrix* m, void* out, int out_dtype, int64_t ld_out, int
  * (elements).  x_dtype / y_dtype: SQ_F16 or SQ_BF16 (y may also be SQ_F32).
  * Replaces proto_runs.gemv (reference shapequant/kernels/proto_runs.py:505-571), cuda_gemv.gemv
  * (cuda_gemv.py:148-172), PackedLinear.gemv (gemv.py:142-156) and RunsBatch.run
- * (batched_runs.py:745-771).  Pieces with M > 1 need workspace (see sq_workspace_bytes). */
+ * (batched_runs.py:745-771).  Pieces with M > 1 need workspace (see sq_workspace_bytes); from 11 activation
+ * rows on, a stack that has column orders (and C % 64 == 0, 16-byte aligned x, ldx % 8 == 0) is decoded to
+ * fp16 in the workspace and multiplied by the tile GEMM, which is faster than its decode-time kernel there. */
 #define SQ_SMALL_BMAX 32
 int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx,
                     void* y, int y_dtype, int64_t ldy, int32_t B, void* workspace, size_t ws_bytes,

@@ -1,4 +1,5 @@
 // extern "C" surface of libsqhip.so: argument checks, error text, dispatch to the launchers.
+#include <algorithm>
 #include <stdarg.h>
 #include <stdio.h>
 #include "sq_stream.h"
@@ -94,6 +95,9 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
     if (B > SQ_SMALL_BMAX) return fail(SQ_EINVAL, "sq_linear_small: B %d > %d", B, SQ_SMALL_BMAX);
     if (B == 0 || n_mats == 0) return SQ_OK;
     const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
+    if (small_takes_gemm_route(mats, n_mats, B, x, ldx))
+        return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
+                           has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
     return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
                         has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
 }
@@ -121,7 +125,9 @@ int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C,
 
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which) {
     if (!mats || n_mats <= 0 || rows <= 0) return 0;
-    const size_t inner = which == 0 ? small_workspace(mats, n_mats, rows) : gemm_workspace(mats, n_mats, rows);
+    // which = 0 covers both kernels a stack with column orders may take (the caller's x decides, see sq_linear_small)
+    const size_t inner = which == 0 ? std::max(small_workspace(mats, n_mats, rows), small_gemm_route_workspace(mats, n_mats, rows))
+                                    : gemm_workspace(mats, n_mats, rows);
     return inner ? inner + SQ_WS_HEADER : 0;
 }
 

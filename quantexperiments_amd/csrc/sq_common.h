@@ -85,6 +85,9 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
 size_t small_workspace(const sq_matrix* mats, int n, int B);
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                 int64_t ldy, int T, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s);
+// stacks with column orders and more than a few activation rows: sq_linear_small runs the decode + tile GEMM route
+bool small_takes_gemm_route(const sq_matrix* mats, int n, int B, const void* x, int64_t ldx);
+size_t small_gemm_route_workspace(const sq_matrix* mats, int n, int B);
 // most activation rows for which passes of SQ_SMALL_BMAX rows through the decode-time kernel beat decode + GEMM
 // for these pieces (0: never)
 int small_pass_limit(const sq_matrix* mats, int n);

@@ -162,6 +162,34 @@ static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 static bool fused_ok(const sq_matrix& m) { return (m.d == 8 || m.d == 4) && !m.perms && ((uintptr_t)m.table & 15) == 0; }
 static size_t dense_bytes(const sq_matrix& m) { return (((size_t)m.R * m.C * 2) + 255) & ~(size_t)255; }
 
+// The decode + 256 x 256 tile route: from GEMM256_MIN_T rows, and for stacks with column orders at any row count
+// (their decode-time kernel is the slow one: 27B-shaped layer with 16 orders, 880 us at 16 rows and 1746 us at 32
+// against 625 us here).
+static bool big_route(const sq_matrix* mats, int n, int T) {
+    if (mats[0].C % 64) return false;
+    if (T >= GEMM256_MIN_T) return true;
+    for (int i = 0; i < n; ++i)
+        if (mats[i].perms) return true;
+    return false;
+}
+
+// Activation rows from which sq_linear_small hands a stack with column orders to the route above.
+constexpr int MASKED_GEMM_FROM = 11;
+
+bool small_takes_gemm_route(const sq_matrix* mats, int n, int B, const void* x, int64_t ldx) {
+    if (B < MASKED_GEMM_FROM || mats[0].C % 64 || !x_vec_ok(x, ldx, mats[0].C)) return false;
+    for (int i = 0; i < n; ++i)
+        if (mats[i].perms) return true;
+    return false;
+}
+
+size_t small_gemm_route_workspace(const sq_matrix* mats, int n, int B) {
+    if (B < MASKED_GEMM_FROM || mats[0].C % 64) return 0;
+    for (int i = 0; i < n; ++i)
+        if (mats[i].perms) return gemm_workspace(mats, n, B);
+    return 0;
+}
+
 size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
     if (T > SQ_SMALL_BMAX && T <= small_pass_limit(mats, n)) {
         // full passes and the last, shorter one may run different kernels with different needs
@@ -170,7 +198,7 @@ size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
         return std::max(full, last);
     }
     size_t need = 0;
-    const bool big = T >= GEMM256_MIN_T && mats[0].C % 64 == 0;
+    const bool big = big_route(mats, n, T);
     for (int i = 0; i < n; ++i)
         if ((big || !fused_ok(mats[i])) && dense_bytes(mats[i]) > need) need = dense_bytes(mats[i]);
     if (big) {
@@ -231,7 +259,7 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
     }
     if (gemm_workspace(mats, n, T) > ws_bytes)
         return fail(SQ_EWORKSPACE, "sq_linear_gemm: workspace %zu < %zu", ws_bytes, gemm_workspace(mats, n, T));
-    if (T >= GEMM256_MIN_T && mats[0].C % 64 == 0) {
+    if (big_route(mats, n, T)) {
         const int C = mats[0].C;
         const uint16_t* xh = (const uint16_t*)x;
         int64_t ldxh = ldx;

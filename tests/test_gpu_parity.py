@@ -233,14 +233,15 @@ def test_stream_gemv_matches_oracle_and_row_path(case, dtype):
     y2 = torch.empty_like(y32)
     linear_small([lin], x.cuda(), y2)
     assert torch.equal(y2, y32)
-    # several activation rows per pass (1, 2, 4 or 8; more passes beyond 8 rows with column orders): every row
-    # must equal its own batch-1 result bit for bit, since its sums are formed in the same order
-    for B in (2, 3, 5, 8) + ((11,) if M > 1 else ()):
+    # several activation rows per pass (1, 2, 4 or 8; a second pass for 9 and 10 rows with column orders): every
+    # row must equal its own batch-1 result bit for bit, since its sums are formed in the same order.  From 11 rows
+    # a matrix with column orders (and C % 64 == 0) is decoded and multiplied by the tile GEMM instead: oracle only.
+    for B in (2, 3, 5, 8) + ((10, 11, 19) if M > 1 else ()):
         xb = rand_x(B, C, dtype, seed=R + B)
         yb = torch.full((B, R + 3), 5.0, dtype=torch.float32, device="cuda")
         linear_small([lin], xb.cuda(), yb[:, :R])
         assert rel_max_err(yb[:, :R].cpu().numpy(), _ref(s, xb)) < TOL and (yb[:, R:] == 5.0).all()
-        if M > 1:                                       # (without column orders small matrices take the matrix-core kernel)
+        if M > 1 and (B < 11 or C % 64):                # (without column orders small matrices take the matrix-core kernel)
             for b in range(B):
                 linear_small([lin], xb[b:b + 1].cuda(), y2)
                 assert torch.equal(y2[0], yb[b, :R]), (B, b)
