@@ -160,12 +160,16 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
 }
 
 // Passes of 32 rows through the matrix-core decode kernel against decode + tile GEMM (7B layer): 104 us per pass
-// against 600-640 us when the codebook sits in LDS (d = 4), 201 us per pass when its gathers go to L2.
+// against 600-640 us when the codebook sits in LDS (d = 4), 201 us per pass when its gathers go to L2.  A
+// codebook that fills most of LDS leaves room for fewer waves per workgroup and doubles the cost of a pass
+// (27B layer, 4 books of 4096: 246 us per pass against 800 us).
 int small_pass_limit(const sq_matrix* mats, int n) {
     int limit = 160;
     for (int i = 0; i < n; ++i) {
         if (!mma_shape(mats[i])) return 0;
-        if (!mma_table_bytes(mats[i])) limit = 64;
+        const size_t tab = mma_table_bytes(mats[i]);
+        const int li = tab == 0 ? 64 : tab > 64 * 1024 ? 96 : 160;
+        if (li < limit) limit = li;
     }
     return n > 0 ? limit : 0;
 }
