@@ -190,6 +190,32 @@ size_t small_gemm_route_workspace(const sq_matrix* mats, int n, int B) {
     return 0;
 }
 
+// Pieces that are neighbours in Y are decoded one behind the other and multiplied in ONE tile GEMM over all their
+// rows (their row scales copied into one array): a 512-row k or v projection alone is 2 tiles of 256 rows, a
+// launch that leaves the chip idle (7B q|k|v at 64-255 rows: 139 us as three products, the o projection of q's
+// size: 62 us).
+constexpr size_t STACK_MAX_BYTES = (size_t)1 << 30;
+static bool stacked_route(const sq_matrix* mats, int n) {
+    if (n < 2) return false;
+    size_t tot = 0;
+    for (int i = 0; i < n; ++i) {
+        if (mats[i].R <= 0) return false;
+        if (i + 1 < n && mats[i + 1].y_off != mats[i].y_off + mats[i].R) return false;
+        tot += dense_bytes(mats[i]);
+    }
+    return tot <= STACK_MAX_BYTES;
+}
+static int stacked_rows(const sq_matrix* mats, int n) {
+    int r = 0;
+    for (int i = 0; i < n; ++i) r += mats[i].R;
+    return r;
+}
+
+__global__ __launch_bounds__(256) void copy_u16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
 size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
     if (T > SQ_SMALL_BMAX && T <= small_pass_limit(mats, n)) {
         // full passes and the last, shorter one may run different kernels with different needs
@@ -199,6 +225,11 @@ size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
     }
     size_t need = 0;
     const bool big = big_route(mats, n, T);
+    if (big && stacked_route(mats, n)) {
+        const int R = stacked_rows(mats, n);
+        for (int i = 0; i < n; ++i) need += dense_bytes(mats[i]);
+        return need + align256((size_t)R * 2) + align256((size_t)T * mats[0].C * 2) + gemm256_part_bytes(T, R, mats[0].C, device_cus());
+    }
     for (int i = 0; i < n; ++i)
         if ((big || !fused_ok(mats[i])) && dense_bytes(mats[i]) > need) need = dense_bytes(mats[i]);
     if (big) {
@@ -271,6 +302,28 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
             ldxh = C;
         }
         wd += align256((size_t)T * C * 2);
+        const int cus0 = device_cus();
+        if (stacked_route(mats, n)) {
+            const int R = stacked_rows(mats, n);
+            char* next = wd;
+            for (int i = 0; i < n; ++i) next += dense_bytes(mats[i]);
+            uint16_t* scales = (uint16_t*)next;
+            float* part = (float*)(next + align256((size_t)R * 2));
+            char* w = wd;
+            int r0 = 0;
+            for (int i = 0; i < n; ++i) {
+                const sq_matrix& m = mats[i];
+                int rc = launch_dequant(m, w, SQ_F16, C, 0, m.R, s, /*raw=*/true);
+                if (rc) return rc;
+                hipLaunchKernelGGL(copy_u16_kernel, dim3((unsigned)((m.R + 255) / 256)), dim3(256), 0, s, m.row_scale, scales + r0, m.R);
+                rc = check_launch("sq_linear_gemm(row scales)");
+                if (rc) return rc;
+                w += (size_t)m.R * C * 2;                       // rows follow each other without gaps
+                r0 += m.R;
+            }
+            return launch_gemm256(xh, ldxh, (const uint16_t*)wd, C, scales, y, y_dtype, ldy, mats[0].y_off, T, R, C,
+                                  gemm256_part_bytes(T, R, C, cus0) ? part : nullptr, cus0, s);
+        }
         size_t dense = 0;
         for (int i = 0; i < n; ++i) dense = std::max(dense, dense_bytes(mats[i]));
         float* part = (float*)(wd + dense);

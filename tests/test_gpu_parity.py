@@ -327,9 +327,37 @@ def test_gemm_dense_matches_float64():
     assert rel_max_err(y.cpu().numpy(), ref) < 1e-5
 
 
+def test_gemm_of_neighbouring_and_scattered_pieces():
+    # pieces that follow each other in Y are multiplied in one tile GEMM over all their rows; pieces with gaps
+    # between their column slices (or in another order) one by one.  Both through the raw C ABI.
+    import ctypes
+    from quantexperiments_amd import _lib
+    ss = [synth(R, 1280, 4, 12, seed=R) for R in (300, 64, 64)]
+    lins = [to_device(s) for s in ss]
+    L = _lib.lib()
+    T = 200
+    x = rand_x(T, 1280, torch.bfloat16, seed=5)
+    refs = [_ref(s, x) for s in ss]
+    for offs in ([0, 300, 364], [70, 0, 400], [0, 310, 380]):
+        width = max(o + s.R for o, s in zip(offs, ss)) + 5
+        mats = _lib.matrix_array([p.descriptor(o) for p, o in zip(lins, offs)])
+        need = L.sq_workspace_bytes(mats, 3, T, 1)
+        ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+        y = torch.full((T, width), 3.0, dtype=torch.float32, device="cuda")
+        xd = x.cuda()
+        _lib.check(L.sq_linear_gemm(mats, 3, xd.data_ptr(), _lib.SQ_BF16, 1280, y.data_ptr(), _lib.SQ_F32, width, T,
+                                    ws.data_ptr(), need, _lib.stream_ptr(y.device)))
+        covered = torch.zeros(width, dtype=torch.bool)
+        for o, s, ref in zip(offs, ss, refs):
+            assert rel_max_err(y[:, o:o + s.R].cpu().numpy(), ref) < TOL
+            covered[o:o + s.R] = True
+        assert (y[:, ~covered.cuda()] == 3.0).all()
+        assert not ws[:4096].any()                      # the counter header is left at zero
+
+
 # ------------------------------------------------------------------ the layer object and the op
 @pytest.mark.parametrize("large", ["fused", "dequant", "chunked"])
-@pytest.mark.parametrize("M", [0, 1, 3, 32, 33, 100])
+@pytest.mark.parametrize("M", [0, 1, 3, 32, 33, 100, 200, 300])
 def test_packed_shards_forward(large, M):
     # reference tests/test_vllm_ext_core.py:35-58
     from quantexperiments_amd.vllm_ext import core
