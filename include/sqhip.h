@@ -86,7 +86,10 @@ int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_d
 
 /* Dense fp16/bf16 weight [R, C] (row stride ldw) times X: the GEMM half of the reference's
  * "dequant + GEMM" large-M route (reference shapequant/vllm_ext/core.py:396-406, where it is a
- * cuBLAS call).  w_dtype: SQ_F16 or SQ_BF16, independent of x_dtype (both are multiplied as fp16). */
+ * cuBLAS call).  w_dtype: SQ_F16 or SQ_BF16, independent of x_dtype (both are multiplied as fp16); y_dtype any of
+ * the three, independent of both.  fp16 weights with fp16 activations (16-byte aligned, strides % 8 == 0,
+ * C % 64 == 0) run on the 256 x 256 tile kernel from 33 activation rows on; other combinations on a 128 x 128 tile
+ * kernel that converts while it loads. */
 int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype,
                   int64_t ldx, void* y, int y_dtype, int64_t ldy, int32_t T, void* stream);
 

@@ -116,7 +116,7 @@ int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C,
                   void* y, int y_dtype, int64_t ldy, int32_t T, void* stream) {
     if (x_dtype != SQ_F16 && x_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense: x_dtype %d", x_dtype);
     if (w_dtype != SQ_F16 && w_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense: w_dtype %d", w_dtype);
-    if (y_dtype != SQ_F32 && y_dtype != x_dtype) return fail(SQ_EINVAL, "sq_gemm_dense: y_dtype %d", y_dtype);
+    if (y_dtype != SQ_F32 && y_dtype != SQ_F16 && y_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense: y_dtype %d", y_dtype);
     if (R < 0 || C <= 0 || T < 0) return fail(SQ_EINVAL, "sq_gemm_dense: R %d C %d T %d", R, C, T);
     if (R == 0 || T == 0) return SQ_OK;
     if (!w || !x || !y || ldw < C || ldx < C || ldy < R) return fail(SQ_EINVAL, "sq_gemm_dense: bad pointer or stride");

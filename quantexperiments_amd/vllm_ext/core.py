@@ -216,6 +216,8 @@ class PackedShards:
         if self.large == "chunked":
             rows = min(rows, max(128, (self.chunk_bytes // (2 * self.C)) // 128 * 128))
         scratch = _Workspace.get(rows * self.C * 2, x.device, kind="dense").view(torch.float16)
+        if x.dtype != torch.float16 and M > BMAX and self.C % 64 == 0:
+            x = x.to(torch.float16)                     # fp16 x fp16 takes the 256 x 256 tile kernel; y keeps its dtype
         for rl, off in zip(self.rls, self.offs):
             for r0 in range(0, rl.R, rows):
                 r1 = min(rl.R, r0 + rows)
