@@ -336,28 +336,50 @@ __global__ __launch_bounds__(256, RING == 2 ? 4 : 3) void q8_mfma_kernel(Q8MfmaA
     }
 }
 
+// N consecutive outputs of type T from fp32 values: 16-byte stores when the destination allows it.
+template <int DT, int N>
+__device__ __forceinline__ void store_run(typename store_as<DT>::type* dst, const float (&v)[N], bool vec) {
+    typedef typename store_as<DT>::type T;
+    if (vec) {
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int k = 0; k < N; k += 4)
+                *reinterpret_cast<float4v*>(dst + k) = float4v{v[k], v[k + 1], v[k + 2], v[k + 3]};
+        } else {
+#pragma unroll
+            for (int k = 0; k < N; k += 8) {
+                u32x4 p;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    p[e] = (uint32_t)store_as<DT>::cvt(v[k + 2 * e]) | ((uint32_t)store_as<DT>::cvt(v[k + 2 * e + 1]) << 16);
+                *reinterpret_cast<u32x4*>(dst + k) = p;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < N; ++k) dst[k] = store_as<DT>::cvt(v[k]);
+    }
+}
+
 // Rows [r0, r1) as dense values, one 16-byte load (16 weights, half a block) per thread.
 template <int DT>
 __global__ __launch_bounds__(256) void q8_dequant_kernel(const int8_t* __restrict__ q, const uint16_t* __restrict__ sc,
                                                          int C, typename store_as<DT>::type* __restrict__ out,
-                                                         int64_t ld_out, int r0, int64_t n16) {
-    typedef typename store_as<DT>::type T;
+                                                         int64_t ld_out, int r0, int64_t n16, int vec) {
     const int per_row = C >> 4;
     for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < n16; t += (int64_t)gridDim.x * 256) {
         const int rr = (int)(t / per_row), c = (int)(t - (int64_t)rr * per_row) * 16;
         const int64_t row = r0 + rr;
         const u32x4 v = *reinterpret_cast<const u32x4*>(q + row * C + c);
         const float s = h2f(sc[row * (C >> 5) + (c >> 5)]);
-        T o[16];
+        float o[16];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const uint32_t w = v[k];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[4 * k + e] = store_as<DT>::cvt((float)(int8_t)(w >> (8 * e)) * s);
+            for (int e = 0; e < 4; ++e) o[4 * k + e] = (float)(int8_t)(w >> (8 * e)) * s;
         }
-        T* dst = out + (int64_t)rr * ld_out + c;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) dst[k] = o[k];
+        store_run<DT, 16>(out + (int64_t)rr * ld_out + c, o, vec != 0);
     }
 }
 
@@ -365,7 +387,7 @@ __global__ __launch_bounds__(256) void q8_dequant_kernel(const int8_t* __restric
 template <int DT>
 __global__ __launch_bounds__(256) void q4_embed_kernel(const uint8_t* __restrict__ q, const uint16_t* __restrict__ sc,
                                                        int V, int C, const int64_t* __restrict__ ids, int64_t n_ids,
-                                                       typename store_as<DT>::type* __restrict__ out, int64_t ld_out) {
+                                                       typename store_as<DT>::type* __restrict__ out, int64_t ld_out, int vec) {
     typedef typename store_as<DT>::type T;
     const int nblk = C >> 5;
     const int64_t total = n_ids * nblk;
@@ -374,20 +396,21 @@ __global__ __launch_bounds__(256) void q4_embed_kernel(const uint8_t* __restrict
         const int b = (int)(t - i * nblk);
         const int64_t id = ids[i];
         T* dst = out + i * ld_out + b * 32;
+        float o[32];
         if (id < 0 || id >= V) {
 #pragma unroll
-            for (int k = 0; k < 32; ++k) dst[k] = store_as<DT>::cvt(0.f);
-            continue;
-        }
-        const u32x4 v = *reinterpret_cast<const u32x4*>(q + id * (C >> 1) + b * 16);
-        const float s = h2f(sc[id * nblk + b]);
+            for (int k = 0; k < 32; ++k) o[k] = 0.f;
+        } else {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(q + id * (C >> 1) + b * 16);
+            const float s = h2f(sc[id * nblk + b]);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t w = v[k];
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t w = v[k];
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                dst[8 * k + e] = store_as<DT>::cvt((float)((int)((w >> (4 * e)) & 15u) - 8) * s);
+                for (int e = 0; e < 8; ++e) o[8 * k + e] = (float)((int)((w >> (4 * e)) & 15u) - 8) * s;
+            }
         }
+        store_run<DT, 32>(dst, o, vec != 0);
     }
 }
 
@@ -474,12 +497,14 @@ int launch_q8_dequant(const int8_t* q, const uint16_t* sc, int C, void* out, int
     if (n16 == 0) return SQ_OK;
     const int64_t want = (n16 + 255) / 256;
     const unsigned grid = (unsigned)(want < 65536 ? want : 65536);
+    const int64_t per16 = out_dtype == SQ_F32 ? 4 : 8;          // elements per 16 bytes
+    const int vec = ((uintptr_t)out & 15) == 0 && ld_out % per16 == 0;
     if (out_dtype == SQ_F32)
-        hipLaunchKernelGGL(q8_dequant_kernel<SQ_F32>, dim3(grid), dim3(256), 0, s, q, sc, C, (float*)out, ld_out, r0, n16);
+        hipLaunchKernelGGL(q8_dequant_kernel<SQ_F32>, dim3(grid), dim3(256), 0, s, q, sc, C, (float*)out, ld_out, r0, n16, vec);
     else if (out_dtype == SQ_F16)
-        hipLaunchKernelGGL(q8_dequant_kernel<SQ_F16>, dim3(grid), dim3(256), 0, s, q, sc, C, (uint16_t*)out, ld_out, r0, n16);
+        hipLaunchKernelGGL(q8_dequant_kernel<SQ_F16>, dim3(grid), dim3(256), 0, s, q, sc, C, (uint16_t*)out, ld_out, r0, n16, vec);
     else
-        hipLaunchKernelGGL(q8_dequant_kernel<SQ_BF16>, dim3(grid), dim3(256), 0, s, q, sc, C, (uint16_t*)out, ld_out, r0, n16);
+        hipLaunchKernelGGL(q8_dequant_kernel<SQ_BF16>, dim3(grid), dim3(256), 0, s, q, sc, C, (uint16_t*)out, ld_out, r0, n16, vec);
     return check_launch("q8_dequant_kernel");
 }
 
@@ -489,12 +514,14 @@ int launch_q4_embed(const uint8_t* q, const uint16_t* sc, int V, int C, const in
     if (total == 0) return SQ_OK;
     const int64_t want = (total + 255) / 256;
     const unsigned grid = (unsigned)(want < 65536 ? want : 65536);
+    const int64_t per16 = out_dtype == SQ_F32 ? 4 : 8;
+    const int vec = ((uintptr_t)out & 15) == 0 && ld_out % per16 == 0;
     if (out_dtype == SQ_F32)
-        hipLaunchKernelGGL(q4_embed_kernel<SQ_F32>, dim3(grid), dim3(256), 0, s, q, sc, V, C, ids, n_ids, (float*)out, ld_out);
+        hipLaunchKernelGGL(q4_embed_kernel<SQ_F32>, dim3(grid), dim3(256), 0, s, q, sc, V, C, ids, n_ids, (float*)out, ld_out, vec);
     else if (out_dtype == SQ_F16)
-        hipLaunchKernelGGL(q4_embed_kernel<SQ_F16>, dim3(grid), dim3(256), 0, s, q, sc, V, C, ids, n_ids, (uint16_t*)out, ld_out);
+        hipLaunchKernelGGL(q4_embed_kernel<SQ_F16>, dim3(grid), dim3(256), 0, s, q, sc, V, C, ids, n_ids, (uint16_t*)out, ld_out, vec);
     else
-        hipLaunchKernelGGL(q4_embed_kernel<SQ_BF16>, dim3(grid), dim3(256), 0, s, q, sc, V, C, ids, n_ids, (uint16_t*)out, ld_out);
+        hipLaunchKernelGGL(q4_embed_kernel<SQ_BF16>, dim3(grid), dim3(256), 0, s, q, sc, V, C, ids, n_ids, (uint16_t*)out, ld_out, vec);
     return check_launch("q4_embed_kernel");
 }
 
