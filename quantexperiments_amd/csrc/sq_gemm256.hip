@@ -42,7 +42,10 @@ struct Gemm256Args {
     // part[(tail tile * kt + kz)][256][256] for gemm256_reduce_kernel.
     int main_tiles, kt;
     float* part;
+    int vec_y;                // y rows allow 16-byte stores of 16-bit results (y 16-byte aligned, ldy % 8 == y_off % 8 == 0)
 };
+
+constexpr int G_EP_PITCH = 64 * 2 + 16;      // bytes per token row of a wave's 128 x 64 output tile in LDS
 
 // s_waitcnt immediate that waits until at most n vector-memory operations are outstanding and leaves the
 // other counters alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
@@ -196,7 +199,45 @@ __global__ __launch_bounds__(G_WAVES * 64) void gemm256_kernel(Gemm256Args a) {
     }
 #undef SQ_SB
 
-    // epilogue
+    // Epilogue.  In the accumulator layout a lane holds one weight row and 4 consecutive tokens, so direct stores
+    // are 2-byte pieces (49 us of a 376 us product at the 2048 x 18944 output).  16-bit results therefore go
+    // through the now idle LDS: every wave lays its 128 x 64 tile out token-major and writes it in 16-byte
+    // pieces, 128 contiguous bytes per token.
+    if (nparts == 1 && a.vec_y && a.y_dtype != SQ_F32) {
+        __syncthreads();                                        // every wave is done with the operand ring
+        unsigned char* my = smem + wave * (128 * G_EP_PITCH);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int rl = j * 32 + (lane & 31);
+            const int r = r0 + wn + rl;
+            const float sc_r = a.row_scale ? h2f(a.row_scale[r < a.R ? r : a.R - 1]) : 1.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int tl = i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                    const float val = acc[i][j][v] * sc_r;
+                    *reinterpret_cast<uint16_t*>(my + tl * G_EP_PITCH + rl * 2) = a.y_dtype == SQ_BF16 ? f2bf(val) : f2h(val);
+                }
+        }
+        uint16_t* yb = reinterpret_cast<uint16_t*>(a.y);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int idx = k * 64 + lane, tl = idx >> 3, piece = idx & 7;
+            const int t = t0 + wm + tl, r = r0 + wn + piece * 8;
+            if (t >= a.T || r >= a.R) continue;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(my + tl * G_EP_PITCH + piece * 16);
+            uint16_t* dst = yb + (int64_t)t * a.ldy + a.y_off + r;
+            if (r + 8 <= a.R) {
+                *reinterpret_cast<u32x4*>(dst) = v;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (r + e < a.R) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int r = r0 + wn + j * 32 + (lane & 31);
@@ -291,6 +332,7 @@ int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ld
     a.main_tiles = pl.main_tiles;
     a.kt = pl.kt;
     a.part = part;
+    a.vec_y = ((uintptr_t)y & 15) == 0 && ldy % 8 == 0 && y_off % 8 == 0;
     const unsigned grid = (unsigned)(8 * ((pl.main_tiles + 7) / 8 + (pl.tail_tiles * pl.kt + 7) / 8));
     hipLaunchKernelGGL(gemm256_kernel, dim3(grid), dim3(G_WAVES * 64), G_SLOTS * G_SLOT_BYTES, s, a);
     int rc = check_launch("sq_linear_gemm(gemm256)");
