@@ -218,6 +218,7 @@ struct Q8MfmaArgs {
     int64_t ldy;
     int ldxh;
     int V, C, B, y_dtype, tasks;
+    int vec_y;              // y rows allow 8-byte stores of 16-bit results (y 8-byte aligned, ldy % 4 == 0)
 };
 
 constexpr int q8_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }   // wait on vmcnt only
@@ -329,6 +330,25 @@ __global__ __launch_bounds__(256, RING == 2 ? 4 : 3) void q8_mfma_kernel(Q8MfmaA
         }
     }
     if (!active || r >= a.B) return;
+    // a lane holds 4 x 4 consecutive weight rows of activation row r: 8-byte stores of 16-bit results when aligned
+    if (a.vec_y && a.y_dtype != SQ_F32) {
+        uint16_t* yb = reinterpret_cast<uint16_t*>(a.y) + (int64_t)r * a.ldy;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int orow = task * 32 + g * 8 + h * 4;
+            uint16_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = a.y_dtype == SQ_BF16 ? f2bf(acc[4 * g + e]) : f2h(acc[4 * g + e]);
+            if (orow + 4 <= a.V) {
+                *reinterpret_cast<u32x2*>(yb + orow) = u32x2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (orow + e < a.V) yb[orow + e] = o[e];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int jj = 0; jj < 16; ++jj) {
         const int orow = task * 32 + (jj >> 2) * 8 + h * 4 + (jj & 3);
@@ -455,6 +475,7 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
         a.ldxh = (int)ldxh;
         a.y = (char*)y + (size_t)b0 * ldy * ys;
         a.ldy = ldy; a.V = V; a.C = C; a.B = B - b0 < 32 ? B - b0 : 32; a.y_dtype = y_dtype; a.tasks = tasks;
+        a.vec_y = ((uintptr_t)a.y & 7) == 0 && ldy % 4 == 0;
         hipLaunchKernelGGL(q8_mfma_kernel<Q8_RING>, dim3((unsigned)((tasks + 3) / 4)), dim3(256), 0, s, a);
         rc = check_launch("q8_mfma_kernel");
         if (rc) return rc;
