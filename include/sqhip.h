@@ -79,7 +79,8 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
  * M > 1 are decoded with their column orders into workspace and multiplied from there.  Between
  * SQ_SMALL_BMAX + 1 and 160 rows (64 when the codebook does not fit LDS) pieces without column orders
  * run as passes of SQ_SMALL_BMAX rows through sq_linear_small's kernels, which is cheaper than decoding
- * the matrix first; sq_workspace_bytes(which = 1) accounts for whichever route T takes. */
+ * the matrix first, and up to SQ_SMALL_BMAX rows the call is sq_linear_small; sq_workspace_bytes(which = 1)
+ * accounts for whichever route T takes. */
 int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx,
                    void* y, int y_dtype, int64_t ldy, int32_t T, void* workspace, size_t ws_bytes,
                    void* stream);

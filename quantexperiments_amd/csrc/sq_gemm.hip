@@ -176,18 +176,19 @@ static bool big_route(const sq_matrix* mats, int n, int T) {
 // Activation rows from which sq_linear_small hands a stack with column orders to the route above.
 constexpr int MASKED_GEMM_FROM = 11;
 
-bool small_takes_gemm_route(const sq_matrix* mats, int n, int B, const void* x, int64_t ldx) {
-    if (B < MASKED_GEMM_FROM || mats[0].C % 64 || !x_vec_ok(x, ldx, mats[0].C)) return false;
+static bool masked_gemm(const sq_matrix* mats, int n, int B) {
+    if (B < MASKED_GEMM_FROM || mats[0].C % 64) return false;
     for (int i = 0; i < n; ++i)
         if (mats[i].perms) return true;
     return false;
 }
 
+bool small_takes_gemm_route(const sq_matrix* mats, int n, int B, const void* x, int64_t ldx) {
+    return masked_gemm(mats, n, B) && x_vec_ok(x, ldx, mats[0].C);
+}
+
 size_t small_gemm_route_workspace(const sq_matrix* mats, int n, int B) {
-    if (B < MASKED_GEMM_FROM || mats[0].C % 64) return 0;
-    for (int i = 0; i < n; ++i)
-        if (mats[i].perms) return gemm_workspace(mats, n, B);
-    return 0;
+    return masked_gemm(mats, n, B) ? gemm_workspace(mats, n, B) : 0;
 }
 
 // Pieces that are neighbours in Y are decoded one behind the other and multiplied in ONE tile GEMM over all their
@@ -216,7 +217,17 @@ __global__ __launch_bounds__(256) void copy_u16_kernel(const uint16_t* __restric
     if (i < n) dst[i] = src[i];
 }
 
+static size_t gemm_workspace_beyond_small(const sq_matrix* mats, int n, int T);
+
 size_t gemm_workspace(const sq_matrix* mats, int n, int T) {
+    // up to SQ_SMALL_BMAX rows sq_linear_gemm is sq_linear_small, unless the stack goes the other way (see above);
+    // which of the two runs then depends on the alignment of x, so the workspace covers both
+    if (T > SQ_SMALL_BMAX) return gemm_workspace_beyond_small(mats, n, T);
+    const size_t small = small_workspace(mats, n, T);
+    return masked_gemm(mats, n, T) ? std::max(small, gemm_workspace_beyond_small(mats, n, T)) : small;
+}
+
+static size_t gemm_workspace_beyond_small(const sq_matrix* mats, int n, int T) {
     if (T > SQ_SMALL_BMAX && T <= small_pass_limit(mats, n)) {
         // full passes and the last, shorter one may run different kernels with different needs
         const size_t full = small_workspace(mats, n, SQ_SMALL_BMAX);
@@ -265,6 +276,8 @@ int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, con
 
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                 int64_t ldy, int T, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s) {
+    if (T <= SQ_SMALL_BMAX && !small_takes_gemm_route(mats, n, T, x, ldx))
+        return launch_small(mats, n, x, x_dtype, ldx, y, y_dtype, ldy, T, ws, ws_bytes, counters, s);
     if (T > SQ_SMALL_BMAX && T <= small_pass_limit(mats, n) && x_vec_ok(x, ldx, mats[0].C)) {
         // a few passes of the decode-time kernel read the packed tags a few times; decoding to fp16 first
         // (below) writes and reads 8 to 16 times as many bytes once

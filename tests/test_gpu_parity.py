@@ -316,6 +316,30 @@ def test_gemm_matches_oracle(case, dtype):
     _check_lowp(y, ref)
 
 
+def test_gemm_entry_point_with_few_rows_is_the_decode_path():
+    # up to 32 activation rows sq_linear_gemm runs sq_linear_small's kernels: identical bits; a stack with column
+    # orders switches to decode + tile GEMM at 11 rows through either entry point
+    from quantexperiments_amd.kernels import linear_gemm, linear_small
+    plain, masked = synth(200, 1280, 4, 12, seed=7), synth(96, 256, 8, 16, 1, 4, seed=8)
+    lp, lm = to_device(plain), to_device(masked)
+    for T in (1, 5, 32):
+        x = rand_x(T, 1280, torch.bfloat16, seed=T).cuda()
+        ya, yb = torch.empty(T, 200, dtype=torch.float32, device="cuda"), torch.empty(T, 200, dtype=torch.float32, device="cuda")
+        linear_gemm([lp], x, ya)
+        linear_small([lp], x, yb)
+        assert torch.equal(ya, yb)
+    for T in (4, 10, 11, 32):
+        x = rand_x(T, 256, torch.bfloat16, seed=T)
+        ya, yb = torch.empty(T, 96, dtype=torch.float32, device="cuda"), torch.empty(T, 96, dtype=torch.float32, device="cuda")
+        linear_gemm([lm], x.cuda(), ya)
+        linear_small([lm], x.cuda(), yb)
+        assert torch.equal(ya, yb) and rel_max_err(ya.cpu().numpy(), _ref(masked, x)) < TOL
+        xo = torch.zeros(T, 256 + 8, dtype=torch.bfloat16, device="cuda")[:, 3:259]   # x that is not 16-byte aligned
+        xo.copy_(x)
+        linear_small([lm], xo, yb)
+        assert rel_max_err(yb.cpu().numpy(), _ref(masked, x)) < TOL
+
+
 def test_gemm_dense_matches_float64():
     from quantexperiments_amd.kernels import gemm_dense
     g = torch.Generator().manual_seed(5)
