@@ -181,23 +181,23 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_kernel(Q8Args a) {
     }
 }
 
-// ---- 5 .. Q8_MFMA_MAX_ROWS activation rows: fp16 MFMA, 32 activation rows per pass.
-// v_mfma_f32_32x32x16_f16 operand layout, lane l: A row / B column l % 32, k = 8 * (l / 32) .. + 7; result register
-// jj of lane l is D[(jj / 4) * 8 + (l / 32) * 4 + jj % 4][l % 32].  Weights are the A operand, loaded straight into
-// registers: a wave owns 32 rows, and per step of 128 columns lane (r, h) takes 16 bytes of row r at column
-// 128 s + 32 j + 16 h for j = 0..3, issued back to back, so the two lanes of a row consume a whole 128-byte line
-// while it is in flight.  Each 16-byte piece feeds two MFMAs; the k index of MFMA m of piece j is column
-// 128 s + 32 j + 16 h + 8 m + e, and the activations (B operand) are read with the same mapping from LDS, where
-// the workgroup keeps the current 256-column chunk of the fp16 activations (global_load_lds, double buffered).
-// One wave alone moves only 5 GB/s (latency), so the design is many small waves: one 32-row block each, <= 128
-// registers, 16 waves per CU, two steps of loads in flight each.  What is left between this kernel (4 TB/s) and
-// the 4-row kernel (5.7 TB/s) is the address pattern the MFMA operand layout forces on direct loads: the 16
-// lanes of a quarter wave always belong to 16 different weight rows, i.e. 16 cache lines per quarter wave.
-// The block scale is folded into the fp16 weight (one rounding, as the reference's tile kernel does,
+// ---- 5 .. Q8_MFMA_MAX_ROWS activation rows, 3 and 4 too when C % 1024 != 0 (C % 256 == 0): fp16 MFMA, 32 activation rows per pass.
+// v_mfma_f32_16x16x32_f16 operand layout: A: lane l supplies weight row l % 16, k = 8 * (l / 16) .. + 7; B: token
+// l % 16, the same k; D: lane l holds token l % 16, weight rows 4 * (l / 16) .. + 3.  Weights are the A operand,
+// loaded straight into registers: a wave owns 16 rows, and per step of 128 columns lane (r, g) takes 16 bytes of
+// row r at column 128 s + 64 j + 16 g for j = 0, 1, issued back to back, so the four lanes of a row consume a whole
+// 128-byte line while it is in flight.  Each 16-byte piece feeds two MFMAs per block of 16 tokens; the k index of
+// MFMA m of piece j is column 128 s + 64 j + 16 g + 8 m + e, and the activations (B operand) are read with the
+// same mapping from LDS, where a workgroup of 8 waves (128 rows) keeps the current 256-column chunk of the fp16
+// activations (global_load_lds, double buffered).  One wave alone moves only 5 GB/s (latency), so the design is
+// many small waves: 16 rows and < 80 registers each, 24 waves per CU, two steps of loads in flight each.  What is
+// left between this kernel (4.1-4.4 TB/s) and the 4-row kernel (5.7 TB/s) is mostly the address pattern the MFMA
+// operand layout forces on direct loads (the 16 lanes of a quarter wave belong to 16 different weight rows); a
+// first version with 32 rows per wave on the 32x32x16 instruction (32 bytes per row and instruction) was 7 %
+// slower.  The block scale is folded into the fp16 weight (one rounding, as the reference's tile kernel does,
 // shapequant/kernels/batched_runs.py:442-447): all 8 weights a lane feeds to one MFMA sit in one block.
 constexpr int Q8_MFMA_MAX_ROWS = 128;           // up to here passes of 32 beat decode + tile GEMM
 constexpr int Q8_XC = 256;                      // columns of x per LDS chunk (2 steps)
-constexpr int Q8_RING = 2;                      // steps of weight loads in flight per wave (2 or 4; measured equal)
 
 // x [B, C] (fp16 or bf16, any stride) -> fp16 [B, C] contiguous.
 __global__ __launch_bounds__(256) void q8_x_kernel(const uint16_t* __restrict__ x, int64_t ldx, int B, int C, int x_dtype,
@@ -223,136 +223,115 @@ struct Q8MfmaArgs {
 
 constexpr int q8_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }   // wait on vmcnt only
 
-template <int RING>
-__global__ __launch_bounds__(256, RING == 2 ? 4 : 3) void q8_mfma_kernel(Q8MfmaArgs a) {
-    // x chunk in LDS: [32 activation rows][32 pieces of 16 bytes], piece p of row n stored in slot p ^ (n & 15),
-    // so the 16 lanes of a ds_read_b128 (16 different rows, same piece) hit 16 different bank groups
+template <int NBLK>     // 16-token blocks: 1 (up to 16 activation rows) or 2
+__global__ __launch_bounds__(512, 2) void q8_mfma_kernel(Q8MfmaArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char xs[2][32 * Q8_XC * 2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int task_raw = blockIdx.x * 4 + wave;
-    const bool active = task_raw < a.tasks;                 // idle waves still copy x and meet the barriers
+    const int task_raw = blockIdx.x * 8 + wave;
+    const bool active = task_raw < a.tasks;
     const int task = active ? task_raw : a.tasks - 1;
-    const int r = lane & 31, h = lane >> 5;
-    const int C = a.C, nblk = C >> 5, nsteps = C >> 7;      // C % 256 == 0: an even number of 128-column steps
-    const int nchunks = nsteps >> 1;
-    const int row = min(task * 32 + r, a.V - 1);
-    const int8_t* wp = a.q + (int64_t)row * C + h * 16;
+    const int r = lane & 15, g = lane >> 4;
+    const int C = a.C, nblk = C >> 5, nsteps = C >> 7, nchunks = nsteps >> 1;
+    const int row = min(task * 16 + r, a.V - 1);
+    const int8_t* wp = a.q + (int64_t)row * C + g * 16;
     const char* sp = (const char*)(a.sc + (int64_t)row * nblk);
 
-    // x copies: one instruction moves 1 KB = two activation rows of the chunk; wave w brings rows 8 w .. 8 w + 7.
-    // The lane that lands in slot (lane & 31) of its row fetches the piece the swizzle puts there.
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    uint32_t xsrc[4];
+    uint32_t xsrc[2];                           // wave w copies activation rows 4 w .. 4 w + 3, two per instruction
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int rowx = wave * 8 + 2 * i + h;
+    for (int i = 0; i < 2; ++i) {
+        const int rowx = wave * 4 + 2 * i + (lane >> 5);
         const int piece = (lane & 31) ^ (rowx & 15);
-        xsrc[i] = (uint32_t)(min(rowx, a.B - 1) * a.ldxh + piece * 8);    // halves
+        xsrc[i] = (uint32_t)(min(rowx, a.B - 1) * a.ldxh + piece * 8);
     }
     auto copy_x = [&](int c) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 2; ++i)
             __builtin_amdgcn_global_load_lds((gptr_t)(a.xh + c * Q8_XC + xsrc[i]),
-                                             (lptr_t)(&xs[c & 1][(wave * 8 + 2 * i) * (Q8_XC * 2)]), 16, 0, 0);
+                                             (lptr_t)(&xs[c & 1][(wave * 4 + 2 * i) * (Q8_XC * 2)]), 16, 0, 0);
     };
-    const uint32_t xrow = (uint32_t)r * (Q8_XC * 2), xsw = (uint32_t)(r & 15);
+    const uint32_t xrow = (uint32_t)r * (Q8_XC * 2), xsw = (uint32_t)r;
+    const uint32_t sshift = (uint32_t)(g >> 1) << 4;        // which half of a scale pair this lane's pieces use
 
-    float16v acc;
+    float4v acc[NBLK];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) acc[k] = 0.f;
-
-    u32x4 wr[RING][4];
-    u32x2 sr[RING];
+    for (int nb = 0; nb < NBLK; ++nb) acc[nb] = float4v{0.f, 0.f, 0.f, 0.f};
+    u32x4 wr[2][2];
+    u32x2 sr[2];
     copy_x(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int p = 0; p < RING; ++p) {
-        const int sp_ = p < nsteps ? p : nsteps - 1;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) wr[p][j] = *reinterpret_cast<const u32x4*>(wp + sp_ * 128 + j * 32);
-        sr[p] = *reinterpret_cast<const u32x2*>(sp + sp_ * 8);
+    for (int p = 0; p < 2; ++p) {
+        const int s0 = p < nsteps ? p : nsteps - 1;
+        wr[p][0] = *reinterpret_cast<const u32x4*>(wp + s0 * 128);
+        wr[p][1] = *reinterpret_cast<const u32x4*>(wp + s0 * 128 + 64);
+        sr[p] = *reinterpret_cast<const u32x2*>(sp + s0 * 8);
     }
-    for (int c0 = 0; c0 < nchunks; c0 += 2) {
+    for (int c = 0; c < nchunks; ++c) {
+        // chunk c was requested one chunk ago, before the 6 loads of that chunk's two refills
+        if (c == 0 || c == nchunks - 1) __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
+        else __builtin_amdgcn_s_waitcnt(q8_vmcnt(6));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if (c + 1 < nchunks) copy_x(c + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned char* xc = &xs[c & 1][0] + xrow;
 #pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-            const int c = c0 + cc;
-            if (c < nchunks) {
-                // chunk c was requested one chunk ago, before the 10 loads of that chunk's two refills; the
-                // first chunk (prologue) and the last one (no refills left) wait for everything
-                if (c == 0 || c == nchunks - 1) __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
-                else __builtin_amdgcn_s_waitcnt(q8_vmcnt(10));
-                __builtin_amdgcn_s_barrier();
-                __builtin_amdgcn_sched_barrier(0);
-                if (c + 1 < nchunks) copy_x(c + 1);
-                __builtin_amdgcn_sched_barrier(0);
-                const unsigned char* xc = &xs[cc][0] + xrow;
+        for (int sl = 0; sl < 2; ++sl) {
+            const int s = c * 2 + sl;
 #pragma unroll
-                for (int sl = 0; sl < 2; ++sl) {
-                    const int slot = (cc * 2 + sl) % RING;
-                    const int s = c * 2 + sl;
+            for (int j = 0; j < 2; ++j) {
+                const half_t sh = __builtin_bit_cast(half_t, (uint16_t)(sr[sl][j] >> sshift));
+                const half2v s2 = {sh, sh};
+                half2v p[8];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint32_t spair = sr[slot][j >> 1];
-                        const uint16_t sbits = (j & 1) ? (uint16_t)(spair >> 16) : (uint16_t)(spair & 0xFFFFu);
-                        const half_t sh = __builtin_bit_cast(half_t, sbits);
-                        const half2v s2 = {sh, sh};
-                        half2v p[8];
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t wk = wr[sl][j][k];
+                    i8x4_to_h2(wk, p[2 * k], p[2 * k + 1]);
+                }
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            const uint32_t wk = wr[slot][j][k];
-                            i8x4_to_h2(wk, p[2 * k], p[2 * k + 1]);
-                        }
+                for (int k = 0; k < 8; ++k) p[k] = p[k] * s2;
+                half8v a0, a1;
 #pragma unroll
-                        for (int k = 0; k < 8; ++k) p[k] = p[k] * s2;
-                        half8v a0, a1;
+                for (int k = 0; k < 4; ++k) {
+                    a0[2 * k] = p[k][0]; a0[2 * k + 1] = p[k][1];
+                    a1[2 * k] = p[4 + k][0]; a1[2 * k + 1] = p[4 + k][1];
+                }
+                const uint32_t p0 = (uint32_t)(sl * 16 + j * 8 + g * 2);      // pieces p0, p0 + 1 of the token's row
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            a0[2 * k] = p[k][0]; a0[2 * k + 1] = p[k][1];
-                            a1[2 * k] = p[4 + k][0]; a1[2 * k + 1] = p[4 + k][1];
-                        }
-                        // pieces sl * 16 + j * 4 + h * 2 + m of this lane's activation row
-                        const uint32_t p0 = (uint32_t)(sl * 16 + j * 4 + h * 2);
-                        const half8v x0 = *reinterpret_cast<const half8v*>(xc + ((p0 ^ xsw) << 4));
-                        const half8v x1 = *reinterpret_cast<const half8v*>(xc + (((p0 + 1) ^ xsw) << 4));
-                        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, x0, acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, x1, acc, 0, 0, 0);
-                    }
-                    // the slot is free: refill it RING steps ahead
-                    if (s + RING < nsteps) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            wr[slot][j] = *reinterpret_cast<const u32x4*>(wp + (s + RING) * 128 + j * 32);
-                        sr[slot] = *reinterpret_cast<const u32x2*>(sp + (s + RING) * 8);
-                    }
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    const unsigned char* xt = xc + nb * (16 * Q8_XC * 2);
+                    const half8v x0 = *reinterpret_cast<const half8v*>(xt + ((p0 ^ xsw) << 4));
+                    const half8v x1 = *reinterpret_cast<const half8v*>(xt + (((p0 + 1) ^ xsw) << 4));
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, x0, acc[nb], 0, 0, 0);
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, x1, acc[nb], 0, 0, 0);
                 }
             }
-        }
-    }
-    if (!active || r >= a.B) return;
-    // a lane holds 4 x 4 consecutive weight rows of activation row r: 8-byte stores of 16-bit results when aligned
-    if (a.vec_y && a.y_dtype != SQ_F32) {
-        uint16_t* yb = reinterpret_cast<uint16_t*>(a.y) + (int64_t)r * a.ldy;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int orow = task * 32 + g * 8 + h * 4;
-            uint16_t o[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = a.y_dtype == SQ_BF16 ? f2bf(acc[4 * g + e]) : f2h(acc[4 * g + e]);
-            if (orow + 4 <= a.V) {
-                *reinterpret_cast<u32x2*>(yb + orow) = u32x2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (orow + e < a.V) yb[orow + e] = o[e];
+            if (s + 2 < nsteps) {
+                wr[sl][0] = *reinterpret_cast<const u32x4*>(wp + (s + 2) * 128);
+                wr[sl][1] = *reinterpret_cast<const u32x4*>(wp + (s + 2) * 128 + 64);
+                sr[sl] = *reinterpret_cast<const u32x2*>(sp + (s + 2) * 8);
             }
         }
-        return;
     }
+    if (!active) return;
+    const int orow = task * 16 + g * 4;
 #pragma unroll
-    for (int jj = 0; jj < 16; ++jj) {
-        const int orow = task * 32 + (jj >> 2) * 8 + h * 4 + (jj & 3);
-        if (orow < a.V) store_y(a.y, a.y_dtype, (int64_t)r * a.ldy + orow, acc[jj]);
+    for (int nb = 0; nb < NBLK; ++nb) {
+        const int tok = nb * 16 + r;
+        if (tok >= a.B) continue;
+        if (a.vec_y && a.y_dtype != SQ_F32 && orow + 4 <= a.V) {
+            uint16_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = a.y_dtype == SQ_BF16 ? f2bf(acc[nb][e]) : f2h(acc[nb][e]);
+            *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(a.y) + (int64_t)tok * a.ldy + orow) =
+                u32x2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (orow + e < a.V) store_y(a.y, a.y_dtype, (int64_t)tok * a.ldy + orow + e, acc[nb][e]);
+        }
     }
 }
 
@@ -444,7 +423,11 @@ static int q8_pass_rows(int B, int C) {
 // 32-bit offsets.
 static bool q8_mfma_ok(int C) { return C % 256 == 0 && (int64_t)C * 32 < ((int64_t)1 << 31); }
 
-bool q8_mid(int C, int B) { return B > 4 && B <= Q8_MFMA_MAX_ROWS && q8_mfma_ok(C); }
+// 3 and 4 rows: the 4-row kernel walks a row in 1 KB steps and is VALU-bound there, so it wins when C fills its last
+// step (248,320 x 5,120: 255 us against 312 us on the MFMA passes) and loses otherwise (152,064 x 3,584: 148 against 131)
+bool q8_mid(int C, int B) {
+    return B <= Q8_MFMA_MAX_ROWS && q8_mfma_ok(C) && (B > 4 || (B > 2 && C % 1024 != 0));
+}
 
 size_t q8_mid_workspace(int C, int B) { return q8_mid(C, B) ? (((size_t)B * C * 2) + 255) & ~(size_t)255 : 0; }
 
@@ -467,7 +450,7 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
         xh = (const uint16_t*)ws;
         ldxh = C;
     }
-    const int tasks = (V + 31) / 32;
+    const int tasks = (V + 15) / 16;
     for (int b0 = 0; b0 < B; b0 += 32) {
         Q8MfmaArgs a{};
         a.q = q; a.sc = sc;
@@ -476,7 +459,8 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
         a.y = (char*)y + (size_t)b0 * ldy * ys;
         a.ldy = ldy; a.V = V; a.C = C; a.B = B - b0 < 32 ? B - b0 : 32; a.y_dtype = y_dtype; a.tasks = tasks;
         a.vec_y = ((uintptr_t)a.y & 7) == 0 && ldy % 4 == 0;
-        hipLaunchKernelGGL(q8_mfma_kernel<Q8_RING>, dim3((unsigned)((tasks + 3) / 4)), dim3(256), 0, s, a);
+        if (a.B > 16) hipLaunchKernelGGL(q8_mfma_kernel<2>, dim3((unsigned)((tasks + 7) / 8)), dim3(512), 0, s, a);
+        else hipLaunchKernelGGL(q8_mfma_kernel<1>, dim3((unsigned)((tasks + 7) / 8)), dim3(512), 0, s, a);
         rc = check_launch("q8_mfma_kernel");
         if (rc) return rc;
     }

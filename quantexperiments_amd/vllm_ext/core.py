@@ -232,7 +232,7 @@ class Q8Head:
     (reference shapequant/vllm_ext/core.py:489-591, same constructor, attributes and forward / R interface
     as PackedShards, so it runs through the shapequant::linear op).
 
-      M <= small_max: sq_q8_linear streams the int8 rows once per four activation rows, straight into y;
+      M <= small_max: sq_q8_linear streams the int8 rows once per 32 activation rows, straight into y;
       M >  small_max: row chunks decoded to fp16 and multiplied by the tile GEMM (sq_q8_linear's second route).
 
     The kernels read the file's natural layout at full cache-line width, so no tile-major copy is made:
