@@ -165,6 +165,27 @@ int sq_q8_dequant(const int8_t* q, const uint16_t* scale, int32_t V, int32_t C, 
 int sq_q4_embed(const uint8_t* q, const uint16_t* scale, int32_t V, int32_t C, const int64_t* ids, int64_t n_ids, void* out,
                 int out_dtype, int64_t ld_out, void* stream);
 
+/* ---- The elementwise neighbours of the decode-time products ----
+ *
+ * sq_addnorm: residual add + RMS norm that writes the next product's input, for B activation rows:
+ *     v[b, i]      = h_in[b * ld_h + i] + add[b * ld_add + i]            (fp32; add may be NULL)
+ *     h_out[b, i]  = v[b, i]                                            (h_out may be NULL, or h_in when perms is NULL)
+ *     act[b, i]    = round(v[b, i] * rsqrt(mean_i(v[b, i]^2) + eps) * w[i])   to out_dtype (SQ_F16 / SQ_BF16)
+ *     out[(b * M + m) * C + i] = act[b, perms[m * C + i]]                (perms NULL: M = 1 and the identity)
+ * It replaces addnorm_perm (reference shapequant/kernels/decode_e2e.py:84-108) and the EPI 1 epilogue of gemv_runs
+ * (shapequant/kernels/proto_runs.py:223-268).  perms are a piece's column orders (sq_matrix.perms); the products of
+ * this library read x through them themselves, so callers inside it pass NULL.  With perms C <= 32256.
+ *
+ * sq_silu_mul: out = silu(gate) * up, SiLU in fp32 rounded to `dtype`, the product rounded to `dtype` (the model
+ * code's arithmetic), gate / up / out all of `dtype`, rows b at gate + b * ld and up + b * ld (gate | up of one
+ * stacked product: up = gate + C, ld = 2 C), out[(b * M + m) * C + i] as above.  It replaces silu_mul_perm
+ * (reference shapequant/kernels/decode_e2e.py:125-136) and the EPI 2 epilogue (proto_runs.py:269-276). */
+int sq_addnorm(const float* h_in, float* h_out, int64_t ld_h, const void* add, int add_dtype, int64_t ld_add, const void* w,
+               int w_dtype, const int32_t* perms, int32_t M, int32_t B, int32_t C, float eps, void* out, int out_dtype,
+               void* stream);
+int sq_silu_mul(const void* gate, const void* up, int dtype, int64_t ld, const int32_t* perms, int32_t M, int32_t B, int32_t C,
+                void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -21,6 +21,8 @@ multi-threaded baseline), the arithmetic of the reference's CPU path:
   q8_pack                    shapequant/kernels/proto_formats.py:464-471   8-bit block-32 head
   q8_rows                    shapequant/packed.py:155-158
   q8_linear                  shapequant/kernels/batched_runs.py:376-440 (per-block sum times block scale)
+  addnorm                    shapequant/kernels/decode_e2e.py:84-108 (addnorm_perm), proto_runs.py:246-268 (EPI 1)
+  silu_mul                   shapequant/kernels/decode_e2e.py:125-136 (silu_mul_perm), proto_runs.py:269-276 (EPI 2)
 
 Pinning status (what fixes each function besides this file's own formula):
   pack_bits/unpack_bits  known-answer layout vectors of the reference's tests, closed forms for
@@ -38,6 +40,11 @@ Pinning status (what fixes each function besides this file's own formula):
                          scale/2 that any correct round-to-nearest block quantizer meets.
   q4_embed_rows/q8_rows  the same known-answer blocks decoded back, pure-Python loops on small inputs.
   q8_linear              float64 dense product of q8_rows (the two must agree to fp32 rounding).
+  addnorm                torch.nn.functional.rms_norm on the same fp32 residual, closed forms (a constant row
+                         normalises to its sign times w, scaling the row by 2 changes nothing at eps = 0),
+                         the copies by a double loop over (m, i).
+  silu_mul               torch.nn.functional.silu and scipy.special.expit, fixed points (0, large |a|), the
+                         rounding points by hand-picked fp16 values whose product is not representable.
 """
 
 from __future__ import annotations
@@ -312,3 +319,41 @@ def q8_linear(x, q, sc, acc=np.float64) -> np.ndarray:
     V, C = q.shape
     part = np.einsum("bkc,vkc->bvk", x.reshape(x.shape[0], C // 32, 32), q.reshape(V, C // 32, 32))
     return (part * np.asarray(sc).astype(acc)[None]).sum(-1)
+
+
+# ----------------------------------------------------------------------------- elementwise neighbours
+
+def _round16(v, dtype: str) -> np.ndarray:
+    if dtype == "bf16":
+        return round_bf16(v)
+    if dtype == "fp16":
+        return round_fp16(v)
+    raise ValueError(dtype)
+
+
+def _copies(act, perms) -> np.ndarray:
+    """out[b, m, i] = act[b, perms[m, i]]; perms None: one copy in natural order."""
+    if perms is None:
+        return act[:, None, :]
+    return act[:, np.asarray(perms, dtype=np.int64)]
+
+
+def addnorm(h_in, add, w, eps: float, perms=None, dtype: str = "fp16"):
+    """v = h_in + add in fp32 (add may be None); h_out = v; act = round(v * rsqrt(mean(v^2) + eps) * w) to `dtype`;
+    returns (h_out [B, C] fp32, out [B, M, C] with the values of `dtype` held in fp32).  The mean is taken in
+    float64 and the factor rounded to fp32 once, where the GPU sums in fp32: the two differ by an ulp of fp32 at
+    most, i.e. by one rounding step of `dtype` on rare ties."""
+    v = np.atleast_2d(np.asarray(h_in, dtype=np.float32))
+    if add is not None:
+        v = v + np.atleast_2d(np.asarray(add, dtype=np.float32))
+    rstd = (1.0 / np.sqrt((v.astype(np.float64) ** 2).mean(-1, keepdims=True) + np.float64(np.float32(eps)))).astype(np.float32)
+    act = _round16((v * rstd) * np.asarray(w, dtype=np.float32)[None], dtype)
+    return v, _copies(act, perms)
+
+
+def silu_mul(gate, up, perms=None, dtype: str = "fp16") -> np.ndarray:
+    """out = round(round(silu(gate)) * up), both roundings to `dtype`; [B, M, C]."""
+    g = np.atleast_2d(np.asarray(gate, dtype=np.float32)).astype(np.float64)
+    s = _round16((g / (1.0 + np.exp(-g))).astype(np.float32), dtype)
+    act = _round16(s * np.atleast_2d(np.asarray(up, dtype=np.float32)), dtype)
+    return _copies(act, perms)

@@ -65,8 +65,11 @@ def lib() -> ctypes.CDLL:
         L.sq_q8_workspace_bytes.restype = sz
         L.sq_q8_dequant.argtypes = [vp, vp, i32, i32, vp, ctypes.c_int, i64, i32, i32, vp]
         L.sq_q4_embed.argtypes = [vp, vp, i32, i32, vp, i64, vp, ctypes.c_int, i64, vp]
+        L.sq_addnorm.argtypes = [vp, vp, i64, vp, ctypes.c_int, i64, vp, ctypes.c_int, vp, i32, i32, i32, ctypes.c_float, vp,
+                                 ctypes.c_int, vp]
+        L.sq_silu_mul.argtypes = [vp, vp, ctypes.c_int, i64, vp, i32, i32, i32, vp, vp]
         for f in (L.sq_dequant, L.sq_linear_small, L.sq_linear_gemm, L.sq_gemm_dense, L.sq_q8_linear, L.sq_q8_dequant,
-                  L.sq_q4_embed):
+                  L.sq_q4_embed, L.sq_addnorm, L.sq_silu_mul):
             f.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -74,7 +77,7 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
            "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build", "sq_q8_linear", "sq_q8_workspace_bytes",
-           "sq_q8_dequant", "sq_q4_embed")
+           "sq_q8_dequant", "sq_q4_embed", "sq_addnorm", "sq_silu_mul")
 
 
 def check(rc: int) -> None:

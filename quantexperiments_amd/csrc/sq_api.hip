@@ -74,7 +74,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 102; }
+int sq_version(void) { return 103; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -209,6 +209,33 @@ int sq_q4_embed(const uint8_t* q, const uint16_t* scale, int32_t V, int32_t C, c
     if (!ids || !out || ld_out < C) return fail(SQ_EINVAL, "sq_q4_embed: ids %p out %p ld_out %lld", (const void*)ids, out, (long long)ld_out);
     if ((uintptr_t)ids & 7) return fail(SQ_EINVAL, "sq_q4_embed: ids must be 8-byte aligned");
     return launch_q4_embed(q, scale, V, C, ids, n_ids, out, out_dtype, ld_out, (hipStream_t)stream);
+}
+
+static bool is16(int dt) { return dt == SQ_F16 || dt == SQ_BF16; }
+
+int sq_addnorm(const float* h_in, float* h_out, int64_t ld_h, const void* add, int add_dtype, int64_t ld_add, const void* w,
+               int w_dtype, const int32_t* perms, int32_t M, int32_t B, int32_t C, float eps, void* out, int out_dtype,
+               void* stream) {
+    if (B < 0 || C <= 0) return fail(SQ_EINVAL, "sq_addnorm: B %d C %d", B, C);
+    if (!is16(w_dtype) || !is16(out_dtype) || (add && !is16(add_dtype)))
+        return fail(SQ_EINVAL, "sq_addnorm: add / w / out must be fp16 or bf16 (%d / %d / %d)", add_dtype, w_dtype, out_dtype);
+    if (perms && M <= 0) return fail(SQ_EINVAL, "sq_addnorm: %d column orders", M);
+    if (B == 0) return SQ_OK;
+    if (!h_in || !w || !out) return fail(SQ_EINVAL, "sq_addnorm: null h_in / w / out");
+    if (B > 1 && (ld_h < C || (add && ld_add < C))) return fail(SQ_EINVAL, "sq_addnorm: ld_h %lld / ld_add %lld too small", (long long)ld_h, (long long)ld_add);
+    if (perms && h_out == h_in) return fail(SQ_EINVAL, "sq_addnorm: with column orders h_out must not be h_in");
+    return launch_addnorm(h_in, h_out, ld_h, add, add_dtype, ld_add, w, w_dtype, perms, M, B, C, eps, out, out_dtype, (hipStream_t)stream);
+}
+
+int sq_silu_mul(const void* gate, const void* up, int dtype, int64_t ld, const int32_t* perms, int32_t M, int32_t B, int32_t C,
+                void* out, void* stream) {
+    if (B < 0 || C <= 0) return fail(SQ_EINVAL, "sq_silu_mul: B %d C %d", B, C);
+    if (!is16(dtype)) return fail(SQ_EINVAL, "sq_silu_mul: dtype %d", dtype);
+    if (perms && M <= 0) return fail(SQ_EINVAL, "sq_silu_mul: %d column orders", M);
+    if (B == 0) return SQ_OK;
+    if (!gate || !up || !out) return fail(SQ_EINVAL, "sq_silu_mul: null gate / up / out");
+    if (B > 1 && ld < C) return fail(SQ_EINVAL, "sq_silu_mul: ld %lld too small", (long long)ld);
+    return launch_silu_mul(gate, up, dtype, ld, perms, M, B, C, out, (hipStream_t)stream);
 }
 
 }  // extern "C"

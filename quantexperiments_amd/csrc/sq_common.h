@@ -115,4 +115,10 @@ int launch_q8_dequant(const int8_t* q, const uint16_t* sc, int C, void* out, int
 int launch_q4_embed(const uint8_t* q, const uint16_t* sc, int V, int C, const int64_t* ids, int64_t n_ids, void* out,
                     int out_dtype, int64_t ld_out, hipStream_t s);
 
+// elementwise neighbours of the decode-time products (sq_neighbours.hip)
+int launch_addnorm(const float* h_in, float* h_out, int64_t ld_h, const void* add, int add_dtype, int64_t ld_add, const void* w,
+                   int w_dtype, const int32_t* perms, int M, int B, int C, float eps, void* out, int out_dtype, hipStream_t s);
+int launch_silu_mul(const void* gate, const void* up, int dtype, int64_t ld, const int32_t* perms, int M, int B, int C, void* out,
+                    hipStream_t s);
+
 }  // namespace sq

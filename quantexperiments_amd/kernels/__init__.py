@@ -313,3 +313,58 @@ def q4_rows(q: torch.Tensor, sc: torch.Tensor, ids: torch.Tensor, dtype: torch.d
         _lib.check(_lib.lib().sq_q4_embed(q.data_ptr(), sc.data_ptr(), V, C, ids.data_ptr(), ids.shape[0], out.data_ptr(),
                                           _lib.DTYPES[dtype], C, _lib.stream_ptr(dev)))
     return out
+
+
+# ------------------------------------------------------------------ elementwise neighbours of the decode-time products
+
+def _perm_args(perms, C: int, dev, who: str):
+    if perms is None:
+        return 0, 1
+    if perms.dtype != torch.int32 or perms.dim() != 2 or perms.shape[1] != C or not perms.is_contiguous() or perms.device != dev:
+        raise ValueError(f"{who}: perms must be a contiguous int32 [M, {C}] tensor on {dev}")
+    return perms.data_ptr(), perms.shape[0]
+
+
+def addnorm(h_in: torch.Tensor, add, w: torch.Tensor, eps: float, out: torch.Tensor, h_out=None, perms=None) -> torch.Tensor:
+    """Residual add + RMS norm for the next product (sq_addnorm): h_in fp32 [B, C], add fp16 / bf16 [B, C] or None,
+    w fp16 / bf16 [C]; writes out [B, C] (or [B, M, C] with int32 column orders perms [M, C]) in its dtype and, if
+    given, h_out fp32 [B, C] = h_in + add (may be h_in when perms is None).  The reference's addnorm_perm
+    (shapequant/kernels/decode_e2e.py:84-108)."""
+    dev = h_in.device
+    if h_in.dtype != torch.float32 or h_in.dim() != 2 or h_in.stride(1) != 1:
+        raise ValueError("addnorm: h_in must be fp32 [B, C] with unit column stride")
+    B, C = h_in.shape
+    pp, M = _perm_args(perms, C, dev, "addnorm")
+    if out.dtype not in _lib.DTYPES or out.dtype == torch.float32 or not out.is_contiguous() or out.numel() != B * M * C:
+        raise ValueError("addnorm: out must be a contiguous fp16 / bf16 tensor of B * M * C elements")
+    if w.dtype == torch.float32 or w.dtype not in _lib.DTYPES or w.numel() != C or not w.is_contiguous():
+        raise ValueError("addnorm: w must be a contiguous fp16 / bf16 [C]")
+    if add is not None and (add.dtype == torch.float32 or add.dtype not in _lib.DTYPES or add.shape != h_in.shape or add.stride(1) != 1):
+        raise ValueError("addnorm: add must be fp16 / bf16 [B, C] with unit column stride")
+    if h_out is not None and (h_out.dtype != torch.float32 or h_out.shape != h_in.shape or h_out.stride() != h_in.stride()):
+        raise ValueError("addnorm: h_out must match h_in")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().sq_addnorm(h_in.data_ptr(), 0 if h_out is None else h_out.data_ptr(), h_in.stride(0),
+                                         0 if add is None else add.data_ptr(), _lib.DTYPES[add.dtype] if add is not None else 0,
+                                         add.stride(0) if add is not None else 0, w.data_ptr(), _lib.DTYPES[w.dtype], pp, M, B, C,
+                                         float(eps), out.data_ptr(), _lib.DTYPES[out.dtype], _lib.stream_ptr(dev)))
+    return out
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, perms=None) -> torch.Tensor:
+    """out = silu(gate) * up in the tensors' dtype (sq_silu_mul): gate / up fp16 or bf16 [B, C] with the same row
+    stride (the two halves of a stacked gate | up output), out [B, C] or [B, M, C] with column orders.  The
+    reference's silu_mul_perm (shapequant/kernels/decode_e2e.py:125-136)."""
+    dev = gate.device
+    if gate.dtype == torch.float32 or gate.dtype not in _lib.DTYPES or gate.dim() != 2 or gate.stride(1) != 1:
+        raise ValueError("silu_mul: gate must be fp16 / bf16 [B, C] with unit column stride")
+    if up.dtype != gate.dtype or up.shape != gate.shape or up.stride() != gate.stride():
+        raise ValueError("silu_mul: up must match gate in dtype, shape and strides")
+    B, C = gate.shape
+    pp, M = _perm_args(perms, C, dev, "silu_mul")
+    if out.dtype != gate.dtype or not out.is_contiguous() or out.numel() != B * M * C:
+        raise ValueError("silu_mul: out must be a contiguous tensor of gate's dtype with B * M * C elements")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().sq_silu_mul(gate.data_ptr(), up.data_ptr(), _lib.DTYPES[gate.dtype], gate.stride(0), pp, M, B, C,
+                                          out.data_ptr(), _lib.stream_ptr(dev)))
+    return out

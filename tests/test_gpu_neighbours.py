@@ -1,0 +1,170 @@
+"""GPU parity of the elementwise neighbours of the decode-time products (residual add + RMS norm, SiLU * up),
+called through the C ABI, against the CPU oracle.  The residual is bit-exact (one fp32 add).  The normalised
+output and the SiLU product may differ from the oracle by one rounding step of the 16-bit output type where the
+value sits on a tie: the GPU sums squares in fp32 and uses the hardware exponential, the oracle float64; such
+entries must be rare.  Column-order copies are exact gathers of the natural-order result.  Shapes follow the
+reference's decode engine (hidden 896 / 3584 / 5120, intermediate 18944, M = 1 and M = 16 column orders;
+reference tests/test_decode_e2e.py:203-226 checks its epilogues against these same separate kernels)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sq_oracle as O
+from tests.helpers import rand_x
+
+pytestmark = pytest.mark.gpu
+NAMES = {torch.float16: "fp16", torch.bfloat16: "bf16"}
+
+
+def _one_step(got: np.ndarray, ref: np.ndarray, dtype, rare=0.01):
+    step = np.abs(ref) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10) + (0 if dtype == torch.bfloat16 else 2.0 ** -24)
+    d = np.abs(got.astype(np.float64) - ref)
+    assert np.all(d <= step * 1.001), float((d / np.maximum(step, 1e-30)).max())
+    assert (d > 0).mean() <= rare, float((d > 0).mean())
+
+
+def _perms(M, C, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.stack([torch.randperm(C, generator=g) for _ in range(M)]).to(torch.int32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("B,C,M", [(1, 3584, 0), (1, 896, 0), (3, 5120, 0), (32, 64, 0), (1, 3584, 16), (2, 896, 4), (1, 100, 3),
+                                   (1, 18944, 16), (5, 1, 0)])
+def test_addnorm_matches_oracle(B, C, M, dtype):
+    from quantexperiments_amd.kernels import addnorm
+    g = torch.Generator().manual_seed(B * 1000 + C + M)
+    h = torch.randn(B, C, generator=g) * 2
+    add = rand_x(B, C, dtype, seed=C)
+    w = (torch.rand(C, generator=g) + 0.5).to(dtype)
+    perms = _perms(M, C, C) if M else None
+    h_ref, out_ref = O.addnorm(h.numpy(), add.float().numpy(), w.float().numpy(), 1e-6,
+                               perms=None if perms is None else perms.numpy(), dtype=NAMES[dtype])
+    out = torch.full((B, max(M, 1), C), float("nan"), dtype=dtype, device="cuda")
+    h_out = torch.full((B, C), float("nan"), device="cuda")
+    addnorm(h.cuda(), add.cuda(), w.cuda(), 1e-6, out, h_out=h_out, perms=None if perms is None else perms.cuda())
+    assert np.array_equal(h_out.cpu().numpy(), h_ref)
+    _one_step(out.float().cpu().numpy(), out_ref, dtype)
+    if perms is not None:                                   # the copies are exact gathers of one row of results
+        plain = torch.empty(B, C, dtype=dtype, device="cuda")
+        addnorm(h.cuda(), add.cuda(), w.cuda(), 1e-6, plain)
+        assert torch.equal(out, plain[:, perms.long().cuda()])
+
+
+def test_addnorm_without_add_in_place_and_strided_rows():
+    from quantexperiments_amd.kernels import addnorm
+    g = torch.Generator().manual_seed(7)
+    big = torch.randn(4, 600, generator=g).cuda()
+    h = big[:, 40:552]                                      # row stride 600
+    w = torch.ones(512, dtype=torch.float16, device="cuda")
+    ref = O.addnorm(h.cpu().numpy(), None, np.ones(512, dtype=np.float32), 1e-5)
+    out = torch.empty(4, 512, dtype=torch.float16, device="cuda")
+    addnorm(h, None, w, 1e-5, out)                          # no residual, h_out not asked for
+    _one_step(out.float().cpu().numpy(), ref[1][:, 0], torch.float16)
+    add = rand_x(4, 600, torch.float16, seed=1).cuda()[:, 8:520]
+    ref2 = O.addnorm(h.cpu().numpy(), add.float().cpu().numpy(), np.ones(512, dtype=np.float32), 1e-5)
+    keep = big.clone()
+    addnorm(h, add, w, 1e-5, out, h_out=h)                  # the residual updated in place
+    assert np.array_equal(h.cpu().numpy(), ref2[0])
+    assert torch.equal(big[:, :40], keep[:, :40]) and torch.equal(big[:, 552:], keep[:, 552:])
+    _one_step(out.float().cpu().numpy(), ref2[1][:, 0], torch.float16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("B,C,M", [(1, 18944, 0), (1, 4864, 0), (4, 17408, 0), (32, 96, 0), (1, 18944, 16), (3, 4864, 2), (1, 7, 0)])
+def test_silu_mul_matches_oracle(B, C, M, dtype):
+    from quantexperiments_amd.kernels import silu_mul
+    gu = rand_x(B, 2 * C, dtype, seed=C + B, scale=3.0)    # gate | up as one stacked product writes them
+    perms = _perms(M, C, C + 1) if M else None
+    ref = O.silu_mul(gu[:, :C].float().numpy(), gu[:, C:].float().numpy(), perms=None if perms is None else perms.numpy(),
+                     dtype=NAMES[dtype])
+    d = gu.cuda()
+    out = torch.full((B, max(M, 1), C), float("nan"), dtype=dtype, device="cuda")
+    silu_mul(d[:, :C], d[:, C:], out, perms=None if perms is None else perms.cuda())
+    # two roundings follow the hardware exponential, so a tie may fall the other way twice
+    step = np.abs(ref) * (2.0 ** -6 if dtype == torch.bfloat16 else 2.0 ** -9) + 2.0 ** -23
+    diff = np.abs(out.float().cpu().numpy().astype(np.float64) - ref)
+    assert np.all(diff <= step) and (diff > 0).mean() <= 0.01
+    if perms is not None:
+        plain = torch.empty(B, C, dtype=dtype, device="cuda")
+        silu_mul(d[:, :C], d[:, C:], plain)
+        assert torch.equal(out, plain[:, perms.long().cuda()])
+
+
+def test_silu_mul_special_values():
+    from quantexperiments_amd.kernels import silu_mul
+    g = torch.tensor([[0.0, -0.0, 20.0, -20.0, 60000.0, -60000.0, 1.0, float("inf")]], dtype=torch.float16, device="cuda")
+    u = torch.tensor([[7.0, 7.0, 0.5, 1.0, 1.0, 1.0, 1.0, 0.0]], dtype=torch.float16, device="cuda")
+    out = torch.empty(1, 8, dtype=torch.float16, device="cuda")
+    silu_mul(g, u, out)
+    o = out.float().cpu().numpy()[0]
+    assert o[0] == 0 and o[1] == 0 and o[2] == 10.0 and abs(o[3]) < 1e-6 and o[4] == 60000.0 and o[5] == 0
+    assert o[6] == np.float32(np.float16(1.0 / (1.0 + np.exp(-1.0)))) and np.isnan(o[7])       # inf * 0
+
+
+def test_neighbours_reject_bad_arguments():
+    from quantexperiments_amd import _lib
+    from quantexperiments_amd.kernels import addnorm, silu_mul
+    h = torch.zeros(2, 64, device="cuda")
+    w = torch.ones(64, dtype=torch.float16, device="cuda")
+    out = torch.empty(2, 64, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        addnorm(h.half(), None, w, 1e-6, out)               # residual must be fp32
+    with pytest.raises(ValueError):
+        addnorm(h, None, w.float(), 1e-6, out)
+    with pytest.raises(ValueError):
+        addnorm(h, None, w, 1e-6, out[:1])
+    with pytest.raises(ValueError):
+        addnorm(h, None, w, 1e-6, out, perms=torch.zeros(2, 64, dtype=torch.int64, device="cuda"))
+    p = _perms(2, 64, 1).cuda()
+    with pytest.raises(_lib.SqError):                       # several workgroups per row would race on the residual
+        addnorm(h, None, w, 1e-6, torch.empty(2, 2, 64, dtype=torch.float16, device="cuda"), h_out=h, perms=p)
+    with pytest.raises(ValueError):
+        silu_mul(out, out.bfloat16(), out)
+    with pytest.raises(ValueError):
+        silu_mul(out, out, out.float())
+    L = _lib.lib()
+    assert L.sq_addnorm(h.data_ptr(), None, 64, None, 0, 0, w.data_ptr(), _lib.SQ_F16, None, 1, 2, 64, 1e-6, out.data_ptr(),
+                        _lib.SQ_F32, None) == _lib.SQ_EINVAL
+    assert L.sq_addnorm(h.data_ptr(), None, 64, None, 0, 0, w.data_ptr(), _lib.SQ_F16, None, 1, 0, 64, 1e-6, None,
+                        _lib.SQ_F16, None) == _lib.SQ_OK                      # no rows
+    assert L.sq_silu_mul(out.data_ptr(), out.data_ptr(), _lib.SQ_F32, 64, None, 1, 2, 64, out.data_ptr(), None) == _lib.SQ_EINVAL
+    assert L.sq_silu_mul(out.data_ptr(), out.data_ptr(), _lib.SQ_F16, 32, None, 1, 2, 64, out.data_ptr(), None) == _lib.SQ_EINVAL
+    big = torch.zeros(1, 40000, device="cuda")
+    with pytest.raises(_lib.SqError):                       # a row with column orders is staged in LDS
+        addnorm(big, None, torch.ones(40000, dtype=torch.float16, device="cuda"), 1e-6,
+                torch.empty(1, 1, 40000, dtype=torch.float16, device="cuda"),
+                perms=torch.arange(40000, dtype=torch.int32, device="cuda")[None].contiguous())
+
+
+def test_decode_layer_chain_under_graph():
+    # o projection -> add + norm -> gate | up -> silu * up, captured and replayed: the neighbours take the products'
+    # outputs where the products left them and allocate nothing
+    from quantexperiments_amd.kernels import addnorm, silu_mul
+    g = torch.Generator().manual_seed(11)
+    C, I = 896, 4864
+    h = torch.randn(1, C, generator=g).cuda()
+    yo = rand_x(1, C, torch.bfloat16, seed=2).cuda()
+    w = (torch.rand(C, generator=g) + 0.5).bfloat16().cuda()
+    gu = rand_x(1, 2 * I, torch.bfloat16, seed=3, scale=2.0).cuda()
+    x2 = torch.empty(1, C, dtype=torch.bfloat16, device="cuda")
+    act = torch.empty(1, I, dtype=torch.bfloat16, device="cuda")
+    h2 = torch.empty_like(h)
+
+    def step():
+        addnorm(h, yo, w, 1e-6, x2, h_out=h2)
+        silu_mul(gu[:, :I], gu[:, I:], act)
+
+    step()
+    torch.cuda.synchronize()
+    e = (x2.clone(), act.clone(), h2.clone())
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr):
+        step()
+    for _ in range(3):
+        x2.zero_(); act.zero_(); h2.zero_()
+        torch.cuda.synchronize()
+        gr.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(x2, e[0]) and torch.equal(act, e[1]) and torch.equal(h2, e[2])

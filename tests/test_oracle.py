@@ -291,3 +291,90 @@ def test_host_packers_agree_with_oracle():
     with pytest.raises(ValueError):
         P.q8_pack(torch.zeros(2, 40))
     assert P.aux_bits({"vocab": 10, "hidden": 64}) == {"embed": 640 * 4.5, "lm_head": 640 * 8.5}
+
+
+# ------------------------------------------------------------------ elementwise neighbours (addnorm, silu_mul)
+def _ulp16(ref, dtype):
+    return np.abs(ref) * (2.0 ** -7 if dtype == "bf16" else 2.0 ** -10) + (0 if dtype == "bf16" else 2.0 ** -24)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_addnorm_matches_library_rms_norm(dtype):
+    g = torch.Generator().manual_seed(3)
+    h = torch.randn(5, 896, generator=g) * 3
+    add = (torch.randn(5, 896, generator=g)).to(torch.float16 if dtype == "fp16" else torch.bfloat16)
+    w = (torch.rand(896, generator=g) + 0.5).to(add.dtype)
+    h_out, out = O.addnorm(h.numpy(), add.float().numpy(), w.float().numpy(), 1e-6, dtype=dtype)
+    v = h + add.float()
+    assert np.array_equal(h_out, v.numpy())                                   # one fp32 add
+    lib = torch.nn.functional.rms_norm(v, (896,), w.float(), 1e-6).numpy()
+    assert out.shape == (5, 1, 896)
+    d = np.abs(out[:, 0] - lib)
+    assert np.all(d <= _ulp16(lib, dtype)) and (d > 0.51 * _ulp16(lib, dtype)).mean() < 0.01
+
+
+def test_addnorm_closed_forms():
+    ones = np.ones(64, dtype=np.float32)
+    # a constant row normalises to its sign; mean, not sum; eps inside the root
+    assert np.array_equal(O.addnorm(np.full((1, 64), 3.0), None, ones, 0.0)[1][0, 0], ones)
+    assert np.array_equal(O.addnorm(np.full((1, 64), -0.25), None, ones, 0.0)[1][0, 0], -ones)
+    assert np.array_equal(O.addnorm(np.ones((1, 64)), None, ones * 3, 3.0)[1][0, 0], ones * 1.5)    # 1 / sqrt(1 + 3) = 1/2
+    assert np.array_equal(O.addnorm(np.zeros((1, 64)), None, ones, 0.25)[1][0, 0], 0 * ones)
+    # the residual is added before the norm: 1 + 2 = 3 -> sign 1, and h_out = 3
+    h_out, out = O.addnorm(np.ones((1, 64)), np.full((1, 64), 2.0), ones, 0.0)
+    assert np.array_equal(h_out, np.full((1, 64), 3.0, dtype=np.float32)) and np.array_equal(out[0, 0], ones)
+    # scaling the row by a power of two changes nothing at eps = 0
+    g = np.random.default_rng(1)
+    v = g.standard_normal((3, 96)).astype(np.float32)
+    w = g.standard_normal(96).astype(np.float16).astype(np.float32)
+    assert np.array_equal(O.addnorm(v, None, w, 0.0)[1], O.addnorm(4 * v, None, w, 0.0)[1])
+    # every element of a two-valued row: v = (+a, -a, ...) has mean square a^2
+    v = np.tile(np.array([2.0, -2.0], dtype=np.float32), 32)[None]
+    assert np.array_equal(O.addnorm(v, None, ones, 0.0)[1][0, 0], np.sign(v[0]))
+
+
+def test_neighbour_copies_by_double_loop():
+    g = np.random.default_rng(2)
+    v = g.standard_normal((2, 40)).astype(np.float32)
+    w = np.ones(40, dtype=np.float32)
+    perms = np.stack([g.permutation(40) for _ in range(3)])
+    plain = O.addnorm(v, None, w, 1e-5)[1]
+    out = O.addnorm(v, None, w, 1e-5, perms=perms)[1]
+    su = O.silu_mul(v, v[::-1], perms=perms)
+    sp = O.silu_mul(v, v[::-1])
+    assert out.shape == (2, 3, 40) and su.shape == (2, 3, 40)
+    for b in range(2):
+        for m in range(3):
+            for i in range(40):
+                assert out[b, m, i] == plain[b, 0, perms[m, i]] and su[b, m, i] == sp[b, 0, perms[m, i]]
+
+
+def test_silu_mul_against_library_routines():
+    from scipy.special import expit
+    g = torch.Generator().manual_seed(5)
+    a = (torch.randn(4, 512, generator=g) * 4).half()
+    u = torch.randn(4, 512, generator=g).half()
+    out = O.silu_mul(a.float().numpy(), u.float().numpy())[:, 0]
+    # fp16: numpy's float16 arithmetic rounds each operation once
+    s16 = (a.double().numpy() * expit(a.double().numpy())).astype(np.float16)
+    assert np.array_equal(out, (s16 * u.numpy()).astype(np.float32))
+    # the two roundings are not one: somewhere the single-rounded product differs
+    single = (a.double().numpy() * expit(a.double().numpy()) * u.double().numpy()).astype(np.float16).astype(np.float32)
+    assert (single != out).any()
+    # torch's silu in the model dtype agrees to one unit in the last place of the SiLU value
+    t = (torch.nn.functional.silu(a.float()).half() * u).float().numpy()
+    assert np.all(np.abs(t - out) <= _ulp16(out, "fp16") * 1.01 + 2.0 ** -24 * np.abs(u.float().numpy()))
+    # bf16 through torch's bf16 multiply
+    ab, ub = a.bfloat16(), u.bfloat16()
+    ob = O.silu_mul(ab.float().numpy(), ub.float().numpy(), dtype="bf16")[:, 0]
+    sb = torch.from_numpy((ab.double().numpy() * expit(ab.double().numpy())).astype(np.float32)).bfloat16()
+    assert np.array_equal(ob, (sb * ub).float().numpy())
+
+
+def test_silu_mul_fixed_points():
+    one = np.ones((1, 4), dtype=np.float32)
+    assert np.array_equal(O.silu_mul(np.zeros((1, 4)), one * 7)[0, 0], np.zeros(4))
+    assert np.array_equal(O.silu_mul(np.full((1, 4), 20.0), one * 0.5)[0, 0], np.full(4, 10.0))     # silu(20) rounds to 20
+    assert np.all(np.abs(O.silu_mul(np.full((1, 4), -20.0), one)[0, 0]) < 1e-7)
+    assert np.array_equal(O.silu_mul(np.full((1, 4), 1.0), one)[0, 0],
+                          np.full(4, np.float16(1.0 / (1.0 + math.exp(-1.0))), dtype=np.float32))
