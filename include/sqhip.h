@@ -186,6 +186,35 @@ int sq_addnorm(const float* h_in, float* h_out, int64_t ld_h, const void* add, i
 int sq_silu_mul(const void* gate, const void* up, int dtype, int64_t ld, const int32_t* perms, int32_t M, int32_t B, int32_t C,
                 void* out, void* stream);
 
+/* sq_linear_small whose activations X [B, C] are produced by one of the two neighbours above instead of being read:
+ * the same results, bit for bit, as sq_addnorm / sq_silu_mul (perms = NULL) into x_out followed by sq_linear_small
+ * on x_out.  For one activation row of pieces that run on the tag-stream kernel (codebooks beyond LDS, or column
+ * orders) the producer is fused into that kernel: every workgroup computes its part of the row while it stages it
+ * (the mean square of the whole row included, in the stand-alone kernel's summation order), so no launch and no
+ * dependency bubble sit between the two; otherwise the library launches the stand-alone kernel first.  This is the
+ * counterpart of the reference's epi argument (reference shapequant/kernels/proto_runs.py:505-571, EPI 1 / EPI 2 at
+ * :223-287), turned round: there the producing kernel's last blocks write the next product's input, here the
+ * consuming kernel's workgroups compute it, which needs no launch-wide ticket and no cross-die visibility.
+ * mode SQ_FROM_ADDNORM: X = round(v * rsqrt(mean(v^2) + eps) * w), v = h_in + add (add NULL: v = h_in), h_out = v
+ * if not NULL (h_out must not be h_in).  mode SQ_FROM_SILU_MUL: X = silu(add) * up.  add / up / w / x_out hold
+ * x_dtype; rows b of h_in / h_out at b * ld_h, of add / up at b * ld_in, of x_out at b * C.  x_out is always
+ * written (it must be 16-byte aligned and C % 8 == 0). */
+#define SQ_FROM_ADDNORM 1
+#define SQ_FROM_SILU_MUL 2
+typedef struct sq_producer {
+    int32_t mode;
+    float eps;
+    const float* h_in;
+    float* h_out;
+    const void* add;
+    const void* up;
+    const void* w;
+    void* x_out;
+    int64_t ld_h, ld_in;
+} sq_producer;
+int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_producer* from, int x_dtype, void* y, int y_dtype,
+                         int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

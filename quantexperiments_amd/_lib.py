@@ -27,6 +27,16 @@ class SqMatrix(ctypes.Structure):
                 ("stream", ctypes.c_void_p), ("stream_runs", ctypes.c_int32), ("stream_groups", ctypes.c_int32)]
 
 
+class SqProducer(ctypes.Structure):
+    """struct sq_producer of include/sqhip.h."""
+    _fields_ = [("mode", ctypes.c_int32), ("eps", ctypes.c_float), ("h_in", ctypes.c_void_p), ("h_out", ctypes.c_void_p),
+                ("add", ctypes.c_void_p), ("up", ctypes.c_void_p), ("w", ctypes.c_void_p), ("x_out", ctypes.c_void_p),
+                ("ld_h", ctypes.c_int64), ("ld_in", ctypes.c_int64)]
+
+
+SQ_FROM_ADDNORM, SQ_FROM_SILU_MUL = 1, 2
+
+
 class SqError(RuntimeError):
     def __init__(self, code: int, msg: str):
         super().__init__(f"sqhip error {code}: {msg}")
@@ -68,8 +78,9 @@ def lib() -> ctypes.CDLL:
         L.sq_addnorm.argtypes = [vp, vp, i64, vp, ctypes.c_int, i64, vp, ctypes.c_int, vp, i32, i32, i32, ctypes.c_float, vp,
                                  ctypes.c_int, vp]
         L.sq_silu_mul.argtypes = [vp, vp, ctypes.c_int, i64, vp, i32, i32, i32, vp, vp]
+        L.sq_linear_small_from.argtypes = [mp, i32, ctypes.POINTER(SqProducer), ctypes.c_int, vp, ctypes.c_int, i64, i32, vp, sz, vp]
         for f in (L.sq_dequant, L.sq_linear_small, L.sq_linear_gemm, L.sq_gemm_dense, L.sq_q8_linear, L.sq_q8_dequant,
-                  L.sq_q4_embed, L.sq_addnorm, L.sq_silu_mul):
+                  L.sq_q4_embed, L.sq_addnorm, L.sq_silu_mul, L.sq_linear_small_from):
             f.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -77,7 +88,8 @@ def lib() -> ctypes.CDLL:
 
 EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
            "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build", "sq_q8_linear", "sq_q8_workspace_bytes",
-           "sq_q8_dequant", "sq_q4_embed", "sq_addnorm", "sq_silu_mul")
+           "sq_q8_dequant", "sq_q4_embed", "sq_addnorm", "sq_silu_mul",
+           "sq_linear_small_from")
 
 
 def check(rc: int) -> None:

@@ -74,7 +74,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 103; }
+int sq_version(void) { return 104; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -100,6 +100,39 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
                            has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
     return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
                         has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
+}
+
+int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_producer* from, int x_dtype, void* y, int y_dtype,
+                         int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream) {
+    const char* who = "sq_linear_small_from";
+    if (!from) return fail(SQ_EINVAL, "%s: null producer", who);
+    if (from->mode != SQ_FROM_ADDNORM && from->mode != SQ_FROM_SILU_MUL) return fail(SQ_EINVAL, "%s: mode %d", who, from->mode);
+    int rc = check_xy(who, mats, n_mats, from->x_out, x_dtype, n_mats > 0 ? mats[0].C : 0, y, y_dtype, ldy, B);
+    if (rc) return rc;
+    if (B > SQ_SMALL_BMAX) return fail(SQ_EINVAL, "%s: B %d > %d", who, B, SQ_SMALL_BMAX);
+    if (B == 0 || n_mats == 0) return SQ_OK;
+    const int C = mats[0].C;
+    const bool addnorm = from->mode == SQ_FROM_ADDNORM;
+    if (C % 8 || ((uintptr_t)from->x_out & 15)) return fail(SQ_EINVAL, "%s: x_out must be 16-byte aligned and C %% 8 == 0", who);
+    if (addnorm && (!from->h_in || !from->w)) return fail(SQ_EINVAL, "%s: null h_in / w", who);
+    if (addnorm && from->h_out == from->h_in) return fail(SQ_EINVAL, "%s: h_out must not be h_in", who);
+    if (!addnorm && (!from->add || !from->up)) return fail(SQ_EINVAL, "%s: null gate / up", who);
+    if (B > 1 && ((addnorm && from->ld_h < C) || ((from->add || !addnorm) && from->ld_in < C)))
+        return fail(SQ_EINVAL, "%s: ld_h %lld / ld_in %lld too small", who, (long long)from->ld_h, (long long)from->ld_in);
+    hipStream_t s = (hipStream_t)stream;
+    const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
+    void* ws = has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr;
+    const size_t wsb = has_ws ? ws_bytes - SQ_WS_HEADER : 0;
+    const bool aligned = (((uintptr_t)from->h_in | (uintptr_t)from->h_out | (uintptr_t)from->add | (uintptr_t)from->up | (uintptr_t)from->w) & 15) == 0;
+    if (aligned && small_fuses_producer(mats, n_mats, B))
+        return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, (unsigned*)workspace, s, from);
+    rc = addnorm ? launch_addnorm(from->h_in, from->h_out, from->ld_h, from->add, x_dtype, from->ld_in, from->w, x_dtype, nullptr, 1, B,
+                                  C, from->eps, from->x_out, x_dtype, s)
+                 : launch_silu_mul(from->add, from->up, x_dtype, from->ld_in, nullptr, 1, B, C, from->x_out, s);
+    if (rc) return rc;
+    if (small_takes_gemm_route(mats, n_mats, B, from->x_out, C))
+        return launch_gemm(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, (unsigned*)workspace, s);
+    return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, (unsigned*)workspace, s);
 }
 
 int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,

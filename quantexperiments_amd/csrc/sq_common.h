@@ -81,7 +81,10 @@ int device_cus();       // compute units of the current device (cached)
 int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s,
                    bool raw = false);
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s);
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s,
+                 const sq_producer* from = nullptr);
+// one activation row of these pieces is a single launch of the tag-stream kernel, which can produce its own x
+bool small_fuses_producer(const sq_matrix* mats, int n, int B);
 size_t small_workspace(const sq_matrix* mats, int n, int B);
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                 int64_t ldy, int T, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s);

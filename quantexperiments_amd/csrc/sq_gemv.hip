@@ -253,8 +253,16 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
     return SQ_OK;
 }
 
+bool small_fuses_producer(const sq_matrix* mats, int n, int B) {
+    if (B != 1 || n < 1 || n > GEMV_MAX_PIECES_STREAM) return false;
+    for (int i = 0; i < n; ++i)
+        if (mats[i].R <= 0 || !stream_rows(mats[i], 1) || mats[i].bits != mats[0].bits) return false;
+    return true;
+}
+
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s) {
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s, const sq_producer* from) {
+    if (from && !small_fuses_producer(mats, n, B)) return fail(SQ_EUNSUPPORTED, "sq_linear_small_from: no fused kernel for this stack");
     if (small_workspace(mats, n, B) > ws_bytes)
         return fail(SQ_EWORKSPACE, "sq_linear_small: workspace %zu < %zu", ws_bytes, small_workspace(mats, n, B));
     const int cus = device_cus();
@@ -266,7 +274,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         const sq_matrix& m0 = mats[i];
         if (m0.R == 0) { ++i; continue; }
         const int ud = unit_dwords(m0.bits);
-        if (stream_rows(m0, B) && x_ok) {
+        if (stream_rows(m0, B) && (x_ok || from)) {
             int j = i + 1;
             while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_rows(mats[j], B) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
             const size_t ws0 = ws_off, ysz = y_dtype == SQ_F32 ? 4 : 2;
@@ -277,7 +285,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
                 counters_used = c0;
                 int rc = launch_stream_group(mats + i, j - i, (const char*)x + (size_t)b0 * ldx * 2, x_dtype, ldx,
                                              (char*)y + (size_t)b0 * ldy * ysz, y_dtype, ldy, B - b0 < 8 ? B - b0 : 8, B,
-                                             (char*)ws, ws_off, counters, counters_used, s);
+                                             (char*)ws, ws_off, counters, counters_used, s, from);
                 if (rc) return rc;
                 ws_end = ws_off;
             }

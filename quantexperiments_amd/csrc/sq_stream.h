@@ -29,6 +29,6 @@ bool stream_shape(const sq_matrix& m);
 size_t stream_part_bytes(const sq_matrix& m, int B);
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                         int64_t ldy, int nb, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
-                        hipStream_t s);
+                        hipStream_t s, const sq_producer* from = nullptr);
 
 }  // namespace sq

@@ -239,7 +239,84 @@ struct StreamArgs {
     int64_t ldx, ldy;
     int nb;                           // activation rows of this pass (<= NB)
     int x_dtype, y_dtype;
+    // Producer of the activation row (stream_kernel<1, NW, PRO> with PRO != 0 only): the row is computed while it is
+    // staged instead of being read from x.  PRO 1: round(v * rsqrt(mean(v^2) + eps) * w) with v = h_in + add;
+    // PRO 2: silu(add) * up.  add / up / w / x_out hold x_dtype; x_out (and h_out) are written once per launch.
+    const float* h_in;
+    float* h_out;
+    const uint16_t* add;
+    const uint16_t* up;
+    const uint16_t* w;
+    uint16_t* x_out;
+    float eps;
 };
+
+// element i of the produced activation row, as 16 bits of dtype
+__device__ __forceinline__ uint16_t pro_round(float v, int dtype) { return dtype == SQ_BF16 ? f2bf(v) : f2h(v); }
+__device__ __forceinline__ float pro_load(const uint16_t* p, int dtype, int i) { return dtype == SQ_BF16 ? bf2f(p[i]) : h2f(p[i]); }
+__device__ __forceinline__ uint16_t pro_silu_mul(uint16_t g, uint16_t u, int dtype) {
+    if (dtype == SQ_BF16) {
+        const float a = bf2f(g);
+        return f2bf(bf2f(f2bf(a / (1.f + __expf(-a)))) * bf2f(u));
+    }
+    const float a = h2f(g);
+    const half_t sv = (half_t)(a / (1.f + __expf(-a)));
+    return __builtin_bit_cast(uint16_t, (half_t)(sv * __builtin_bit_cast(half_t, u)));
+}
+// The operands of one chunk (8 elements) of the produced row, fetched first and finished once the row's scale is known.
+// PRO 1: h, lo = add, hi = w.  PRO 2: lo = gate, hi = up.
+struct ProRaw { float h[8]; uint32_t lo[4], hi[4]; };
+
+// chunk ci in natural order: 16-byte loads (every pointer 16-byte aligned)
+template <int PRO>
+__device__ __forceinline__ ProRaw pro_fetch(const StreamArgs& a, int ci) {
+    ProRaw r;
+    const u32x4 hi = reinterpret_cast<const u32x4*>(PRO == 1 ? a.w : a.up)[ci];
+    u32x4 lo = u32x4{0u, 0u, 0u, 0u};
+    if (PRO == 2 || a.add) lo = reinterpret_cast<const u32x4*>(a.add)[ci];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { r.lo[k] = lo[k]; r.hi[k] = hi[k]; }
+    if (PRO == 1) {
+        const float4v h0 = reinterpret_cast<const float4v*>(a.h_in)[2 * ci], h1 = reinterpret_cast<const float4v*>(a.h_in)[2 * ci + 1];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { r.h[k] = h0[k]; r.h[4 + k] = h1[k]; }
+    }
+    return r;
+}
+// the 8 elements idx[0..7] (a chunk of a column order)
+template <int PRO>
+__device__ __forceinline__ ProRaw pro_gather(const StreamArgs& a, const int32_t* idx) {
+    ProRaw r;
+    const uint16_t* hp = PRO == 1 ? a.w : a.up;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int i0 = idx[2 * k], i1 = idx[2 * k + 1];
+        r.hi[k] = (uint32_t)hp[i0] | ((uint32_t)hp[i1] << 16);
+        r.lo[k] = (PRO == 2 || a.add) ? ((uint32_t)a.add[i0] | ((uint32_t)a.add[i1] << 16)) : 0u;
+        if (PRO == 1) { r.h[2 * k] = a.h_in[i0]; r.h[2 * k + 1] = a.h_in[i1]; }
+    }
+    return r;
+}
+__device__ __forceinline__ float pro_f(uint32_t pair, int k, int dtype) {
+    const uint16_t b = (uint16_t)(pair >> (16 * (k & 1)));
+    return dtype == SQ_BF16 ? bf2f(b) : h2f(b);
+}
+// v = h + add of element k of a fetched chunk (PRO 1)
+__device__ __forceinline__ float pro_v(const StreamArgs& a, const ProRaw& r, int k) {
+    return a.add ? r.h[k] + pro_f(r.lo[k >> 1], k, a.x_dtype) : r.h[k];
+}
+template <int PRO>
+__device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r, float rstd) {
+    uint32_t e[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        if (PRO == 2)
+            e[k] = pro_silu_mul((uint16_t)(r.lo[k >> 1] >> (16 * (k & 1))), (uint16_t)(r.hi[k >> 1] >> (16 * (k & 1))), a.x_dtype);
+        else
+            e[k] = pro_round(pro_v(a, r, k) * rstd * pro_f(r.hi[k >> 1], k, a.x_dtype), a.x_dtype);
+    }
+    return u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+}
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
 constexpr int STREAM_XS = STREAM_PART_MAX * 16;   // LDS bytes of one activation row's part of x
@@ -254,8 +331,9 @@ struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
 
 // NB activation rows per pass (every entry's codeword is gathered once and multiplied with NB x chunks), NW waves.
 // LDS: [codebook slice 64 KB][NB x parts of 10 KB][two words of flags].
-template <int NB, int NW>
+template <int NB, int NW, int PRO = 0>
 __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
+    static_assert(PRO == 0 || NB == 1, "produced activations: one row");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int pi = 0;
@@ -317,10 +395,99 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
         for (int k = 0; k < NT; ++k) t[k] = src[tid + k * NW * 64];
         const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
+        if (PRO != 0) {
+            // every operand of the produced row is requested before anything waits: this thread's chunks, then
+            // (PRO 1) its share of the whole row for the mean square
+            const int32_t* pm = P.perms ? P.perms + (size_t)run[2] * P.C : nullptr;
+            ProRaw raw[NX];
+#pragma unroll
+            for (int k = 0; k < NX; ++k) {
+                const int ci = c0 + min(tid + k * NW * 64, nc - 1);
+                raw[k] = pm ? pro_gather<PRO>(a, pm + (size_t)ci * 8) : pro_fetch<PRO>(a, ci);
+            }
+            float rstd = 0.f;
+            if (PRO == 1) {
+                // Mean square of the whole row in the stand-alone kernel's order, so both give the same bits: slot j
+                // of 1024 adds the squares of chunks j, j + 1024, ... element by element with fused multiply-adds, each
+                // block of 64 slots is folded by the wave butterfly, the 16 block sums are added in turn.  A thread
+                // here owns slots tid and tid + 512.
+                static_assert(PRO != 1 || NW * 64 == 512, "two slots per thread");
+                float* red = reinterpret_cast<float*>(flag + 4);
+                float ps[2] = {0.f, 0.f};
+                if (pm == nullptr && nc == P.U && P.U <= NX * 512) {
+                    // one column part, natural order: this thread's chunks are its slots' chunks, already fetched
+#pragma unroll
+                    for (int k = 0; k < NX; ++k)
+                        if (tid + k * 512 < P.U) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) { const float v = pro_v(a, raw[k], e); ps[k & 1] = __builtin_fmaf(v, v, ps[k & 1]); }
+                        }
+                } else if (P.U <= 1024) {                       // one chunk per slot, both fetched together
+                    ProRaw r2[2];
+#pragma unroll
+                    for (int m = 0; m < 2; ++m) r2[m] = pro_fetch<1>(a, min(tid + m * 512, P.U - 1));
+#pragma unroll
+                    for (int m = 0; m < 2; ++m)
+                        if (tid + m * 512 < P.U) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) { const float v = pro_v(a, r2[m], e); ps[m] = __builtin_fmaf(v, v, ps[m]); }
+                        }
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 2; ++m)
+                        for (int c = tid + m * 512; c < P.U; c += 1024) {
+                            const ProRaw r = pro_fetch<1>(a, c);
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) { const float v = pro_v(a, r, e); ps[m] = __builtin_fmaf(v, v, ps[m]); }
+                        }
+                }
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    ps[m] = wave_sum(ps[m]);
+                    if (lane == 0) red[m * NW + wave] = ps[m];
+                }
+                __syncthreads();
+                float tot = 0.f;
+#pragma unroll
+                for (int q = 0; q < 16; ++q) tot += red[q];
+                rstd = rsqrtf(tot / (float)P.C + a.eps);
+            }
+#pragma unroll
+            for (int k = 0; k < NX; ++k) xq[0][k] = pro_finish<PRO>(a, raw[k], rstd);
+            if (pi == 0 && s == 0 && wi == 0) {
+                // one workgroup per column part leaves the produced row (and the updated residual) in memory
+                if (pm == nullptr) {
+#pragma unroll
+                    for (int k = 0; k < NX; ++k) {
+                        const int c = tid + k * NW * 64;
+                        if (c >= nc) continue;
+                        reinterpret_cast<u32x4*>(a.x_out)[c0 + c] = xq[0][k];
+                        if (PRO == 1 && a.h_out) {
+                            float4v o0, o1;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) { o0[e] = pro_v(a, raw[k], e); o1[e] = pro_v(a, raw[k], 4 + e); }
+                            reinterpret_cast<float4v*>(a.h_out)[2 * (c0 + c)] = o0;
+                            reinterpret_cast<float4v*>(a.h_out)[2 * (c0 + c) + 1] = o1;
+                        }
+                    }
+                } else {
+                    for (int c = tid; c < nc; c += NW * 64) {
+                        const ProRaw r = pro_fetch<PRO>(a, c0 + c);
+                        reinterpret_cast<u32x4*>(a.x_out)[c0 + c] = pro_finish<PRO>(a, r, rstd);
+                        if (PRO == 1 && a.h_out) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) a.h_out[(c0 + c) * 8 + e] = pro_v(a, r, e);
+                        }
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const uint16_t* xr = a.x + (int64_t)min(b, a.nb - 1) * a.ldx;
-            if (P.perms == nullptr) {
+            if (PRO != 0) {
+                // filled above
+            } else if (P.perms == nullptr) {
                 const u32x4* xs = reinterpret_cast<const u32x4*>(xr) + c0;
 #pragma unroll
                 for (int k = 0; k < NX; ++k) xq[b][k] = xs[min(tid + k * NW * 64, nc - 1)];
@@ -496,16 +663,16 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     SQ_TRACE_POINT(6);
 }
 
-template <int NB, int NW>
+template <int NB, int NW, int PRO = 0>
 static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
     static bool raised = false;
     if (!raised) {
-        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NW, PRO>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         (void)hipGetLastError();
         raised = true;
     }
-    const size_t smem = (size_t)STREAM_TAB + (size_t)NB * STREAM_XS + 16;
-    hipLaunchKernelGGL((stream_kernel<NB, NW>), dim3((unsigned)grid), dim3(NW * 64), smem, s, a);
+    const size_t smem = (size_t)STREAM_TAB + (size_t)NB * STREAM_XS + 16 + (PRO == 1 ? 64 : 0);   // + 16 block sums
+    hipLaunchKernelGGL((stream_kernel<NB, NW, PRO>), dim3((unsigned)grid), dim3(NW * 64), smem, s, a);
     return check_launch("sq_linear_small(stream)");
 }
 
@@ -526,8 +693,13 @@ size_t stream_part_bytes(const sq_matrix& m, int B) {
 // of the workspace.
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                         int64_t ldy, int nb, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
-                        hipStream_t s) {
+                        hipStream_t s, const sq_producer* from) {
     StreamArgs a;
+    a.h_in = nullptr; a.h_out = nullptr; a.add = a.up = a.w = nullptr; a.x_out = nullptr; a.eps = 0.f;
+    if (from) {
+        a.h_in = from->h_in; a.h_out = from->h_out; a.add = (const uint16_t*)from->add; a.up = (const uint16_t*)from->up;
+        a.w = (const uint16_t*)from->w; a.x_out = (uint16_t*)from->x_out; a.eps = from->eps;
+    }
     a.n = cnt;
     a.x = (const uint16_t*)x;
     a.y = y;
@@ -561,6 +733,10 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         wg += g.NV * nwg;
     }
     for (int k = cnt; k < GEMV_MAX_PIECES_STREAM; ++k) a.p[k] = a.p[0];
+    if (from) {
+        if (nb != 1) return fail(SQ_EINVAL, "sq_linear_small_from: fused producers take one activation row");
+        return from->mode == 1 ? stream_launch<1, 8, 1>(a, wg, s) : stream_launch<1, 8, 2>(a, wg, s);
+    }
     switch (stream_pass_rows(nb)) {
         case 1: return stream_launch<1, 8>(a, wg, s);           // 74 KB of LDS: two workgroups of 8 waves per CU
         case 2: return stream_launch<2, 16>(a, wg, s);          // from here one workgroup of 16 waves per CU

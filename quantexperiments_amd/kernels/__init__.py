@@ -368,3 +368,56 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, perms=None
         _lib.check(_lib.lib().sq_silu_mul(gate.data_ptr(), up.data_ptr(), _lib.DTYPES[gate.dtype], gate.stride(0), pp, M, B, C,
                                           out.data_ptr(), _lib.stream_ptr(dev)))
     return out
+
+
+def _row_ld(t: torch.Tensor) -> int:
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def linear_small_from(pieces, y: torch.Tensor, x_out: torch.Tensor, *, h_in=None, add=None, w=None, eps: float = 0.0, h_out=None,
+                      gate=None, up=None) -> torch.Tensor:
+    """sq_linear_small over activations produced on the way in (sq_linear_small_from), the same bits as the
+    stand-alone neighbour into x_out followed by linear_small(pieces, x_out, y):
+
+      h_in (+ add), w, eps [, h_out]:  x_out = rmsnorm(h_in + add) * w, h_out = h_in + add   (addnorm)
+      gate, up:                        x_out = silu(gate) * up                                 (silu_mul)
+
+    x_out [B, C] (contiguous, fp16 / bf16) is always written.  One activation row of pieces on the tag-stream kernel
+    runs as ONE launch (the producer fused into the product); everything else as two.  The reference's epi argument
+    of proto_runs.gemv (shapequant/kernels/proto_runs.py:505-571)."""
+    norm = h_in is not None
+    if norm == (gate is not None):
+        raise ValueError("linear_small_from: give either h_in / w or gate / up")
+    if not x_out.is_contiguous() or x_out.dim() != 2 or x_out.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("linear_small_from: x_out must be a contiguous fp16 / bf16 [B, C]")
+    mats, _, ldy = _prep(pieces, x_out, y)
+    dev, dt = x_out.device, x_out.dtype
+    pr = _lib.SqProducer()
+    pr.x_out = x_out.data_ptr()
+    pr.eps = float(eps)
+    if norm:
+        if h_in.dtype != torch.float32 or h_in.shape != x_out.shape or h_in.stride(1) != 1:
+            raise ValueError("linear_small_from: h_in must be fp32 [B, C] with unit column stride")
+        if w is None or w.dtype != dt or w.numel() != x_out.shape[1] or not w.is_contiguous():
+            raise ValueError("linear_small_from: w must be a contiguous [C] of x_out's dtype")
+        if add is not None and (add.dtype != dt or add.shape != x_out.shape or add.stride(1) != 1):
+            raise ValueError("linear_small_from: add must match x_out in dtype and shape")
+        if h_out is not None and (h_out.dtype != torch.float32 or h_out.shape != h_in.shape or h_out.stride() != h_in.stride()):
+            raise ValueError("linear_small_from: h_out must match h_in")
+        pr.mode, pr.h_in, pr.ld_h, pr.w = _lib.SQ_FROM_ADDNORM, h_in.data_ptr(), _row_ld(h_in), w.data_ptr()
+        pr.h_out = None if h_out is None else h_out.data_ptr()
+        if add is not None:
+            pr.add, pr.ld_in = add.data_ptr(), _row_ld(add)
+    else:
+        if gate.dtype != dt or gate.shape != x_out.shape or gate.stride(1) != 1 or up.dtype != dt or up.shape != gate.shape \
+                or up.stride() != gate.stride():
+            raise ValueError("linear_small_from: gate / up must match x_out in dtype and shape and each other in strides")
+        pr.mode, pr.add, pr.up, pr.ld_in = _lib.SQ_FROM_SILU_MUL, gate.data_ptr(), up.data_ptr(), _row_ld(gate)
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        need = L.sq_workspace_bytes(mats, len(pieces), x_out.shape[0], 0)
+        ws = _Workspace.get(need, dev) if need else None
+        _lib.check(L.sq_linear_small_from(mats, len(pieces), ctypes.byref(pr), _lib.DTYPES[dt], y.data_ptr(), _lib.DTYPES[y.dtype],
+                                          ldy, x_out.shape[0], None if ws is None else ws.data_ptr(),
+                                          0 if ws is None else ws.numel(), _lib.stream_ptr(dev)))
+    return y

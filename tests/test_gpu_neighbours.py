@@ -168,3 +168,117 @@ def test_decode_layer_chain_under_graph():
         gr.replay()
         torch.cuda.synchronize()
         assert torch.equal(x2, e[0]) and torch.equal(act, e[1]) and torch.equal(h2, e[2])
+
+
+# ------------------------------------------------------------------ products that compute their own activations
+def _stack(shapes, bits, M, seed, d=8):
+    from quantexperiments_amd.kernels import prepare_stack
+    from tests.helpers import synth, to_device
+    ss = [synth(R, C, d, bits, 1, M, seed=seed + i) for i, (R, C) in enumerate(shapes)]
+    lins = [to_device(s) for s in ss]
+    prepare_stack(lins)
+    return ss, lins
+
+
+FROM = [  # piece row counts, C, tag bits, M, d: tag-stream stacks (fused), and stacks on other kernels (two launches)
+    ((260, 70, 70), 3584, 16, 1, 8), ((130,), 896, 16, 1, 8), ((300, 300), 5120, 16, 16, 8), ((65,), 18944, 16, 1, 8),
+    ((40,), 17408, 16, 16, 8), ((333,), 2048, 14, 1, 8), ((96, 40), 512, 12, 1, 4), ((64,), 256, 10, 4, 4),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", FROM, ids=lambda c: "x".join(map(str, c[0])) + f"_C{c[1]}_b{c[2]}_M{c[3]}")
+@pytest.mark.parametrize("B", [1, 3])
+def test_linear_small_from_equals_two_calls(case, dtype, B):
+    # reference tests/test_decode_e2e.py:203-226: the fused form against the separate kernels, bit for bit
+    from quantexperiments_amd.kernels import addnorm, linear_small, linear_small_from, silu_mul
+    rows, C, bits, M, d = case
+    ss, lins = _stack([(R, C) for R in rows], bits, M, seed=C + bits, d=d)
+    g = torch.Generator().manual_seed(C)
+    h = (torch.randn(B, C, generator=g) * 2).cuda()
+    add = rand_x(B, C, dtype, seed=1).cuda()
+    w = (torch.rand(C, generator=g) + 0.5).to(dtype).cuda()
+    gu = rand_x(B, 2 * C, dtype, seed=2, scale=2.0).cuda()
+    R = sum(rows)
+    for mode in ("addnorm", "addnorm_no_add", "silu"):
+        x_ref = torch.empty(B, C, dtype=dtype, device="cuda")
+        h_ref = torch.full((B, C), float("nan"), device="cuda")
+        if mode == "silu":
+            silu_mul(gu[:, :C], gu[:, C:], x_ref)
+        else:
+            addnorm(h, add if mode == "addnorm" else None, w, 1e-6, x_ref, h_out=h_ref)
+        y_ref = torch.empty(B, R, dtype=torch.float32, device="cuda")
+        linear_small(lins, x_ref, y_ref)
+        x_out = torch.full((B, C), float("nan"), dtype=dtype, device="cuda")
+        h_out = torch.full((B, C), float("nan"), device="cuda")
+        y = torch.full((B, R), float("nan"), dtype=torch.float32, device="cuda")
+        if mode == "silu":
+            linear_small_from(lins, y, x_out, gate=gu[:, :C], up=gu[:, C:])
+        else:
+            linear_small_from(lins, y, x_out, h_in=h, add=add if mode == "addnorm" else None, w=w, eps=1e-6, h_out=h_out)
+            assert torch.equal(h_out, h_ref), mode
+        assert torch.equal(x_out, x_ref), mode
+        assert torch.equal(y, y_ref), mode
+    # and against the oracle end to end (one mode is enough: the pieces above are bit-equal)
+    from tests.test_gpu_parity import _ref
+    ref = np.concatenate([_ref(s, x_ref.cpu()) for s in ss], axis=1)
+    assert float(np.abs(y_ref.cpu().numpy() - ref).max() / np.abs(ref).max()) < 1e-3
+
+
+def test_linear_small_from_rejects_bad_arguments():
+    from quantexperiments_amd import _lib
+    from quantexperiments_amd.kernels import linear_small_from
+    ss, lins = _stack([(70, 512)], 16, 1, seed=3)
+    y = torch.empty(1, 70, dtype=torch.float32, device="cuda")
+    x_out = torch.empty(1, 512, dtype=torch.bfloat16, device="cuda")
+    h = torch.zeros(1, 512, device="cuda")
+    w = torch.ones(512, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        linear_small_from(lins, y, x_out)                                   # no producer
+    with pytest.raises(ValueError):
+        linear_small_from(lins, y, x_out, h_in=h, w=w, gate=x_out, up=x_out)
+    with pytest.raises(ValueError):
+        linear_small_from(lins, y, x_out, h_in=h, w=w.half())
+    with pytest.raises(ValueError):
+        linear_small_from(lins, y, x_out, h_in=h.half(), w=w)
+    with pytest.raises(_lib.SqError):
+        linear_small_from(lins, y, x_out, h_in=h, w=w, h_out=h)             # workgroups still read h_in while one writes
+    with pytest.raises(ValueError):
+        linear_small_from(lins, y, x_out, gate=x_out, up=x_out.half())
+
+
+def test_decode_layer_with_fused_producers_under_graph():
+    # qkv-like -> o -> (add + norm fused into) gate | up -> (silu * up fused into) down, captured and replayed
+    from quantexperiments_amd.kernels import linear_small, linear_small_from
+    C, I = 512, 1024
+    _, o = _stack([(C, C)], 16, 1, seed=1)
+    _, gu = _stack([(I, C), (I, C)], 16, 1, seed=2)
+    _, dn = _stack([(C, I)], 16, 1, seed=3)
+    g = torch.Generator().manual_seed(4)
+    attn = rand_x(1, C, torch.bfloat16, seed=5).cuda()
+    h0 = torch.randn(1, C, generator=g).cuda()
+    w = (torch.rand(C, generator=g) + 0.5).bfloat16().cuda()
+    yo = torch.empty(1, C, dtype=torch.bfloat16, device="cuda")
+    ygu = torch.empty(1, 2 * I, dtype=torch.bfloat16, device="cuda")
+    yd = torch.empty(1, C, dtype=torch.bfloat16, device="cuda")
+    x1 = torch.empty(1, C, dtype=torch.bfloat16, device="cuda")
+    act = torch.empty(1, I, dtype=torch.bfloat16, device="cuda")
+    h1 = torch.empty_like(h0)
+
+    def step():
+        linear_small(o, attn, yo)
+        linear_small_from(gu, ygu, x1, h_in=h0, add=yo, w=w, eps=1e-6, h_out=h1)
+        linear_small_from(dn, yd, act, gate=ygu[:, :I], up=ygu[:, I:])
+
+    step()
+    torch.cuda.synchronize()
+    eager = (yd.clone(), h1.clone(), act.clone())
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr):
+        step()
+    for _ in range(3):
+        yd.zero_(); h1.zero_(); act.zero_()
+        torch.cuda.synchronize()
+        gr.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(yd, eager[0]) and torch.equal(h1, eager[1]) and torch.equal(act, eager[2])
