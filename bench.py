@@ -15,7 +15,8 @@ the packed file's bytes, which is what the metric is quoted on.
 value = packed (algorithmic) bytes of a layer / time per layer, in GB/s.  The same JSON line
 carries us_per_layer, the roofline of the dominant kernel (gate|up launch, HIP events around graph
 replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s, the 8-bit block-32 output head
-(152,064 x 3,584) at a few decode batch sizes, and the CPU baseline (the reference's CPU route, oracle
+(152,064 x 3,584) at a few decode batch sizes, the layer with its three elementwise neighbours (add + RMS
+norm twice, SiLU * up) as separate launches and fused into the consuming products, and the CPU baseline (the reference's CPU route, oracle
 port, on the host cores).
 """
 
@@ -150,6 +151,45 @@ def lm_head(torch, dev, rows=(1, 4, 8, 32), reps=3):
     return res
 
 
+def neighbours(torch, dev, layers, x, y):
+    """One decoder layer with the three elementwise neighbours of its products (add + RMS norm before q|k|v and
+    before gate|up, SiLU * up before down), as separate launches and fused into the consuming products; and the
+    two stand-alone kernels by themselves.  Microseconds per layer / per launch inside a HIP graph."""
+    from quantexperiments_amd.kernels import addnorm, linear_small, linear_small_from, silu_mul
+    L, I = LAUNCHES, SHAPES_7B["gate"][0]
+    h = [torch.randn(1, 3584, device=dev), torch.empty(1, 3584, device=dev)]
+    w = torch.ones(3584, device=dev, dtype=torch.bfloat16)
+    x1 = torch.empty(1, 3584, device=dev, dtype=torch.bfloat16)
+    act = torch.empty(1, I, device=dev, dtype=torch.bfloat16)
+    gate, up = y[L[2]][:, :I], y[L[2]][:, I:]
+
+    def separate():
+        for Ly in layers:
+            addnorm(h[1], y[L[3]], w, 1e-6, x1, h_out=h[0])
+            linear_small([Ly[n] for n in L[0]], x1, y[L[0]])
+            linear_small([Ly[n] for n in L[1]], x[3584], y[L[1]])          # (attention sits between q|k|v and o)
+            addnorm(h[0], y[L[1]], w, 1e-6, x1, h_out=h[1])
+            linear_small([Ly[n] for n in L[2]], x1, y[L[2]])
+            silu_mul(gate, up, act)
+            linear_small([Ly[n] for n in L[3]], act, y[L[3]])
+
+    def fused():
+        for Ly in layers:
+            linear_small_from([Ly[n] for n in L[0]], y[L[0]], x1, h_in=h[1], add=y[L[3]], w=w, eps=1e-6, h_out=h[0])
+            linear_small([Ly[n] for n in L[1]], x[3584], y[L[1]])
+            linear_small_from([Ly[n] for n in L[2]], y[L[2]], x1, h_in=h[0], add=y[L[1]], w=w, eps=1e-6, h_out=h[1])
+            linear_small_from([Ly[n] for n in L[3]], y[L[3]], act, gate=gate, up=up)
+
+    res = {}
+    for name, fn, per in (("layer_separate_us", separate, len(layers)), ("layer_fused_us", fused, len(layers)),
+                          ("addnorm_us", lambda: [addnorm(h[0], y[L[1]], w, 1e-6, x1, h_out=h[1]) for _ in range(28)], 28),
+                          ("silu_mul_us", lambda: [silu_mul(gate, up, act) for _ in range(28)], 28)):
+        ms, g = timed_graph(torch, fn, reps=3)
+        del g
+        res[name] = ms * 1e3 / per
+    return res
+
+
 def copy_probe(torch, dev):
     """Three 256 MiB device-to-device copies: a kernel of known HBM traffic to scale profiler counters by."""
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -172,6 +212,7 @@ def main():
                     help="run only the dominant launch (gate|up) and print only its roofline object: the command "
                          "the rocprofv3 summaries under profiles/ are made with")
     ap.add_argument("--no-head", action="store_true", help="skip the 8-bit lm_head GEMV")
+    ap.add_argument("--no-neighbours", action="store_true", help="skip the layer with its elementwise neighbours")
     ap.add_argument("--head-only", action="store_true",
                     help="run only the 8-bit lm_head GEMV and print only its object (the command its rocprofv3 "
                          "summary under profiles/ is made with)")
@@ -279,6 +320,8 @@ def main():
         out["prefill"] = {"M": 2048, "gate_18944x3584": pf["gate"], "down_3584x18944": pf["down"],
                           "peak_tflops": MFMA_PEAK_TFLOPS,
                           "frac_of_peak": min(pf["gate"]["tflops"], pf["down"]["tflops"]) / MFMA_PEAK_TFLOPS}
+    if not args.no_neighbours:
+        out["layer_with_neighbours"] = neighbours(torch, dev, layers, x, y)
     if not args.no_head:
         del layers[1:]                           # the head needs 0.6 GB; the rotated layers are no longer used
         out["lm_head_q8"] = lm_head(torch, dev)
