@@ -63,6 +63,10 @@ def lib() -> ctypes.CDLL:
         L.sq_linear_small.argtypes = [mp, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
         L.sq_linear_gemm.argtypes = [mp, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
         L.sq_gemm_dense.argtypes = [vp, ctypes.c_int, i64, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp]
+        L.sq_gemm_dense_ws.argtypes = [vp, ctypes.c_int, i64, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
+        L.sq_gemm_dense_ws.restype = ctypes.c_int
+        L.sq_gemm_dense_workspace_bytes.argtypes = [i32, i32, i32]
+        L.sq_gemm_dense_workspace_bytes.restype = sz
         L.sq_workspace_bytes.argtypes = [mp, i32, i32, ctypes.c_int]
         L.sq_workspace_bytes.restype = sz
         ip = ctypes.POINTER(ctypes.c_int32)
@@ -89,7 +93,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
            "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build", "sq_q8_linear", "sq_q8_workspace_bytes",
            "sq_q8_dequant", "sq_q4_embed", "sq_addnorm", "sq_silu_mul",
-           "sq_linear_small_from")
+           "sq_linear_small_from", "sq_gemm_dense_ws", "sq_gemm_dense_workspace_bytes")
 
 
 def check(rc: int) -> None:

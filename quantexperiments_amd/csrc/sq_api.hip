@@ -74,7 +74,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 104; }
+int sq_version(void) { return 105; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -154,6 +154,26 @@ int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C,
     if (R == 0 || T == 0) return SQ_OK;
     if (!w || !x || !y || ldw < C || ldx < C || ldy < R) return fail(SQ_EINVAL, "sq_gemm_dense: bad pointer or stride");
     return launch_gemm_dense(w, w_dtype, ldw, R, C, x, x_dtype, ldx, y, y_dtype, ldy, T, (hipStream_t)stream);
+}
+
+int sq_gemm_dense_ws(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype, int64_t ldx,
+                     void* y, int y_dtype, int64_t ldy, int32_t T, void* workspace, size_t ws_bytes, void* stream) {
+    if (!workspace || ws_bytes <= SQ_WS_HEADER || ((uintptr_t)workspace & 255))
+        return sq_gemm_dense(w, w_dtype, ldw, R, C, x, x_dtype, ldx, y, y_dtype, ldy, T, stream);
+    if (x_dtype != SQ_F16 && x_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense_ws: x_dtype %d", x_dtype);
+    if (w_dtype != SQ_F16 && w_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense_ws: w_dtype %d", w_dtype);
+    if (y_dtype != SQ_F32 && y_dtype != SQ_F16 && y_dtype != SQ_BF16) return fail(SQ_EINVAL, "sq_gemm_dense_ws: y_dtype %d", y_dtype);
+    if (R < 0 || C <= 0 || T < 0) return fail(SQ_EINVAL, "sq_gemm_dense_ws: R %d C %d T %d", R, C, T);
+    if (R == 0 || T == 0) return SQ_OK;
+    if (!w || !x || !y || ldw < C || ldx < C || ldy < R) return fail(SQ_EINVAL, "sq_gemm_dense_ws: bad pointer or stride");
+    return launch_gemm_dense(w, w_dtype, ldw, R, C, x, x_dtype, ldx, y, y_dtype, ldy, T, (hipStream_t)stream,
+                             (char*)workspace + SQ_WS_HEADER, ws_bytes - SQ_WS_HEADER);
+}
+
+size_t sq_gemm_dense_workspace_bytes(int32_t R, int32_t C, int32_t T) {
+    if (R <= 0 || C <= 0 || T <= 0) return 0;
+    const size_t inner = gemm_dense_workspace(R, C, T);
+    return inner ? inner + SQ_WS_HEADER : 0;
 }
 
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which) {

@@ -96,7 +96,8 @@ size_t small_gemm_route_workspace(const sq_matrix* mats, int n, int B);
 int small_pass_limit(const sq_matrix* mats, int n);
 size_t gemm_workspace(const sq_matrix* mats, int n, int T);
 int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, const void* x, int x_dtype, int64_t ldx,
-                      void* y, int y_dtype, int64_t ldy, int T, hipStream_t s);
+                      void* y, int y_dtype, int64_t ldy, int T, hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
+size_t gemm_dense_workspace(int R, int C, int T);
 
 // tile-major copy of the tags for the matrix-core decode kernel (host routines, sq_gemv.hip)
 bool tiled_format_ok(int R, int W, int C, int d, int bits);

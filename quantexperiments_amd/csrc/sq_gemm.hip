@@ -260,12 +260,20 @@ static int run(const GemmArgs& a, int d, bool dense, hipStream_t s) {
     return check_launch("sq_linear_gemm");
 }
 
+size_t gemm_dense_workspace(int R, int C, int T) {
+    return (T >= GEMM256_MIN_T && C % 64 == 0) ? gemm256_part_bytes(T, R, C, device_cus()) : 0;
+}
+
 int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, const void* x, int x_dtype, int64_t ldx,
-                      void* y, int y_dtype, int64_t ldy, int T, hipStream_t s) {
+                      void* y, int y_dtype, int64_t ldy, int T, hipStream_t s, void* ws, size_t ws_bytes) {
     if (!x_vec_ok(x, ldx, C) || !x_vec_ok(w, ldw, C))
         return fail(SQ_EUNSUPPORTED, "sq_gemm_dense: C, ldx, ldw must be multiples of 8 and pointers 16-byte aligned");
-    if (x_dtype == SQ_F16 && w_dtype == SQ_F16 && T >= GEMM256_MIN_T && gemm256_ok(C, ldx, ldw, x, w))
-        return launch_gemm256((const uint16_t*)x, ldx, (const uint16_t*)w, ldw, nullptr, y, y_dtype, ldy, 0, T, R, C, nullptr, 0, s);
+    if (x_dtype == SQ_F16 && w_dtype == SQ_F16 && T >= GEMM256_MIN_T && gemm256_ok(C, ldx, ldw, x, w)) {
+        const size_t part = gemm256_part_bytes(T, R, C, device_cus());
+        const bool split = ws && part && ws_bytes >= part;
+        return launch_gemm256((const uint16_t*)x, ldx, (const uint16_t*)w, ldw, nullptr, y, y_dtype, ldy, 0, T, R, C,
+                              split ? (float*)ws : nullptr, split ? device_cus() : 0, s);
+    }
     GemmArgs a{};
     a.m.R = R; a.m.C = C; a.m.y_off = 0;
     a.wd = (const uint16_t*)w; a.ldw = ldw;

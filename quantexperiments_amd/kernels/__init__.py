@@ -242,12 +242,17 @@ def linear_gemm(pieces, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
 
 
 def gemm_dense(w: torch.Tensor, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
-    """Y = X . W^T for a dense fp16 / bf16 weight [R, C] (sq_gemm_dense)."""
+    """Y = X . W^T for a dense fp16 / bf16 weight [R, C] (sq_gemm_dense_ws: with the shared workspace the last partial
+    round of tiles is split along K)."""
     dev = x.device
+    L = _lib.lib()
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().sq_gemm_dense(w.data_ptr(), _lib.DTYPES[w.dtype], w.stride(0), w.shape[0], w.shape[1], x.data_ptr(),
-                                            _lib.DTYPES[x.dtype], x.stride(0), y.data_ptr(), _lib.DTYPES[y.dtype],
-                                            y.stride(0), x.shape[0], _lib.stream_ptr(dev)))
+        need = L.sq_gemm_dense_workspace_bytes(w.shape[0], w.shape[1], x.shape[0])
+        ws = _Workspace.get(need, dev) if need else None
+        _lib.check(L.sq_gemm_dense_ws(w.data_ptr(), _lib.DTYPES[w.dtype], w.stride(0), w.shape[0], w.shape[1], x.data_ptr(),
+                                      _lib.DTYPES[x.dtype], x.stride(0), y.data_ptr(), _lib.DTYPES[y.dtype],
+                                      y.stride(0), x.shape[0], None if ws is None else ws.data_ptr(),
+                                      0 if ws is None else ws.numel(), _lib.stream_ptr(dev)))
     return y
 
 

@@ -351,6 +351,28 @@ def test_gemm_dense_matches_float64():
     assert rel_max_err(y.cpu().numpy(), ref) < 1e-5
 
 
+def test_gemm_dense_with_workspace_splits_the_last_round():
+    # 8 tiles of 256 x 256 on 256 CUs: with a workspace each is cut into 4 parts along K and reduced
+    from quantexperiments_amd import _lib
+    from quantexperiments_amd.kernels import gemm_dense
+    g = torch.Generator().manual_seed(6)
+    R, C, T = 2048, 4096, 250
+    assert _lib.lib().sq_gemm_dense_workspace_bytes(R, C, T) == 4096 + 8 * 4 * 256 * 256 * 4
+    assert _lib.lib().sq_gemm_dense_workspace_bytes(R, C, 32) == 0 and _lib.lib().sq_gemm_dense_workspace_bytes(R, 4000, T) == 0
+    w = (torch.randn(R, C, generator=g) * 0.05).half().cuda()
+    x = torch.randn(T, C, generator=g).half().cuda()
+    ref = x.double().cpu().numpy() @ w.double().cpu().numpy().T
+    for dtype in (torch.float32, torch.bfloat16):
+        y = torch.full((T, R + 8), float("nan"), dtype=dtype, device="cuda")
+        gemm_dense(w, x, y[:, :R])
+        assert rel_max_err(y[:, :R].float().cpu().numpy(), ref) < (1e-5 if dtype == torch.float32 else 5e-3)
+        assert torch.isnan(y[:, R:]).all()
+        plain = torch.empty(T, R, dtype=dtype, device="cuda")
+        _lib.check(_lib.lib().sq_gemm_dense(w.data_ptr(), _lib.SQ_F16, C, R, C, x.data_ptr(), _lib.SQ_F16, C, plain.data_ptr(),
+                                            _lib.DTYPES[dtype], R, T, _lib.stream_ptr(x.device)))
+        assert rel_max_err(plain.float().cpu().numpy(), y[:, :R].float().cpu().numpy().astype(np.float64)) < (1e-5 if dtype == torch.float32 else 1e-2)
+
+
 def test_gemm_of_neighbouring_and_scattered_pieces():
     # pieces that follow each other in Y are multiplied in one tile GEMM over all their rows; pieces with gaps
     # between their column slices (or in another order) one by one.  Both through the raw C ABI.
