@@ -181,22 +181,25 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_kernel(Q8Args a) {
     }
 }
 
-// ---- 5 .. Q8_MFMA_MAX_ROWS activation rows, 3 and 4 too when C % 1024 != 0 (C % 256 == 0): fp16 MFMA, 32 activation rows per pass.
+// ---- 3 .. Q8_MFMA_MAX_ROWS activation rows (C % 256 == 0): fp16 MFMA, 16 or 32 activation rows per pass.
 // v_mfma_f32_16x16x32_f16 operand layout: A: lane l supplies weight row l % 16, k = 8 * (l / 16) .. + 7; B: token
-// l % 16, the same k; D: lane l holds token l % 16, weight rows 4 * (l / 16) .. + 3.  Weights are the A operand,
-// loaded straight into registers: a wave owns 16 rows, and per step of 128 columns lane (r, g) takes 16 bytes of
-// row r at column 128 s + 64 j + 16 g for j = 0, 1, issued back to back, so the four lanes of a row consume a whole
-// 128-byte line while it is in flight.  Each 16-byte piece feeds two MFMAs per block of 16 tokens; the k index of
-// MFMA m of piece j is column 128 s + 64 j + 16 g + 8 m + e, and the activations (B operand) are read with the
-// same mapping from LDS, where a workgroup of 8 waves (128 rows) keeps the current 256-column chunk of the fp16
-// activations (global_load_lds, double buffered).  One wave alone moves only 5 GB/s (latency), so the design is
-// many small waves: 16 rows and < 80 registers each, 24 waves per CU, two steps of loads in flight each.  What is
-// left between this kernel (4.1-4.4 TB/s) and the 4-row kernel (5.7 TB/s) is mostly the address pattern the MFMA
-// operand layout forces on direct loads (the 16 lanes of a quarter wave belong to 16 different weight rows); a
-// first version with 32 rows per wave on the 32x32x16 instruction (32 bytes per row and instruction) was 7 %
-// slower.  The block scale is folded into the fp16 weight (one rounding, as the reference's tile kernel does,
-// shapequant/kernels/batched_runs.py:442-447): all 8 weights a lane feeds to one MFMA sit in one block.
-constexpr int Q8_MFMA_MAX_ROWS = 128;           // up to here passes of 32 beat decode + tile GEMM
+// l % 16, the same k; D: lane l holds token l % 16, weight rows 4 * (l / 16) .. + 3.  Weights are the A operand and a
+// wave owns 16 rows.  The rows reach the wave through LDS: global_load_lds (no registers in between) fetches them in
+// lane order ALONG the row, one instruction = 8 rows x 128 bytes, whole cache lines with 8 consecutive lanes per
+// line, into a private ring of D steps per wave (a step = 16 rows x 128 columns = 2 KB); the wave reads its
+// fragments back in the operand layout (lane (r, g) takes pieces 2 g and 2 g + 1 of row r, 32 bytes per step), so
+// the weights need no barrier, only counted waits.  Rows are XOR-swizzled in 16-byte pieces (piece p of row r at
+// slot p ^ ((r >> 1) & 7), applied through the source addresses of the copy), so the 16 lanes of an LDS read clock
+// hit 16 different bank groups.  Block scales travel the same way (a 4-byte copy per lane: 16 bytes per row and
+// chunk of 256 columns).  Each 16-byte piece feeds two MFMAs per block of 16 tokens; the k index of MFMA m of piece
+// j is column 128 s + 16 (2 g + j) + 8 m + e, and the activations (B operand) are read with the same mapping from
+// LDS, where the workgroup keeps the current 256-column chunk of the fp16 activations (global_load_lds, double
+// buffered, one barrier per chunk).  The block scale is folded into the fp16 weight (one rounding, as the
+// reference's tile kernel does, shapequant/kernels/batched_runs.py:442-447): all 16 weights of a piece sit in one
+// block.  A first form loaded the operand layout straight from memory (lane = row, 16 bytes per lane): every
+// quarter wave then touches 16 different cache lines, and it stayed at 4.1-4.4 TB/s where this one reaches
+// 5.2-5.5 TB/s (the one-row kernel: 5.7); 32 rows per wave on the 32x32x16 instruction was slower still.
+constexpr int Q8_MFMA_MAX_ROWS = 192;           // up to here passes of 32 beat decode + tile GEMM (129 rows: 630 against 780 us)
 constexpr int Q8_XC = 256;                      // columns of x per LDS chunk (2 steps)
 
 // x [B, C] (fp16 or bf16, any stride) -> fp16 [B, C] contiguous.
@@ -223,97 +226,134 @@ struct Q8MfmaArgs {
 
 constexpr int q8_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }   // wait on vmcnt only
 
-template <int NBLK>     // 16-token blocks: 1 (up to 16 activation rows) or 2
-__global__ __launch_bounds__(512, 2) void q8_mfma_kernel(Q8MfmaArgs a) {
-    __shared__ __attribute__((aligned(16))) unsigned char xs[2][32 * Q8_XC * 2];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int task_raw = blockIdx.x * 8 + wave;
+// weights ring + scales of d - 1 chunks (with a ring of 4 steps the scales of chunk c + 2 are requested while chunk c
+// is still being multiplied)
+constexpr int q8l_wave_bytes(int d) { return d * 2048 + (d - 1) * 256; }
+constexpr int q8l_lds_bytes(int nblk, int waves, int d) { return 2 * nblk * 16 * Q8_XC * 2 + waves * q8l_wave_bytes(d); }
+
+// NBLK 16-token blocks, WAVES waves per workgroup (the first 8 NBLK copy two tokens of every x chunk each), ring of D
+// steps per wave (one being multiplied, D - 1 in flight)
+template <int NBLK, int WAVES, int D>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void q8_mfma_kernel(Q8MfmaArgs a) {
+    static_assert(D == 3 || D == 4, "wait counts below are written out for these depths");
+    constexpr int Q8L_D = D, Q8L_WAVE_BYTES = q8l_wave_bytes(D);
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char* xs = smem;                                   // [2][16 NBLK tokens][512 bytes]
+    constexpr int XBUF = NBLK * 16 * Q8_XC * 2;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    unsigned char* wl = smem + 2 * XBUF + wave * Q8L_WAVE_BYTES;  // this wave's ring
+    unsigned char* sl_ = wl + Q8L_D * 2048;                        // this wave's scales: [D - 1][16 rows][16 bytes]
+    const int task_raw = blockIdx.x * WAVES + wave;
     const bool active = task_raw < a.tasks;
     const int task = active ? task_raw : a.tasks - 1;
     const int r = lane & 15, g = lane >> 4;
     const int C = a.C, nblk = C >> 5, nsteps = C >> 7, nchunks = nsteps >> 1;
-    const int row = min(task * 16 + r, a.V - 1);
-    const int8_t* wp = a.q + (int64_t)row * C + g * 16;
-    const char* sp = (const char*)(a.sc + (int64_t)row * nblk);
 
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    uint32_t xsrc[2];                           // wave w copies activation rows 4 w .. 4 w + 3, two per instruction
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int rowx = wave * 4 + 2 * i + (lane >> 5);
+    // activations: wave w copies tokens 2 w and 2 w + 1 of a chunk (one instruction: 2 x 512 bytes); the 16-byte piece
+    // p of token t is kept at slot p ^ (t % 16), so the 16 lanes of a read clock (16 tokens, one piece) spread over
+    // 16 bank groups
+    uint32_t xsrc;
+    {
+        const int rowx = wave * 2 + (lane >> 5);
         const int piece = (lane & 31) ^ (rowx & 15);
-        xsrc[i] = (uint32_t)(min(rowx, a.B - 1) * a.ldxh + piece * 8);
+        xsrc = (uint32_t)(min(rowx, a.B - 1) * a.ldxh + piece * 8);
     }
+    const bool xo = wave < 8 * NBLK;                            // this wave takes part in the x copies
     auto copy_x = [&](int c) {
+        if (xo) __builtin_amdgcn_global_load_lds((gptr_t)(a.xh + c * Q8_XC + xsrc), (lptr_t)(xs + (c & 1) * XBUF + wave * 2 * (Q8_XC * 2)), 16, 0, 0);
+    };
+    // weights: instruction n of a step fills rows 8 n .. 8 n + 7; lane i lands in row 8 n + i / 8, slot i % 8 and
+    // fetches the piece the swizzle keeps there
+    const int8_t* wsrc[2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(a.xh + c * Q8_XC + xsrc[i]),
-                                             (lptr_t)(&xs[c & 1][(wave * 4 + 2 * i) * (Q8_XC * 2)]), 16, 0, 0);
+    for (int n = 0; n < 2; ++n) {
+        const int rw = 8 * n + (lane >> 3);
+        const int piece = (lane & 7) ^ ((rw >> 1) & 7);
+        wsrc[n] = a.q + (int64_t)min(task * 16 + rw, a.V - 1) * C + piece * 16;
+    }
+    auto copy_w = [&](int s) {
+#pragma unroll
+        for (int n = 0; n < 2; ++n)
+            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[n] + s * 128), (lptr_t)(wl + (s % Q8L_D) * 2048 + n * 1024), 16, 0, 0);
+    };
+    // scales of chunk c: lane i fetches dword i % 4 of row i / 4
+    const char* ssrc = (const char*)(a.sc + (int64_t)min(task * 16 + (lane >> 2), a.V - 1) * nblk) + (lane & 3) * 4;
+    auto copy_s = [&](int c) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(ssrc + c * 16), (lptr_t)(sl_ + (c % (D - 1)) * 256), 4, 0, 0);
     };
     const uint32_t xrow = (uint32_t)r * (Q8_XC * 2), xsw = (uint32_t)r;
-    const uint32_t sshift = (uint32_t)(g >> 1) << 4;        // which half of a scale pair this lane's pieces use
+    const uint32_t wsw = (uint32_t)((r >> 1) & 7);
+    const uint32_t w0 = (uint32_t)r * 128 + (((uint32_t)(2 * g) ^ wsw) << 4), w1 = (uint32_t)r * 128 + (((uint32_t)(2 * g + 1) ^ wsw) << 4);
 
     float4v acc[NBLK];
 #pragma unroll
     for (int nb = 0; nb < NBLK; ++nb) acc[nb] = float4v{0.f, 0.f, 0.f, 0.f};
-    u32x4 wr[2][2];
-    u32x2 sr[2];
+
+    // Issue order per wave (X = this wave's x copy of a chunk, S = scales of a chunk, W = the 2 copies of a step):
+    // S(c) goes right before W(2c); step s starts (even s: after the wait and the barrier, then X(s/2 + 1)) with the
+    // refill of step s + D - 1.  Waits count the operations that may stay in flight:
+    //   even s (needs X, S, W of its chunk):  D = 3: W(s+1) -> 2;           D = 4: W(s+1) S W(s+2) -> 5
+    //   odd s (needs W(s)):  D = 3: X S W(s+1) W(s+2) -> 5 + x;  D = 4: S W(s+1) X W(s+2) S W(s+3) -> 8 + x
+    // and fall back to "everything" near the end of the row, where refills stop.
+    auto refill = [&](int f) {
+        if (f < nsteps) {
+            if (!(f & 1)) copy_s(f >> 1);
+            copy_w(f);
+        }
+    };
     copy_x(0);
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-        const int s0 = p < nsteps ? p : nsteps - 1;
-        wr[p][0] = *reinterpret_cast<const u32x4*>(wp + s0 * 128);
-        wr[p][1] = *reinterpret_cast<const u32x4*>(wp + s0 * 128 + 64);
-        sr[p] = *reinterpret_cast<const u32x2*>(sp + s0 * 8);
-    }
-    for (int c = 0; c < nchunks; ++c) {
-        // chunk c was requested one chunk ago, before the 6 loads of that chunk's two refills
-        if (c == 0 || c == nchunks - 1) __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
-        else __builtin_amdgcn_s_waitcnt(q8_vmcnt(6));
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        if (c + 1 < nchunks) copy_x(c + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        const unsigned char* xc = &xs[c & 1][0] + xrow;
-#pragma unroll
-        for (int sl = 0; sl < 2; ++sl) {
-            const int s = c * 2 + sl;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const half_t sh = __builtin_bit_cast(half_t, (uint16_t)(sr[sl][j] >> sshift));
-                const half2v s2 = {sh, sh};
-                half2v p[8];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const uint32_t wk = wr[sl][j][k];
-                    i8x4_to_h2(wk, p[2 * k], p[2 * k + 1]);
-                }
-#pragma unroll
-                for (int k = 0; k < 8; ++k) p[k] = p[k] * s2;
-                half8v a0, a1;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    a0[2 * k] = p[k][0]; a0[2 * k + 1] = p[k][1];
-                    a1[2 * k] = p[4 + k][0]; a1[2 * k + 1] = p[4 + k][1];
-                }
-                const uint32_t p0 = (uint32_t)(sl * 16 + j * 8 + g * 2);      // pieces p0, p0 + 1 of the token's row
-#pragma unroll
-                for (int nb = 0; nb < NBLK; ++nb) {
-                    const unsigned char* xt = xc + nb * (16 * Q8_XC * 2);
-                    const half8v x0 = *reinterpret_cast<const half8v*>(xt + ((p0 ^ xsw) << 4));
-                    const half8v x1 = *reinterpret_cast<const half8v*>(xt + (((p0 + 1) ^ xsw) << 4));
-                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, x0, acc[nb], 0, 0, 0);
-                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, x1, acc[nb], 0, 0, 0);
-                }
-            }
-            if (s + 2 < nsteps) {
-                wr[sl][0] = *reinterpret_cast<const u32x4*>(wp + (s + 2) * 128);
-                wr[sl][1] = *reinterpret_cast<const u32x4*>(wp + (s + 2) * 128 + 64);
-                sr[sl] = *reinterpret_cast<const u32x2*>(sp + (s + 2) * 8);
+    for (int t = 0; t < D - 1; ++t) refill(t);
+    for (int s = 0; s < nsteps; ++s) {
+        const int c = s >> 1, odd = s & 1;
+        if (!odd) {
+            if (s + D - 2 < nsteps) __builtin_amdgcn_s_waitcnt(q8_vmcnt(D == 3 ? 2 : 5));
+            else __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            if (c + 1 < nchunks) copy_x(c + 1);
+            refill(s + D - 1);
+        } else {
+            refill(s + D - 1);
+            if (s + D - 1 < nsteps) {
+                if (xo) __builtin_amdgcn_s_waitcnt(q8_vmcnt(D == 3 ? 6 : 9));
+                else __builtin_amdgcn_s_waitcnt(q8_vmcnt(D == 3 ? 5 : 8));
+            } else {
+                __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned char* st = wl + (s % Q8L_D) * 2048;
+        const u32x4 wq[2] = {*reinterpret_cast<const u32x4*>(st + w0), *reinterpret_cast<const u32x4*>(st + w1)};
+        const half_t sh = __builtin_bit_cast(half_t, *reinterpret_cast<const uint16_t*>(sl_ + (c % (D - 1)) * 256 + r * 16 + odd * 8 + g * 2));
+        const half2v s2 = {sh, sh};
+        const unsigned char* xc = xs + (c & 1) * XBUF + xrow;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            half2v p[8];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) i8x4_to_h2(wq[j][k], p[2 * k], p[2 * k + 1]);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) p[k] = p[k] * s2;
+            half8v a0, a1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                a0[2 * k] = p[k][0]; a0[2 * k + 1] = p[k][1];
+                a1[2 * k] = p[4 + k][0]; a1[2 * k + 1] = p[4 + k][1];
+            }
+            const uint32_t p0 = (uint32_t)(odd * 16 + (2 * g + j) * 2);   // x pieces (8 halves each) of these 16 columns
+#pragma unroll
+            for (int nb = 0; nb < NBLK; ++nb) {
+                const unsigned char* xt = xc + nb * (16 * Q8_XC * 2);
+                const half8v x0 = *reinterpret_cast<const half8v*>(xt + ((p0 ^ xsw) << 4));
+                const half8v x1 = *reinterpret_cast<const half8v*>(xt + (((p0 + 1) ^ xsw) << 4));
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, x0, acc[nb], 0, 0, 0);
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, x1, acc[nb], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
     if (!active) return;
     const int orow = task * 16 + g * 4;
@@ -423,12 +463,9 @@ static int q8_pass_rows(int B, int C) {
 // 32-bit offsets.
 static bool q8_mfma_ok(int C) { return C % 256 == 0 && (int64_t)C * 32 < ((int64_t)1 << 31); }
 
-// 3 and 4 rows: the 4-row kernel walks a row in 1 KB steps and is VALU-bound there, so it wins when C fills its last
-// step (248,320 x 5,120: 255 us against 312 us on the MFMA passes) and loses otherwise (152,064 x 3,584: 148 against 131)
-bool q8_mid(int C, int B) {
-    return B <= Q8_MFMA_MAX_ROWS && q8_mfma_ok(C) && (B > 4 || (B > 2 && C % 1024 != 0));
-}
-
+// from 3 rows the MFMA passes win over the 4-row kernel (152,064 x 3,584: 106 against 148 us; 248,320 x 5,120: 246
+// against 255 us); 2 rows stay on the exact-product kernel (106-115 / 228 us)
+bool q8_mid(int C, int B) { return B > 2 && B <= Q8_MFMA_MAX_ROWS && q8_mfma_ok(C); }
 size_t q8_mid_workspace(int C, int B) { return q8_mid(C, B) ? (((size_t)B * C * 2) + 255) & ~(size_t)255 : 0; }
 
 int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
@@ -459,8 +496,19 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
         a.y = (char*)y + (size_t)b0 * ldy * ys;
         a.ldy = ldy; a.V = V; a.C = C; a.B = B - b0 < 32 ? B - b0 : 32; a.y_dtype = y_dtype; a.tasks = tasks;
         a.vec_y = ((uintptr_t)a.y & 7) == 0 && ldy % 4 == 0;
-        if (a.B > 16) hipLaunchKernelGGL(q8_mfma_kernel<2>, dim3((unsigned)((tasks + 7) / 8)), dim3(512), 0, s, a);
-        else hipLaunchKernelGGL(q8_mfma_kernel<1>, dim3((unsigned)((tasks + 7) / 8)), dim3(512), 0, s, a);
+        static bool raised = false;
+        if (!raised) {
+            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<1, 8, 3>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<2, 16, 3>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipGetLastError();
+            raised = true;
+        }
+        // up to 16 rows: 8 waves per workgroup, 68 KB of LDS, two workgroups per CU; 17-32 rows: the x chunks double,
+        // so one workgroup of 16 waves per CU shares them (136 KB)
+        if (a.B > 16)
+            hipLaunchKernelGGL((q8_mfma_kernel<2, 16, 3>), dim3((unsigned)((tasks + 15) / 16)), dim3(1024), q8l_lds_bytes(2, 16, 3), s, a);
+        else
+            hipLaunchKernelGGL((q8_mfma_kernel<1, 8, 3>), dim3((unsigned)((tasks + 7) / 8)), dim3(512), q8l_lds_bytes(1, 8, 3), s, a);
         rc = check_launch("q8_mfma_kernel");
         if (rc) return rc;
     }
