@@ -229,17 +229,17 @@ constexpr int q8_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | 
 // weights ring + scales of d - 1 chunks (with a ring of 4 steps the scales of chunk c + 2 are requested while chunk c
 // is still being multiplied)
 constexpr int q8l_wave_bytes(int d) { return d * 2048 + (d - 1) * 256; }
-constexpr int q8l_lds_bytes(int nblk, int waves, int d) { return 2 * nblk * 16 * Q8_XC * 2 + waves * q8l_wave_bytes(d); }
+constexpr int q8l_lds_bytes(int nblk, int waves, int d, int xs) { return 2 * nblk * 16 * xs * 256 + waves * q8l_wave_bytes(d); }
 
-// NBLK 16-token blocks, WAVES waves per workgroup (the first 8 NBLK copy two tokens of every x chunk each), ring of D
-// steps per wave (one being multiplied, D - 1 in flight)
-template <int NBLK, int WAVES, int D>
+// NBLK 16-token blocks, WAVES waves per workgroup, ring of D steps per wave (one being multiplied, D - 1 in flight),
+// x chunks of XS steps (128 XS columns; the first 16 NBLK XS / 4 waves copy 4 / XS tokens of every chunk each)
+template <int NBLK, int WAVES, int D, int XS>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void q8_mfma_kernel(Q8MfmaArgs a) {
-    static_assert(D == 3 || D == 4, "wait counts below are written out for these depths");
+    static_assert((D == 3 || D == 4) && (XS == 2 || (XS == 1 && D == 3)), "wait counts below are written out for these");
     constexpr int Q8L_D = D, Q8L_WAVE_BYTES = q8l_wave_bytes(D);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    unsigned char* xs = smem;                                   // [2][16 NBLK tokens][512 bytes]
-    constexpr int XBUF = NBLK * 16 * Q8_XC * 2;
+    unsigned char* xs = smem;                                   // [2][16 NBLK tokens][256 XS bytes]
+    constexpr int XPITCH = XS * 256, XBUF = NBLK * 16 * XPITCH;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     unsigned char* wl = smem + 2 * XBUF + wave * Q8L_WAVE_BYTES;  // this wave's ring
     unsigned char* sl_ = wl + Q8L_D * 2048;                        // this wave's scales: [D - 1][16 rows][16 bytes]
@@ -247,22 +247,22 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void q8_mfma_kernel
     const bool active = task_raw < a.tasks;
     const int task = active ? task_raw : a.tasks - 1;
     const int r = lane & 15, g = lane >> 4;
-    const int C = a.C, nblk = C >> 5, nsteps = C >> 7, nchunks = nsteps >> 1;
+    const int C = a.C, nblk = C >> 5, nsteps = C >> 7, nchunks = nsteps / XS;
 
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    // activations: wave w copies tokens 2 w and 2 w + 1 of a chunk (one instruction: 2 x 512 bytes); the 16-byte piece
-    // p of token t is kept at slot p ^ (t % 16), so the 16 lanes of a read clock (16 tokens, one piece) spread over
-    // 16 bank groups
+    // activations: one copy instruction moves 1 KB = 4 / XS tokens of a chunk; the 16-byte piece p of token t is kept
+    // at slot p ^ (t % 16), so the 16 lanes of a read clock (16 tokens, one piece) spread over 16 bank groups
+    constexpr int TPI = 4 / XS, LPT = 64 / TPI;                 // tokens per instruction, lanes (= pieces) per token
     uint32_t xsrc;
     {
-        const int rowx = wave * 2 + (lane >> 5);
-        const int piece = (lane & 31) ^ (rowx & 15);
+        const int rowx = wave * TPI + lane / LPT;
+        const int piece = (lane % LPT) ^ (rowx & 15);
         xsrc = (uint32_t)(min(rowx, a.B - 1) * a.ldxh + piece * 8);
     }
-    const bool xo = wave < 8 * NBLK;                            // this wave takes part in the x copies
+    const bool xo = wave * TPI < 16 * NBLK;                     // this wave takes part in the x copies
     auto copy_x = [&](int c) {
-        if (xo) __builtin_amdgcn_global_load_lds((gptr_t)(a.xh + c * Q8_XC + xsrc), (lptr_t)(xs + (c & 1) * XBUF + wave * 2 * (Q8_XC * 2)), 16, 0, 0);
+        if (xo) __builtin_amdgcn_global_load_lds((gptr_t)(a.xh + c * (XS * 128) + xsrc), (lptr_t)(xs + (c & 1) * XBUF + wave * TPI * XPITCH), 16, 0, 0);
     };
     // weights: instruction n of a step fills rows 8 n .. 8 n + 7; lane i lands in row 8 n + i / 8, slot i % 8 and
     // fetches the piece the swizzle keeps there
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void q8_mfma_kernel
     auto copy_s = [&](int c) {
         __builtin_amdgcn_global_load_lds((gptr_t)(ssrc + c * 16), (lptr_t)(sl_ + (c % (D - 1)) * 256), 4, 0, 0);
     };
-    const uint32_t xrow = (uint32_t)r * (Q8_XC * 2), xsw = (uint32_t)r;
+    const uint32_t xrow = (uint32_t)r * XPITCH, xsw = (uint32_t)r;
     const uint32_t wsw = (uint32_t)((r >> 1) & 7);
     const uint32_t w0 = (uint32_t)r * 128 + (((uint32_t)(2 * g) ^ wsw) << 4), w1 = (uint32_t)r * 128 + (((uint32_t)(2 * g + 1) ^ wsw) << 4);
 
@@ -307,13 +307,21 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void q8_mfma_kernel
 #pragma unroll
     for (int t = 0; t < D - 1; ++t) refill(t);
     for (int s = 0; s < nsteps; ++s) {
-        const int c = s >> 1, odd = s & 1;
-        if (!odd) {
+        const int c = s >> 1, odd = s & 1, cx = s / XS;         // chunk of scales, step in it, chunk of x
+        if (XS == 1) {
+            // every step opens an x chunk: X(s) was issued one step ago, before [S] W(s + 1)
+            if (s + 1 < nsteps) { if (odd) __builtin_amdgcn_s_waitcnt(q8_vmcnt(3)); else __builtin_amdgcn_s_waitcnt(q8_vmcnt(2)); }
+            else __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            if (cx + 1 < nchunks) copy_x(cx + 1);
+            refill(s + D - 1);
+        } else if (!odd) {
             if (s + D - 2 < nsteps) __builtin_amdgcn_s_waitcnt(q8_vmcnt(D == 3 ? 2 : 5));
             else __builtin_amdgcn_s_waitcnt(q8_vmcnt(0));
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
-            if (c + 1 < nchunks) copy_x(c + 1);
+            if (cx + 1 < nchunks) copy_x(cx + 1);
             refill(s + D - 1);
         } else {
             refill(s + D - 1);
@@ -329,7 +337,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void q8_mfma_kernel
         const u32x4 wq[2] = {*reinterpret_cast<const u32x4*>(st + w0), *reinterpret_cast<const u32x4*>(st + w1)};
         const half_t sh = __builtin_bit_cast(half_t, *reinterpret_cast<const uint16_t*>(sl_ + (c % (D - 1)) * 256 + r * 16 + odd * 8 + g * 2));
         const half2v s2 = {sh, sh};
-        const unsigned char* xc = xs + (c & 1) * XBUF + xrow;
+        const unsigned char* xc = xs + (cx & 1) * XBUF + xrow;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             half2v p[8];
@@ -343,10 +351,10 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void q8_mfma_kernel
                 a0[2 * k] = p[k][0]; a0[2 * k + 1] = p[k][1];
                 a1[2 * k] = p[4 + k][0]; a1[2 * k + 1] = p[4 + k][1];
             }
-            const uint32_t p0 = (uint32_t)(odd * 16 + (2 * g + j) * 2);   // x pieces (8 halves each) of these 16 columns
+            const uint32_t p0 = (uint32_t)((s % XS) * 16 + (2 * g + j) * 2);   // x pieces (8 halves each) of these 16 columns
 #pragma unroll
             for (int nb = 0; nb < NBLK; ++nb) {
-                const unsigned char* xt = xc + nb * (16 * Q8_XC * 2);
+                const unsigned char* xt = xc + nb * (16 * XPITCH);
                 const half8v x0 = *reinterpret_cast<const half8v*>(xt + ((p0 ^ xsw) << 4));
                 const half8v x1 = *reinterpret_cast<const half8v*>(xt + (((p0 + 1) ^ xsw) << 4));
                 acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, x0, acc[nb], 0, 0, 0);
@@ -498,17 +506,24 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
         a.vec_y = ((uintptr_t)a.y & 7) == 0 && ldy % 4 == 0;
         static bool raised = false;
         if (!raised) {
-            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<1, 8, 3>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<2, 16, 3>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<1, 8, 3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<2, 16, 3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<2, 8, 3, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             (void)hipGetLastError();
             raised = true;
         }
-        // up to 16 rows: 8 waves per workgroup, 68 KB of LDS, two workgroups per CU; 17-32 rows: the x chunks double,
-        // so one workgroup of 16 waves per CU shares them (136 KB)
-        if (a.B > 16)
-            hipLaunchKernelGGL((q8_mfma_kernel<2, 16, 3>), dim3((unsigned)((tasks + 15) / 16)), dim3(1024), q8l_lds_bytes(2, 16, 3), s, a);
+        // 17-32 rows: one workgroup of 16 waves per CU sharing 256-column x chunks, unless its workgroups fill the last
+        // round of the chip badly; then 8 waves with 128-column chunks (a barrier per step, two workgroups per CU).
+        // Measured: 152,064 x 3,584 (594 workgroups of 16 waves, 2.3 rounds) 126 against 116 us; 248,320 x 5,120
+        // (970, 3.8 rounds) 265 against 278 us.
+        const int cus = device_cus(), n16 = (tasks + 15) / 16;
+        const bool x128 = (double)n16 / ((double)((n16 + cus - 1) / cus) * cus) < 0.85;
+        if (a.B > 16 && x128)
+            hipLaunchKernelGGL((q8_mfma_kernel<2, 8, 3, 1>), dim3((unsigned)((tasks + 7) / 8)), dim3(512), q8l_lds_bytes(2, 8, 3, 1), s, a);
+        else if (a.B > 16)
+            hipLaunchKernelGGL((q8_mfma_kernel<2, 16, 3, 2>), dim3((unsigned)((tasks + 15) / 16)), dim3(1024), q8l_lds_bytes(2, 16, 3, 2), s, a);
         else
-            hipLaunchKernelGGL((q8_mfma_kernel<1, 8, 3>), dim3((unsigned)((tasks + 7) / 8)), dim3(512), q8l_lds_bytes(1, 8, 3), s, a);
+            hipLaunchKernelGGL((q8_mfma_kernel<1, 8, 3, 2>), dim3((unsigned)((tasks + 7) / 8)), dim3(512), q8l_lds_bytes(1, 8, 3, 2), s, a);
         rc = check_launch("q8_mfma_kernel");
         if (rc) return rc;
     }
