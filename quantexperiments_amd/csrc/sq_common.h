@@ -41,6 +41,26 @@ __device__ __forceinline__ uint32_t bf2h_x2(uint32_t v) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
+// 16-bit activations of a run-time dtype (SQ_F16 / SQ_BF16)
+__device__ __forceinline__ float load16(const void* p, int dtype, int64_t i) {
+    const uint16_t b = reinterpret_cast<const uint16_t*>(p)[i];
+    return dtype == SQ_BF16 ? bf2f(b) : h2f(b);
+}
+__device__ __forceinline__ uint16_t round16(float v, int dtype) { return dtype == SQ_BF16 ? f2bf(v) : f2h(v); }
+
+// silu(g) * u with the reference's rounding points (shapequant/kernels/decode_e2e.py:125-136): SiLU in fp32 rounded
+// to the model dtype, then the product rounded to the model dtype.  One definition, because the stand-alone kernel
+// and the products that compute their own input must agree bit for bit.
+__device__ __forceinline__ uint16_t silu_mul_one(uint16_t g, uint16_t u, int dtype) {
+    if (dtype == SQ_BF16) {
+        const float a = bf2f(g);
+        return f2bf(bf2f(f2bf(a / (1.f + __expf(-a)))) * bf2f(u));
+    }
+    const float a = h2f(g);
+    const half_t s = (half_t)(a / (1.f + __expf(-a)));
+    return __builtin_bit_cast(uint16_t, (half_t)(s * __builtin_bit_cast(half_t, u)));
+}
+
 template <int DT> struct store_as;
 template <> struct store_as<SQ_F32> { typedef float type; static __device__ __forceinline__ float cvt(float f) { return f; } };
 template <> struct store_as<SQ_F16> { typedef uint16_t type; static __device__ __forceinline__ uint16_t cvt(float f) { return f2h(f); } };

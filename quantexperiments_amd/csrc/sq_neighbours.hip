@@ -11,12 +11,6 @@ namespace sq {
 constexpr int NB_THREADS = 1024;
 constexpr int NB_MAX_LDS_C = 32256;          // a row staged as 16-bit values for the column-order copies: 63 KB of LDS
 
-__device__ __forceinline__ float load16(const void* p, int dtype, int64_t i) {
-    const uint16_t b = reinterpret_cast<const uint16_t*>(p)[i];
-    return dtype == SQ_BF16 ? bf2f(b) : h2f(b);
-}
-__device__ __forceinline__ uint16_t round16(float v, int dtype) { return dtype == SQ_BF16 ? f2bf(v) : f2h(v); }
-
 // sum over the workgroup, the same value in every thread
 __device__ __forceinline__ float block_sum(float v, float* red) {
     v = wave_sum(v);
@@ -127,18 +121,6 @@ struct SiluArgs {
     int64_t ld;
     int dtype, M, C, blocks_per_row, vec;
 };
-
-// SiLU in fp32 rounded to the model dtype, then the product in the model dtype (what the reference's model code and
-// its kernel do: fp16 silu, fp16 multiply)
-__device__ __forceinline__ uint16_t silu_mul_one(uint16_t g, uint16_t u, int dtype) {
-    if (dtype == SQ_BF16) {
-        const float a = bf2f(g);
-        return f2bf(bf2f(f2bf(a / (1.f + __expf(-a)))) * bf2f(u));
-    }
-    const float a = h2f(g);
-    const half_t s = (half_t)(a / (1.f + __expf(-a)));
-    return __builtin_bit_cast(uint16_t, (half_t)(s * __builtin_bit_cast(half_t, u)));
-}
 
 __global__ __launch_bounds__(NB_THREADS) void silu_mul_kernel(SiluArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint16_t row16[];

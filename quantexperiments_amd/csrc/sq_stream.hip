@@ -251,18 +251,6 @@ struct StreamArgs {
     float eps;
 };
 
-// element i of the produced activation row, as 16 bits of dtype
-__device__ __forceinline__ uint16_t pro_round(float v, int dtype) { return dtype == SQ_BF16 ? f2bf(v) : f2h(v); }
-__device__ __forceinline__ float pro_load(const uint16_t* p, int dtype, int i) { return dtype == SQ_BF16 ? bf2f(p[i]) : h2f(p[i]); }
-__device__ __forceinline__ uint16_t pro_silu_mul(uint16_t g, uint16_t u, int dtype) {
-    if (dtype == SQ_BF16) {
-        const float a = bf2f(g);
-        return f2bf(bf2f(f2bf(a / (1.f + __expf(-a)))) * bf2f(u));
-    }
-    const float a = h2f(g);
-    const half_t sv = (half_t)(a / (1.f + __expf(-a)));
-    return __builtin_bit_cast(uint16_t, (half_t)(sv * __builtin_bit_cast(half_t, u)));
-}
 // The operands of one chunk (8 elements) of the produced row, fetched first and finished once the row's scale is known.
 // PRO 1: h, lo = add, hi = w.  PRO 2: lo = gate, hi = up.
 struct ProRaw { float h[8]; uint32_t lo[4], hi[4]; };
@@ -311,9 +299,9 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         if (PRO == 2)
-            e[k] = pro_silu_mul((uint16_t)(r.lo[k >> 1] >> (16 * (k & 1))), (uint16_t)(r.hi[k >> 1] >> (16 * (k & 1))), a.x_dtype);
+            e[k] = silu_mul_one((uint16_t)(r.lo[k >> 1] >> (16 * (k & 1))), (uint16_t)(r.hi[k >> 1] >> (16 * (k & 1))), a.x_dtype);
         else
-            e[k] = pro_round(pro_v(a, r, k) * rstd * pro_f(r.hi[k >> 1], k, a.x_dtype), a.x_dtype);
+            e[k] = round16(pro_v(a, r, k) * rstd * pro_f(r.hi[k >> 1], k, a.x_dtype), a.x_dtype);
     }
     return u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
 }
