@@ -206,7 +206,9 @@ int sq_silu_mul(const void* gate, const void* up, int dtype, int64_t ld, const i
  * mode SQ_FROM_ADDNORM: X = round(v * rsqrt(mean(v^2) + eps) * w), v = h_in + add (add NULL: v = h_in), h_out = v
  * if not NULL (h_out must not be h_in).  mode SQ_FROM_SILU_MUL: X = silu(add) * up.  add / up / w / x_out hold
  * x_dtype; rows b of h_in / h_out at b * ld_h, of add / up at b * ld_in, of x_out at b * C.  x_out is always
- * written (it must be 16-byte aligned and C % 8 == 0). */
+ * written (it must be 16-byte aligned and C % 8 == 0); x_out and h_out must not overlap h_in / add / up / w (the
+ * reference lets its epilogue write into x's buffer because it runs after every block has read x; here workgroups
+ * still read the operands while one of them writes). */
 #define SQ_FROM_ADDNORM 1
 #define SQ_FROM_SILU_MUL 2
 typedef struct sq_producer {

@@ -116,6 +116,18 @@ int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_produce
     if (C % 8 || ((uintptr_t)from->x_out & 15)) return fail(SQ_EINVAL, "%s: x_out must be 16-byte aligned and C %% 8 == 0", who);
     if (addnorm && (!from->h_in || !from->w)) return fail(SQ_EINVAL, "%s: null h_in / w", who);
     if (addnorm && from->h_out == from->h_in) return fail(SQ_EINVAL, "%s: h_out must not be h_in", who);
+    {
+        // workgroups read the producer's operands while others already write x_out / h_out: no overlap allowed
+        auto overlap = [](const void* p, size_t n, const void* q, size_t m) {
+            return p && q && (const char*)p < (const char*)q + m && (const char*)q < (const char*)p + n;
+        };
+        const size_t xo = (size_t)B * C * 2, in16 = ((size_t)(B - 1) * (size_t)(B > 1 ? from->ld_in : 0) + C) * 2;
+        const size_t h32 = ((size_t)(B - 1) * (size_t)(B > 1 ? from->ld_h : 0) + C) * 4;
+        if (overlap(from->x_out, xo, from->add, in16) || overlap(from->x_out, xo, from->up, in16) ||
+            (addnorm && (overlap(from->x_out, xo, from->h_in, h32) || overlap(from->x_out, xo, from->w, (size_t)C * 2) ||
+                         overlap(from->h_out, h32, from->add, in16) || overlap(from->h_out, h32, from->h_in, h32))))
+            return fail(SQ_EINVAL, "%s: x_out / h_out must not overlap the producer's operands", who);
+    }
     if (!addnorm && (!from->add || !from->up)) return fail(SQ_EINVAL, "%s: null gate / up", who);
     if (B > 1 && ((addnorm && from->ld_h < C) || ((from->add || !addnorm) && from->ld_in < C)))
         return fail(SQ_EINVAL, "%s: ld_h %lld / ld_in %lld too small", who, (long long)from->ld_h, (long long)from->ld_in);

@@ -245,6 +245,12 @@ def test_linear_small_from_rejects_bad_arguments():
         linear_small_from(lins, y, x_out, h_in=h, w=w, h_out=h)             # workgroups still read h_in while one writes
     with pytest.raises(ValueError):
         linear_small_from(lins, y, x_out, gate=x_out, up=x_out.half())
+    add = torch.zeros(1, 512, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.SqError):
+        linear_small_from(lins, y, add, h_in=h, add=add, w=w)                # the row would be overwritten while it is read
+    gu = torch.zeros(1, 1024, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.SqError):
+        linear_small_from(lins, y, gu[:, :512], gate=gu[:, :512], up=gu[:, 512:])
 
 
 def test_decode_layer_with_fused_producers_under_graph():
