@@ -148,12 +148,12 @@ int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, i
  * sq_q8_linear: Y[b, v] = sum_c X[b, c] * w[v, c] for B activation rows, fp32 accumulation with the block scale
  * applied to each block's fp32 sum (the reference kernel's arithmetic, shapequant/kernels/batched_runs.py:376-440).
  * One or two rows (up to SQ_SMALL_BMAX when C % 256 != 0, 4 per pass) stream q through an exact-product kernel that
- * needs no workspace; otherwise 3 .. 192 rows run fp16 MFMA passes of up to 32 rows with the block scale
+ * needs no workspace; otherwise 3 .. 320 rows run fp16 MFMA passes of up to 64 rows with the block scale
  * folded into the fp16 weight (one rounding) and need the workspace sq_q8_workspace_bytes names (an fp16 copy of
  * the activations).  It replaces gemv_q8_batched /
  * gemv_q8_tile (reference shapequant/kernels/batched_runs.py:826-861, called from vllm_ext/core.py:575-583) and
  * proto_formats.gemv_q8 (shapequant/kernels/proto_formats.py:474-482); it reads the file's natural layout, so
- * there is no counterpart of the reference's tile-major copy.  B > 192 (B > SQ_SMALL_BMAX when C % 256 != 0) decodes row chunks to fp16 in
+ * there is no counterpart of the reference's tile-major copy.  B > 320 (B > SQ_SMALL_BMAX when C % 256 != 0) decodes row chunks to fp16 in
  * the workspace (scale folded in, one rounding) and multiplies them with the tile GEMM, as the reference's chunked
  * route does (vllm_ext/core.py:584-591); sq_q8_workspace_bytes gives the size (0 for B <= 2), with the
  * same rules as sq_workspace_bytes.  x_dtype / y_dtype as in sq_linear_small. */

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_kernel(Q8Args a) {
     }
 }
 
-// ---- 3 .. Q8_MFMA_MAX_ROWS activation rows (C % 256 == 0): fp16 MFMA, 16 or 32 activation rows per pass.
+// ---- 3 .. Q8_MFMA_MAX_ROWS activation rows (C % 256 == 0): fp16 MFMA, 16, 32 or 64 activation rows per pass.
 // v_mfma_f32_16x16x32_f16 operand layout: A: lane l supplies weight row l % 16, k = 8 * (l / 16) .. + 7; B: token
 // l % 16, the same k; D: lane l holds token l % 16, weight rows 4 * (l / 16) .. + 3.  Weights are the A operand and a
 // wave owns 16 rows.  The rows reach the wave through LDS: global_load_lds (no registers in between) fetches them in
@@ -199,7 +199,8 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_kernel(Q8Args a) {
 // block.  A first form loaded the operand layout straight from memory (lane = row, 16 bytes per lane): every
 // quarter wave then touches 16 different cache lines, and it stayed at 4.1-4.4 TB/s where this one reaches
 // 5.2-5.5 TB/s (the one-row kernel: 5.7); 32 rows per wave on the 32x32x16 instruction was slower still.
-constexpr int Q8_MFMA_MAX_ROWS = 192;           // up to here passes of 32 beat decode + tile GEMM (129 rows: 630 against 780 us)
+constexpr int Q8_MFMA_MAX_ROWS = 320;           // up to here passes of 64 beat decode + tile GEMM (152,064 x 3,584: 151 us per pass,
+                                                // 5 passes 755 us against ~880; 8 passes 1208 against 961 at 512 rows)
 constexpr int Q8_XC = 256;                      // columns of x per LDS chunk (2 steps)
 
 // x [B, C] (fp16 or bf16, any stride) -> fp16 [B, C] contiguous.
@@ -467,9 +468,9 @@ static int q8_pass_rows(int B, int C) {
     return nb;
 }
 
-// The MFMA passes need C % 256 == 0 (whole 256-column chunks of x) and 32 activation rows of C halves within
+// The MFMA passes need C % 256 == 0 (whole 256-column chunks of x) and 64 activation rows of C halves within
 // 32-bit offsets.
-static bool q8_mfma_ok(int C) { return C % 256 == 0 && (int64_t)C * 32 < ((int64_t)1 << 31); }
+static bool q8_mfma_ok(int C) { return C % 256 == 0 && (int64_t)C * 64 < ((int64_t)1 << 31); }
 
 // from 3 rows the MFMA passes win over the 4-row kernel (152,064 x 3,584: 106 against 148 us; 248,320 x 5,120: 246
 // against 255 us); 2 rows stay on the exact-product kernel (106-115 / 228 us)
@@ -485,7 +486,7 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
     const uint16_t* xh = (const uint16_t*)x;
     int64_t ldxh = ldx;
     int rc;
-    if (x_dtype != SQ_F16 || ((uintptr_t)x & 15) || ldx % 8 || ldx * 32 >= ((int64_t)1 << 31)) {
+    if (x_dtype != SQ_F16 || ((uintptr_t)x & 15) || ldx % 8 || ldx * 64 >= ((int64_t)1 << 31)) {
         const int64_t n = (int64_t)B * C;
         const int64_t want = (n + 255) / 256;
         hipLaunchKernelGGL(q8_x_kernel, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, s, (const uint16_t*)x, ldx, B,
@@ -496,19 +497,21 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
         ldxh = C;
     }
     const int tasks = (V + 15) / 16;
-    for (int b0 = 0; b0 < B; b0 += 32) {
+    for (int b0 = 0; b0 < B;) {
+        const int pass = B - b0 > 32 ? 64 : 32;                  // activation rows of this pass at most
         Q8MfmaArgs a{};
         a.q = q; a.sc = sc;
         a.xh = xh + (int64_t)b0 * ldxh;
         a.ldxh = (int)ldxh;
         a.y = (char*)y + (size_t)b0 * ldy * ys;
-        a.ldy = ldy; a.V = V; a.C = C; a.B = B - b0 < 32 ? B - b0 : 32; a.y_dtype = y_dtype; a.tasks = tasks;
+        a.ldy = ldy; a.V = V; a.C = C; a.B = B - b0 < pass ? B - b0 : pass; a.y_dtype = y_dtype; a.tasks = tasks;
         a.vec_y = ((uintptr_t)a.y & 7) == 0 && ldy % 4 == 0;
         static bool raised = false;
         if (!raised) {
             (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<1, 8, 3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<2, 16, 3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<2, 8, 3, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)q8_mfma_kernel<4, 16, 3, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             (void)hipGetLastError();
             raised = true;
         }
@@ -518,7 +521,9 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
         // (970, 3.8 rounds) 265 against 278 us.
         const int cus = device_cus(), n16 = (tasks + 15) / 16;
         const bool x128 = (double)n16 / ((double)((n16 + cus - 1) / cus) * cus) < 0.85;
-        if (a.B > 16 && x128)
+        if (a.B > 32)                                           // 33-64 rows: 16 waves share 128-column chunks of 64 tokens
+            hipLaunchKernelGGL((q8_mfma_kernel<4, 16, 3, 1>), dim3((unsigned)((tasks + 15) / 16)), dim3(1024), q8l_lds_bytes(4, 16, 3, 1), s, a);
+        else if (a.B > 16 && x128)
             hipLaunchKernelGGL((q8_mfma_kernel<2, 8, 3, 1>), dim3((unsigned)((tasks + 7) / 8)), dim3(512), q8l_lds_bytes(2, 8, 3, 1), s, a);
         else if (a.B > 16)
             hipLaunchKernelGGL((q8_mfma_kernel<2, 16, 3, 2>), dim3((unsigned)((tasks + 15) / 16)), dim3(1024), q8l_lds_bytes(2, 16, 3, 2), s, a);
@@ -526,6 +531,7 @@ int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void*
             hipLaunchKernelGGL((q8_mfma_kernel<1, 8, 3, 2>), dim3((unsigned)((tasks + 7) / 8)), dim3(512), q8l_lds_bytes(1, 8, 3, 2), s, a);
         rc = check_launch("q8_mfma_kernel");
         if (rc) return rc;
+        b0 += a.B;
     }
     return SQ_OK;
 }

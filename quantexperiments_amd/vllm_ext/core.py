@@ -232,8 +232,8 @@ class Q8Head:
     (reference shapequant/vllm_ext/core.py:489-591, same constructor, attributes and forward / R interface
     as PackedShards, so it runs through the shapequant::linear op).
 
-      sq_q8_linear routes by row count: one or two rows through an exact-product kernel, up to 192 rows in passes of
-      up to 32 rows on the matrix cores (the int8 rows streamed once per pass, straight into y), beyond that row
+      sq_q8_linear routes by row count: one or two rows through an exact-product kernel, up to 320 rows in passes of
+      up to 64 rows on the matrix cores (the int8 rows streamed once per pass, straight into y), beyond that row
       chunks decoded to fp16 and multiplied by the tile GEMM (the reference's chunked route).
 
     The kernels read the file's natural layout at full cache-line width, so no tile-major copy is made:

@@ -101,14 +101,14 @@ def test_block32_entry_points_check_arguments_on_the_host():
     assert L.sq_q8_workspace_bytes(64, 64, 32) == 0
     assert L.sq_q8_workspace_bytes(64, 64, 40) == 4096 + 64 * 64 * 2 + 40 * 64 * 2      # decoded rows + fp16 x
     assert L.sq_q8_workspace_bytes(64, 48, 40) == 0
-    # 3 .. 192 rows with C % 256 == 0: an fp16 copy of the activations
+    # 3 .. 320 rows with C % 256 == 0: an fp16 copy of the activations
     assert L.sq_q8_workspace_bytes(64, 256, 2) == 0
     assert L.sq_q8_workspace_bytes(64, 256, 3) == 4096 + 3 * 256 * 2
     assert L.sq_q8_workspace_bytes(64, 1024, 4) == 4096 + 4 * 1024 * 2
     assert L.sq_q8_workspace_bytes(64, 256, 8) == 4096 + 8 * 256 * 2
     assert L.sq_q8_workspace_bytes(64, 256, 128) == 4096 + 128 * 256 * 2
-    assert L.sq_q8_workspace_bytes(64, 256, 192) == 4096 + 192 * 256 * 2
-    assert L.sq_q8_workspace_bytes(64, 256, 193) == 4096 + 64 * 256 * 2 + 193 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 320) == 4096 + 320 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 321) == 4096 + 64 * 256 * 2 + 321 * 256 * 2
     assert L.sq_q8_linear(q, sc, 64, 256, x, bf, 256, y, bf, 64, 8, None, 0, None) == _lib.SQ_EWORKSPACE
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 64, 3, 65, None) == _lib.SQ_EINVAL                    # rows outside
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 32, 0, 4, None) == _lib.SQ_EINVAL                     # ld_out < C
