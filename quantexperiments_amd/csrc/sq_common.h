@@ -127,7 +127,7 @@ void tiled_build(const uint32_t* tags, int R, int W, int bits, uint32_t* out);
 // the block-32 side formats (8-bit output head, 4-bit embedding)
 int launch_q8_small(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
                     int y_dtype, int64_t ldy, int B, hipStream_t s);
-bool q8_mid(int C, int B);                  // 5 .. 128 activation rows on MFMA passes of 32
+bool q8_mid(int C, int B);                  // 3 .. 320 activation rows (C % 256 == 0) on MFMA passes of up to 64
 size_t q8_mid_workspace(int C, int B);
 int launch_q8_mid(const int8_t* q, const uint16_t* sc, int V, int C, const void* x, int x_dtype, int64_t ldx, void* y,
                   int y_dtype, int64_t ldy, int B, void* ws, size_t ws_bytes, hipStream_t s);
