@@ -92,6 +92,29 @@ def test_silu_mul_matches_oracle(B, C, M, dtype):
         assert torch.equal(out, plain[:, perms.long().cuda()])
 
 
+def test_neighbours_at_prefill_row_counts():
+    # 2048 activation rows: one workgroup per row (add + norm), 8 elements per thread (SiLU * up); rows sampled
+    from quantexperiments_amd.kernels import addnorm, silu_mul
+    g = torch.Generator().manual_seed(21)
+    B, C, I = 2048, 3584, 4864
+    h = torch.randn(B, C, generator=g)
+    add = rand_x(B, C, torch.bfloat16, seed=3)
+    w = (torch.rand(C, generator=g) + 0.5).bfloat16()
+    out = torch.empty(B, C, dtype=torch.bfloat16, device="cuda")
+    hd = h.cuda()
+    addnorm(hd, add.cuda(), w.cuda(), 1e-6, out, h_out=hd)
+    rows = torch.tensor([0, 1, 777, 2047])
+    h_ref, o_ref = O.addnorm(h[rows].numpy(), add[rows].float().numpy(), w.float().numpy(), 1e-6, dtype="bf16")
+    assert np.array_equal(hd[rows.cuda()].cpu().numpy(), h_ref)
+    _one_step(out[rows.cuda()].float().cpu().numpy(), o_ref[:, 0], torch.bfloat16)
+    gu = rand_x(B, 2 * I, torch.float16, seed=4, scale=3.0).cuda()
+    act = torch.empty(B, I, dtype=torch.float16, device="cuda")
+    silu_mul(gu[:, :I], gu[:, I:], act)
+    ref = O.silu_mul(gu[rows.cuda(), :I].float().cpu().numpy(), gu[rows.cuda(), I:].float().cpu().numpy())[:, 0]
+    d = np.abs(act[rows.cuda()].float().cpu().numpy() - ref)
+    assert np.all(d <= np.abs(ref) * 2.0 ** -9 + 2.0 ** -23) and (d > 0).mean() <= 0.01
+
+
 def test_silu_mul_special_values():
     from quantexperiments_amd.kernels import silu_mul
     g = torch.tensor([[0.0, -0.0, 20.0, -20.0, 60000.0, -60000.0, 1.0, float("inf")]], dtype=torch.float16, device="cuda")
