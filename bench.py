@@ -15,7 +15,7 @@ the packed file's bytes, which is what the metric is quoted on.
 value = packed (algorithmic) bytes of a layer / time per layer, in GB/s.  The same JSON line
 carries us_per_layer, the roofline of the dominant kernel (gate|up launch, HIP events around graph
 replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s, the 8-bit block-32 output head
-(152,064 x 3,584) at a few decode batch sizes, the layer with its three elementwise neighbours (add + RMS
+(152,064 x 3,584) at decode batch sizes 1 to 64, the layer with its three elementwise neighbours (add + RMS
 norm twice, SiLU * up) as separate launches and fused into the consuming products, and the CPU baseline (the reference's CPU route, oracle
 port, on the host cores).
 """
@@ -129,7 +129,7 @@ def prefill(torch, dev, layer, steps=3):
     return res
 
 
-def lm_head(torch, dev, rows=(1, 4, 8, 32), reps=3):
+def lm_head(torch, dev, rows=(1, 4, 8, 16, 32, 64), reps=3):
     """The 7B model's 8-bit block-32 output head (152,064 x 3,584 int8 + fp16 block scales = 579 MB, more than
     twice the last-level cache): microseconds and weight bytes per second for a few decode batch sizes."""
     from quantexperiments_amd.kernels import q8_linear
