@@ -108,7 +108,8 @@ def test_q4_embedding_from_pinned_host_memory():
 
 
 # ------------------------------------------------------------------ the head product
-Q8_SHAPES = [(100, 64), (257, 896), (1000, 3584), (70, 5120), (31, 1056), (40, 8192), (24, 12288)]
+Q8_SHAPES = [(100, 64), (257, 896), (1000, 3584), (70, 5120), (31, 1056), (40, 8192), (24, 12288), (50, 256), (33, 512),
+             (300, 768)]
 
 
 @pytest.mark.parametrize("V,C", Q8_SHAPES, ids=lambda v: str(v))
