@@ -201,7 +201,6 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_kernel(Q8Args a) {
 // 5.2-5.5 TB/s (the one-row kernel: 5.7); 32 rows per wave on the 32x32x16 instruction was slower still.
 constexpr int Q8_MFMA_MAX_ROWS = 320;           // up to here passes of 64 beat decode + tile GEMM (152,064 x 3,584: 151 us per pass,
                                                 // 5 passes 755 us against ~880; 8 passes 1208 against 961 at 512 rows)
-constexpr int Q8_XC = 256;                      // columns of x per LDS chunk (2 steps)
 
 // x [B, C] (fp16 or bf16, any stride) -> fp16 [B, C] contiguous.
 __global__ __launch_bounds__(256) void q8_x_kernel(const uint16_t* __restrict__ x, int64_t ldx, int B, int C, int x_dtype,
