@@ -33,6 +33,9 @@ def test_struct_layout_matches_header():
     # 7 pointers + 8 int32 + 1 pointer + 2 int32
     assert ctypes.sizeof(_lib.SqMatrix) == 7 * 8 + 8 * 4 + 8 + 8
     assert _lib.SqMatrix.R.offset == 56 and _lib.SqMatrix.y_off.offset == 56 + 28 and _lib.SqMatrix.stream.offset == 88 and _lib.SqMatrix.stream_groups.offset == 100
+    # sq_producer: int32 mode, float eps, 6 pointers, 2 int64
+    assert ctypes.sizeof(_lib.SqProducer) == 8 + 6 * 8 + 2 * 8
+    assert _lib.SqProducer.eps.offset == 4 and _lib.SqProducer.h_in.offset == 8 and _lib.SqProducer.x_out.offset == 48 and _lib.SqProducer.ld_in.offset == 64
 
 
 def test_host_side_argument_checks():
@@ -119,3 +122,27 @@ def test_block32_entry_points_check_arguments_on_the_host():
     assert L.sq_q4_embed(q, sc, 64, 64, None, 3, y, bf, 64, None) == _lib.SQ_EINVAL
     assert L.sq_q4_embed(q, sc, 64, 64, x, 3, y, bf, 48, None) == _lib.SQ_EINVAL                        # ld_out < C
     assert L.sq_q4_embed(q, sc, 64, 64, x, 0, y, bf, 64, None) == _lib.SQ_OK
+
+
+def test_neighbour_entry_points_check_arguments_on_the_host():
+    L = _lib.lib()
+    f16, bf, f32 = _lib.SQ_F16, _lib.SQ_BF16, _lib.SQ_F32
+    p = 0x10000
+    assert L.sq_addnorm(p, None, 64, None, 0, 0, p, f16, None, 1, 1, 0, 1e-6, p, f16, None) == _lib.SQ_EINVAL       # C = 0
+    assert L.sq_addnorm(p, None, 64, None, 0, 0, p, f32, None, 1, 1, 64, 1e-6, p, f16, None) == _lib.SQ_EINVAL      # fp32 weights
+    assert L.sq_addnorm(p, None, 64, p, f32, 64, p, f16, None, 1, 1, 64, 1e-6, p, f16, None) == _lib.SQ_EINVAL      # fp32 add
+    assert L.sq_addnorm(None, None, 64, None, 0, 0, p, f16, None, 1, 1, 64, 1e-6, p, f16, None) == _lib.SQ_EINVAL   # no h_in
+    assert L.sq_addnorm(p, None, 32, None, 0, 0, p, f16, None, 1, 2, 64, 1e-6, p, f16, None) == _lib.SQ_EINVAL      # ld_h < C
+    assert L.sq_addnorm(p, p, 64, None, 0, 0, p, f16, p, 2, 1, 64, 1e-6, p, f16, None) == _lib.SQ_EINVAL            # in place with orders
+    assert L.sq_addnorm(p, None, 64, None, 0, 0, p, f16, p, 0, 1, 64, 1e-6, p, f16, None) == _lib.SQ_EINVAL         # M = 0
+    assert L.sq_addnorm(p, None, 64, None, 0, 0, p, f16, None, 1, 0, 64, 1e-6, None, f16, None) == _lib.SQ_OK       # no rows
+    assert L.sq_silu_mul(p, p, f32, 64, None, 1, 1, 64, p, None) == _lib.SQ_EINVAL
+    assert L.sq_silu_mul(p, None, bf, 64, None, 1, 1, 64, p, None) == _lib.SQ_EINVAL
+    assert L.sq_silu_mul(p, p, bf, 64, None, 1, 0, 64, None, None) == _lib.SQ_OK
+    pr = _lib.SqProducer()
+    m = _lib.matrix_array([])
+    assert L.sq_linear_small_from(m, 0, None, bf, p, bf, 64, 1, None, 0, None) == _lib.SQ_EINVAL                    # no producer
+    pr.mode = 3
+    assert L.sq_linear_small_from(m, 0, ctypes.byref(pr), bf, p, bf, 64, 1, None, 0, None) == _lib.SQ_EINVAL        # unknown mode
+    pr.mode = _lib.SQ_FROM_SILU_MUL
+    assert L.sq_linear_small_from(m, 0, ctypes.byref(pr), bf, p, bf, 64, 1, None, 0, None) == _lib.SQ_OK            # no pieces
