@@ -328,7 +328,7 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
     for (int k = 1; k < GEMV_MAX_PIECES_STREAM; ++k)
         if (k < a.n && (int)blockIdx.x >= a.p[k].wg_begin) pi = k;
-    const StreamPiece& P = a.p[pi];
+    const StreamPiece P = a.p[pi];                             // by value: the piece's fields arrive in one batch of scalar loads
     const int local = (int)blockIdx.x - P.wg_begin;
     const int v = local / P.nwg, wi = local - v * P.nwg;
     const int s = v % P.NS, kp = v / P.NS;
@@ -350,12 +350,27 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     // that every wave draws the next unclaimed group from a counter in LDS, so all waves stay busy to the end.
     // The head of a group (its first step, its step count, the lane's row and count) is fetched one group
     // ahead; the first one goes out before the staging loads.
+    // A run with at most NW / 2 groups would leave waves idle while the others walk their steps a few fetches at
+    // a time; there `split` (2, 4 or 8) waves share a group, each takes a contiguous share of its steps, and
+    // the shares are added in wave order through LDS before the partial sum is stored.
+    // The share count follows from the group count alone (at most 8 waves share), so a row's sums are formed in the
+    // same order whatever NB and NW are.
+    int split = 1;
+    while (ng * split * 2 <= 8) split *= 2;
+    const int sub = wave & (split - 1);
     auto head = [&](int k) {
         StreamHead h{0u, 0, STREAM_NO_ROW};
         if (k < ng) {
             h.st0 = goff[k];
             h.nst = (int)(goff[k + 1] - h.st0);
             h.slot = slots[(size_t)k * 64 + lane];
+            if (split > 1) {                                    // uniform in the workgroup
+                const int s0 = h.nst * sub / split, s1 = h.nst * (sub + 1) / split;
+                const int cnt = max((int)(h.slot >> STREAM_ROW_BITS) - 4 * s0, 0);
+                h.st0 += (uint32_t)s0;
+                h.nst = s1 - s0;
+                h.slot = (h.slot & STREAM_NO_ROW) | ((uint32_t)cnt << STREAM_ROW_BITS);
+            }
         }
         return h;
     };
@@ -367,6 +382,10 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
         }
     };
     int kcur = wave, knext = 2 * NW - 1 - wave;
+    if (split > 1) {                                            // one share of one group per wave, or nothing
+        kcur = wave < ng * split ? wave / split : ng;
+        knext = ng;
+    }
     StreamHead hn = head(kcur);
     u32x3 nx[STREAM_PF];
 #pragma unroll
@@ -511,6 +530,10 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     __syncthreads();
     SQ_TRACE_POINT(1);
 
+    float acc_share[NB];                                        // split > 1: this wave's share of its group
+    uint32_t row_share = STREAM_NO_ROW;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc_share[b] = 0.f;
     while (kcur < ng) {
         const StreamHead h = hn;
         hn = head(knext);
@@ -566,12 +589,33 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
         if (nst == 0) first_steps(hn, nx);                      // a group without steps fetched nothing for its successor
         // device-scope stores: written through to memory, so other XCDs' L2s never hold a stale copy and no
         // cache-wide write-back is needed before the workgroup counts itself off
-        if (row != STREAM_NO_ROW) {
+        if (split > 1) {
+            row_share = row;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) acc_share[b] = acc[b];
+        } else if (row != STREAM_NO_ROW) {
 #pragma unroll
             for (int b = 0; b < NB; ++b) __hip_atomic_store(part + b * np + row, acc[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         kcur = knext;
         knext = kafter;
+    }
+    if (split > 1) {
+        // the x rows are no longer needed once every wave has left the loop: their LDS holds the shares
+        float* share = reinterpret_cast<float*>(lds + STREAM_TAB);
+        static_assert(NW * 64 * 4 <= STREAM_XS, "shares of one activation row fit its part of x");
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < NB; ++b) share[(wave * NB + b) * 64 + lane] = acc_share[b];
+        __syncthreads();
+        if (sub == 0 && row_share != STREAM_NO_ROW) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                float sum = 0.f;
+                for (int j = 0; j < split; ++j) sum += share[((wave + j) * NB + b) * 64 + lane];
+                __hip_atomic_store(part + b * np + row_share, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
     }
 
     // Count this workgroup off once all its partial sums have been acknowledged (the barrier waits for every
@@ -601,32 +645,47 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
         return P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
     };
     if (P.NV <= 16) {
+        // Every load below is unconditional (indices are clamped, missing terms are dropped afterwards): a load the
+        // compiler must guard with a branch is waited for before the next one goes out, and the 64 partial sums
+        // of a thread would take four trips to memory instead of one.
         for (int ib = tid; ib < items; ib += 4 * NW * 64) {
-            float t[4][16];
+            float t[4][16], rs[4];
             uint32_t rr[4];
             int bb[4];
+            bool live[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int it = ib + q * NW * 64;
-                bb[q] = it < items ? it / nl : 0;
-                rr[q] = it < items ? row_of(it - bb[q] * nl) : STREAM_NO_ROW;
+                live[q] = ib + q * NW * 64 < items;
+                const int it = min(ib + q * NW * 64, items - 1);
+                bb[q] = it / nl;
+            }
+            if (P.perms) {                                      // the four row ids in one trip
+#pragma unroll
+                for (int q = 0; q < 4; ++q) rr[q] = rows0[min(ib + q * NW * 64, items - 1) - bb[q] * nl];
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) rr[q] = row_of(min(ib + q * NW * 64, items - 1) - bb[q] * nl);
             }
 #pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (!live[q]) rr[q] = STREAM_NO_ROW;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) rs[q] = h2f(P.row_scale[rr[q] != STREAM_NO_ROW ? rr[q] : 0u]);
+#pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int it = ib + q * NW * 64;
+                const int it = min(ib + q * NW * 64, items - 1);
                 const uint32_t off = (uint32_t)(bb[q] * (int)np + (it - bb[q] * nl));  // uniform base + 32-bit lane offset
 #pragma unroll
                 for (int k = 0; k < 16; ++k)
-                    t[q][k] = (it < items && k < P.NV)
-                                  ? __hip_atomic_load(pp + (size_t)k * NB * np + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+                    t[q][k] = __hip_atomic_load(pp + (size_t)min(k, P.NV - 1) * NB * np + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 float sum = 0.f;
 #pragma unroll
-                for (int k = 0; k < 16; ++k) sum += t[q][k];
+                for (int k = 0; k < 16; ++k) sum += k < P.NV ? t[q][k] : 0.f;
                 if (rr[q] != STREAM_NO_ROW)
-                    store_y((char*)a.y + (size_t)bb[q] * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + rr[q], sum * h2f(P.row_scale[rr[q]]));
+                    store_y((char*)a.y + (size_t)bb[q] * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + rr[q], sum * rs[q]);
             }
         }
     } else {
