@@ -358,21 +358,24 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     int split = 1;
     while (ng * split * 2 <= 8) split *= 2;
     const int sub = wave & (split - 1);
-    auto head = [&](int k) {
-        StreamHead h{0u, 0, STREAM_NO_ROW};
-        if (k < ng) {
-            h.st0 = goff[k];
-            h.nst = (int)(goff[k + 1] - h.st0);
-            h.slot = slots[(size_t)k * 64 + lane];
-            if (split > 1) {                                    // uniform in the workgroup
-                const int s0 = h.nst * sub / split, s1 = h.nst * (sub + 1) / split;
-                const int cnt = max((int)(h.slot >> STREAM_ROW_BITS) - 4 * s0, 0);
-                h.st0 += (uint32_t)s0;
-                h.nst = s1 - s0;
-                h.slot = (h.slot & STREAM_NO_ROW) | ((uint32_t)cnt << STREAM_ROW_BITS);
-            }
+    // The head of group k from its three loaded words (first step, end step, this lane's slot).
+    auto head_from = [&](int k, uint32_t ga, uint32_t gb, uint32_t sl) {
+        StreamHead h{ga, (int)(gb - ga), sl};
+        if (k >= ng) h = StreamHead{0u, 0, STREAM_NO_ROW};
+        else if (split > 1) {                                   // uniform in the workgroup
+            const int s0 = h.nst * sub / split, s1 = h.nst * (sub + 1) / split;
+            const int cnt = max((int)(h.slot >> STREAM_ROW_BITS) - 4 * s0, 0);
+            h.st0 += (uint32_t)s0;
+            h.nst = s1 - s0;
+            h.slot = (h.slot & STREAM_NO_ROW) | ((uint32_t)cnt << STREAM_ROW_BITS);
         }
         return h;
+    };
+    // (loads without a branch around them, from a clamped index: the compiler then knows how many loads are in
+    // flight and later waits do not have to cover these)
+    auto head = [&](int k) {
+        const int kc = min(k, ng - 1);
+        return head_from(k, goff[kc], goff[kc + 1], slots[(size_t)kc * 64 + lane]);
     };
     auto first_steps = [&](const StreamHead& h, u32x3* nx) {
         if (h.nst > 0) {                                        // wave-uniform
@@ -381,12 +384,22 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
             for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, h.nst - 1) * 768);
         }
     };
+    // the same without a branch, for the prologue: a wave without steps reads step 0 of the stream and ignores it
+    auto first_steps_always = [&](const StreamHead& h, u32x3* nx) {
+        const unsigned char* en = steps + (size_t)h.st0 * 768;
+#pragma unroll
+        for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, max(h.nst - 1, 0)) * 768);
+    };
     int kcur = wave, knext = 2 * NW - 1 - wave;
     if (split > 1) {                                            // one share of one group per wave, or nothing
         kcur = wave < ng * split ? wave / split : ng;
         knext = ng;
     }
-    StreamHead hn = head(kcur);
+    // the first head's words are requested here and used only after the staging loads have gone out
+    const int kc0 = min(kcur, ng - 1);
+    const uint32_t head_a = goff[kc0], head_b = goff[kc0 + 1], head_s = slots[(size_t)kc0 * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
+    StreamHead hn;
     u32x3 nx[STREAM_PF];
 #pragma unroll
     for (int q = 0; q < STREAM_PF; ++q) nx[q] = u32x3{0u, 0u, 0u};
@@ -511,7 +524,9 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
                 }
             }
         }
-        first_steps(hn, nx);
+        __builtin_amdgcn_sched_barrier(0);
+        hn = head_from(kcur, head_a, head_b, head_s);
+        first_steps_always(hn, nx);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
