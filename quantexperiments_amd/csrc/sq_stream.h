@@ -7,6 +7,7 @@ namespace sq {
 
 constexpr int STREAM_SLICE_BITS = 12;        // 4096 codewords of 16 bytes per LDS slice
 constexpr int STREAM_PART_MAX = 640;         // most chunks in one column part (10 bits of an entry are enough)
+constexpr int STREAM_ZERO_CHUNK = STREAM_PART_MAX;   // chunk index of padding entries: a chunk of x kept at zero
 constexpr int STREAM_ROW_BITS = 19;          // slot = row | count << 19
 constexpr uint32_t STREAM_NO_ROW = (1u << STREAM_ROW_BITS) - 1u;
 constexpr int GEMV_MAX_PIECES_STREAM = 4;

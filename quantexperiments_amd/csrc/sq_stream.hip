@@ -193,10 +193,11 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
     for (size_t k = 0; k < (size_t)g.NV * g.NG * 64; ++k) slots[k] = STREAM_NO_ROW;
     unsigned char* steps = out + g.off_steps;
     parallel_rows(R, [&](int a, int b) {
-        std::vector<uint32_t> q(g.NV);
+        std::vector<uint32_t> q(g.NV), last(g.NV);
         for (int r = a; r < b; ++r) {
             const uint32_t* row = tags + (size_t)r * W;
             std::fill(q.begin(), q.end(), 0u);
+            std::fill(last.begin(), last.end(), 0u);
             for (int v = 0; v < g.NV; ++v) {
                 const uint32_t k = P.pos[(size_t)v * R + r];
                 slots[(size_t)v * g.NG * 64 + k] = place[r] | ((uint32_t)P.cnt[(size_t)v * R + r] << STREAM_ROW_BITS);
@@ -209,6 +210,21 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
                 unsigned char* rec = steps + ((size_t)P.goff[(size_t)v * g.NG + (k >> 6)] + (n >> 2)) * 768 + (k & 63) * 12 +
                                      (n & 3) * 3;
                 rec[0] = (unsigned char)e; rec[1] = (unsigned char)(e >> 8); rec[2] = (unsigned char)(e >> 16);
+                last[v] = e & ((1u << STREAM_SLICE_BITS) - 1u);
+            }
+            // Padding up to the group's longest row: the row's last codeword of the bucket again, at the chunk of x
+            // that the kernel keeps at zero, so padding adds exactly nothing and needs no test in the inner loop
+            // (a codeword that is not finite is already part of the row's sum; a row without entries in the
+            // bucket is dropped by its count).
+            for (int v = 0; v < g.NV; ++v) {
+                const uint32_t k = P.pos[(size_t)v * R + r];
+                const size_t gi = (size_t)v * g.NG + (k >> 6);
+                const uint32_t cap = (P.goff[gi + 1] - P.goff[gi]) * 4u;
+                const uint32_t e = last[v] | ((uint32_t)STREAM_ZERO_CHUNK << STREAM_SLICE_BITS);
+                for (uint32_t n = q[v]; n < cap; ++n) {
+                    unsigned char* rec = steps + ((size_t)P.goff[gi] + (n >> 2)) * 768 + (k & 63) * 12 + (n & 3) * 3;
+                    rec[0] = (unsigned char)e; rec[1] = (unsigned char)(e >> 8); rec[2] = (unsigned char)(e >> 16);
+                }
             }
         }
     });
@@ -307,7 +323,7 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 }
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
-constexpr int STREAM_XS = STREAM_PART_MAX * 16;   // LDS bytes of one activation row's part of x
+constexpr int STREAM_XS = (STREAM_PART_MAX + 1) * 16;   // LDS bytes of one activation row's part of x, plus the zero chunk
 constexpr int STREAM_PF = 4;          // steps fetched ahead
 
 struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
@@ -344,6 +360,7 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     const unsigned char* steps = P.stream + P.off_steps + lane * 12;
     const size_t np = (size_t)P.NG * 64;
     float* part = P.part + (size_t)v * NB * np;
+    const unsigned char* ldsx = lds + STREAM_TAB;
     unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_TAB + NB * STREAM_XS);   // [0] arrival result, [1] next group
 
     // The groups of a run are sorted longest first.  Wave w starts with group w, then group 2 NW - 1 - w; after
@@ -385,8 +402,9 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
         }
     };
     // the same without a branch, for the prologue: a wave without steps reads step 0 of the stream and ignores it
+    // (a group without steps may begin where the stream ends: it must not read from its own first step)
     auto first_steps_always = [&](const StreamHead& h, u32x3* nx) {
-        const unsigned char* en = steps + (size_t)h.st0 * 768;
+        const unsigned char* en = steps + (size_t)(h.nst > 0 ? h.st0 : 0u) * 768;
 #pragma unroll
         for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, max(h.nst - 1, 0)) * 768);
     };
@@ -538,6 +556,8 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
                 if (tid + k * NW * 64 < nc) xd[tid + k * NW * 64] = q;
             }
         }
+        if (tid < NB)                                            // the chunk that padding entries multiply with
+            reinterpret_cast<u32x4*>(lds + STREAM_TAB + tid * STREAM_XS)[STREAM_ZERO_CHUNK] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
         for (int k = 0; k < NT; ++k) dst[tid + k * NW * 64] = t[k];
         if (tid == 0) flag[1] = 2 * NW;
@@ -579,27 +599,38 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
             for (int q = 0; q < STREAM_PF; ++q) {
                 if (t0 + q >= nst) break;                       // wave-uniform
-                const uint32_t e[4] = {cur[q].x & 0xFFFFFFu, (cur[q].x >> 24) | ((cur[q].y & 0xFFFFu) << 8),
-                                       (cur[q].y >> 16) | ((cur[q].z & 0xFFu) << 16), cur[q].z >> 8};
+                // (bits above an entry's 24 are left in place: the address fields are cut out below)
+                const uint32_t e[4] = {cur[q].x, (cur[q].x >> 24) | (cur[q].y << 8), (cur[q].y >> 16) | (cur[q].z << 16), cur[q].z >> 8};
+                // the LDS reads of EB entries go out together, then their products: a wave does not sit out one
+                // LDS round trip per entry
+                constexpr int EB = NB == 1 ? 4 : NB == 2 ? 2 : 1;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t ta = (e[j] << 4) & 0xFFF0u;
-                    const uint32_t xa = ((e[j] >> 8) & 0xFFFF0u) | (uint32_t)STREAM_TAB;
-                    const u32x4 cw = *reinterpret_cast<const u32x4*>(lds + ta);
-                    const bool valid = (t0 + q) * 4 + j < cnt;
+                for (int j0 = 0; j0 < 4; j0 += EB) {
+                    u32x4 cw[EB], xv[EB][NB];
 #pragma unroll
-                    for (int b = 0; b < NB; ++b) {
-                        const u32x4 xv = *reinterpret_cast<const u32x4*>(lds + xa + b * STREAM_XS);
-                        float dsum = 0.f;
+                    for (int jj = 0; jj < EB; ++jj) {
+                        const uint32_t ta = (e[j0 + jj] & 0xFFFu) << 4, xa = ((e[j0 + jj] >> 12) & 0xFFFu) << 4;
+                        cw[jj] = *reinterpret_cast<const u32x4*>(lds + ta);
 #pragma unroll
-                        for (int hh = 0; hh < 4; ++hh) {
-                            const uint32_t cwh = cw[hh], xvh = xv[hh];  // bit_cast straight from a vector element misreads it
-                            dsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, cwh), __builtin_bit_cast(half2v, xvh), dsum, false);
+                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * STREAM_XS + xa);
+                    }
+#pragma unroll
+                    for (int jj = 0; jj < EB; ++jj) {
+#pragma unroll
+                        for (int b = 0; b < NB; ++b) {
+#pragma unroll
+                            for (int hh = 0; hh < 4; ++hh) {
+                                const uint32_t cwh = cw[jj][hh], xvh = xv[jj][b][hh];  // bit_cast straight from a vector element misreads it
+                                acc[b] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, cwh), __builtin_bit_cast(half2v, xvh), acc[b], false);
+                            }
                         }
-                        acc[b] += valid ? dsum : 0.f;
                     }
                 }
             }
+        }
+        if (cnt == 0) {                                         // a row without entries in this bucket (or share)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) acc[b] = 0.f;
         }
         if (nst == 0) first_steps(hn, nx);                      // a group without steps fetched nothing for its successor
         // device-scope stores: written through to memory, so other XCDs' L2s never hold a stale copy and no

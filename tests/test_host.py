@@ -251,7 +251,8 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
                     assert (e[lane] == 0).all()
                     continue
                 c = int(cnts[k])
-                assert (e[lane, c:] == 0).all()                               # padding is zero
+                # padding: the row's last codeword of the bucket again (0 when it has none), at the zero chunk of x
+                assert (e[lane, c:] == ((e[lane, c - 1] & 0xFFF if c else 0) | 640 << 12)).all()
                 chunk = (e[lane, :c] >> 12) + kp * PC
                 assert (np.diff(chunk.astype(np.int64)) > 0).all() and (chunk < min(U, (kp + 1) * PC)).all()
                 assert (tags[rows[k], chunk] == -1).all()
