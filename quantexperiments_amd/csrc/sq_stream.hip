@@ -174,6 +174,84 @@ size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int b
     return P.g.off_steps + (size_t)P.g.total_steps * 768;
 }
 
+// Orders the entries of 16 neighbouring lanes of a group (see the second pass of stream_build_host).
+struct BankMatch {
+    static constexpr uint32_t NONE = 0xFFFFFFFFu;
+    std::vector<uint32_t> by[16][16];        // [lane][codeword bank group]: entries not yet placed
+    uint32_t rep[16][16];                    // one tag of the lane per bank group (for padding), NONE = none
+    uint32_t cnt[16];
+    int lane_of[16], grp_of[16];
+    bool seen[16];
+    uint32_t slot_n;
+
+    bool avail(int l, int k) const { return cnt[l] > slot_n ? !by[l][k].empty() : rep[l][k] != NONE; }
+    bool augment(int l) {
+        for (int k = 0; k < 16; ++k) {
+            if (!avail(l, k) || seen[k]) continue;
+            seen[k] = true;
+            if (lane_of[k] < 0 || augment(lane_of[k])) { lane_of[k] = l; grp_of[l] = k; return true; }
+        }
+        return false;
+    }
+    static unsigned char* rec_of(unsigned char* base, int lane, uint32_t n) {
+        return base + (size_t)(n >> 2) * 768 + lane * 12 + (n & 3) * 3;
+    }
+    void order_lanes(unsigned char* base, const uint32_t* sl, int q0, uint32_t ns) {
+        bool any = false;
+        for (int l = 0; l < 16; ++l) {
+            const uint32_t s0 = sl[q0 + l];
+            cnt[l] = (s0 & STREAM_NO_ROW) == STREAM_NO_ROW ? 0u : s0 >> STREAM_ROW_BITS;
+            for (int k = 0; k < 16; ++k) { by[l][k].clear(); rep[l][k] = NONE; }
+            for (uint32_t n = 0; n < cnt[l]; ++n) {
+                const unsigned char* r = rec_of(base, q0 + l, n);
+                const uint32_t e = r[0] | (uint32_t)r[1] << 8 | (uint32_t)r[2] << 16;
+                by[l][e & 15u].push_back(e);
+                rep[l][e & 15u] = e & ((1u << STREAM_SLICE_BITS) - 1u);
+            }
+            any = any || cnt[l] > 0;
+        }
+        if (!any) return;
+        for (uint32_t n = 0; n < ns; ++n) {
+            slot_n = n;
+            for (int k = 0; k < 16; ++k) lane_of[k] = grp_of[k] = -1;
+            // lanes that must place an entry first, then those that only repeat one
+            for (int pass = 0; pass < 2; ++pass)
+                for (int l = 0; l < 16; ++l) {
+                    if (cnt[l] == 0 || (cnt[l] > n) != (pass == 0)) continue;
+                    int best = -1;
+                    for (int k = 0; k < 16; ++k)
+                        if (lane_of[k] < 0 && avail(l, k) && (best < 0 || by[l][k].size() > by[l][best].size())) best = k;
+                    if (best >= 0) { lane_of[best] = l; grp_of[l] = best; continue; }
+                    for (int k = 0; k < 16; ++k) seen[k] = false;
+                    if (augment(l)) continue;
+                    for (int k = 0; k < 16; ++k)                 // no bank group to itself: the fullest one
+                        if (avail(l, k) && (best < 0 || by[l][k].size() > by[l][best].size())) best = k;
+                    grp_of[l] = best;
+                }
+            int xuse[16] = {};
+            for (int l = 0; l < 16; ++l) {
+                if (cnt[l] == 0) continue;
+                const int k = grp_of[l];
+                uint32_t e;
+                if (cnt[l] > n) {
+                    std::vector<uint32_t>& c = by[l][k];
+                    size_t bi = 0;
+                    for (size_t i = 1; i < c.size(); ++i)
+                        if (xuse[(c[i] >> STREAM_SLICE_BITS) & 15u] < xuse[(c[bi] >> STREAM_SLICE_BITS) & 15u]) bi = i;
+                    e = c[bi];
+                    ++xuse[(e >> STREAM_SLICE_BITS) & 15u];
+                    c[bi] = c.back();
+                    c.pop_back();
+                } else {
+                    e = rep[l][k] | ((uint32_t)STREAM_ZERO_CHUNK << STREAM_SLICE_BITS);
+                }
+                unsigned char* r = rec_of(base, q0 + l, n);
+                r[0] = (unsigned char)e; r[1] = (unsigned char)(e >> 8); r[2] = (unsigned char)(e >> 16);
+            }
+        }
+    }
+};
+
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                       unsigned char* out, size_t bytes, int* runs_out, int* groups_out) {
     StreamPlan P;
@@ -226,6 +304,24 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
                     rec[0] = (unsigned char)e; rec[1] = (unsigned char)(e >> 8); rec[2] = (unsigned char)(e >> 16);
                 }
             }
+        }
+    });
+    // Second pass, group by group: the order of a lane's entries is free (padding stays behind them), so it is
+    // chosen to keep the LDS gathers apart.  A 16-byte LDS read of a wave takes four clocks of 16 consecutive lanes
+    // each, and two lanes of a clock collide when their addresses differ but fall into the same group of four banks
+    // (address / 16 mod 16).  For every entry slot and every 16 lanes the entries are picked by a bipartite
+    // matching of lanes to codeword bank groups (greedy, a lane prefers the bank group it has most entries left
+    // in, then Kuhn's augmenting paths for the lanes left without one); among a lane's entries of its bank group
+    // the one whose chunk of x falls into the bank group least used in this slot goes first.  A lane that has run
+    // out repeats whichever of its codewords fits.
+    parallel_rows(g.NV * g.NG, [&](int a, int b) {
+        BankMatch bm;
+        for (int vg = a; vg < b; ++vg) {
+            const uint32_t st0 = P.goff[vg], ns = (P.goff[vg + 1] - st0) * 4;
+            if (ns == 0) continue;
+            const uint32_t* sl = slots + (size_t)vg * 64;
+            unsigned char* base = steps + (size_t)st0 * 768;
+            for (int q0 = 0; q0 < 64; q0 += 16) bm.order_lanes(base, sl, q0, ns);
         }
     });
     if (runs_out) *runs_out = g.runs;

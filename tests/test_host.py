@@ -251,10 +251,12 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
                     assert (e[lane] == 0).all()
                     continue
                 c = int(cnts[k])
-                # padding: the row's last codeword of the bucket again (0 when it has none), at the zero chunk of x
-                assert (e[lane, c:] == ((e[lane, c - 1] & 0xFFF if c else 0) | 640 << 12)).all()
+                # padding: one of the row's codewords of the bucket again (0 when it has none), at the zero chunk of x
+                assert (e[lane, c:] >> 12 == 640).all()
+                assert set((e[lane, c:] & 0xFFF).tolist()) <= (set((e[lane, :c] & 0xFFF).tolist()) if c else {0})
+                # the entries of a lane come in an order chosen for the LDS banks: every chunk once, any order
                 chunk = (e[lane, :c] >> 12) + kp * PC
-                assert (np.diff(chunk.astype(np.int64)) > 0).all() and (chunk < min(U, (kp + 1) * PC)).all()
+                assert len(set(chunk.tolist())) == c and (chunk >= kp * PC).all() and (chunk < min(U, (kp + 1) * PC)).all()
                 assert (tags[rows[k], chunk] == -1).all()
                 tags[rows[k], chunk] = (e[lane, :c] & 0xFFF) + (s << 12)
     return tags
