@@ -74,7 +74,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 105; }
+int sq_version(void) { return 106; }
 
 const char* sq_last_error(void) { return g_err; }
 
