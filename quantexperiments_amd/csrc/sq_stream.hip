@@ -123,6 +123,16 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
         for (int q : ngm) { n += (q + GR - 1) / GR; whole = whole && q <= GR; }
         if (n <= runs || whole) break;
     }
+    // A run of 5 to 7 groups leaves one to three of a workgroup's eight waves without a group (shorter runs share
+    // their groups among the waves, longer ones deal groups out as waves finish): 8 groups per run instead.  With
+    // one column order the kernel derives the cut from the run count alone, as ceil(groups / runs) per run.
+    if (GR > 4 && GR < 8) {
+        GR = 8;
+        if (ngm.size() == 1) {
+            const int n = (ngm[0] + GR - 1) / GR;
+            GR = (ngm[0] + n - 1) / n;
+        }
+    }
     P.runs.clear();
     P.base.clear();
     for (size_t i = 0; i < ngm.size(); ++i) {

@@ -217,6 +217,9 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
     # runs tile the groups in order; every run has one column order
     assert rt[0, 0] == 0 and (rt[1:, 0] == rt[:-1, 0] + rt[:-1, 1]).all() and rt[-1, 0] + rt[-1, 1] == NG
     assert (rt[:, 1] >= 1).all() and (rt[:, 3] == 0).all() and (np.diff(rt[:, 2]) >= 0).all()
+    if row_mask is None:                                                      # the cut the kernel derives from the run count
+        gr = -(-NG // runs)
+        assert (rt[:, 0] == np.arange(runs) * gr).all() and (rt[:, 1] == np.minimum(gr, NG - rt[:, 0])).all()
     steps = np.frombuffer(buf, np.uint8, int(goff[-1]) * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.uint32)
     ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
     tags = np.full((R, U), -1, np.int64)
