@@ -51,6 +51,67 @@ __global__ __launch_bounds__(256) void dequant_kernel(sq_matrix m, typename stor
     }
 }
 
+// d = 8 without column orders: four chunks per thread, 256 chunks apart, so that a thread has four tag loads and then
+// four 16-byte table gathers in flight instead of one (the decode is bound by the rate and latency of those gathers,
+// which hit L2, not HBM).  Same arithmetic as dequant_kernel; `vec`: 16-byte aligned rows of a 16-bit type, stored
+// as one 16-byte piece per chunk; raw fp16 output copies the codeword's bits.
+template <int DT>
+__global__ __launch_bounds__(256) void dequant8x4_kernel(sq_matrix m, typename store_as<DT>::type* __restrict__ out,
+                                                         int64_t ld_out, int r0, int r1, int raw, int vec) {
+    typedef typename store_as<DT>::type T;
+    const int nch = m.C / 8;
+    const int total = (r1 - r0) * nch;                          // < 2^31, checked by the launcher
+    const int base = (int)blockIdx.x * 1024 + (int)threadIdx.x;
+    int rr[4], j[4];
+    bool ok[4];
+    uint32_t tag[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        int idx = base + k * 256;
+        ok[k] = idx < total;
+        idx = min(idx, total - 1);
+        rr[k] = idx / nch;
+        j[k] = idx - rr[k] * nch;
+        const uint32_t* row = reinterpret_cast<const uint32_t*>(m.tags) + (int64_t)(r0 + rr[k]) * m.W;
+        tag[k] = tag_at(row, m.W, m.bits, j[k]);
+    }
+    if (m.row_book) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) tag[k] += (uint32_t)m.row_book[r0 + rr[k]] << m.bits;
+    }
+    u32x4 cw[4];
+    float s[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        cw[k] = *reinterpret_cast<const u32x4*>(m.table + (int64_t)tag[k] * 8);
+        s[k] = raw ? 1.f : h2f(m.row_scale[r0 + rr[k]]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        if (!ok[k]) continue;
+        T* o = out + (int64_t)rr[k] * ld_out + j[k] * 8;
+        if (DT == SQ_F16 && raw && vec) {
+            *reinterpret_cast<u32x4*>(o) = cw[k];
+            continue;
+        }
+        T t[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            t[2 * e] = store_as<DT>::cvt(h2f((uint16_t)(cw[k][e] & 0xFFFFu)) * s[k]);
+            t[2 * e + 1] = store_as<DT>::cvt(h2f((uint16_t)(cw[k][e] >> 16)) * s[k]);
+        }
+        if (DT != SQ_F32 && vec) {
+            u32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = (uint32_t)t[2 * e] | ((uint32_t)t[2 * e + 1] << 16);
+            *reinterpret_cast<u32x4*>(o) = v;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = t[e];
+        }
+    }
+}
+
 // Matrices with column orders: scattering 2-byte values straight to HBM costs 4x the plain decode, so a
 // workgroup decodes one row at a time into LDS at its permuted positions (ds_write of one element each, the
 // order read as whole 16/32-byte pieces) and then writes the row out in 16-byte pieces.
@@ -118,6 +179,11 @@ static int launch_dt(const sq_matrix& m, void* out, int64_t ld_out, int r0, int 
         const unsigned rgrid = (unsigned)(r1 - r0 < want ? r1 - r0 : want);
         if (m.d == 8) hipLaunchKernelGGL((dequant_rows_lds_kernel<DT, 8>), dim3(rgrid), dim3(256), row_bytes, s, m, (T*)out, ld_out, r0, r1, raw, vec_out);
         else hipLaunchKernelGGL((dequant_rows_lds_kernel<DT, 4>), dim3(rgrid), dim3(256), row_bytes, s, m, (T*)out, ld_out, r0, r1, raw, vec_out);
+        return check_launch("sq_dequant");
+    }
+    if (m.d == 8 && !m.perms && n < ((int64_t)1 << 31) - 1024 && ((uintptr_t)m.table & 15) == 0) {
+        const int vec = sizeof(T) == 2 && ((uintptr_t)out & 15) == 0 && ld_out % 8 == 0;
+        hipLaunchKernelGGL((dequant8x4_kernel<DT>), dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw, vec);
         return check_launch("sq_dequant");
     }
     const unsigned grid = (unsigned)((n + 255) / 256);
