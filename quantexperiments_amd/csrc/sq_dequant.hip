@@ -56,12 +56,12 @@ __global__ __launch_bounds__(256) void dequant_kernel(sq_matrix m, typename stor
 // which hit L2, not HBM).  Same arithmetic as dequant_kernel; `vec`: 16-byte aligned rows of a 16-bit type, stored
 // as one 16-byte piece per chunk; raw fp16 output copies the codeword's bits.
 template <int DT>
-__global__ __launch_bounds__(256) void dequant8x4_kernel(sq_matrix m, typename store_as<DT>::type* __restrict__ out,
-                                                         int64_t ld_out, int r0, int r1, int raw, int vec) {
+__device__ __forceinline__ void dequant8x4_block(const sq_matrix& m, typename store_as<DT>::type* __restrict__ out, int64_t ld_out,
+                                                 int r0, int r1, int raw, int vec, int block) {
     typedef typename store_as<DT>::type T;
     const int nch = m.C / 8;
     const int total = (r1 - r0) * nch;                          // < 2^31, checked by the launcher
-    const int base = (int)blockIdx.x * 1024 + (int)threadIdx.x;
+    const int base = block * 1024 + (int)threadIdx.x;
     int rr[4], j[4];
     bool ok[4];
     uint32_t tag[4];
@@ -110,6 +110,32 @@ __global__ __launch_bounds__(256) void dequant8x4_kernel(sq_matrix m, typename s
             for (int e = 0; e < 8; ++e) o[e] = t[e];
         }
     }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void dequant8x4_kernel(sq_matrix m, typename store_as<DT>::type* __restrict__ out,
+                                                         int64_t ld_out, int r0, int r1, int raw, int vec) {
+    dequant8x4_block<DT>(m, out, ld_out, r0, r1, raw, vec, (int)blockIdx.x);
+}
+
+// The raw fp16 decode of a whole matrix and the fp16 copy of a bf16 activation matrix in one launch: the decode is
+// bound by table gathers out of L2, the copy by HBM, so the copy's `nc` workgroups (8 elements per thread) are dealt
+// evenly among the decode's `nd` and the two overlap instead of running one after the other.
+__global__ __launch_bounds__(256) void dequant8x4_cvt_kernel(sq_matrix m, uint16_t* __restrict__ out, int64_t ld_out,
+                                                             const uint16_t* __restrict__ x, int64_t ldx, int T, int C,
+                                                             uint16_t* __restrict__ xout, int nd, int nc) {
+    const int64_t b = blockIdx.x, total = (int64_t)nd + nc;
+    const int cb = (int)(b * nc / total);                       // copy workgroups before this one
+    if ((int)((b + 1) * nc / total) == cb) {
+        dequant8x4_block<SQ_F16>(m, out, ld_out, 0, m.R, 1, 1, (int)b - cb);
+        return;
+    }
+    const int64_t i = ((int64_t)cb * 256 + threadIdx.x) * 8;
+    if (i >= (int64_t)T * C) return;
+    const int t = (int)(i / C), c = (int)(i - (int64_t)t * C);
+    u32x4 v = *reinterpret_cast<const u32x4*>(x + (int64_t)t * ldx + c);
+    v.x = bf2h_x2(v.x); v.y = bf2h_x2(v.y); v.z = bf2h_x2(v.z); v.w = bf2h_x2(v.w);
+    *reinterpret_cast<u32x4*>(xout + i) = v;
 }
 
 // Matrices with column orders: scattering 2-byte values straight to HBM costs 4x the plain decode, so a
@@ -164,6 +190,10 @@ __global__ __launch_bounds__(256) void dequant_rows_lds_kernel(sq_matrix m, type
     }
 }
 
+static bool dequant8x4_ok(const sq_matrix& m, int64_t n) {
+    return m.d == 8 && !m.perms && n > 0 && n < ((int64_t)1 << 31) - 1024 && ((uintptr_t)m.table & 15) == 0;
+}
+
 template <int DT>
 static int launch_dt(const sq_matrix& m, void* out, int64_t ld_out, int r0, int r1, hipStream_t s, int raw) {
     typedef typename store_as<DT>::type T;
@@ -181,7 +211,7 @@ static int launch_dt(const sq_matrix& m, void* out, int64_t ld_out, int r0, int 
         else hipLaunchKernelGGL((dequant_rows_lds_kernel<DT, 4>), dim3(rgrid), dim3(256), row_bytes, s, m, (T*)out, ld_out, r0, r1, raw, vec_out);
         return check_launch("sq_dequant");
     }
-    if (m.d == 8 && !m.perms && n < ((int64_t)1 << 31) - 1024 && ((uintptr_t)m.table & 15) == 0) {
+    if (dequant8x4_ok(m, n)) {
         const int vec = sizeof(T) == 2 && ((uintptr_t)out & 15) == 0 && ld_out % 8 == 0;
         hipLaunchKernelGGL((dequant8x4_kernel<DT>), dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw, vec);
         return check_launch("sq_dequant");
@@ -191,6 +221,20 @@ static int launch_dt(const sq_matrix& m, void* out, int64_t ld_out, int r0, int 
     else if (m.d == 4) hipLaunchKernelGGL((dequant_kernel<DT, 4>), dim3(grid), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw);
     else hipLaunchKernelGGL((dequant_kernel<DT, 0>), dim3(grid), dim3(256), 0, s, m, (T*)out, ld_out, r0, r1, raw);
     return check_launch("sq_dequant");
+}
+
+// Raw fp16 decode of every row of `m` into out[r * ld_out + c] together with the fp16 copy of the bf16 matrix x
+// [T, C] (row stride ldx, 16-byte aligned rows, C % 8 == 0) into xout [T, C].  Returns 1 without launching
+// anything when the matrix does not take the four-chunk kernel; the caller then launches the two steps itself.
+int launch_dequant_with_cvt(const sq_matrix& m, void* out, int64_t ld_out, const uint16_t* x, int64_t ldx, int T, int C,
+                            uint16_t* xout, hipStream_t s) {
+    const int64_t n = (int64_t)m.R * (m.C / (m.d ? m.d : 1)), ne = (int64_t)T * C;
+    if (!dequant8x4_ok(m, n) || ((uintptr_t)out & 15) || ld_out % 8 || ne <= 0 || ne >= ((int64_t)1 << 40)) return 1;
+    const int64_t nd = (n + 1023) / 1024, nc = (ne / 8 + 255) / 256;
+    if (nd + nc >= ((int64_t)1 << 31)) return 1;
+    hipLaunchKernelGGL(dequant8x4_cvt_kernel, dim3((unsigned)(nd + nc)), dim3(256), 0, s, m, (uint16_t*)out, ld_out, x, ldx, T, C, xout,
+                       (int)nd, (int)nc);
+    return check_launch("sq_linear_gemm(decode + fp16 copy)");
 }
 
 int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s, bool raw) {

@@ -150,6 +150,8 @@ size_t gemm256_part_bytes(int T, int R, int C, int cus);
 int launch_gemm256(const uint16_t* x, int64_t ldx, const uint16_t* w, int64_t ldw, const uint16_t* row_scale, void* y,
                    int y_dtype, int64_t ldy, int y_off, int T, int R, int C, float* part, int cus, hipStream_t s);
 int launch_bf16_to_f16(const uint16_t* x, int64_t ldx, int T, int C, uint16_t* out, hipStream_t s);
+int launch_dequant_with_cvt(const sq_matrix& m, void* out, int64_t ld_out, const uint16_t* x, int64_t ldx, int T, int C,
+                            uint16_t* xout, hipStream_t s);
 
 static bool x_vec_ok(const void* x, int64_t ldx, int C) { return C % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x & 15) == 0; }
 // Activation rows from which the large-tile route (decode each piece once into the workspace as raw fp16
@@ -316,12 +318,23 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
         const uint16_t* xh = (const uint16_t*)x;
         int64_t ldxh = ldx;
         char* wd = (char*)ws;
-        if (x_dtype == SQ_BF16) {
-            int rc = launch_bf16_to_f16((const uint16_t*)x, ldx, T, C, (uint16_t*)ws, s);
-            if (rc) return rc;
+        // bf16 activations are copied to fp16 once; the copy rides along with the first decode when that takes
+        // the four-chunk kernel (the two overlap in one launch), else it is a launch of its own
+        bool copy_pending = x_dtype == SQ_BF16;
+        if (copy_pending) {
             xh = (const uint16_t*)ws;
             ldxh = C;
         }
+        auto decode = [&](const sq_matrix& m, void* w) -> int {
+            if (copy_pending) {
+                copy_pending = false;
+                const int rc = launch_dequant_with_cvt(m, w, C, (const uint16_t*)x, ldx, T, C, (uint16_t*)ws, s);
+                if (rc <= 0) return rc;
+                const int rc2 = launch_bf16_to_f16((const uint16_t*)x, ldx, T, C, (uint16_t*)ws, s);
+                if (rc2) return rc2;
+            }
+            return launch_dequant(m, w, SQ_F16, C, 0, m.R, s, /*raw=*/true);
+        };
         wd += align256((size_t)T * C * 2);
         const int cus0 = device_cus();
         if (stacked_route(mats, n)) {
@@ -334,7 +347,7 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
             int r0 = 0;
             for (int i = 0; i < n; ++i) {
                 const sq_matrix& m = mats[i];
-                int rc = launch_dequant(m, w, SQ_F16, C, 0, m.R, s, /*raw=*/true);
+                int rc = decode(m, w);
                 if (rc) return rc;
                 hipLaunchKernelGGL(copy_u16_kernel, dim3((unsigned)((m.R + 255) / 256)), dim3(256), 0, s, m.row_scale, scales + r0, m.R);
                 rc = check_launch("sq_linear_gemm(row scales)");
@@ -352,7 +365,7 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
         for (int i = 0; i < n; ++i) {
             const sq_matrix& m = mats[i];
             if (m.R == 0) continue;
-            int rc = launch_dequant(m, wd, SQ_F16, C, 0, m.R, s, /*raw=*/true);
+            int rc = decode(m, wd);
             if (rc) return rc;
             rc = launch_gemm256(xh, ldxh, (const uint16_t*)wd, C, m.row_scale, y, y_dtype, ldy, m.y_off, T, m.R, C,
                                 gemm256_part_bytes(T, m.R, C, cus) ? part : nullptr, cus, s);
