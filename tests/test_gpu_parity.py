@@ -373,6 +373,32 @@ def test_gemm_dense_with_workspace_splits_the_last_round():
         assert rel_max_err(plain.float().cpu().numpy(), y[:, :R].float().cpu().numpy().astype(np.float64)) < (1e-5 if dtype == torch.float32 else 1e-2)
 
 
+def test_gemm_stacked_large_codebook_pieces_and_the_activation_copy():
+    # bf16 activations are copied to fp16 once per call; the copy shares the launch of the first decode when that piece
+    # has d = 8 and no column orders, and is a launch of its own otherwise.  Both orders of a plain and a masked piece,
+    # at token counts below, at and above one copy workgroup's 2048 elements per row boundary, and an fp16 call (no copy).
+    from quantexperiments_amd.kernels import linear_gemm
+    plain, masked = synth(300, 1024, 8, 16, seed=31), synth(70, 1024, 8, 15, 1, 4, seed=32)
+    lp, lm = to_device(plain), to_device(masked)
+    for T in (256, 257, 700):
+        for dtype in (torch.bfloat16, torch.float16):
+            x = rand_x(T, 1024, dtype, seed=T)
+            for order in ((plain, lp, masked, lm), (masked, lm, plain, lp)):
+                y = torch.full((T, 370 + 6), 2.0, dtype=torch.float32, device="cuda")
+                linear_gemm([order[1], order[3]], x.cuda(), y[:, :370])
+                ref = np.concatenate([_ref(order[0], x), _ref(order[2], x)], axis=1)
+                assert rel_max_err(y[:, :370].cpu().numpy(), ref) < TOL, (T, dtype)
+                assert (y[:, 370:] == 2.0).all()
+    # one plain piece alone, ragged sizes: the copy's workgroups are dealt among the decode's
+    for (R, C, T) in ((1, 64, 256), (257, 3584, 300), (40, 18944, 256)):
+        s1 = synth(R, C, 8, 16, seed=R + T)
+        l1 = to_device(s1)
+        x = rand_x(T, C, torch.bfloat16, seed=R)
+        y = torch.empty(T, R, dtype=torch.float32, device="cuda")
+        linear_gemm([l1], x.cuda(), y)
+        assert rel_max_err(y.cpu().numpy(), _ref(s1, x)) < TOL, (R, C, T)
+
+
 def test_gemm_of_neighbouring_and_scattered_pieces():
     # pieces that follow each other in Y are multiplied in one tile GEMM over all their rows; pieces with gaps
     # between their column slices (or in another order) one by one.  Both through the raw C ABI.
