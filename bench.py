@@ -200,6 +200,71 @@ def copy_probe(torch, dev):
     return {"bytes_read": 256 << 20, "bytes_written": 256 << 20, "launches": 3}
 
 
+SHAPES_27B = {"q": (5120, 5120), "k": (1024, 5120), "v": (1024, 5120), "o": (5120, 5120), "gate": (17408, 5120),
+              "up": (17408, 5120), "down": (5120, 17408)}
+
+
+def sweep(torch, dev, spec: str, rows: str, n_layers: int):
+    """Other formats and shapes than the headline's, one layer (4 launches) per activation-row count:
+    spec = "<7b|27b>,d,bits,G,M", e.g. "7b,4,12,1,1" (cfg3), "27b,8,16,1,16" (cfg5), "27b,4,12,4,1" (the shipped 27B
+    format).  Up to 32 rows through sq_linear_small, above through sq_linear_gemm; n_layers distinct layers rotated
+    in one HIP graph, HIP events around the replay, median of 5."""
+    from quantexperiments_amd.kernels import PackedLinear, linear_small, linear_gemm, prepare_stack
+    model, d, bits, G, M = spec.split(",")
+    d, bits, G, M = int(d), int(bits), int(G), int(M)
+    shapes = SHAPES_7B if model == "7b" else SHAPES_27B
+    gen = torch.Generator(device=dev).manual_seed(0)
+
+    def make():
+        out = {}
+        for nm, (R, C) in shapes.items():
+            W = (C // d) * bits // 32
+            words = torch.randint(-2**31, 2**31, (R, W), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
+            table = torch.randn(G << bits, d, device=dev, generator=gen).half()
+            rs = (torch.randn(R, device=dev, generator=gen) * 0.005 + 0.02).abs().half()
+            rb = torch.randint(0, G, (R,), device=dev, generator=gen).to(torch.uint8) if G > 1 else None
+            rm = torch.randint(0, M, (R,), device=dev, generator=gen).to(torch.uint8) if M > 1 else None
+            perms = (torch.stack([torch.randperm(C, device=dev, generator=gen) for _ in range(M)]) if M > 1
+                     else torch.arange(C, device=dev)[None])
+            out[nm] = PackedLinear(words, table, rs, rb, rm, perms, 1 << bits, d)
+        for l in LAUNCHES:
+            prepare_stack([out[n] for n in l])
+        return out
+
+    layers = [make() for _ in range(n_layers)]
+    res = {}
+    for B in [int(b) for b in rows.split(",")]:
+        f = linear_small if B <= 32 else linear_gemm
+        xs = {C: torch.randn(B, C, device=dev, generator=gen).to(torch.bfloat16) for C in {c for _, c in shapes.values()}}
+        per, tot = {}, 0.0
+        for l in LAUNCHES:
+            C = shapes[l[0]][1]
+            y = torch.empty(B, sum(shapes[n][0] for n in l), device=dev, dtype=torch.bfloat16)
+
+            def run():
+                for L in layers:
+                    f([L[n] for n in l], xs[C], y)
+            run()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                run()
+            g.replay()
+            torch.cuda.synchronize()
+            ts = []
+            for _ in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(); g.replay(); e1.record()
+                torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1))
+            per["|".join(l)] = sorted(ts)[2] * 1e3 / n_layers
+            tot += per["|".join(l)]
+        nbytes = sum(L.words.numel() * 4 + L.table.numel() * 2 + L.R * 2 for L in layers[0].values())
+        res[f"B{B}"] = {"us_per_layer": tot, "GBps_packed": nbytes / tot / 1e3,
+                        "tflops": 2.0 * B * sum(R * C for R, C in shapes.values()) / tot / 1e6, "per_launch_us": per}
+    return {"sweep": spec, "layers_rotated": n_layers, "rows": res}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,6 +281,10 @@ def main():
     ap.add_argument("--head-only", action="store_true",
                     help="run only the 8-bit lm_head GEMV and print only its object (the command its rocprofv3 "
                          "summary under profiles/ is made with)")
+    ap.add_argument("--sweep", default="", metavar="MODEL,d,bits,G,M",
+                    help="time one layer of another format / shape set instead of the headline workload and print only "
+                         "that object, e.g. 7b,4,12,1,1 (cfg3), 27b,8,16,1,16 (cfg5); see --rows")
+    ap.add_argument("--rows", default="1", help="activation-row counts for --sweep, comma separated")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic to scale rocprofv3 counters by)")
     args = ap.parse_args()
@@ -230,6 +299,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.head_only:
         print(json.dumps({"lm_head": lm_head(torch, dev)}))
+        return
+    if args.sweep:
+        print(json.dumps(sweep(torch, dev, args.sweep, args.rows, min(args.layers, 8 if args.sweep.startswith("27b") else 16))))
         return
     gen = torch.Generator(device=dev).manual_seed(0)
     layers = [make_layer(torch, dev, gen) for _ in range(args.layers)]
