@@ -281,6 +281,33 @@ def test_stream_builder_keeps_every_tag(R, C, bits, runs, M):
     assert np.array_equal(_walk_stream(buf, R, C, 8, bits, eff, NG, row_mask), tags)
 
 
+def test_stream_builder_orders_entries_for_the_lds_banks():
+    """Per entry slot, the 16 lanes of an LDS clock should name codewords in different groups of four banks
+    (tag mod 16): count, for every slot and 16 lanes, the most lanes that share a group with different tags.  Random
+    order gives about 3; the builder's matching has to stay well below 2 on a matrix with full groups."""
+    rng = np.random.default_rng(17)
+    R, C, bits = 512, 3584, 16
+    tags = rng.integers(0, 1 << bits, size=(R, C // 8))
+    buf, runs, NG = _build_stream(O.pack_bits(tags, bits), R, C, bits, None, 1)
+    NV = 16
+    off_slots = ((NV * NG + 1) * 4 + 255) & ~255
+    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
+    off_rows = (off_runs + runs * 16 + 255) & ~255
+    off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
+    goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
+    steps = np.frombuffer(buf, np.uint8, int(goff[-1]) * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.int64)
+    ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
+    e = ent.transpose(0, 2, 1).reshape(-1, 16)                                # [slot x 16-lane clock, lane]
+    tag = e & 0xFFF
+    worst = np.zeros(len(e), np.int64)
+    for g in range(16):
+        t = np.where((tag & 15) == g, tag, -1)
+        t.sort(axis=1)
+        distinct = ((np.diff(t, axis=1) != 0) & (t[:, 1:] >= 0)).sum(1) + (t[:, 0] >= 0)
+        worst = np.maximum(worst, distinct)
+    assert worst.mean() < 1.8, worst.mean()
+
+
 def test_stream_builder_rejects_other_formats():
     import ctypes
     from quantexperiments_amd import _lib
