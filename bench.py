@@ -34,8 +34,8 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes one gate|up launch of stream_kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (37,828.2 KiB x 1.9998 read + 15,263.5 KiB x 1.0 written; scale factors from a 256 MiB copy in the same runs)
-GATE_UP_TRAFFIC_BYTES = 93_090_000
+# (30,601.1 KiB x 1.9998 read + 15,263.3 KiB x 1.0 written; scale factors from a 256 MiB copy in the same runs)
+GATE_UP_TRAFFIC_BYTES = 78_290_000
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16
 
 SHAPES_7B = {"q": (3584, 3584), "k": (512, 3584), "v": (512, 3584), "o": (3584, 3584),
