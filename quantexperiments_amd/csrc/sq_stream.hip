@@ -451,17 +451,17 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     for (int k = 1; k < GEMV_MAX_PIECES_STREAM; ++k)
         if (k < a.n && (int)blockIdx.x >= a.p[k].wg_begin) pi = k;
     const StreamPiece P = a.p[pi];                             // by value: the piece's fields arrive in one batch of scalar loads
-    // Workgroups go to the 8 XCDs in turn (workgroup i to XCD i mod 8), each with an L2 of its own.  With 8 or 16
-    // slices the slice is made a function of the workgroup index modulo 8, so an XCD only ever stages an eighth
-    // of the codebook (one fetch from memory, then hits in its L2), and the workgroups of all buckets that
-    // share a run are neighbours in the grid and arrive together.  Any other mapping is as correct.
+    // Workgroups go to the 8 XCDs in turn (workgroup i to XCD i mod 8), each with an L2 of its own.  When the
+    // bucket count is a multiple of 8 the bucket (and with it the slice) is made a function of the workgroup index
+    // modulo 8, so an XCD only ever stages an eighth of the buckets' slices (one fetch from memory, then hits in
+    // its L2), and the workgroups of all buckets that share a run are neighbours in the grid and arrive together.
+    // Any other mapping is as correct.
     const int local = (int)blockIdx.x - P.wg_begin;
     int v, wi;
-    if ((P.NS & 7) == 0 && (P.wg_begin & 7) == 0) {
-        const int per = P.NS >> 3, rest = local >> 3;           // slices per XCD; index among that XCD's workgroups
-        const int sl = (local & 7) + 8 * (rest % per), rest2 = rest / per;
-        wi = rest2 % P.nwg;
-        v = (rest2 / P.nwg) * P.NS + sl;
+    if ((P.NV & 7) == 0 && (P.wg_begin & 7) == 0) {
+        const int per = P.NV >> 3, rest = local >> 3;           // buckets per XCD; index among that XCD's workgroups
+        v = (local & 7) + 8 * (rest % per);
+        wi = rest / per;
     } else {
         v = local / P.nwg;
         wi = local - v * P.nwg;
