@@ -184,79 +184,159 @@ size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int b
     return P.g.off_steps + (size_t)P.g.total_steps * 768;
 }
 
-// Orders the entries of 16 neighbouring lanes of a group (see the second pass of stream_build_host).
+// The lanes of a wave that one clock of a 16-byte LDS read serves.  A ds_read_b128 takes four clocks; measured on
+// gfx950 (two lanes reading different rows of one bank group while every other lane reads a third address: one extra
+// clock exactly for the pairs listed together here; 256 random address patterns then fit "sum over the four sets of
+// the most distinct addresses in one group of four banks" to within 1 percent), the sets are not 16 consecutive lanes:
+static const int LDS_CLOCK_LANES[4][16] = {
+    {0, 1, 2, 3, 12, 13, 14, 15, 20, 21, 22, 23, 24, 25, 26, 27},
+    {4, 5, 6, 7, 8, 9, 10, 11, 16, 17, 18, 19, 28, 29, 30, 31},
+    {32, 33, 34, 35, 44, 45, 46, 47, 52, 53, 54, 55, 56, 57, 58, 59},
+    {36, 37, 38, 39, 40, 41, 42, 43, 48, 49, 50, 51, 60, 61, 62, 63}};
+
+// Orders the entries of the 16 lanes of one LDS clock (see the second pass of stream_build_host): every entry slot
+// should hold, over the 16 lanes, 16 different codeword bank groups (tag mod 16) and 16 different bank groups of x
+// (chunk mod 16).  A greedy fill (each lane takes the entry that collides least with the lanes before it) followed by
+// hill climbing over the whole group: a lane that collides in a slot swaps that entry with one of its other slots when
+// the two slots together get cheaper.
 struct BankMatch {
     static constexpr uint32_t NONE = 0xFFFFFFFFu;
-    std::vector<uint32_t> by[16][16];        // [lane][codeword bank group]: entries not yet placed
-    uint32_t rep[16][16];                    // one tag of the lane per bank group (for padding), NONE = none
+    std::vector<uint32_t> ent[16];           // [lane][slot]: the lane's real entries in slot order
+    std::vector<uint8_t> ha, hb;             // [slot][16]: lanes per codeword / x bank group
+    std::vector<uint8_t> mx;                 // [slot][4]: fullest codeword group, groups that full; the same for x
     uint32_t cnt[16];
-    int lane_of[16], grp_of[16];
-    bool seen[16];
-    uint32_t slot_n;
 
-    bool avail(int l, int k) const { return cnt[l] > slot_n ? !by[l][k].empty() : rep[l][k] != NONE; }
-    bool augment(int l) {
-        for (int k = 0; k < 16; ++k) {
-            if (!avail(l, k) || seen[k]) continue;
-            seen[k] = true;
-            if (lane_of[k] < 0 || augment(lane_of[k])) { lane_of[k] = l; grp_of[l] = k; return true; }
-        }
-        return false;
-    }
     static unsigned char* rec_of(unsigned char* base, int lane, uint32_t n) {
         return base + (size_t)(n >> 2) * 768 + lane * 12 + (n & 3) * 3;
     }
-    void order_lanes(unsigned char* base, const uint32_t* sl, int q0, uint32_t ns) {
-        bool any = false;
+    static void put(unsigned char* r, uint32_t e) { r[0] = (unsigned char)e; r[1] = (unsigned char)(e >> 8); r[2] = (unsigned char)(e >> 16); }
+    static int ga(uint32_t e) { return (int)(e & 15u); }
+    static int gb(uint32_t e) { return (int)((e >> STREAM_SLICE_BITS) & 15u); }
+    void add(uint32_t n, uint32_t e, int d) { ha[n * 16 + ga(e)] += d; hb[n * 16 + gb(e)] += d; }
+
+    void order_lanes(unsigned char* base, const uint32_t* sl, const int* lanes, uint32_t ns) {
+        uint32_t most = 0;
         for (int l = 0; l < 16; ++l) {
-            const uint32_t s0 = sl[q0 + l];
+            const uint32_t s0 = sl[lanes[l]];
             cnt[l] = (s0 & STREAM_NO_ROW) == STREAM_NO_ROW ? 0u : s0 >> STREAM_ROW_BITS;
-            for (int k = 0; k < 16; ++k) { by[l][k].clear(); rep[l][k] = NONE; }
+            ent[l].resize(cnt[l]);
             for (uint32_t n = 0; n < cnt[l]; ++n) {
-                const unsigned char* r = rec_of(base, q0 + l, n);
-                const uint32_t e = r[0] | (uint32_t)r[1] << 8 | (uint32_t)r[2] << 16;
-                by[l][e & 15u].push_back(e);
-                rep[l][e & 15u] = e & ((1u << STREAM_SLICE_BITS) - 1u);
+                const unsigned char* r = rec_of(base, lanes[l], n);
+                ent[l][n] = r[0] | (uint32_t)r[1] << 8 | (uint32_t)r[2] << 16;
             }
-            any = any || cnt[l] > 0;
+            most = std::max(most, cnt[l]);
         }
-        if (!any) return;
-        for (uint32_t n = 0; n < ns; ++n) {
-            slot_n = n;
-            for (int k = 0; k < 16; ++k) lane_of[k] = grp_of[k] = -1;
-            // lanes that must place an entry first, then those that only repeat one
-            for (int pass = 0; pass < 2; ++pass)
+        if (most == 0) return;
+        ha.assign((size_t)ns * 16, 0);
+        hb.assign((size_t)ns * 16, 0);
+        // greedy fill, slot by slot; the lanes with the fewest entries left choose first
+        int order[16];
+        for (int l = 0; l < 16; ++l) order[l] = l;
+        std::sort(order, order + 16, [this](int x, int y) { return cnt[x] != cnt[y] ? cnt[x] < cnt[y] : x < y; });
+        for (uint32_t n = 0; n < most; ++n)
+            for (int d = 0; d < 16; ++d) {
+                const int l = order[d];
+                if (cnt[l] <= n) continue;
+                uint32_t bi = n;
+                int bc = 1 << 30;
+                for (uint32_t i = n; i < cnt[l]; ++i) {
+                    const int c = ha[n * 16 + ga(ent[l][i])] + hb[n * 16 + gb(ent[l][i])];
+                    if (c < bc) { bc = c; bi = i; if (c == 0) break; }
+                }
+                std::swap(ent[l][n], ent[l][bi]);
+                add(n, ent[l][n], 1);
+            }
+        // Hill climbing.  What a slot costs is the fullest bank group of its codeword reads plus that of its x reads
+        // (clocks); with 16 lanes on 16 bank groups some collisions are forced, and they are cheapest when they share
+        // slots.  A lane in a fullest group swaps that entry with one of its other slots when the clocks of the two
+        // slots together go down (ties: when the sum of squared group counts does).  The fullest group's count after
+        // moving one lane from group p to group q follows from the count, the current maximum and how many groups hold
+        // it, so a candidate costs a few operations.
+        mx.assign((size_t)most * 4, 0);
+        auto rescan = [&](uint32_t n) {
+            uint8_t* m4 = &mx[n * 4];
+            m4[0] = m4[1] = m4[2] = m4[3] = 0;
+            for (int k = 0; k < 16; ++k) {
+                const uint8_t a = ha[n * 16 + k], b = hb[n * 16 + k];
+                if (a > m4[0]) { m4[0] = a; m4[1] = 1; } else if (a == m4[0]) ++m4[1];
+                if (b > m4[2]) { m4[2] = b; m4[3] = 1; } else if (b == m4[2]) ++m4[3];
+            }
+        };
+        // fullest count of histogram h (maximum M held by `at` groups) once a lane leaves group p and joins group q
+        auto moved = [](const uint8_t* h, int M, int at, int p, int q) {
+            if (p == q) return M;
+            if (h[q] + 1 > M) return h[q] + 1;
+            return (h[p] == M && at == 1 && h[q] + 1 < M) ? M - 1 : M;
+        };
+        for (uint32_t n = 0; n < most; ++n) rescan(n);
+        for (int pass = 0; pass < 1; ++pass) {
+            bool improved = false;
+            for (uint32_t n = 0; n < most; ++n) {
+                const uint8_t* an = &ha[n * 16];
+                const uint8_t* bn = &hb[n * 16];
+                const uint8_t* xn = &mx[n * 4];
+                if (xn[0] + xn[2] <= 2) continue;
                 for (int l = 0; l < 16; ++l) {
-                    if (cnt[l] == 0 || (cnt[l] > n) != (pass == 0)) continue;
-                    int best = -1;
-                    for (int k = 0; k < 16; ++k)
-                        if (lane_of[k] < 0 && avail(l, k) && (best < 0 || by[l][k].size() > by[l][best].size())) best = k;
-                    if (best >= 0) { lane_of[best] = l; grp_of[l] = best; continue; }
-                    for (int k = 0; k < 16; ++k) seen[k] = false;
-                    if (augment(l)) continue;
-                    for (int k = 0; k < 16; ++k)                 // no bank group to itself: the fullest one
-                        if (avail(l, k) && (best < 0 || by[l][k].size() > by[l][best].size())) best = k;
-                    grp_of[l] = best;
+                    if (cnt[l] <= n) continue;
+                    const uint32_t e = ent[l][n];
+                    const int ae = ga(e), be = gb(e);
+                    if (!((an[ae] == xn[0] && xn[0] > 1) || (bn[be] == xn[2] && xn[2] > 1))) continue;
+                    int best = 0;
+                    uint32_t bm = n;
+                    for (uint32_t m = 0; m < cnt[l]; ++m) {
+                        if (m == n) continue;
+                        const uint32_t f = ent[l][m];
+                        const int af = ga(f), bf = gb(f);
+                        const uint8_t* am = &ha[m * 16];
+                        const uint8_t* bq = &hb[m * 16];
+                        const uint8_t* xm = &mx[m * 4];
+                        const int clocks = moved(an, xn[0], xn[1], ae, af) + moved(bn, xn[2], xn[3], be, bf) +
+                                           moved(am, xm[0], xm[1], af, ae) + moved(bq, xm[2], xm[3], bf, be) -
+                                           (xn[0] + xn[2] + xm[0] + xm[2]);
+                        if (clocks > 0) continue;
+                        int sq = 0;
+                        if (af != ae) sq += 4 + 2 * ((int)an[af] - an[ae] + am[ae] - am[af]);
+                        if (bf != be) sq += 4 + 2 * ((int)bn[bf] - bn[be] + bq[be] - bq[bf]);
+                        const int delta = clocks * 1024 + sq;
+                        if (delta < best) { best = delta; bm = m; }
+                    }
+                    if (bm != n) {
+                        const uint32_t f = ent[l][bm];
+                        add(n, e, -1); add(bm, f, -1); add(n, f, 1); add(bm, e, 1);
+                        std::swap(ent[l][n], ent[l][bm]);
+                        rescan(n);
+                        rescan(bm);
+                        improved = true;
+                        if (xn[0] + xn[2] <= 2) break;
+                    }
                 }
-            int xuse[16] = {};
+            }
+            if (!improved) break;
+        }
+        // Write the slots back.  A lane that has run out repeats one of its own codewords (from the least used bank
+        // group) against one of the 16 chunks of x that are kept at zero (one per bank group).  A lane without a row,
+        // or whose row has no entry here, reads what a neighbour reads (the same addresses are one broadcast read); the
+        // kernel drops its sum.
+        for (uint32_t n = 0; n < ns; ++n) {
+            uint32_t chosen[16];
+            int donor = -1;
+            for (int l = 0; l < 16; ++l)
+                if (cnt[l] > n) { chosen[l] = ent[l][n]; if (donor < 0) donor = l; }
             for (int l = 0; l < 16; ++l) {
-                if (cnt[l] == 0) continue;
-                const int k = grp_of[l];
-                uint32_t e;
-                if (cnt[l] > n) {
-                    std::vector<uint32_t>& c = by[l][k];
-                    size_t bi = 0;
-                    for (size_t i = 1; i < c.size(); ++i)
-                        if (xuse[(c[i] >> STREAM_SLICE_BITS) & 15u] < xuse[(c[bi] >> STREAM_SLICE_BITS) & 15u]) bi = i;
-                    e = c[bi];
-                    ++xuse[(e >> STREAM_SLICE_BITS) & 15u];
-                    c[bi] = c.back();
-                    c.pop_back();
-                } else {
-                    e = rep[l][k] | ((uint32_t)STREAM_ZERO_CHUNK << STREAM_SLICE_BITS);
-                }
-                unsigned char* r = rec_of(base, q0 + l, n);
-                r[0] = (unsigned char)e; r[1] = (unsigned char)(e >> 8); r[2] = (unsigned char)(e >> 16);
+                if (cnt[l] > n || cnt[l] == 0) continue;
+                uint32_t bi = 0;
+                for (uint32_t i = 1; i < cnt[l]; ++i)
+                    if (ha[n * 16 + ga(ent[l][i])] < ha[n * 16 + ga(ent[l][bi])]) bi = i;
+                int kb = 0;
+                for (int k = 1; k < 16; ++k)
+                    if (hb[n * 16 + k] < hb[n * 16 + kb]) kb = k;
+                chosen[l] = (ent[l][bi] & ((1u << STREAM_SLICE_BITS) - 1u)) | ((uint32_t)(STREAM_ZERO_CHUNK + kb) << STREAM_SLICE_BITS);
+                add(n, chosen[l], 1);
+                if (donor < 0) donor = l;
+            }
+            for (int l = 0; l < 16; ++l) {
+                if (cnt[l] == 0) chosen[l] = donor >= 0 ? chosen[donor] : 0u;
+                put(rec_of(base, lanes[l], n), chosen[l]);
             }
         }
     }
@@ -317,13 +397,9 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
         }
     });
     // Second pass, group by group: the order of a lane's entries is free (padding stays behind them), so it is
-    // chosen to keep the LDS gathers apart.  A 16-byte LDS read of a wave takes four clocks of 16 consecutive lanes
-    // each, and two lanes of a clock collide when their addresses differ but fall into the same group of four banks
-    // (address / 16 mod 16).  For every entry slot and every 16 lanes the entries are picked by a bipartite
-    // matching of lanes to codeword bank groups (greedy, a lane prefers the bank group it has most entries left
-    // in, then Kuhn's augmenting paths for the lanes left without one); among a lane's entries of its bank group
-    // the one whose chunk of x falls into the bank group least used in this slot goes first.  A lane that has run
-    // out repeats whichever of its codewords fits.
+    // chosen to keep the LDS gathers apart.  A 16-byte LDS read of a wave takes four clocks of 16 lanes each
+    // (LDS_CLOCK_LANES), and two lanes of a clock collide when their addresses differ but fall into the same group
+    // of four banks (address / 16 mod 16): BankMatch arranges the entries of each clock's lanes.
     parallel_rows(g.NV * g.NG, [&](int a, int b) {
         BankMatch bm;
         for (int vg = a; vg < b; ++vg) {
@@ -331,7 +407,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             if (ns == 0) continue;
             const uint32_t* sl = slots + (size_t)vg * 64;
             unsigned char* base = steps + (size_t)st0 * 768;
-            for (int q0 = 0; q0 < 64; q0 += 16) bm.order_lanes(base, sl, q0, ns);
+            for (int q = 0; q < 4; ++q) bm.order_lanes(base, sl, LDS_CLOCK_LANES[q], ns);
         }
     });
     if (runs_out) *runs_out = g.runs;
@@ -429,7 +505,7 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 }
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
-constexpr int STREAM_XS = (STREAM_PART_MAX + 1) * 16;   // LDS bytes of one activation row's part of x, plus the zero chunk
+constexpr int STREAM_XS = (STREAM_PART_MAX + 16) * 16;  // LDS bytes of one activation row's part of x, plus 16 zero chunks (one per bank group)
 constexpr int STREAM_PF = 4;          // steps fetched ahead
 
 struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
@@ -675,8 +751,8 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
                 if (tid + k * NW * 64 < nc) xd[tid + k * NW * 64] = q;
             }
         }
-        if (tid < NB)                                            // the chunk that padding entries multiply with
-            reinterpret_cast<u32x4*>(lds + STREAM_TAB + tid * STREAM_XS)[STREAM_ZERO_CHUNK] = u32x4{0u, 0u, 0u, 0u};
+        if (tid < NB * 16)                                       // the chunks that padding entries multiply with
+            reinterpret_cast<u32x4*>(lds + STREAM_TAB + (tid >> 4) * STREAM_XS)[STREAM_ZERO_CHUNK + (tid & 15)] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
         for (int k = 0; k < NT; ++k) dst[tid + k * NW * 64] = t[k];
         if (tid == 0) flag[1] = 2 * NW;

@@ -543,24 +543,61 @@ def test_full_size_gemv_against_c_oracle(shape):
     assert torch.equal(lin.dense(torch.float32).cpu(), torch.from_numpy(w))
 
 
-def test_full_size_gemm_rows_against_gemv():
-    """M = 2048 prefill at 7B gate/up size: every output row of a sample of tokens equals the
-    small path's result for that token within the output rounding (size-independent cross-check),
-    and a sample of outputs is checked against the float64 product."""
+LAYER_7B = (("q", 3584, 3584), ("k", 512, 3584), ("v", 512, 3584), ("o", 3584, 3584), ("gate", 18944, 3584),
+            ("up", 18944, 3584), ("down", 3584, 18944))
+
+
+@pytest.mark.parametrize("launch", [("q", "k", "v"), ("o",), ("gate", "up"), ("down",)], ids="|".join)
+def test_full_7b_layer_stacked_launches_against_c_oracle(launch):
+    """The four launches of one 7B-shaped layer in the headline format (d = 8, 16-bit tags), built the way the
+    benchmark and PackedShards build them (pieces stacked, tag streams cut for the joint launch), one bf16
+    activation row: every output against the float64 product of the C oracle's decode, in fp32 and in bf16
+    (after the reference's stacked forward test, reference tests/test_vllm_ext_core.py:35-58)."""
+    from quantexperiments_amd.kernels import linear_small, prepare_stack
+    shapes = {n: (R, C) for n, R, C in LAYER_7B}
+    C = shapes[launch[0]][1]
+    x = rand_x(1, C, torch.bfloat16, seed=len(launch))
+    pieces, refs = [], []
+    for k, n in enumerate(launch):
+        s = synth(shapes[n][0], C, 8, 16, seed=10 + 7 * k + len(n))
+        pieces.append(to_device(s))
+        w = c_oracle.decode(s.words, 16, C, 8, s.K, s.table, s.row_scale)
+        refs.append(c_oracle.linear(_xf(x), w))
+    prepare_stack(pieces)
+    assert all(p.stream is not None for p in pieces)
+    ref = np.concatenate(refs, axis=1)
+    y = torch.full((1, ref.shape[1]), 7.0, dtype=torch.float32, device="cuda")
+    linear_small(pieces, x.cuda(), y)
+    assert rel_max_err(y.cpu().numpy(), ref) < TOL
+    yb = torch.empty(1, ref.shape[1], dtype=torch.bfloat16, device="cuda")
+    linear_small(pieces, x.cuda(), yb)
+    _check_lowp(yb, ref)
+    assert torch.equal(yb, y.to(torch.bfloat16))              # the 16-bit output is the fp32 one rounded once
+
+
+@pytest.mark.parametrize("shape", [(18944, 3584, 1), (3584, 18944, 1), (5120, 5120, 16)], ids=lambda c: "x".join(map(str, c)))
+def test_full_size_gemm_rows_against_gemv(shape):
+    """M = 2048 prefill at the 7B gate/up and down sizes and at a 27B-class matrix with 16 column orders: every
+    output row of a sample of tokens equals the small path's result for that token within the output rounding
+    (size-independent cross-check), and a sample of outputs is checked against the float64 product."""
     from quantexperiments_amd.kernels import linear_gemm, linear_small
-    s = synth(18944, 3584, 8, 16, seed=0)
+    R, C, M = shape
+    s = synth(R, C, 8, 16, 1, M, seed=0)
     lin = to_device(s)
-    x = rand_x(2048, 3584, torch.bfloat16).cuda()
-    y = torch.empty(2048, 18944, dtype=torch.float32, device="cuda")
+    x = rand_x(2048, C, torch.bfloat16).cuda()
+    y = torch.empty(2048, R, dtype=torch.float32, device="cuda")
     linear_gemm([lin], x, y)
     toks = [0, 1, 127, 128, 1000, 2047]
-    ys = torch.empty(len(toks), 18944, dtype=torch.float32, device="cuda")
+    ys = torch.empty(len(toks), R, dtype=torch.float32, device="cuda")
     linear_small([lin], x[toks].contiguous(), ys)
     a, b = y[toks].cpu().numpy().astype(np.float64), ys.cpu().numpy().astype(np.float64)
     assert np.abs(a - b).max() / np.abs(b).max() < 1e-5
-    w = s.decode()
+    w = c_oracle.decode(s.words, 16, C, 8, s.K, s.table, s.row_scale, None, s.row_mask, s.perms if M > 1 else None)
     ref = c_oracle.linear(x[toks].float().cpu().numpy(), w)
     assert rel_max_err(y[toks].cpu().numpy(), ref) < TOL
+    yb = torch.empty(2048, R, dtype=torch.bfloat16, device="cuda")
+    linear_gemm([lin], x, yb)
+    _check_lowp(yb[toks], ref)
 
 
 # ------------------------------------------------------------------ randomized sweep over the large-codebook paths

@@ -71,7 +71,7 @@ def plugin(monkeypatch):
     monkeypatch.delitem(sys.modules, "quantexperiments_amd.vllm_ext.plugin", raising=False)
     import importlib
     p = importlib.import_module("quantexperiments_amd.vllm_ext.plugin")
-    p._EMBED_BUILT = False
+    p._embedding_is_ours = False
     yield p, mods
     sys.modules.pop("quantexperiments_amd.vllm_ext.plugin", None)
 
@@ -141,15 +141,15 @@ def test_which_method_a_layer_gets(plugin, tmp_path):
     assert c.get_quant_method(voc.ParallelLMHead(), "lm_head") is None
     assert c.get_quant_method(voc.VocabParallelEmbedding(), "model.embed_tokens") is None
     cp = p.ShapeQuantConfig("shapequant.packed", embed_head="packed")
-    assert isinstance(cp.get_quant_method(voc.ParallelLMHead(), "lm_head"), p.ShapeQuantHeadMethod)
-    assert isinstance(cp.get_quant_method(voc.VocabParallelEmbedding(), "model.embed_tokens"), p.ShapeQuantEmbedMethod)
+    assert cp.get_quant_method(voc.ParallelLMHead(), "lm_head").what == "lm_head"
+    assert cp.get_quant_method(voc.VocabParallelEmbedding(), "model.embed_tokens").what == "embed"
     # tensor parallelism is refused before anything touches the GPU
     with pytest.raises(NotImplementedError, match="tensor parallelism"):
         m.create_weights(lin.LinearBase(), 32, [80], 64, 80, torch.bfloat16)
     with pytest.raises(NotImplementedError, match="tensor parallelism"):
         m.create_weights(lin.LinearBase(), 64, [40], 64, 80, torch.bfloat16)
     with pytest.raises(NotImplementedError, match="tensor parallelism"):
-        p.ShapeQuantHeadMethod(cp).create_weights(voc.ParallelLMHead(), 64, [20], 64, 40, torch.bfloat16)
+        p.ShapeQuantAuxMethod(cp, "lm_head").create_weights(voc.ParallelLMHead(), 64, [20], 64, 40, torch.bfloat16)
 
 
 def test_aux_checks_and_head_keep(plugin, tmp_path, monkeypatch):
@@ -158,27 +158,27 @@ def test_aux_checks_and_head_keep(plugin, tmp_path, monkeypatch):
     _packed_dir(tmp_path, aux=False)
     c = p.ShapeQuantConfig("shapequant.packed", embed_head="packed")
     with pytest.raises(ValueError, match="lm_head is None"):
-        p.ShapeQuantHeadMethod(c).create_weights(voc.ParallelLMHead(), 64, [40], 64, 40, torch.bfloat16)
+        p.ShapeQuantAuxMethod(c, "lm_head").create_weights(voc.ParallelLMHead(), 64, [40], 64, 40, torch.bfloat16)
     _packed_dir(tmp_path, aux=True)
     c = p.ShapeQuantConfig("shapequant.packed", embed_head="packed")
     with pytest.raises(ValueError, match=r"\[40, 64\], layer is \[32, 64\]"):        # fewer rows than the file
-        p._aux_check(c, 32, 64, "embed")
+        p._check_aux(c, "embed", 32, 64)
     with pytest.raises(ValueError, match="layer is"):
-        p._aux_check(c, 48, 128, "lm_head")
-    p._aux_check(c, 48, 64, "lm_head")                                               # a padded vocabulary is fine
+        p._check_aux(c, "lm_head", 48, 128)
+    p._check_aux(c, "lm_head", 48, 64)                                               # a padded vocabulary is fine
     with pytest.raises(RuntimeError, match="token embedding was not built"):         # head before embedding
-        p.ShapeQuantHeadMethod(c).create_weights(voc.ParallelLMHead(), 64, [48], 64, 48, torch.bfloat16)
+        p.ShapeQuantAuxMethod(c, "lm_head").create_weights(voc.ParallelLMHead(), 64, [48], 64, 48, torch.bfloat16)
     with pytest.raises(RuntimeError):
-        p.ShapeQuantHeadMethod(c).embedding(voc.ParallelLMHead(), torch.zeros(1, dtype=torch.long))
+        p.ShapeQuantAuxMethod(c, "lm_head").embedding(voc.ParallelLMHead(), torch.zeros(1, dtype=torch.long))
     with pytest.raises(RuntimeError):
-        p.ShapeQuantEmbedMethod(c).apply(voc.VocabParallelEmbedding(), torch.zeros(1, 64))
-    assert p._head_keep() is None
+        p.ShapeQuantAuxMethod(c, "embed").apply(voc.VocabParallelEmbedding(), torch.zeros(1, 64))
+    assert p._kept_token_ids() is None
     np.save(tmp_path / "keep.npy", np.array([0, 3, 2], np.int64))
     monkeypatch.setenv("SHAPEQUANT_HEAD_KEEP", "keep.npy")                           # relative: in the model directory
     with pytest.raises(ValueError, match="ascending"):
-        p._head_keep()
+        p._kept_token_ids()
     np.save(tmp_path / "keep.npy", np.array([0, 2, 39], np.int64))
-    assert p._head_keep().tolist() == [0, 2, 39]
+    assert p._kept_token_ids().tolist() == [0, 2, 39]
 
 
 @pytest.mark.gpu
