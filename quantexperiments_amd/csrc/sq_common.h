@@ -27,7 +27,14 @@ __device__ __forceinline__ uint16_t f2bf(float f) {
     if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
     return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
 }
-__device__ __forceinline__ uint16_t f2h(float f) { return __builtin_bit_cast(uint16_t, (half_t)f); }
+// fp32 -> fp16 bits, round to nearest even.  The empty asm hides where f came from: a multiply feeding this conversion
+// is otherwise folded into v_fma_mixlo_f16, which rounds the exact product to fp16 once, while the same expression
+// elsewhere in a kernel stays v_mul_f32 + v_cvt_f16_f32 (two roundings, the reference's arithmetic) and differs in
+// the last bit of about one value in 2000.
+__device__ __forceinline__ uint16_t f2h(float f) {
+    asm("" : "+v"(f));
+    return __builtin_bit_cast(uint16_t, (half_t)f);
+}
 
 // bf16 bits -> fp16 value (through fp32; exact whenever the value is an fp16 normal,
 // rounds to nearest even in the fp16 subnormal range, +-inf beyond 65504).

@@ -277,19 +277,9 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         if (stream_rows(m0, B) && (x_ok || from)) {
             int j = i + 1;
             while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_rows(mats[j], B) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
-            const size_t ws0 = ws_off, ysz = y_dtype == SQ_F32 ? 4 : 2;
-            const int c0 = counters_used;
-            size_t ws_end = ws0;
-            for (int b0 = 0; b0 < B; b0 += 8) {                 // same partial sums and counters for every pass: one stream
-                ws_off = ws0;
-                counters_used = c0;
-                int rc = launch_stream_group(mats + i, j - i, (const char*)x + (size_t)b0 * ldx * 2, x_dtype, ldx,
-                                             (char*)y + (size_t)b0 * ldy * ysz, y_dtype, ldy, B - b0 < 8 ? B - b0 : 8, B,
-                                             (char*)ws, ws_off, counters, counters_used, s, from);
-                if (rc) return rc;
-                ws_end = ws_off;
-            }
-            ws_off = ws_end;
+            int rc = launch_stream_group(mats + i, j - i, x, x_dtype, ldx, y, y_dtype, ldy, B, (char*)ws, ws_off, counters,
+                                         counters_used, s, from);
+            if (rc) return rc;
             i = j;
             continue;
         }

@@ -6,13 +6,14 @@
 namespace sq {
 
 constexpr int STREAM_SLICE_BITS = 12;        // 4096 codewords of 16 bytes per LDS slice
-constexpr int STREAM_PART_MAX = 640;         // most chunks in one column part (10 bits of an entry are enough)
-constexpr int STREAM_ZERO_CHUNK = STREAM_PART_MAX;   // chunk index of padding entries: a chunk of x kept at zero
+constexpr int STREAM_PART_MAX = 4064;        // most chunks in one column part: its chunks and the 16 zero chunks that padding
+                                             // entries multiply with (chunks PC .. PC + 15 of the part) fit 12 bits of an entry
+constexpr int STREAM_RUN_MAX = 96;           // most groups of 64 rows in one run (a run's partial sums are staged in LDS)
 constexpr int STREAM_ROW_BITS = 19;          // slot = row | count << 19
 constexpr uint32_t STREAM_NO_ROW = (1u << STREAM_ROW_BITS) - 1u;
 constexpr int GEMV_MAX_PIECES_STREAM = 4;
 
-constexpr int STREAM_DEFAULT_WGS = 512;      // workgroups a matrix launched alone should make (2 per CU on 256 CUs)
+constexpr int STREAM_DEFAULT_WGS = 256;      // workgroups a matrix launched alone should make (one per CU on 256 CUs)
 
 struct StreamGeom {
     int U, NS, KP, PC, NV, NG;               // chunks per row, slices, column parts, chunks per part, buckets, groups
@@ -26,10 +27,13 @@ bool stream_format_ok(int R, int C, int d, int bits);
 size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs);
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                       unsigned char* out, size_t bytes, int* runs_out, int* groups_out);
+// sq_matrix.stream_runs is sq_stream_build's runs_out: the run count in the low 16 bits, the groups of the longest run above
+inline int stream_runs_of(const sq_matrix& m) { return m.stream_runs & 0xFFFF; }
+inline int stream_run_max_of(const sq_matrix& m) { return (int)((uint32_t)m.stream_runs >> 16); }
 bool stream_shape(const sq_matrix& m);
 size_t stream_part_bytes(const sq_matrix& m, int B);
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                        int64_t ldy, int nb, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
+                        int64_t ldy, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
                         hipStream_t s, const sq_producer* from = nullptr);
 
 }  // namespace sq

@@ -87,6 +87,7 @@ struct StreamRun { int32_t g0, ng, order, zero; };
 
 struct StreamPlan {
     StreamGeom g;
+    int GR;                          // groups in the longest run
     std::vector<StreamRun> runs;
     std::vector<uint32_t> base;      // [NG * 64]: rows ordered by column order, STREAM_NO_ROW where a group is short
     std::vector<uint16_t> cnt;       // [NV][R]
@@ -123,23 +124,27 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
         for (int q : ngm) { n += (q + GR - 1) / GR; whole = whole && q <= GR; }
         if (n <= runs || whole) break;
     }
-    // A run of 5 to 7 groups leaves one to three of a workgroup's eight waves without a group (shorter runs share
-    // their groups among the waves, longer ones deal groups out as waves finish): 8 groups per run instead.  With
-    // one column order the kernel derives the cut from the run count alone, as ceil(groups / runs) per run.
-    if (GR > 4 && GR < 8) {
-        GR = 8;
-        if (ngm.size() == 1) {
-            const int n = (ngm[0] + GR - 1) / GR;
-            GR = (ngm[0] + n - 1) / n;
+    // A run's partial sums are staged in LDS: no run longer than STREAM_RUN_MAX groups (more runs than asked for then).
+    // With one column order the kernel derives the cut from the run count alone, as ceil(groups / runs) per run: settle
+    // on a run length that this formula gives back.
+    if (GR > STREAM_RUN_MAX) GR = STREAM_RUN_MAX;
+    if (ngm.size() == 1)
+        for (;;) {
+            const int n = (ngm[0] + GR - 1) / GR, g2 = (ngm[0] + n - 1) / n;
+            if (g2 == GR) break;
+            GR = g2;
         }
-    }
+    P.GR = 1;
     P.runs.clear();
     P.base.clear();
     for (size_t i = 0; i < ngm.size(); ++i) {
         const int a = first[i], b = first[i + 1], gbase = (int)(P.base.size() / 64);
         const int m = row_mask ? row_mask[order[a]] : 0;
         for (int k = 0; k < ngm[i] * 64; ++k) P.base.push_back(a + k < b ? order[a + k] : STREAM_NO_ROW);
-        for (int q = 0; q < ngm[i]; q += GR) P.runs.push_back(StreamRun{gbase + q, std::min(GR, ngm[i] - q), m, 0});
+        for (int q = 0; q < ngm[i]; q += GR) {
+            P.runs.push_back(StreamRun{gbase + q, std::min(GR, ngm[i] - q), m, 0});
+            P.GR = std::max(P.GR, std::min(GR, ngm[i] - q));
+        }
     }
     P.g = stream_geom(C, d, bits, (int)(P.base.size() / 64), (int)P.runs.size());
     const StreamGeom& g = P.g;
@@ -214,7 +219,8 @@ struct BankMatch {
     static int gb(uint32_t e) { return (int)((e >> STREAM_SLICE_BITS) & 15u); }
     void add(uint32_t n, uint32_t e, int d) { ha[n * 16 + ga(e)] += d; hb[n * 16 + gb(e)] += d; }
 
-    void order_lanes(unsigned char* base, const uint32_t* sl, const int* lanes, uint32_t ns) {
+    // zero_chunk: the first of the 16 chunks of x that the kernel keeps at zero
+    void order_lanes(unsigned char* base, const uint32_t* sl, const int* lanes, uint32_t ns, uint32_t zero_chunk) {
         uint32_t most = 0;
         for (int l = 0; l < 16; ++l) {
             const uint32_t s0 = sl[lanes[l]];
@@ -330,7 +336,7 @@ struct BankMatch {
                 int kb = 0;
                 for (int k = 1; k < 16; ++k)
                     if (hb[n * 16 + k] < hb[n * 16 + kb]) kb = k;
-                chosen[l] = (ent[l][bi] & ((1u << STREAM_SLICE_BITS) - 1u)) | ((uint32_t)(STREAM_ZERO_CHUNK + kb) << STREAM_SLICE_BITS);
+                chosen[l] = (ent[l][bi] & ((1u << STREAM_SLICE_BITS) - 1u)) | ((uint32_t)(zero_chunk + kb) << STREAM_SLICE_BITS);
                 add(n, chosen[l], 1);
                 if (donor < 0) donor = l;
             }
@@ -348,7 +354,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
     plan_stream(tags, R, W, C, d, bits, row_mask, runs, P);
     const StreamGeom& g = P.g;
     const size_t need = g.off_steps + (size_t)g.total_steps * 768;
-    if (g.total_steps >= ((uint64_t)1 << 32)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: matrix too large");
+    if (g.total_steps >= ((uint64_t)1 << 32) || g.runs >= (1 << 16)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: matrix too large");
     if (bytes < need) return fail(SQ_EINVAL, "sq_stream_build: buffer %zu < %zu", bytes, need);
     memset(out, 0, need);
     memcpy(out, P.goff.data(), P.goff.size() * 4);
@@ -388,7 +394,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
                 const uint32_t k = P.pos[(size_t)v * R + r];
                 const size_t gi = (size_t)v * g.NG + (k >> 6);
                 const uint32_t cap = (P.goff[gi + 1] - P.goff[gi]) * 4u;
-                const uint32_t e = last[v] | ((uint32_t)STREAM_ZERO_CHUNK << STREAM_SLICE_BITS);
+                const uint32_t e = last[v] | ((uint32_t)g.PC << STREAM_SLICE_BITS);
                 for (uint32_t n = q[v]; n < cap; ++n) {
                     unsigned char* rec = steps + ((size_t)P.goff[gi] + (n >> 2)) * 768 + (k & 63) * 12 + (n & 3) * 3;
                     rec[0] = (unsigned char)e; rec[1] = (unsigned char)(e >> 8); rec[2] = (unsigned char)(e >> 16);
@@ -407,10 +413,10 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             if (ns == 0) continue;
             const uint32_t* sl = slots + (size_t)vg * 64;
             unsigned char* base = steps + (size_t)st0 * 768;
-            for (int q = 0; q < 4; ++q) bm.order_lanes(base, sl, LDS_CLOCK_LANES[q], ns);
+            for (int q = 0; q < 4; ++q) bm.order_lanes(base, sl, LDS_CLOCK_LANES[q], ns, (uint32_t)g.PC);
         }
     });
-    if (runs_out) *runs_out = g.runs;
+    if (runs_out) *runs_out = g.runs | (P.GR << 16);
     if (groups_out) *groups_out = g.NG;
     return SQ_OK;
 }
@@ -436,6 +442,8 @@ struct StreamArgs {
     void* y;                          // output row b0
     int64_t ldx, ldy;
     int nb;                           // activation rows of this pass (<= NB)
+    int xs;                           // LDS bytes of one activation row's part of x (its chunks + 16 zero chunks)
+    int nl_max;                       // places of the longest run (64 per group): floats per row of the LDS partial sums
     int x_dtype, y_dtype;
     // Producer of the activation row (stream_kernel<1, NW, PRO> with PRO != 0 only): the row is computed while it is
     // staged instead of being read from x.  PRO 1: round(v * rsqrt(mean(v^2) + eps) * w) with v = h_in + add;
@@ -505,8 +513,11 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 }
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
-constexpr int STREAM_XS = (STREAM_PART_MAX + 16) * 16;  // LDS bytes of one activation row's part of x, plus 16 zero chunks (one per bank group)
 constexpr int STREAM_PF = 4;          // steps fetched ahead
+constexpr int STREAM_NW = 16;         // waves per workgroup: one workgroup per CU
+
+// LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group)
+static inline int stream_xs(int pc) { return (pc + 16) * 16; }
 
 struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
 
@@ -515,11 +526,21 @@ struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
 #define SQ_TRACE_POINT(k)
 #endif
 
-// NB activation rows per pass (every entry's codeword is gathered once and multiplied with NB x chunks), NW waves.
-// LDS: [codebook slice 64 KB][NB x parts of 10 KB][two words of flags].
-template <int NB, int NW, int PRO = 0>
-__global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
+// s_waitcnt immediate that waits until at most n vector-memory operations are outstanding and leaves the other
+// counters alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
+constexpr int stream_vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+typedef const __attribute__((address_space(1))) void* stream_gptr_t;
+typedef __attribute__((address_space(3))) void* stream_lptr_t;
+
+// NB activation rows per pass (every entry's codeword is gathered once and multiplied with NB x chunks), NX chunks of
+// a row's part of x per thread (1: parts of up to 1024 chunks, 4: up to 4096).  One workgroup of 16 waves per CU.
+// LDS: [codebook slice 64 KB][NB x parts of a.xs bytes][partial sums of the run: NB x a.nl_max floats][two words of flags]
+// [16 block sums (PRO 1)].
+template <int NB, int NX, int PRO = 0>
+__global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     static_assert(PRO == 0 || NB == 1, "produced activations: one row");
+    constexpr int NW = STREAM_NW, NTH = NW * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int pi = 0;
@@ -548,28 +569,28 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     // (without column orders every run but the last has ceil(NG / runs) groups: no need to wait for the table)
     const int32_t* run = reinterpret_cast<const int32_t*>(P.stream + P.off_runs) + wi * 4;
     const int gr = (P.NG + P.nwg - 1) / P.nwg;
-    const int g0 = P.perms ? run[0] : wi * gr, ng = P.perms ? run[1] : min(gr, P.NG - g0);
+    const int g0 = P.perms ? run[0] : wi * gr, ng = min(P.perms ? run[1] : min(gr, P.NG - g0), a.nl_max >> 6);
 
     const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG + g0;
     const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
     const unsigned char* steps = P.stream + P.off_steps + lane * 12;
     const size_t np = (size_t)P.NG * 64;
     float* part = P.part + (size_t)v * NB * np;
+    const int xs = a.xs;
     const unsigned char* ldsx = lds + STREAM_TAB;
-    unsigned* flag = reinterpret_cast<unsigned*>(lds + STREAM_TAB + NB * STREAM_XS);   // [0] arrival result, [1] next group
+    float* psum = reinterpret_cast<float*>(lds + STREAM_TAB + NB * xs);          // [NB][a.nl_max], indexed by place - 64 g0
+    unsigned* flag = reinterpret_cast<unsigned*>(psum + (size_t)NB * a.nl_max);  // [0] arrival result, [1] next group
 
     // The groups of a run are sorted longest first.  Wave w starts with group w, then group 2 NW - 1 - w; after
     // that every wave draws the next unclaimed group from a counter in LDS, so all waves stay busy to the end.
     // The head of a group (its first step, its step count, the lane's row and count) is fetched one group
     // ahead; the first one goes out before the staging loads.
     // A run with at most NW / 2 groups would leave waves idle while the others walk their steps a few fetches at
-    // a time; there `split` (2, 4 or 8) waves share a group, each takes a contiguous share of its steps, and
-    // the shares are added in wave order through LDS before the partial sum is stored.
-    // The share count follows from the group count alone (at most 8 waves share), so a row's sums are formed in the
-    // same order whatever NB and NW are.
-    int split = 1;
-    while (ng * split * 2 <= 8) split *= 2;
-    const int sub = wave & (split - 1);
+    // a time; there `split` = 16 / groups waves share a group, each takes a contiguous share of its steps, and
+    // the shares are added in wave order through LDS.  The share count follows from the group count alone, so a
+    // row's sums are formed in the same order whatever NB, NX and PRO are.
+    const int split = ng * 2 <= NW ? NW / ng : 1;
+    const int sub = wave % split;
     // The head of group k from its three loaded words (first step, end step, this lane's slot).
     auto head_from = [&](int k, uint32_t ga, uint32_t gb, uint32_t sl) {
         StreamHead h{ga, (int)(gb - ga), sl};
@@ -617,16 +638,16 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
     for (int q = 0; q < STREAM_PF; ++q) nx[q] = u32x3{0u, 0u, 0u};
 
-    // stage the codebook slice and this part of the NB activation rows (as fp16); the first group's steps are
-    // requested before the LDS stores wait for the staging loads
+    // Stage the codebook slice (copied global -> LDS without passing through registers: a wave instruction moves
+    // 1 KB, lane l to the wave's base + 16 l) and this part of the NB activation rows (as fp16); the first group's
+    // steps are requested before anything waits for the staging loads.
     {
-        const u32x4* src = reinterpret_cast<const u32x4*>(P.table) + (size_t)s * (1 << STREAM_SLICE_BITS);
-        u32x4* dst = reinterpret_cast<u32x4*>(lds);
-        constexpr int NT = (1 << STREAM_SLICE_BITS) / (NW * 64);
-        constexpr int NX = (STREAM_PART_MAX + NW * 64 - 1) / (NW * 64);              // x chunks per thread and row
-        u32x4 t[NT], xq[NB][NX];
+        const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table) + (size_t)s * STREAM_TAB;
 #pragma unroll
-        for (int k = 0; k < NT; ++k) t[k] = src[tid + k * NW * 64];
+        for (int k = 0; k < STREAM_TAB / (NTH * 16); ++k)
+            __builtin_amdgcn_global_load_lds((stream_gptr_t)(src + ((size_t)k * NTH + tid) * 16),
+                                             (stream_lptr_t)(lds + (k * NTH + wave * 64) * 16), 16, 0, 0);
+        u32x4 xq[NB][NX];
         const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
         if (PRO != 0) {
             // every operand of the produced row is requested before anything waits: this thread's chunks, then
@@ -635,54 +656,45 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
             ProRaw raw[NX];
 #pragma unroll
             for (int k = 0; k < NX; ++k) {
-                const int ci = c0 + min(tid + k * NW * 64, nc - 1);
+                const int ci = c0 + min(tid + k * NTH, nc - 1);
                 raw[k] = pm ? pro_gather<PRO>(a, pm + (size_t)ci * 8) : pro_fetch<PRO>(a, ci);
             }
             float rstd = 0.f;
             if (PRO == 1) {
                 // Mean square of the whole row in the stand-alone kernel's order, so both give the same bits: slot j
-                // of 1024 adds the squares of chunks j, j + 1024, ... element by element with fused multiply-adds, each
-                // block of 64 slots is folded by the wave butterfly, the 16 block sums are added in turn.  A thread
-                // here owns slots tid and tid + 512.
-                static_assert(PRO != 1 || NW * 64 == 512, "two slots per thread");
+                // of 1024 (= thread j) adds the squares of chunks j, j + 1024, ... element by element with fused
+                // multiply-adds, each block of 64 slots is folded by the wave butterfly, the 16 block sums are added in
+                // turn.
+                static_assert(NTH == 1024, "one slot per thread");
                 float* red = reinterpret_cast<float*>(flag + 4);
-                float ps[2] = {0.f, 0.f};
-                if (pm == nullptr && nc == P.U && P.U <= NX * 512) {
-                    // one column part, natural order: this thread's chunks are its slots' chunks, already fetched
+                float ps = 0.f;
+                if (pm == nullptr && nc == P.U && P.U <= NX * NTH) {
+                    // one column part, natural order: this thread's chunks are its slot's chunks, already fetched
 #pragma unroll
                     for (int k = 0; k < NX; ++k)
-                        if (tid + k * 512 < P.U) {
+                        if (tid + k * NTH < P.U) {
 #pragma unroll
-                            for (int e = 0; e < 8; ++e) { const float v = pro_v(a, raw[k], e); ps[k & 1] = __builtin_fmaf(v, v, ps[k & 1]); }
+                            for (int e = 0; e < 8; ++e) { const float vv = pro_v(a, raw[k], e); ps = __builtin_fmaf(vv, vv, ps); }
                         }
-                } else if (P.U <= 1024) {                       // one chunk per slot, both fetched together
-                    ProRaw r2[2];
+                } else if (P.U <= NTH) {                        // one chunk per slot
+                    const ProRaw r1 = pro_fetch<1>(a, min(tid, P.U - 1));
+                    if (tid < P.U) {
 #pragma unroll
-                    for (int m = 0; m < 2; ++m) r2[m] = pro_fetch<1>(a, min(tid + m * 512, P.U - 1));
-#pragma unroll
-                    for (int m = 0; m < 2; ++m)
-                        if (tid + m * 512 < P.U) {
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) { const float v = pro_v(a, r2[m], e); ps[m] = __builtin_fmaf(v, v, ps[m]); }
-                        }
+                        for (int e = 0; e < 8; ++e) { const float vv = pro_v(a, r1, e); ps = __builtin_fmaf(vv, vv, ps); }
+                    }
                 } else {
+                    for (int c = tid; c < P.U; c += NTH) {
+                        const ProRaw r = pro_fetch<1>(a, c);
 #pragma unroll
-                    for (int m = 0; m < 2; ++m)
-                        for (int c = tid + m * 512; c < P.U; c += 1024) {
-                            const ProRaw r = pro_fetch<1>(a, c);
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) { const float v = pro_v(a, r, e); ps[m] = __builtin_fmaf(v, v, ps[m]); }
-                        }
+                        for (int e = 0; e < 8; ++e) { const float vv = pro_v(a, r, e); ps = __builtin_fmaf(vv, vv, ps); }
+                    }
                 }
-#pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    ps[m] = wave_sum(ps[m]);
-                    if (lane == 0) red[m * NW + wave] = ps[m];
-                }
+                ps = wave_sum(ps);
+                if (lane == 0) red[wave] = ps;
                 __syncthreads();
                 float tot = 0.f;
 #pragma unroll
-                for (int q = 0; q < 16; ++q) tot += red[q];
+                for (int q = 0; q < NW; ++q) tot += red[q];
                 rstd = rsqrtf(tot / (float)P.C + a.eps);
             }
 #pragma unroll
@@ -692,7 +704,7 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
                 if (pm == nullptr) {
 #pragma unroll
                     for (int k = 0; k < NX; ++k) {
-                        const int c = tid + k * NW * 64;
+                        const int c = tid + k * NTH;
                         if (c >= nc) continue;
                         reinterpret_cast<u32x4*>(a.x_out)[c0 + c] = xq[0][k];
                         if (PRO == 1 && a.h_out) {
@@ -704,7 +716,7 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
                         }
                     }
                 } else {
-                    for (int c = tid; c < nc; c += NW * 64) {
+                    for (int c = tid; c < nc; c += NTH) {
                         const ProRaw r = pro_fetch<PRO>(a, c0 + c);
                         reinterpret_cast<u32x4*>(a.x_out)[c0 + c] = pro_finish<PRO>(a, r, rstd);
                         if (PRO == 1 && a.h_out) {
@@ -721,15 +733,15 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
             if (PRO != 0) {
                 // filled above
             } else if (P.perms == nullptr) {
-                const u32x4* xs = reinterpret_cast<const u32x4*>(xr) + c0;
+                const u32x4* xsrc = reinterpret_cast<const u32x4*>(xr) + c0;
 #pragma unroll
-                for (int k = 0; k < NX; ++k) xq[b][k] = xs[min(tid + k * NW * 64, nc - 1)];
+                for (int k = 0; k < NX; ++k) xq[b][k] = xsrc[min(tid + k * NTH, nc - 1)];
             } else {
                 // chunk j of a row with column order m multiplies x[perm_m[8 j .. 8 j + 7]]
                 const int32_t* pm = P.perms + (size_t)run[2] * P.C + (size_t)c0 * 8;
 #pragma unroll
                 for (int k = 0; k < NX; ++k) {
-                    const int32_t* pk = pm + (size_t)min(tid + k * NW * 64, nc - 1) * 8;
+                    const int32_t* pk = pm + (size_t)min(tid + k * NTH, nc - 1) * 8;
                     const u32x4 i0 = *reinterpret_cast<const u32x4*>(pk), i1 = *reinterpret_cast<const u32x4*>(pk + 4);
                     const uint32_t e0 = xr[i0.x], e1 = xr[i0.y], e2 = xr[i0.z], e3 = xr[i0.w];
                     const uint32_t e4 = xr[i1.x], e5 = xr[i1.y], e6 = xr[i1.z], e7 = xr[i1.w];
@@ -743,25 +755,25 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_TAB + b * STREAM_XS);
+            u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_TAB + b * xs);
 #pragma unroll
             for (int k = 0; k < NX; ++k) {
                 u32x4 q = xq[b][k];
                 if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
-                if (tid + k * NW * 64 < nc) xd[tid + k * NW * 64] = q;
+                if (tid + k * NTH < nc) xd[tid + k * NTH] = q;
             }
         }
         if (tid < NB * 16)                                       // the chunks that padding entries multiply with
-            reinterpret_cast<u32x4*>(lds + STREAM_TAB + (tid >> 4) * STREAM_XS)[STREAM_ZERO_CHUNK + (tid & 15)] = u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int k = 0; k < NT; ++k) dst[tid + k * NW * 64] = t[k];
+            reinterpret_cast<u32x4*>(lds + STREAM_TAB + (tid >> 4) * xs)[P.PC + (tid & 15)] = u32x4{0u, 0u, 0u, 0u};
         if (tid == 0) flag[1] = 2 * NW;
+        // the slice copies were issued before everything except the STREAM_PF loads of the first steps
+        __builtin_amdgcn_s_waitcnt(stream_vmcnt_only(STREAM_PF));
     }
     __syncthreads();
     SQ_TRACE_POINT(1);
 
     float acc_share[NB];                                        // split > 1: this wave's share of its group
-    uint32_t row_share = STREAM_NO_ROW;
+    int k_share = -1;
 #pragma unroll
     for (int b = 0; b < NB; ++b) acc_share[b] = 0.f;
     while (kcur < ng) {
@@ -807,7 +819,7 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
                         const uint32_t ta = (e[j0 + jj] & 0xFFFu) << 4, xa = ((e[j0 + jj] >> 12) & 0xFFFu) << 4;
                         cw[jj] = *reinterpret_cast<const u32x4*>(lds + ta);
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * STREAM_XS + xa);
+                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * xs + xa);
                     }
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
@@ -828,41 +840,54 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
             for (int b = 0; b < NB; ++b) acc[b] = 0.f;
         }
         if (nst == 0) first_steps(hn, nx);                      // a group without steps fetched nothing for its successor
-        // device-scope stores: written through to memory, so other XCDs' L2s never hold a stale copy and no
-        // cache-wide write-back is needed before the workgroup counts itself off
+        // A row's partial sum goes to its place in the run's partial-sum vector in LDS (rows sit at different lanes in
+        // different buckets, so straight from here the 64 lanes would write 64 scattered 4-byte pieces to memory)
         if (split > 1) {
-            row_share = row;
+            k_share = kcur;
 #pragma unroll
             for (int b = 0; b < NB; ++b) acc_share[b] = acc[b];
         } else if (row != STREAM_NO_ROW) {
 #pragma unroll
-            for (int b = 0; b < NB; ++b) __hip_atomic_store(part + b * np + row, acc[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int b = 0; b < NB; ++b) psum[b * a.nl_max + (int)row - g0 * 64] = acc[b];
         }
         kcur = knext;
         knext = kafter;
     }
     if (split > 1) {
-        // the x rows are no longer needed once every wave has left the loop: their LDS holds the shares
-        float* share = reinterpret_cast<float*>(lds + STREAM_TAB);
-        static_assert(NW * 64 * 4 <= STREAM_XS, "shares of one activation row fit its part of x");
+        // the codebook slice is no longer needed once every wave has left the loop: its LDS holds the shares
+        float* share = reinterpret_cast<float*>(lds);
         __syncthreads();
 #pragma unroll
         for (int b = 0; b < NB; ++b) share[(wave * NB + b) * 64 + lane] = acc_share[b];
         __syncthreads();
-        if (sub == 0 && row_share != STREAM_NO_ROW) {
+        if (sub == 0 && k_share >= 0) {
+            const uint32_t row = slots[(size_t)k_share * 64 + lane] & STREAM_NO_ROW;
+            if (row != STREAM_NO_ROW) {
 #pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                float sum = 0.f;
-                for (int j = 0; j < split; ++j) sum += share[((wave + j) * NB + b) * 64 + lane];
-                __hip_atomic_store(part + b * np + row_share, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int b = 0; b < NB; ++b) {
+                    float sum = 0.f;
+                    for (int j = 0; j < split; ++j) sum += share[((wave + j) * NB + b) * 64 + lane];
+                    psum[b * a.nl_max + (int)row - g0 * 64] = sum;
+                }
             }
         }
+    }
+    SQ_TRACE_POINT(2);
+    __syncthreads();
+    // The run's partial sums leave as whole lines (device-scope stores: written through to memory, so other XCDs'
+    // L2s never hold a stale copy and no cache-wide write-back is needed before the workgroup counts itself off).
+    // Places of a short last group hold no row: what is written there is never read.
+    {
+        const int nl = ng * 64;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            for (int i = tid; i < nl; i += NTH)
+                __hip_atomic_store(part + b * np + (size_t)g0 * 64 + i, psum[b * a.nl_max + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // Count this workgroup off once all its partial sums have been acknowledged (the barrier waits for every
     // wave's outstanding stores).  The workgroup that finds every other bucket's workgroup already counted
     // reads all partial sums back with device-scope loads and finishes the rows.
-    SQ_TRACE_POINT(2);
     __builtin_amdgcn_s_waitcnt(0);
     SQ_TRACE_POINT(3);
     __syncthreads();
@@ -889,23 +914,23 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
         // Every load below is unconditional (indices are clamped, missing terms are dropped afterwards): a load the
         // compiler must guard with a branch is waited for before the next one goes out, and the 64 partial sums
         // of a thread would take four trips to memory instead of one.
-        for (int ib = tid; ib < items; ib += 4 * NW * 64) {
+        for (int ib = tid; ib < items; ib += 4 * NTH) {
             float t[4][16], rs[4];
             uint32_t rr[4];
             int bb[4];
             bool live[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                live[q] = ib + q * NW * 64 < items;
-                const int it = min(ib + q * NW * 64, items - 1);
+                live[q] = ib + q * NTH < items;
+                const int it = min(ib + q * NTH, items - 1);
                 bb[q] = it / nl;
             }
             if (P.perms) {                                      // the four row ids in one trip
 #pragma unroll
-                for (int q = 0; q < 4; ++q) rr[q] = rows0[min(ib + q * NW * 64, items - 1) - bb[q] * nl];
+                for (int q = 0; q < 4; ++q) rr[q] = rows0[min(ib + q * NTH, items - 1) - bb[q] * nl];
             } else {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) rr[q] = row_of(min(ib + q * NW * 64, items - 1) - bb[q] * nl);
+                for (int q = 0; q < 4; ++q) rr[q] = row_of(min(ib + q * NTH, items - 1) - bb[q] * nl);
             }
 #pragma unroll
             for (int q = 0; q < 4; ++q)
@@ -914,7 +939,7 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
             for (int q = 0; q < 4; ++q) rs[q] = h2f(P.row_scale[rr[q] != STREAM_NO_ROW ? rr[q] : 0u]);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int it = min(ib + q * NW * 64, items - 1);
+                const int it = min(ib + q * NTH, items - 1);
                 const uint32_t off = (uint32_t)(bb[q] * (int)np + (it - bb[q] * nl));  // uniform base + 32-bit lane offset
 #pragma unroll
                 for (int k = 0; k < 16; ++k)
@@ -930,7 +955,7 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
             }
         }
     } else {
-        for (int it = tid; it < items; it += NW * 64) {
+        for (int it = tid; it < items; it += NTH) {
             const int b = it / nl, i = it - b * nl;
             const uint32_t r = row_of(i);
             if (r == STREAM_NO_ROW) continue;
@@ -951,21 +976,25 @@ __global__ __launch_bounds__(NW * 64) void stream_kernel(StreamArgs a) {
     SQ_TRACE_POINT(6);
 }
 
-template <int NB, int NW, int PRO = 0>
+// LDS bytes of a launch: slice, NB parts of x, NB partial-sum vectors of the longest run, flags, block sums
+static size_t stream_smem(int nb_t, int xs, int nl_max) {
+    return (size_t)STREAM_TAB + (size_t)nb_t * xs + (size_t)nb_t * nl_max * 4 + 16 + 64;
+}
+
+template <int NB, int NX, int PRO = 0>
 static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
     static bool raised = false;
     if (!raised) {
-        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NW, PRO>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NX, PRO>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         (void)hipGetLastError();
         raised = true;
     }
-    const size_t smem = (size_t)STREAM_TAB + (size_t)NB * STREAM_XS + 16 + (PRO == 1 ? 64 : 0);   // + 16 block sums
-    hipLaunchKernelGGL((stream_kernel<NB, NW, PRO>), dim3((unsigned)grid), dim3(NW * 64), smem, s, a);
+    hipLaunchKernelGGL((stream_kernel<NB, NX, PRO>), dim3((unsigned)grid), dim3(STREAM_NW * 64), stream_smem(NB, a.xs, a.nl_max), s, a);
     return check_launch("sq_linear_small(stream)");
 }
 
 bool stream_shape(const sq_matrix& m) {
-    return m.stream && m.stream_runs > 0 && m.stream_groups > 0 && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
+    return m.stream && stream_runs_of(m) > 0 && m.stream_groups > 0 && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
            (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0;
 }
 
@@ -973,14 +1002,15 @@ bool stream_shape(const sq_matrix& m) {
 int stream_pass_rows(int B) { return B > 4 ? 8 : B > 2 ? 4 : B > 1 ? 2 : 1; }
 
 size_t stream_part_bytes(const sq_matrix& m, int B) {
-    const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, m.stream_runs);
+    const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m));
     return (((size_t)g.NV * stream_pass_rows(B) * g.NG * 64 * 4) + 255) & ~(size_t)255;
 }
 
-// Pieces [0, cnt) (same C), activation rows b0 .. b0 + nb - 1 (nb <= 8): one launch.  `counters` is the zeroed head
-// of the workspace.
+// Pieces [0, cnt) (same C), B activation rows in passes of up to 8 (fewer when the parts of x and the runs' partial
+// sums of that many rows do not fit LDS beside the slice): one launch per pass.  `counters` is the zeroed head of the
+// workspace; every pass uses the same partial sums and counters (one stream).
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                        int64_t ldy, int nb, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
+                        int64_t ldy, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
                         hipStream_t s, const sq_producer* from) {
     StreamArgs a;
     a.h_in = nullptr; a.h_out = nullptr; a.add = a.up = a.w = nullptr; a.x_out = nullptr; a.eps = 0.f;
@@ -989,19 +1019,22 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         a.w = (const uint16_t*)from->w; a.x_out = (uint16_t*)from->x_out; a.eps = from->eps;
     }
     a.n = cnt;
-    a.x = (const uint16_t*)x;
-    a.y = y;
     a.ldx = ldx;
     a.ldy = ldy;
-    a.nb = nb;
     a.x_dtype = x_dtype;
     a.y_dtype = y_dtype;
-    int wg = 0;
+    int wg = 0, pc = 0, nl_max = 64;
     for (int k = 0; k < cnt; ++k) {
         const sq_matrix& m = mats[k];
-        const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, m.stream_runs);
-        if (m.stream_groups < (m.R + 63) / 64 || m.stream_runs > m.stream_groups)
-            return fail(SQ_EINVAL, "sq_linear_small: stream_runs %d / stream_groups %d do not fit %d rows", m.stream_runs, m.stream_groups, m.R);
+        const int runs = stream_runs_of(m), run_max = stream_run_max_of(m);
+        const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, runs);
+        if (m.stream_groups < (m.R + 63) / 64 || runs > m.stream_groups || runs < 1 || run_max < 1 || run_max > STREAM_RUN_MAX)
+            return fail(SQ_EINVAL, "sq_linear_small: stream_runs 0x%x / stream_groups %d do not fit %d rows", m.stream_runs, m.stream_groups, m.R);
+        // Without column orders the kernel cuts the groups into runs of ceil(groups / runs) itself: a run count that
+        // leaves the last run empty, or whose runs are longer than the buffer says, is not one the builder made.
+        const int gr = (g.NG + runs - 1) / runs;
+        if (!m.perms && ((runs - 1) * gr >= g.NG || gr != run_max))
+            return fail(SQ_EINVAL, "sq_linear_small: stream_runs 0x%x does not cut %d groups the way the builder does", m.stream_runs, m.stream_groups);
         StreamPiece& P = a.p[k];
         P.stream = (const unsigned char*)m.stream;
         P.table = m.table;
@@ -1019,18 +1052,38 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         P.wg_begin = wg;
         P.nwg = nwg;
         wg += g.NV * nwg;
+        pc = g.PC;                                               // (pieces of one launch share C)
+        nl_max = std::max(nl_max, run_max * 64);
     }
     for (int k = cnt; k < GEMV_MAX_PIECES_STREAM; ++k) a.p[k] = a.p[0];
+    a.xs = stream_xs(pc);
+    a.nl_max = nl_max;
+    if (stream_smem(1, a.xs, a.nl_max) > 160 * 1024)
+        return fail(SQ_EUNSUPPORTED, "sq_linear_small: rows of %d chunks per column part do not fit LDS", pc);
+    const bool nx4 = pc > STREAM_NW * 64;
     if (from) {
-        if (nb != 1) return fail(SQ_EINVAL, "sq_linear_small_from: fused producers take one activation row");
-        return from->mode == 1 ? stream_launch<1, 8, 1>(a, wg, s) : stream_launch<1, 8, 2>(a, wg, s);
+        if (B != 1) return fail(SQ_EINVAL, "sq_linear_small_from: fused producers take one activation row");
+        a.x = (const uint16_t*)x; a.y = y; a.nb = 1;
+        if (from->mode == 1) return nx4 ? stream_launch<1, 4, 1>(a, wg, s) : stream_launch<1, 1, 1>(a, wg, s);
+        return nx4 ? stream_launch<1, 4, 2>(a, wg, s) : stream_launch<1, 1, 2>(a, wg, s);
     }
-    switch (stream_pass_rows(nb)) {
-        case 1: return stream_launch<1, 8>(a, wg, s);           // 74 KB of LDS: two workgroups of 8 waves per CU
-        case 2: return stream_launch<2, 16>(a, wg, s);          // from here one workgroup of 16 waves per CU
-        case 4: return stream_launch<4, 16>(a, wg, s);
-        default: return stream_launch<8, 16>(a, wg, s);
+    int rows = stream_pass_rows(B);
+    while (rows > 1 && stream_smem(rows, a.xs, a.nl_max) > 160 * 1024) rows >>= 1;
+    const size_t ysz = y_dtype == SQ_F32 ? 4 : 2;
+    for (int b0 = 0; b0 < B; b0 += rows) {
+        a.x = (const uint16_t*)((const char*)x + (size_t)b0 * ldx * 2);
+        a.y = (char*)y + (size_t)b0 * ldy * ysz;
+        a.nb = std::min(rows, B - b0);
+        int rc;
+        switch (rows) {
+            case 1: rc = nx4 ? stream_launch<1, 4>(a, wg, s) : stream_launch<1, 1>(a, wg, s); break;
+            case 2: rc = nx4 ? stream_launch<2, 4>(a, wg, s) : stream_launch<2, 1>(a, wg, s); break;
+            case 4: rc = nx4 ? stream_launch<4, 4>(a, wg, s) : stream_launch<4, 1>(a, wg, s); break;
+            default: rc = nx4 ? fail(SQ_ELAUNCH, "sq_linear_small: 8 rows of more than 1024 chunks cannot fit LDS") : stream_launch<8, 1>(a, wg, s); break;
+        }
+        if (rc) return rc;
     }
+    return SQ_OK;
 }
 
 }  // namespace sq

@@ -42,7 +42,7 @@ class PackedLinear(torch.nn.Module):
     """A block linear run from packed tensors."""
 
     def __init__(self, words, table, row_scale, row_book, row_mask, perms, K: int, d: int, bias=None,
-                 stream: bool = True):
+                 stream: bool | str = True):
         super().__init__()
         R, W = words.shape
         dev = words.device
@@ -85,8 +85,12 @@ class PackedLinear(torch.nn.Module):
         self.stream_runs = self.stream_groups = 0
         self.stream_asked = None
         self.stream_tiled = False
-        if stream and self.G == 1 and table.numel() * 2 > 128 * 1024:
-            self.build_stream(0)
+        # stream: True builds now, cut for a launch of this matrix alone; "later" leaves the build to prepare_stack
+        # (pieces that will be launched together are cut for the joint launch, and built once); False: never
+        self.wants_stream = bool(stream) and self.G == 1 and table.numel() * 2 > 128 * 1024 and d == 8 and 12 < self.bits <= 16
+        if self.wants_stream:
+            if stream != "later":
+                self.build_stream(0)
         elif stream and not self.has_mask and d == 4 and table.numel() * 2 <= 128 * 1024:
             # codebooks that live in LDS (d = 4): a tile-major copy of the tags, which the decode-time kernel
             # reads with fully coalesced loads (same call; the library picks the layout by format)
@@ -99,17 +103,19 @@ class PackedLinear(torch.nn.Module):
         self.stream, self.stream_runs, self.stream_groups = build_stream(
             self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs)
         self.stream_asked = runs
+        if self.stream is None:
+            self.wants_stream = False
 
     # ------------------------------------------------------------------ construction
     @classmethod
-    def from_packed(cls, pf, name: str, device="cuda", bias=None):
+    def from_packed(cls, pf, name: str, device="cuda", bias=None, stream: bool | str = True):
         m = pf.meta[name]
         t = pf.tensors(name)
         dev = torch.device(device)
         return cls(t["tags"].to(dev), t["table"].to(dev), t["row_scale"].to(dev),
                    t["row_book"].to(dev) if "row_book" in t else None,
                    t["row_mask"].to(dev) if "row_mask" in t else None,
-                   pf.perms(name).to(dev), m["K"], m["d"], bias=bias)
+                   pf.perms(name).to(dev), m["K"], m["d"], bias=bias, stream=stream)
 
     @property
     def device(self):
@@ -167,8 +173,8 @@ class PackedLinear(torch.nn.Module):
 
 def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, runs: int = 0):
     """(stream, runs, groups): the bucketed tag stream of one matrix (sq_stream_build) as a uint8 tensor on
-    words' device with the run and group counts the library cut it into, or (None, 0, 0) when the format is not
-    covered.  The regrouping itself is the library's host routine; the tags make one trip to host memory at
+    words' device with the library's runs_out (run count and longest run, packed) and group count, to be handed
+    back in sq_matrix, or (None, 0, 0) when the format is not covered.  The regrouping itself is the library's host routine; the tags make one trip to host memory at
     load time."""
     L = _lib.lib()
     host = words.detach().to("cpu", torch.int32).contiguous()
@@ -185,15 +191,24 @@ def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, 
     return out.to(words.device), r.value, g.value
 
 
-def prepare_stack(pieces, workgroups: int = 512) -> None:
+STREAM_PART_MAX = 4064      # chunks per column part of the tag stream (sq_stream.h)
+
+
+def prepare_stack(pieces, workgroups: int | None = None) -> None:
     """Cut the streams of pieces that are launched together so that the launch makes about `workgroups`
-    workgroups in total (two per CU on an MI355X), shared by rows.  Pieces without a stream are left alone."""
-    ps = [p for p in pieces if p.stream is not None and not p.stream_tiled]
+    workgroups in total (default: one per compute unit of the pieces' device), shared by rows.  Pieces without a
+    stream are left alone; a piece whose stream was not built yet (PackedLinear(..., stream="later")) is built here,
+    once."""
+    ps = [p for p in pieces if p.wants_stream and not p.stream_tiled]
+    if not ps:
+        return
+    if workgroups is None:
+        workgroups = torch.cuda.get_device_properties(ps[0].device).multi_processor_count
     rows = sum(p.R for p in ps)
     for p in ps:
-        buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // 640)
+        buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // STREAM_PART_MAX)
         runs = max(1, round(workgroups * p.R / rows / buckets))
-        if runs != p.stream_asked and not (len(ps) == 1 and p.stream_asked == 0):
+        if p.stream is None or (runs != p.stream_asked and not (len(ps) == 1 and p.stream_asked == 0)):
             p.build_stream(runs)
 
 

@@ -141,7 +141,9 @@ class PackedShards:
     @classmethod
     def from_packed(cls, pf, names: list, dev="cuda", **kw) -> "PackedShards":
         with neutral_defaults():
-            return cls([PackedLinear.from_packed(pf, n, device=dev) for n in names], **kw)
+            # stacked pieces get their tag streams in prepare_stack, cut for the joint launch (built once)
+            later = "later" if len(names) > 1 else True
+            return cls([PackedLinear.from_packed(pf, n, device=dev, stream=later) for n in names], **kw)
 
     # ------------------------------------------------------------------ bookkeeping
     def key(self) -> tuple:

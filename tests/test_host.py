@@ -192,13 +192,17 @@ def _build_stream(words, R, C, bits, row_mask, runs):
     args = (ptr, R, W, C, 8, bits, mp, runs, out.ctypes.data_as(ctypes.c_void_p))
     assert L.sq_stream_build(*args, n, ctypes.byref(r), ctypes.byref(g)) == 0
     assert L.sq_stream_build(*args, n - 1, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EINVAL
-    return out.tobytes(), r.value, g.value
+    # runs_out: the run count in the low 16 bits, the groups of the longest run above
+    return out.tobytes(), r.value & 0xFFFF, g.value
+
+
+PART_MAX = 4064     # chunks per column part (sq_stream.h)
 
 
 def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
     """Rebuild the [R, C/d] tag matrix from a stream buffer, checking its structure on the way."""
     U, NS = C // d, 1 << (bits - 12)
-    KP = -(-U // 640)
+    KP = -(-U // PART_MAX)
     PC = -(-U // KP)
     NV = NS * KP
     off_slots = ((NV * NG + 1) * 4 + 255) & ~255
@@ -253,11 +257,11 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
                 if not real[k] or int(cnts[k]) == 0:
                     # a lane without a row or without entries reads valid addresses (what a neighbour reads, or zeros);
                     # the kernel drops its sum
-                    assert ((e[lane] >> 12) < 656).all()
+                    assert ((e[lane] >> 12) < PC + 16).all()
                     continue
                 c = int(cnts[k])
                 # padding: one of the row's codewords of the bucket again, at one of the 16 zero chunks of x
-                assert ((e[lane, c:] >> 12 >= 640) & (e[lane, c:] >> 12 < 656)).all()
+                assert ((e[lane, c:] >> 12 >= PC) & (e[lane, c:] >> 12 < PC + 16)).all()
                 assert set((e[lane, c:] & 0xFFF).tolist()) <= set((e[lane, :c] & 0xFFF).tolist())
                 # the entries of a lane come in an order chosen for the LDS banks: every chunk once, any order
                 chunk = (e[lane, :c] >> 12) + kp * PC
@@ -269,7 +273,9 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
 
 @pytest.mark.parametrize("R,C,bits,runs,M", [(70, 512, 16, 0, 1), (130, 5376, 16, 2, 1), (64, 1024, 13, 5, 1), (1, 8, 14, 0, 1),
                                               (1100, 256, 15, 4, 1), (1100, 256, 15, 7, 1), (300, 512, 16, 3, 4),
-                                              (1000, 256, 14, 2, 16), (5, 64, 16, 0, 3)])
+                                              (1000, 256, 14, 2, 16), (5, 64, 16, 0, 3),
+                                              (12900, 64, 14, 1, 1),          # a run longer than the cap: more runs than asked for
+                                              (70, 32800, 16, 0, 1)])         # more chunks than one column part holds
 def test_stream_builder_keeps_every_tag(R, C, bits, runs, M):
     rng = np.random.default_rng(R + C + M)
     U = C // 8
