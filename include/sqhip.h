@@ -73,6 +73,18 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
                     void* y, int y_dtype, int64_t ldy, int32_t B, void* workspace, size_t ws_bytes,
                     void* stream);
 
+/* sq_linear_small without a workspace argument, for callers that cannot allocate device memory (code under HIP graph
+ * capture that has not grown a workspace beforehand, tight serving loops, harnesses that forbid hipMalloc): same
+ * arguments, same kernels and bit-identical results, with the partial sums and arrival counters kept in a device array
+ * of SQ_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on until the process ends.  It has no
+ * counterpart in the reference (whose launchers grow torch buffers on demand).  Pieces and row counts whose workspace
+ * (sq_workspace_bytes(mats, n_mats, B, 0)) exceeds the array are refused with SQ_EWORKSPACE; nothing is allocated or freed,
+ * here or in anything it calls.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (two streams, two threads) race; calls on one stream are safe. */
+#define SQ_NOALLOC_SCRATCH_BYTES (16u << 20)
+int sq_linear_small_noalloc(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx,
+                            void* y, int y_dtype, int64_t ldy, int32_t B, void* stream);
+
 /* Prefill product for T activation rows: dequantise-into-LDS tile GEMM on fp16 MFMA with fp32
  * accumulation, row scale applied to the accumulator.  Same argument meaning as sq_linear_small.
  * Replaces runs_gemm.gemm (reference shapequant/kernels/runs_gemm.py:471-514).  Pieces with

@@ -13,6 +13,7 @@ LIB_PATH = _HERE / "libsqhip.so"
 SQ_F32, SQ_F16, SQ_BF16 = 0, 1, 2
 SQ_OK, SQ_EINVAL, SQ_EUNSUPPORTED, SQ_EWORKSPACE, SQ_ELAUNCH = 0, -1, -2, -3, -4
 SMALL_BMAX = 32
+NOALLOC_SCRATCH_BYTES = 16 << 20
 
 DTYPES = {torch.float32: SQ_F32, torch.float16: SQ_F16, torch.bfloat16: SQ_BF16}
 
@@ -62,6 +63,8 @@ def lib() -> ctypes.CDLL:
         L.sq_dequant.argtypes = [mp, vp, ctypes.c_int, i64, i32, i32, vp]
         L.sq_linear_small.argtypes = [mp, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
         L.sq_linear_gemm.argtypes = [mp, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
+        L.sq_linear_small_noalloc.argtypes = [mp, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp]
+        L.sq_linear_small_noalloc.restype = ctypes.c_int
         L.sq_gemm_dense.argtypes = [vp, ctypes.c_int, i64, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp]
         L.sq_gemm_dense_ws.argtypes = [vp, ctypes.c_int, i64, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
         L.sq_gemm_dense_ws.restype = ctypes.c_int
@@ -93,7 +96,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
            "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build", "sq_q8_linear", "sq_q8_workspace_bytes",
            "sq_q8_dequant", "sq_q4_embed", "sq_addnorm", "sq_silu_mul",
-           "sq_linear_small_from", "sq_gemm_dense_ws", "sq_gemm_dense_workspace_bytes")
+           "sq_linear_small_from", "sq_gemm_dense_ws", "sq_gemm_dense_workspace_bytes", "sq_linear_small_noalloc")
 
 
 def check(rc: int) -> None:

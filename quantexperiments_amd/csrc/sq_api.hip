@@ -102,6 +102,52 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
                         has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
 }
 
+// ---- sq_linear_small for callers that cannot allocate: the workspace is a device array of this library.
+// In host code `g_static_scratch` is only a handle for hipGetSymbolAddress: the device address it stands for is looked
+// up once per device and kept; kernels are handed that address, never the symbol.
+static __device__ __align__(256) unsigned char g_static_scratch[SQ_NOALLOC_SCRATCH_BYTES];
+static void* g_static_scratch_ptr[64];
+
+__global__ void noalloc_clear_kernel(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// this device's copy of the scratch array (its address, looked up on first use with the device current), or nullptr + error
+static void* static_scratch(hipStream_t s) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { fail(SQ_ELAUNCH, "sq_linear_small_noalloc: no current device"); return nullptr; }
+    if (!g_static_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
+        if (e != hipSuccess || !ptr) { fail(SQ_ELAUNCH, "sq_linear_small_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e)); return nullptr; }
+        // the arrival counters at the head must be zero before the first call (a fill kernel, not a memset node, so
+        // that this is also safe as the first thing a graph capture records)
+        hipLaunchKernelGGL(noalloc_clear_kernel, dim3((unsigned)(SQ_WS_HEADER / 4 / 256)), dim3(256), 0, s, (unsigned*)ptr, (int)(SQ_WS_HEADER / 4));
+        if (check_launch("sq_linear_small_noalloc(clear)")) return nullptr;
+        g_static_scratch_ptr[dev] = ptr;
+    }
+    return g_static_scratch_ptr[dev];
+}
+
+int sq_linear_small_noalloc(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                            int64_t ldy, int32_t B, void* stream) {
+    int rc = check_xy("sq_linear_small_noalloc", mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B);
+    if (rc) return rc;
+    if (B > SQ_SMALL_BMAX) return fail(SQ_EINVAL, "sq_linear_small_noalloc: B %d > %d", B, SQ_SMALL_BMAX);
+    if (B == 0 || n_mats == 0) return SQ_OK;
+    const size_t need = sq_workspace_bytes(mats, n_mats, B, 0);
+    if (need > (size_t)SQ_NOALLOC_SCRATCH_BYTES)
+        return fail(SQ_EWORKSPACE, "sq_linear_small_noalloc: these pieces need %zu bytes of workspace at %d rows, the built-in scratch holds %u "
+                                   "(use sq_linear_small with a workspace of the caller's)", need, B, (unsigned)SQ_NOALLOC_SCRATCH_BYTES);
+    char* ws = (char*)static_scratch((hipStream_t)stream);
+    if (!ws) return SQ_ELAUNCH;
+    const size_t inner = (size_t)SQ_NOALLOC_SCRATCH_BYTES - SQ_WS_HEADER;
+    if (small_takes_gemm_route(mats, n_mats, B, x, ldx))
+        return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, ws + SQ_WS_HEADER, inner, (unsigned*)ws, (hipStream_t)stream);
+    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, ws + SQ_WS_HEADER, inner, (unsigned*)ws, (hipStream_t)stream);
+}
+
 int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_producer* from, int x_dtype, void* y, int y_dtype,
                          int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream) {
     const char* who = "sq_linear_small_from";

@@ -36,6 +36,10 @@
 #include <vector>
 #include "sq_stream.h"
 
+#ifndef SQ_STREAM_CLIMB
+#define SQ_STREAM_CLIMB 1                  // hill-climbing passes of the entry ordering (load time against LDS collisions)
+#endif
+
 namespace sq {
 
 StreamGeom stream_geom(int C, int d, int bits, int groups, int runs) {
@@ -275,7 +279,7 @@ struct BankMatch {
             return (h[p] == M && at == 1 && h[q] + 1 < M) ? M - 1 : M;
         };
         for (uint32_t n = 0; n < most; ++n) rescan(n);
-        for (int pass = 0; pass < 1; ++pass) {
+        for (int pass = 0; pass < SQ_STREAM_CLIMB; ++pass) {
             bool improved = false;
             for (uint32_t n = 0; n < most; ++n) {
                 const uint8_t* an = &ha[n * 16];
@@ -513,7 +517,10 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 }
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
-constexpr int STREAM_PF = 4;          // steps fetched ahead
+#ifndef SQ_STREAM_PF
+#define SQ_STREAM_PF 4
+#endif
+constexpr int STREAM_PF = SQ_STREAM_PF;   // steps fetched ahead
 constexpr int STREAM_NW = 16;         // waves per workgroup: one workgroup per CU
 
 // LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group)
@@ -524,6 +531,9 @@ struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
 // Optional per-wave timeline (debug builds define SQ_TRACE_POINT).
 #ifndef SQ_TRACE_POINT
 #define SQ_TRACE_POINT(k)
+#endif
+#ifndef SQ_TRACE_DEP
+#define SQ_TRACE_DEP(k, reg, v)         // a point taken once value v (in a "s" or "v" register) has arrived
 #endif
 
 // s_waitcnt immediate that waits until at most n vector-memory operations are outstanding and leaves the other
@@ -548,6 +558,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     for (int k = 1; k < GEMV_MAX_PIECES_STREAM; ++k)
         if (k < a.n && (int)blockIdx.x >= a.p[k].wg_begin) pi = k;
     const StreamPiece P = a.p[pi];                             // by value: the piece's fields arrive in one batch of scalar loads
+    SQ_TRACE_DEP(7, "s", P.NV);
     // Workgroups go to the 8 XCDs in turn (workgroup i to XCD i mod 8), each with an L2 of its own.  When the
     // bucket count is a multiple of 8 the bucket (and with it the slice) is made a function of the workgroup index
     // modulo 8, so an XCD only ever stages an eighth of the buckets' slices (one fetch from memory, then hits in
@@ -750,9 +761,11 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        SQ_TRACE_DEP(8, "v", head_s);
         hn = head_from(kcur, head_a, head_b, head_s);
         first_steps_always(hn, nx);
         __builtin_amdgcn_sched_barrier(0);
+        SQ_TRACE_DEP(9, "v", xq[0][0].x);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_TAB + b * xs);
@@ -768,6 +781,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         if (tid == 0) flag[1] = 2 * NW;
         // the slice copies were issued before everything except the STREAM_PF loads of the first steps
         __builtin_amdgcn_s_waitcnt(stream_vmcnt_only(STREAM_PF));
+        SQ_TRACE_POINT(10);
     }
     __syncthreads();
     SQ_TRACE_POINT(1);
@@ -817,9 +831,18 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
                         const uint32_t ta = (e[j0 + jj] & 0xFFFu) << 4, xa = ((e[j0 + jj] >> 12) & 0xFFFu) << 4;
+#if defined(SQ_EXP_NO_CW)                                       /* timing experiments only (wrong results) */
+                        cw[jj] = u32x4{ta, xa, ta, xa};
+#else
                         cw[jj] = *reinterpret_cast<const u32x4*>(lds + ta);
+#endif
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * xs + xa);
+                        for (int b = 0; b < NB; ++b)
+#if defined(SQ_EXP_NO_X)
+                            xv[jj][b] = u32x4{xa, ta, xa, ta};
+#else
+                            xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * xs + xa);
+#endif
                     }
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
