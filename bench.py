@@ -6,18 +6,22 @@ A "step" is one batch-1 pass over the 7 block linears of one Qwen2.5-7B-shaped l
 codebook per matrix, uint16 tags = 2 bits per weight, fp16 row scales, bf16 activations), run as
 the serving path runs it: 4 launches (q|k|v stacked, o, gate|up stacked, down) through the C ABI.
 Steps rotate over enough distinct layers (>= 4x the 256 MB last-level cache) that tags stream from
-HBM.  K steps are captured in one HIP graph and timed between device synchronisations.
+HBM.  K steps are captured in one HIP graph; the graph is replayed several times, each replay timed
+with HIP events on the launch stream, and the median replay counts.
 
-The batch-1 kernels read a load-time regrouping of the tags by codebook slice (about 3.5 bytes per
+The batch-1 kernels read a load-time regrouping of the tags by codebook slice (about 3.4 bytes per
 tag in HBM instead of the file's 2), built by the library when a layer is loaded; value still counts
 the packed file's bytes, which is what the metric is quoted on.
 
 value = packed (algorithmic) bytes of a layer / time per layer, in GB/s.  The same JSON line
 carries us_per_layer, the roofline of the dominant kernel (gate|up launch, HIP events around graph
-replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s, the 8-bit block-32 output head
-(152,064 x 3,584) at decode batch sizes 1 to 64, the layer with its three elementwise neighbours (add + RMS
-norm twice, SiLU * up) as separate launches and fused into the consuming products, and the CPU baseline (the reference's CPU route, oracle
-port, on the host cores).
+replays of that launch alone), the M = 2048 prefill GEMM in TFLOP/s (cfg4), the small-batch crossover
+of the d = 4 / 12-bit format (cfg3), the 27B-class layer with 16 column orders at batch 1 and at 2048
+rows (cfg5), the 8-bit block-32 output head (152,064 x 3,584) at decode batch sizes 1 to 64, the layer
+with its three elementwise neighbours (add + RMS norm twice, SiLU * up) as separate launches and fused
+into the consuming products, and the CPU baseline (the reference's CPU route, oracle port, on the host
+cores).  Synthetic tensors come from one CPU generator (seed 0) consumed in a fixed order: per layer
+and matrix tags, table, row scales, row orders; activations last.
 """
 
 from __future__ import annotations
@@ -33,45 +37,60 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
-# HBM bytes one gate|up launch of stream_kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (30,601.1 KiB x 1.9998 read + 15,263.3 KiB x 1.0 written; scale factors from a 256 MiB copy in the same runs)
-GATE_UP_TRAFFIC_BYTES = 78_290_000
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16
+# HBM bytes one gate|up launch of stream_kernel moves: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of
+# `bench.py --roofline-only --copy-probe`, scaled by the same counters' reading of a 256 MiB copy; the figures and
+# the commands are in the file named here.  It is a property of the kernel as profiled, not measured by this run.
+GATE_UP_TRAFFIC = {"bytes": None, "source": "profiles/stream_kernel_gate_up_7b_bs1.md"}
 
 SHAPES_7B = {"q": (3584, 3584), "k": (512, 3584), "v": (512, 3584), "o": (3584, 3584),
              "gate": (18944, 3584), "up": (18944, 3584), "down": (3584, 18944)}
+SHAPES_27B = {"q": (5120, 5120), "k": (1024, 5120), "v": (1024, 5120), "o": (5120, 5120), "gate": (17408, 5120),
+              "up": (17408, 5120), "down": (5120, 17408)}
 LAUNCHES = (("q", "k", "v"), ("o",), ("gate", "up"), ("down",))
-D, BITS = 8, 16
+REPS = 5
 
 
-def algorithmic_bytes(names, B=1):
-    """tags + table + row scales + x + y of the pieces of one launch, each counted once."""
+def launch_bytes(shapes, names, d, bits, G=1, M=1, B=1):
+    """Algorithmic bytes of one launch: tags + table + row scales (+ row orders and their index) of its pieces, each
+    counted once, + x + y."""
     n = 0
-    C = SHAPES_7B[names[0]][1]
+    C = shapes[names[0]][1]
     for nm in names:
-        R, C = SHAPES_7B[nm]
-        n += R * (C // D) * BITS // 8 + (1 << BITS) * D * 2 + R * 2 + B * R * 2
+        R, C = shapes[nm]
+        n += R * ((C // d) * bits // 32) * 4 + G * (1 << bits) * d * 2 + R * 2 + B * R * 2
+        if G > 1:
+            n += R
+        if M > 1:
+            n += R + M * C * 2
     return n + B * C * 2
 
 
-def make_layer(torch, dev, gen):
-    """One layer of PackedLinear pieces with seeded synthetic contents, generated on the device; the pieces of
-    each launch get their load-time tag streams cut for that launch (as PackedShards does at load)."""
+def make_layer(torch, dev, gen, shapes, d, bits, G=1, M=1):
+    """One layer of PackedLinear pieces with synthetic contents drawn from the CPU generator `gen` (per matrix: tags,
+    table, row scales, codebook ids, row orders); the pieces of each launch get their load-time tag streams cut for
+    that launch (as PackedShards does at load)."""
     from quantexperiments_amd.kernels import PackedLinear, prepare_stack
+    from quantexperiments_amd.masks import seeded_perms
     out = {}
-    for nm, (R, C) in SHAPES_7B.items():
-        W = (C // D) * BITS // 32
-        words = torch.randint(-2 ** 31, 2 ** 31, (R, W), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
-        table = torch.randn(1 << BITS, D, device=dev, generator=gen).to(torch.float16)
-        rs = (torch.randn(R, device=dev, generator=gen) * 0.005 + 0.02).abs().to(torch.float16)
-        out[nm] = PackedLinear(words, table, rs, None, None, torch.arange(C, device=dev)[None], 1 << BITS, D)
+    for i, (nm, (R, C)) in enumerate(shapes.items()):
+        W = (C // d) * bits // 32
+        words = torch.randint(-2 ** 31, 2 ** 31, (R, W), dtype=torch.int64, generator=gen).to(torch.int32)
+        table = torch.randn(G << bits, d, generator=gen).to(torch.float16)
+        rs = (torch.randn(R, generator=gen) * 0.005 + 0.02).abs().to(torch.float16)
+        rb = torch.randint(0, G, (R,), generator=gen).to(torch.uint8) if G > 1 else None
+        rm = torch.randint(0, M, (R,), generator=gen).to(torch.uint8) if M > 1 else None
+        perms = seeded_perms(C, M, gen)
+        t = lambda a: None if a is None else a.to(dev)
+        out[nm] = PackedLinear(t(words), t(table), t(rs), t(rb), t(rm), perms.to(dev), 1 << bits, d, stream="later")
     for l in LAUNCHES:
         prepare_stack([out[n] for n in l])
     return out
 
 
-def timed_graph(torch, fn, reps=5):
-    """ms per replay of a HIP graph of fn(), median of reps; events on torch's current stream."""
+def timed_graph(torch, fn, reps=REPS):
+    """ms per replay of a HIP graph of fn(): median of `reps` replays, each between two events on torch's current
+    stream (the stream the graph's kernels are launched on); one untimed replay first."""
     fn()
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
@@ -87,49 +106,117 @@ def timed_graph(torch, fn, reps=5):
         b.record()
         torch.cuda.synchronize()
         ts.append(a.elapsed_time(b))
-    return sorted(ts)[len(ts) // 2], g
+    del g
+    return sorted(ts)[len(ts) // 2]
 
 
-def cpu_baseline(torch, layer, x):
-    """The reference's CPU route (unpack, gather, scale, fp32 matmul, bf16) on the host cores:
-    one full layer, after a warm-up on k_proj."""
+def cpu_baseline(torch, layer, x, d, bits, shapes):
+    """The reference's CPU route (unpack, gather, scale, fp32 matmul, bf16) on the host cores: one full layer per
+    repetition, median of REPS repetitions after one warm-up."""
     from oracle import sq_oracle as O
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
     host = {nm: (p.words.cpu(), p.table.cpu(), p.row_scale.cpu()) for nm, p in layer.items()}
     xs = {C: x[C].cpu() for C in x}
-    w, t, rs = host["k"]
-    O.torch_cpu_layer(w, t, rs, None, None, BITS, xs[3584])
-    dec = mm = 0.0
-    t0 = time.perf_counter()
-    for nm, (w, t, rs) in host.items():
-        _, a, b = O.torch_cpu_layer(w, t, rs, None, None, BITS, xs[SHAPES_7B[nm][1]])
-        dec += a
-        mm += b
-    total = time.perf_counter() - t0
-    nbytes = sum(algorithmic_bytes(l) for l in LAUNCHES)
+
+    def one_layer():
+        dec = mm = 0.0
+        t0 = time.perf_counter()
+        for nm, (w, t, rs) in host.items():
+            _, a, b = O.torch_cpu_layer(w, t, rs, None, None, bits, xs[shapes[nm][1]])
+            dec += a
+            mm += b
+        return time.perf_counter() - t0, dec, mm
+
+    one_layer()
+    runs = sorted(one_layer() for _ in range(REPS))
+    total, dec, mm = runs[len(runs) // 2]
+    nbytes = sum(launch_bytes(shapes, l, d, bits) for l in LAUNCHES)
     return {"value": nbytes / total / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": "one full 7B-shaped layer (7 matrices, bs=1), 1 repetition after a k_proj warm-up; "
+            "sample": f"one full 7B-shaped layer (7 matrices, bs=1) per repetition, median of {REPS} after one warm-up; "
                       "torch gather + scale + fp32 matmul + bf16 round",
             "us_per_layer": total * 1e6, "decode_s": dec, "matmul_s": mm}
 
 
-def prefill(torch, dev, layer, steps=3):
-    """M = 2048 prefill GEMM at gate/up (18944x3584) and down (3584x18944)."""
+def prefill(torch, dev, layer, shapes, names=("gate", "down"), T=2048):
+    """T-row prefill GEMM of single matrices: ms (median of REPS graph replays) and TFLOP/s."""
     from quantexperiments_amd.kernels import linear_gemm
     res = {}
-    for nm in ("gate", "down"):
-        R, C = SHAPES_7B[nm]
-        x = torch.randn(2048, C, device=dev).to(torch.bfloat16)
-        y = torch.empty(2048, R, device=dev, dtype=torch.bfloat16)
-        ms, g = timed_graph(torch, lambda: linear_gemm([layer[nm]], x, y), reps=steps)
-        del g
-        res[nm] = {"ms": ms, "tflops": 2.0 * 2048 * R * C / (ms * 1e-3) / 1e12}
+    for nm in names:
+        R, C = shapes[nm]
+        x = torch.randn(T, C, device=dev).to(torch.bfloat16)
+        y = torch.empty(T, R, device=dev, dtype=torch.bfloat16)
+        ms = timed_graph(torch, lambda: linear_gemm([layer[nm]], x, y))
+        res[nm] = {"ms": ms, "tflops": 2.0 * T * R * C / (ms * 1e-3) / 1e12}
     return res
 
 
-def lm_head(torch, dev, rows=(1, 4, 8, 16, 32, 64), reps=3):
+def layer_times(torch, dev, layers, shapes, B, fn, gen):
+    """us per launch and per layer of fn(pieces, x, y) over the 4 launches of `layers` rotated inside one graph."""
+    xs = {C: torch.randn(B, C, generator=gen).to(torch.bfloat16).to(dev) for C in sorted({c for _, c in shapes.values()})}
+    per, tot = {}, 0.0
+    for l in LAUNCHES:
+        C = shapes[l[0]][1]
+        y = torch.empty(B, sum(shapes[n][0] for n in l), device=dev, dtype=torch.bfloat16)
+
+        def run():
+            for L in layers:
+                fn([L[n] for n in l], xs[C], y)
+        per["|".join(l)] = timed_graph(torch, run) * 1e3 / len(layers)
+        tot += per["|".join(l)]
+    return tot, per
+
+
+def small_batch_crossover(torch, dev, gen, n_layers):
+    """cfg3: the 7B shapes in the d = 4, K = 4096, 12-bit format (3 bits per weight) at M = 2 .. 32 activation rows:
+    the decode-time kernel (sq_linear_small) against the large-M route (decode to fp16 + tile GEMM), with both
+    rooflines; crossover = the largest M at which the decode-time kernel is still the faster one."""
+    from quantexperiments_amd.kernels import linear_small
+    from quantexperiments_amd.vllm_ext.core import PackedShards
+    d, bits = 4, 12
+    layers = [make_layer(torch, dev, gen, SHAPES_7B, d, bits) for _ in range(n_layers)]
+    shards = [{l: PackedShards([L[n] for n in l], large="dequant") for l in LAUNCHES} for L in layers[:1]]
+    nbytes = sum(launch_bytes(SHAPES_7B, l, d, bits) for l in LAUNCHES)
+    flops1 = 2.0 * sum(R * C for R, C in SHAPES_7B.values())
+    res, cross, small_wins = {}, 0, True
+    for M in (1, 2, 4, 8, 16, 32):
+        small, per = layer_times(torch, dev, layers, SHAPES_7B, M, linear_small, gen)
+        r = {"small_us_per_layer": small, "per_launch_us": per, "GBps_packed": nbytes / small / 1e3,
+             "frac_hbm": nbytes / small / 1e3 / HBM_PEAK_GBS, "tflops": flops1 * M / small / 1e6,
+             "frac_mfma": flops1 * M / small / 1e6 / MFMA_PEAK_TFLOPS}
+        if M > 1:
+            x = {C: torch.randn(M, C, generator=gen).to(torch.bfloat16).to(dev) for C in (3584, 18944)}
+            large = timed_graph(torch, lambda: [shards[0][l]._large(x[SHAPES_7B[l[0]][1]]) for l in LAUNCHES]) * 1e3
+            r["large_us_per_layer"] = large
+            small_wins = small_wins and small <= large
+            if small_wins:
+                cross = M
+        res[f"M{M}"] = r
+    return {"workload": "cfg3: 7B shapes, d=4, K=4096, 12-bit tags (3 bpw), bf16 rows", "layers_rotated": n_layers,
+            "bytes_per_layer": nbytes, "flops_per_row": flops1, "rows": res, "crossover_M": cross,
+            "note": "small = sq_linear_small; large = sq_dequant to fp16 + sq_gemm_dense (the reference's dequant route); "
+                    "crossover_M = largest M of the list up to which small is faster at every M"}
+
+
+def masked_27b(torch, dev, gen, n_layers):
+    """cfg5: the 27B-class layer, d = 8, K = 65,536, 16 column orders per matrix, at batch 1 (HBM roofline) and at
+    2048 rows (MFMA roofline)."""
+    from quantexperiments_amd.kernels import linear_gemm, linear_small
+    d, bits, M = 8, 16, 16
+    layers = [make_layer(torch, dev, gen, SHAPES_27B, d, bits, 1, M) for _ in range(n_layers)]
+    nbytes = sum(launch_bytes(SHAPES_27B, l, d, bits, 1, M) for l in LAUNCHES)
+    flops1 = 2.0 * sum(R * C for R, C in SHAPES_27B.values())
+    us1, per1 = layer_times(torch, dev, layers, SHAPES_27B, 1, linear_small, gen)
+    us2k, per2k = layer_times(torch, dev, layers[:2], SHAPES_27B, 2048, linear_gemm, gen)
+    return {"workload": "cfg5: 27B-class layer (hidden 5120, intermediate 17408), d=8, K=65536, 16 column orders, 4-bit order index per row",
+            "layers_rotated": n_layers, "bytes_per_layer": nbytes,
+            "bs1": {"us_per_layer": us1, "per_launch_us": per1, "GBps_packed": nbytes / us1 / 1e3, "frac_hbm": nbytes / us1 / 1e3 / HBM_PEAK_GBS},
+            "M2048": {"us_per_layer": us2k, "per_launch_us": per2k, "tflops": flops1 * 2048 / us2k / 1e6,
+                      "frac_mfma": flops1 * 2048 / us2k / 1e6 / MFMA_PEAK_TFLOPS}}
+
+
+def lm_head(torch, dev, rows=(1, 4, 8, 16, 32, 64)):
     """The 7B model's 8-bit block-32 output head (152,064 x 3,584 int8 + fp16 block scales = 579 MB, more than
     twice the last-level cache): microseconds and weight bytes per second for a few decode batch sizes."""
     from quantexperiments_amd.kernels import q8_linear
@@ -143,9 +230,7 @@ def lm_head(torch, dev, rows=(1, 4, 8, 16, 32, 64), reps=3):
         x = torch.randn(B, C, device=dev, generator=g).to(torch.bfloat16)
         y = torch.empty(B, V, device=dev, dtype=torch.bfloat16)
         q8_linear(q, sc, x, y)                   # grows the workspace outside capture
-        ms, gr = timed_graph(torch, lambda: [q8_linear(q, sc, x, y) for _ in range(5)], reps=reps)
-        del gr
-        ms /= 5
+        ms = timed_graph(torch, lambda: [q8_linear(q, sc, x, y) for _ in range(5)], reps=3) / 5
         gbs = nbytes / (ms * 1e-3) / 1e9
         res[f"B{B}"] = {"us": ms * 1e3, "achieved": gbs, "frac": gbs / HBM_PEAK_GBS}
     return res
@@ -184,9 +269,7 @@ def neighbours(torch, dev, layers, x, y):
     for name, fn, per in (("layer_separate_us", separate, len(layers)), ("layer_fused_us", fused, len(layers)),
                           ("addnorm_us", lambda: [addnorm(h[0], y[L[1]], w, 1e-6, x1, h_out=h[1]) for _ in range(28)], 28),
                           ("silu_mul_us", lambda: [silu_mul(gate, up, act) for _ in range(28)], 28)):
-        ms, g = timed_graph(torch, fn, reps=3)
-        del g
-        res[name] = ms * 1e3 / per
+        res[name] = timed_graph(torch, fn, reps=3) * 1e3 / per
     return res
 
 
@@ -200,8 +283,20 @@ def copy_probe(torch, dev):
     return {"bytes_read": 256 << 20, "bytes_written": 256 << 20, "launches": 3}
 
 
-SHAPES_27B = {"q": (5120, 5120), "k": (1024, 5120), "v": (1024, 5120), "o": (5120, 5120), "gate": (17408, 5120),
-              "up": (17408, 5120), "down": (5120, 17408)}
+def resident_bytes(layer):
+    """Bytes one layer keeps in HBM, by kind, and per weight."""
+    kinds = {"tags": 0, "tables": 0, "row_scales": 0, "row_orders": 0, "tag_stream": 0}
+    weights = 0
+    for p in layer.values():
+        weights += p.R * p.C
+        size = lambda t: 0 if t is None else t.numel() * t.element_size()
+        kinds["tags"] += size(p.words)
+        kinds["tables"] += size(p.table)
+        kinds["row_scales"] += size(p.row_scale) + size(p.row_book)
+        kinds["row_orders"] += size(p.row_mask) + size(p.perms) + size(p.row_order)
+        kinds["tag_stream"] += size(p.stream)
+    total = sum(kinds.values())
+    return {**kinds, "total": total, "bits_per_weight": 8.0 * total / weights}
 
 
 def sweep(torch, dev, spec: str, rows: str, n_layers: int):
@@ -209,60 +304,19 @@ def sweep(torch, dev, spec: str, rows: str, n_layers: int):
     spec = "<7b|27b>,d,bits,G,M", e.g. "7b,4,12,1,1" (cfg3), "27b,8,16,1,16" (cfg5), "27b,4,12,4,1" (the shipped 27B
     format).  Up to 32 rows through sq_linear_small, above through sq_linear_gemm; n_layers distinct layers rotated
     in one HIP graph, HIP events around the replay, median of 5."""
-    from quantexperiments_amd.kernels import PackedLinear, linear_small, linear_gemm, prepare_stack
+    from quantexperiments_amd.kernels import linear_small, linear_gemm
     model, d, bits, G, M = spec.split(",")
     d, bits, G, M = int(d), int(bits), int(G), int(M)
     shapes = SHAPES_7B if model == "7b" else SHAPES_27B
-    gen = torch.Generator(device=dev).manual_seed(0)
-
-    def make():
-        out = {}
-        for nm, (R, C) in shapes.items():
-            W = (C // d) * bits // 32
-            words = torch.randint(-2**31, 2**31, (R, W), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
-            table = torch.randn(G << bits, d, device=dev, generator=gen).half()
-            rs = (torch.randn(R, device=dev, generator=gen) * 0.005 + 0.02).abs().half()
-            rb = torch.randint(0, G, (R,), device=dev, generator=gen).to(torch.uint8) if G > 1 else None
-            rm = torch.randint(0, M, (R,), device=dev, generator=gen).to(torch.uint8) if M > 1 else None
-            perms = (torch.stack([torch.randperm(C, device=dev, generator=gen) for _ in range(M)]) if M > 1
-                     else torch.arange(C, device=dev)[None])
-            out[nm] = PackedLinear(words, table, rs, rb, rm, perms, 1 << bits, d)
-        for l in LAUNCHES:
-            prepare_stack([out[n] for n in l])
-        return out
-
-    layers = [make() for _ in range(n_layers)]
+    gen = torch.Generator().manual_seed(0)
+    layers = [make_layer(torch, dev, gen, shapes, d, bits, G, M) for _ in range(n_layers)]
+    nbytes = sum(launch_bytes(shapes, l, d, bits, G, M) for l in LAUNCHES)
     res = {}
     for B in [int(b) for b in rows.split(",")]:
-        f = linear_small if B <= 32 else linear_gemm
-        xs = {C: torch.randn(B, C, device=dev, generator=gen).to(torch.bfloat16) for C in {c for _, c in shapes.values()}}
-        per, tot = {}, 0.0
-        for l in LAUNCHES:
-            C = shapes[l[0]][1]
-            y = torch.empty(B, sum(shapes[n][0] for n in l), device=dev, dtype=torch.bfloat16)
-
-            def run():
-                for L in layers:
-                    f([L[n] for n in l], xs[C], y)
-            run()
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                run()
-            g.replay()
-            torch.cuda.synchronize()
-            ts = []
-            for _ in range(5):
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(); g.replay(); e1.record()
-                torch.cuda.synchronize()
-                ts.append(e0.elapsed_time(e1))
-            per["|".join(l)] = sorted(ts)[2] * 1e3 / n_layers
-            tot += per["|".join(l)]
-        nbytes = sum(L.words.numel() * 4 + L.table.numel() * 2 + L.R * 2 for L in layers[0].values())
+        tot, per = layer_times(torch, dev, layers, shapes, B, linear_small if B <= 32 else linear_gemm, gen)
         res[f"B{B}"] = {"us_per_layer": tot, "GBps_packed": nbytes / tot / 1e3,
                         "tflops": 2.0 * B * sum(R * C for R, C in shapes.values()) / tot / 1e6, "per_launch_us": per}
-    return {"sweep": spec, "layers_rotated": n_layers, "rows": res}
+    return {"sweep": spec, "layers_rotated": n_layers, "rows": res, "resident": resident_bytes(layers[0])}
 
 
 def main():
@@ -278,6 +332,7 @@ def main():
                          "the rocprofv3 summaries under profiles/ are made with")
     ap.add_argument("--no-head", action="store_true", help="skip the 8-bit lm_head GEMV")
     ap.add_argument("--no-neighbours", action="store_true", help="skip the layer with its elementwise neighbours")
+    ap.add_argument("--no-configs", action="store_true", help="skip the cfg3 (small-batch crossover) and cfg5 (27B, column orders) objects")
     ap.add_argument("--head-only", action="store_true",
                     help="run only the 8-bit lm_head GEMV and print only its object (the command its rocprofv3 "
                          "summary under profiles/ is made with)")
@@ -301,11 +356,12 @@ def main():
         print(json.dumps({"lm_head": lm_head(torch, dev)}))
         return
     if args.sweep:
-        print(json.dumps(sweep(torch, dev, args.sweep, args.rows, min(args.layers, 8 if args.sweep.startswith("27b") else 16))))
+        print(json.dumps(sweep(torch, dev, args.sweep, args.rows, min(args.layers, 4 if args.sweep.startswith("27b") else 16))))
         return
-    gen = torch.Generator(device=dev).manual_seed(0)
-    layers = [make_layer(torch, dev, gen) for _ in range(args.layers)]
-    x = {C: torch.randn(1, C, device=dev, generator=gen).to(torch.bfloat16) for C in (3584, 18944)}
+    D, BITS = 8, 16
+    gen = torch.Generator().manual_seed(0)
+    layers = [make_layer(torch, dev, gen, SHAPES_7B, D, BITS) for _ in range(args.layers)]
+    x = {C: torch.randn(1, C, generator=gen).to(torch.bfloat16).to(dev) for C in (3584, 18944)}
     y = {l: torch.empty(1, sum(SHAPES_7B[n][0] for n in l), device=dev, dtype=torch.bfloat16) for l in LAUNCHES}
 
     def step(i):
@@ -314,18 +370,23 @@ def main():
             linear_small([L[n] for n in l], x[SHAPES_7B[l[0]][1]], y[l])
 
     gu = LAUNCHES[2]
+    gu_bytes = launch_bytes(SHAPES_7B, gu, D, BITS)
+
+    def gate_up_all():
+        for L in layers:
+            linear_small([L[n] for n in gu], x[3584], y[gu])
+
+    def roofline():
+        dur_us = timed_graph(torch, gate_up_all) * 1e3 / len(layers)
+        achieved = gu_bytes / (dur_us * 1e-6) / 1e9
+        return {"bound": "hbm", "kernel": "sq::stream_kernel (gate|up launch, 2 x 18944x3584)",
+                "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                "bytes_per_launch": gu_bytes, "us_per_launch": dur_us, "traffic": GATE_UP_TRAFFIC["bytes"],
+                "traffic_source": GATE_UP_TRAFFIC["source"],
+                "stream_bytes_per_launch": sum(layers[0][n].stream.numel() for n in gu)}
+
     if args.roofline_only:
-        def gate_up_only():
-            for L in layers:
-                linear_small([L[n] for n in gu], x[3584], y[gu])
-        ms, g2 = timed_graph(torch, gate_up_only)
-        del g2
-        dur_us = ms * 1e3 / len(layers)
-        out = {"roofline": {"bound": "hbm", "kernel": "sq::stream_kernel (gate|up launch, 2 x 18944x3584)",
-                            "achieved": algorithmic_bytes(gu) / (dur_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": algorithmic_bytes(gu) / (dur_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                            "bytes_per_launch": algorithmic_bytes(gu), "us_per_launch": dur_us, "traffic": GATE_UP_TRAFFIC_BYTES,
-                            "stream_bytes_per_launch": sum(layers[0][n].stream.numel() for n in gu)}}
+        out = {"roofline": roofline()}
         if args.copy_probe:
             out["copy_probe"] = copy_probe(torch, dev)
         print(json.dumps(out))
@@ -341,64 +402,65 @@ def main():
             step(i)
     g.replay()                                   # graph upload / first-launch costs stay outside the timed region
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    g.replay()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    layer_bytes = sum(algorithmic_bytes(l) for l in LAUNCHES)
+    replays = []
+    for _ in range(REPS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        g.replay()                               # exactly --steps layer steps
+        e1.record()
+        torch.cuda.synchronize()
+        replays.append(e0.elapsed_time(e1))
+    del g
+    ms_per_step = sorted(replays)[len(replays) // 2] / args.steps
+    layer_bytes = sum(launch_bytes(SHAPES_7B, l, D, BITS) for l in LAUNCHES)
     tag_bytes = sum(R * (C // D) * BITS // 8 for R, C in SHAPES_7B.values())
     value = layer_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # dominant kernel: the gate|up launch alone, over all layers, HIP events around graph replays
-
-    def gate_up_all():
-        for L in layers:
-            linear_small([L[n] for n in gu], x[3584], y[gu])
-    ms, g2 = timed_graph(torch, gate_up_all)
-    del g2
-    dur_us = ms * 1e3 / len(layers)
-    gu_bytes = algorithmic_bytes(gu)
-    achieved = gu_bytes / (dur_us * 1e-6) / 1e9
     per_launch = {}
     for l in LAUNCHES:
         def one(l=l):
             for L in layers:
                 linear_small([L[n] for n in l], x[SHAPES_7B[l[0]][1]], y[l])
-        ms_l, gl = timed_graph(torch, one, reps=3)
-        del gl
-        per_launch["|".join(l)] = {"us": ms_l * 1e3 / len(layers), "bytes": algorithmic_bytes(l)}
+        nb = launch_bytes(SHAPES_7B, l, D, BITS)
+        us = timed_graph(torch, one) * 1e3 / len(layers)
+        per_launch["|".join(l)] = {"us": us, "bytes": nb, "frac_hbm": nb / us / 1e3 / HBM_PEAK_GBS}
 
     out = {
         "metric": "codebook GEMV HBM GB/s + us/layer @7B bs=1; prefill GEMM TFLOP/s @M=2048",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16xf16->f32 (bf16 activations in/out)", "data": "synthetic (seed 0, generated on device)",
+        "dtype": "f16xf16->f32 (bf16 activations in/out)", "data": "synthetic (CPU generator, seed 0)",
         "config": {"workload": "cfg2: one Qwen2.5-7B-shaped layer, 7 block linears, bs=1, d=8, K=65536, uint16 tags "
                                "(2 bpw), fp16 row scales, bf16 x/y; 4 launches per layer (q|k|v, o, gate|up, down)",
-                   "layers_rotated": len(layers), "bytes_per_layer": layer_bytes, "tag_bytes_per_layer": tag_bytes},
+                   "layers_rotated": len(layers), "bytes_per_layer": layer_bytes, "tag_bytes_per_layer": tag_bytes,
+                   "timing": f"HIP events around one graph replay of --steps layer steps, median of {REPS} replays",
+                   "replay_ms": replays},
         "us_per_layer": ms_per_step * 1e3,
+        "frac_hbm": value / HBM_PEAK_GBS,
         "tag_only_GBps": tag_bytes / (ms_per_step * 1e-3) / 1e9,
         "per_launch": per_launch,
-        "roofline": {"bound": "hbm", "kernel": "sq::stream_kernel (gate|up launch, 2 x 18944x3584)",
-                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "bytes_per_launch": gu_bytes, "us_per_launch": dur_us, "traffic": GATE_UP_TRAFFIC_BYTES,
-                     "stream_bytes_per_launch": sum(layers[0][n].stream.numel() for n in gu)},
+        "resident": resident_bytes(layers[0]),
+        "roofline": roofline(),
     }
     if args.copy_probe:
         out["copy_probe"] = copy_probe(torch, dev)
     if not args.no_prefill:
-        pf = prefill(torch, dev, layers[0])
+        pf = prefill(torch, dev, layers[0], SHAPES_7B)
         out["prefill"] = {"M": 2048, "gate_18944x3584": pf["gate"], "down_3584x18944": pf["down"],
                           "peak_tflops": MFMA_PEAK_TFLOPS,
                           "frac_of_peak": min(pf["gate"]["tflops"], pf["down"]["tflops"]) / MFMA_PEAK_TFLOPS}
     if not args.no_neighbours:
         out["layer_with_neighbours"] = neighbours(torch, dev, layers, x, y)
+    cpu_layer = layers[0] if not args.no_cpu else None
+    del layers[1:]                               # the rotated layers are no longer used
+    if not args.no_configs:
+        out["cfg3_small_batch"] = small_batch_crossover(torch, dev, gen, 8)
+        out["cfg5_masked_27b"] = masked_27b(torch, dev, gen, 4)
     if not args.no_head:
-        del layers[1:]                           # the head needs 0.6 GB; the rotated layers are no longer used
         out["lm_head_q8"] = lm_head(torch, dev)
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(torch, layers[0], x)
+    if cpu_layer is not None:
+        out["cpu_baseline"] = cpu_baseline(torch, cpu_layer, x, D, BITS, SHAPES_7B)
     print(json.dumps(out))
 
 
