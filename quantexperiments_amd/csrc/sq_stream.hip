@@ -36,9 +36,7 @@
 #include <vector>
 #include "sq_stream.h"
 
-#ifndef SQ_STREAM_CLIMB
-#define SQ_STREAM_CLIMB 1                  // hill-climbing passes of the entry ordering (load time against LDS collisions)
-#endif
+constexpr int STREAM_CLIMB = 1;      // hill-climbing passes of the entry ordering (load time against LDS collisions)
 
 namespace sq {
 
@@ -279,7 +277,7 @@ struct BankMatch {
             return (h[p] == M && at == 1 && h[q] + 1 < M) ? M - 1 : M;
         };
         for (uint32_t n = 0; n < most; ++n) rescan(n);
-        for (int pass = 0; pass < SQ_STREAM_CLIMB; ++pass) {
+        for (int pass = 0; pass < STREAM_CLIMB; ++pass) {
             bool improved = false;
             for (uint32_t n = 0; n < most; ++n) {
                 const uint8_t* an = &ha[n * 16];
@@ -517,10 +515,7 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 }
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
-#ifndef SQ_STREAM_PF
-#define SQ_STREAM_PF 4
-#endif
-constexpr int STREAM_PF = SQ_STREAM_PF;   // steps fetched ahead
+constexpr int STREAM_PF = 3;          // steps fetched ahead (2 to 4 measure alike, 6 and 8 slower: the loop runs at the memory system's rate)
 constexpr int STREAM_NW = 16;         // waves per workgroup: one workgroup per CU
 
 // LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group)
@@ -640,6 +635,17 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         kcur = wave < ng * split ? wave / split : ng;
         knext = ng;
     }
+    // The codebook slice is copied global -> LDS without passing through registers (a wave instruction moves 1 KB, lane l
+    // to the wave's base + 16 l).  It goes out first: loads are accounted for in the order they were issued, and the
+    // small scattered reads of the group heads below come back later than this bulk copy does.
+    {
+        const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table) + (size_t)s * STREAM_TAB;
+#pragma unroll
+        for (int k = 0; k < STREAM_TAB / (NTH * 16); ++k)
+            __builtin_amdgcn_global_load_lds((stream_gptr_t)(src + ((size_t)k * NTH + tid) * 16),
+                                             (stream_lptr_t)(lds + (k * NTH + wave * 64) * 16), 16, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     // the first head's words are requested here and used only after the staging loads have gone out
     const int kc0 = min(kcur, ng - 1);
     const uint32_t head_a = goff[kc0], head_b = goff[kc0 + 1], head_s = slots[(size_t)kc0 * 64 + lane];
@@ -649,15 +655,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
     for (int q = 0; q < STREAM_PF; ++q) nx[q] = u32x3{0u, 0u, 0u};
 
-    // Stage the codebook slice (copied global -> LDS without passing through registers: a wave instruction moves
-    // 1 KB, lane l to the wave's base + 16 l) and this part of the NB activation rows (as fp16); the first group's
-    // steps are requested before anything waits for the staging loads.
+    // Stage this part of the NB activation rows (as fp16); the first group's steps are requested before anything waits
+    // for the staging loads.
     {
-        const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table) + (size_t)s * STREAM_TAB;
-#pragma unroll
-        for (int k = 0; k < STREAM_TAB / (NTH * 16); ++k)
-            __builtin_amdgcn_global_load_lds((stream_gptr_t)(src + ((size_t)k * NTH + tid) * 16),
-                                             (stream_lptr_t)(lds + (k * NTH + wave * 64) * 16), 16, 0, 0);
         u32x4 xq[NB][NX];
         const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
         if (PRO != 0) {
@@ -831,18 +831,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
                         const uint32_t ta = (e[j0 + jj] & 0xFFFu) << 4, xa = ((e[j0 + jj] >> 12) & 0xFFFu) << 4;
-#if defined(SQ_EXP_NO_CW)                                       /* timing experiments only (wrong results) */
-                        cw[jj] = u32x4{ta, xa, ta, xa};
-#else
                         cw[jj] = *reinterpret_cast<const u32x4*>(lds + ta);
-#endif
 #pragma unroll
-                        for (int b = 0; b < NB; ++b)
-#if defined(SQ_EXP_NO_X)
-                            xv[jj][b] = u32x4{xa, ta, xa, ta};
-#else
-                            xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * xs + xa);
-#endif
+                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * xs + xa);
                     }
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
