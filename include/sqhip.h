@@ -33,7 +33,8 @@ enum { SQ_F32 = 0, SQ_F16 = 1, SQ_BF16 = 2 };
 /* One packed matrix resident in device memory (the tensors the reference keeps in
  * kernels/gemv.py:107-131 PackedLinear, same meaning, file layout unchanged). */
 typedef struct sq_matrix {
-    const int32_t*  tags;       /* [R, W] */
+    const int32_t*  tags;       /* [R, W]; may be NULL for a matrix that keeps only its slice stream (below): every entry
+                                 * point then works from the stream (one resident copy, the reference's `compact`) */
     const uint16_t* table;      /* fp16 bits [G*K, d] */
     const uint16_t* row_scale;  /* fp16 bits [R] */
     const uint8_t*  row_book;   /* [R] or NULL when G == 1 */
@@ -43,7 +44,7 @@ typedef struct sq_matrix {
     int32_t R, C, d, bits, G, M, W;
     int32_t y_off;              /* first output column of this piece in the stacked Y */
     const void*     stream;     /* optional: device copy of the buffer sq_stream_build wrote for `tags`; NULL = none */
-    int32_t stream_runs;        /* runs_out of sq_stream_build for that buffer */
+    int32_t stream_runs;        /* runs_out of sq_stream_build for that buffer (opaque: run count and longest run, packed) */
     int32_t stream_groups;      /* groups_out of sq_stream_build for that buffer */
 } sq_matrix;
 
@@ -128,13 +129,16 @@ size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, i
  * HOST pointers: `tags_host` is the file's tag tensor in host memory, `row_mask_host` the file's row_mask
  * (NULL when the matrix has one column order), `out_host` receives sq_stream_bytes() bytes that the caller
  * copies to the device (16-byte aligned) and names in sq_matrix.stream, together with *runs_out and
- * *groups_out in sq_matrix.stream_runs / stream_groups.  sq_stream_bytes returns 0 for formats the stream does
- * not cover.  `runs` asks for that many row runs; each run becomes 2^(bits - 12) * ceil(C / 5120) workgroups
- * of the batch-1 launch, so pick it to give the pieces launched together about two workgroups per CU in
- * total (0 = a good value for a matrix launched alone); rows with different column orders never share a run,
- * so *runs_out can exceed the request.  A matrix with column orders must be given to sq_linear_small with
- * the same row_mask and with perms on the device.  The tags tensor stays the source of truth (sq_dequant,
- * B > 1 and the prefill GEMM read it); this plays the part of the reference's load-time layouts (reference
+ * *groups_out in sq_matrix.stream_runs / stream_groups (both opaque to the caller).  sq_stream_bytes returns 0 for
+ * formats the stream does not cover.  `runs` asks for that many row runs; each run becomes
+ * 2^(bits - 12) * ceil(C / 8 / 4064) workgroups of 1024 threads in the batch-1 launch, one per compute unit, so
+ * pick it to give the pieces launched together about one workgroup per CU in total (0 = a good value for a matrix
+ * launched alone on 256 CUs); rows with different column orders never share a run and no run is longer than 6144
+ * rows, so the run count can exceed the request.  A matrix with column orders must be given to sq_linear_small with
+ * the same row_mask and with perms on the device.  Once the stream is on the device the tags are optional: with
+ * sq_matrix.tags == NULL sq_dequant, every row count of sq_linear_small and sq_linear_gemm work from the stream
+ * alone (decode-time speed is kept, the other paths get slower; x must then be 16-byte aligned with ldx % 8 == 0).
+ * This plays the part of the reference's load-time layouts (reference
  * shapequant/kernels/proto_runs.py:295-349 pack_lane_major / RunsLinear, batched_runs.py:213-373 tile_words),
  * with a layout chosen for LDS gathers.
  *
@@ -143,7 +147,8 @@ size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, i
  * each 16-row tile stored unit by unit, as large as the tags rounded up to 16 rows) that lets the decode-time
  * kernel read with fully coalesced loads; `runs` is ignored, *runs_out = *groups_out = 0, and the caller passes
  * the device copy in sq_matrix.stream with stream_runs = stream_groups = 0.  It is optional like the slice
- * stream (the reference keeps such a copy too: shapequant/kernels/batched_runs.py tile_words). */
+ * stream (the reference keeps such a copy too: shapequant/kernels/batched_runs.py tile_words); these formats
+ * always need their tags. */
 size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
                        const uint8_t* row_mask_host, int32_t runs);
 int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,

@@ -35,7 +35,8 @@ int device_cus() {
 }
 
 static int check_matrix(const sq_matrix& m, const char* who) {
-    if (!m.tags || !m.table || !m.row_scale) return fail(SQ_EINVAL, "%s: null tags/table/row_scale", who);
+    if (!m.table || !m.row_scale) return fail(SQ_EINVAL, "%s: null table/row_scale", who);
+    if (!m.tags && !stream_shape(m)) return fail(SQ_EINVAL, "%s: null tags (only a matrix with a slice stream may drop them)", who);
     if (m.R < 0 || m.C <= 0 || m.d <= 0 || m.C % m.d) return fail(SQ_EINVAL, "%s: R %d C %d d %d", who, m.R, m.C, m.d);
     if (m.bits < 1 || m.bits > 16) return fail(SQ_EINVAL, "%s: tag bits %d outside 1..16", who, m.bits);
     if (m.G < 1 || m.G > 256 || (m.G > 1 && !m.row_book)) return fail(SQ_EINVAL, "%s: G %d needs row_book", who, m.G);

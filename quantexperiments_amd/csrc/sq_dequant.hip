@@ -2,7 +2,7 @@
 //   out[r, perm[mask[r]][j*d + k]] = rn_T( f32(table[book[r]*K + tag[r, j]][k]) * f32(row_scale[r]) )
 // The fp32 product of two fp16 values is exact, so T = fp32 reproduces the CPU decode bit
 // for bit and T = fp16 / bf16 differ from it by exactly one round-to-nearest-even.
-#include "sq_common.h"
+#include "sq_stream.h"
 
 namespace sq {
 
@@ -229,7 +229,7 @@ static int launch_dt(const sq_matrix& m, void* out, int64_t ld_out, int r0, int 
 int launch_dequant_with_cvt(const sq_matrix& m, void* out, int64_t ld_out, const uint16_t* x, int64_t ldx, int T, int C,
                             uint16_t* xout, hipStream_t s) {
     const int64_t n = (int64_t)m.R * (m.C / (m.d ? m.d : 1)), ne = (int64_t)T * C;
-    if (!dequant8x4_ok(m, n) || ((uintptr_t)out & 15) || ld_out % 8 || ne <= 0 || ne >= ((int64_t)1 << 40)) return 1;
+    if (!m.tags || !dequant8x4_ok(m, n) || ((uintptr_t)out & 15) || ld_out % 8 || ne <= 0 || ne >= ((int64_t)1 << 40)) return 1;
     const int64_t nd = (n + 1023) / 1024, nc = (ne / 8 + 255) / 256;
     if (nd + nc >= ((int64_t)1 << 31)) return 1;
     hipLaunchKernelGGL(dequant8x4_cvt_kernel, dim3((unsigned)(nd + nc)), dim3(256), 0, s, m, (uint16_t*)out, ld_out, x, ldx, T, C, xout,
@@ -238,6 +238,7 @@ int launch_dequant_with_cvt(const sq_matrix& m, void* out, int64_t ld_out, const
 }
 
 int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s, bool raw) {
+    if (!m.tags) return launch_stream_dequant(m, out, out_dtype, ld_out, r0, r1, s, raw);    // one-copy residency
     switch (out_dtype) {
         case SQ_F32: return launch_dt<SQ_F32>(m, out, ld_out, r0, r1, s, raw ? 1 : 0);
         case SQ_F16: return launch_dt<SQ_F16>(m, out, ld_out, r0, r1, s, raw ? 1 : 0);

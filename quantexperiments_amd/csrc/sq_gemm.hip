@@ -161,7 +161,7 @@ static bool x_vec_ok(const void* x, int64_t ldx, int C) { return C % 8 == 0 && l
 // used from the first row count sq_linear_small does not take.
 constexpr int GEMM256_MIN_T = SQ_SMALL_BMAX + 1;
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
-static bool fused_ok(const sq_matrix& m) { return (m.d == 8 || m.d == 4) && !m.perms && ((uintptr_t)m.table & 15) == 0; }
+static bool fused_ok(const sq_matrix& m) { return m.tags && (m.d == 8 || m.d == 4) && !m.perms && ((uintptr_t)m.table & 15) == 0; }
 static size_t dense_bytes(const sq_matrix& m) { return (((size_t)m.R * m.C * 2) + 255) & ~(size_t)255; }
 
 // The decode + 256 x 256 tile route: from GEMM256_MIN_T rows, and for stacks with column orders at any row count
@@ -301,6 +301,8 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
         return SQ_OK;
     }
     if (!x_vec_ok(x, ldx, mats[0].C)) {
+        for (int i = 0; i < n; ++i)
+            if (!mats[i].tags) return fail(SQ_EUNSUPPORTED, "sq_linear_gemm: a matrix held as its tag stream only needs 16-byte aligned x with ldx %% 8 == 0");
         // odd strides: the any-shape kernel, SQ_SMALL_BMAX activation rows at a time
         for (int t = 0; t < T; t += SQ_SMALL_BMAX) {
             const int nb = T - t < SQ_SMALL_BMAX ? T - t : SQ_SMALL_BMAX;

@@ -46,6 +46,7 @@ int launch_small_generic(const sq_matrix* mats, int n, const void* x, int x_dtyp
 static int unit_dwords(int bits) { return bits == 12 ? 3 : bits == 10 ? 5 : 4; }
 
 static bool fast_shape(const sq_matrix& m) {
+    if (!m.tags) return false;                                   // held as its tag stream only
     const bool fmt = (m.d == 8 && m.bits == 16) || (m.d == 4 && (m.bits == 12 || m.bits == 10 || m.bits == 8));
     if (!fmt) return false;
     if (m.W % unit_dwords(m.bits)) return false;                 // rows must be whole units
@@ -120,6 +121,7 @@ static Plan plan_for(int U, int bits, int d) {
 // against 14 us).
 static bool stream_rows(const sq_matrix& m, int B) {
     if (!stream_shape(m)) return false;
+    if (!m.tags) return true;                                    // one-copy residency: the stream is all there is
     return B == 1 || m.perms != nullptr || (B <= 4 && (int64_t)m.R * m.C >= (int64_t)32 << 20);
 }
 
@@ -294,6 +296,8 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
             continue;
         }
         const Plan pl = (fast_shape(m0) && x_ok) ? plan_for(m0.W / ud, m0.bits, m0.d) : Plan{0, 0, 0};
+        if (pl.TS == 0 && !m0.tags)
+            return fail(SQ_EUNSUPPORTED, "sq_linear_small: a matrix held as its tag stream only needs 16-byte aligned x with ldx %% 8 == 0");
         if (pl.TS == 0) {
             int rc = launch_small_generic(mats + i, 1, x, x_dtype, ldx, y, y_dtype, ldy, B, s);
             if (rc) return rc;

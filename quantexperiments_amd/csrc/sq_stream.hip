@@ -1007,6 +1007,97 @@ static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
     return check_launch("sq_linear_small(stream)");
 }
 
+// ---- dense rows from the tag stream alone (a matrix held in one copy: sq_matrix.tags == NULL).  One wave per (bucket,
+// group): lane = row, as in the product; every real entry writes its chunk of 8 weights, so over all buckets each
+// (row, chunk) is written exactly once.  Same arithmetic as dequant_kernel: f32(codeword) * f32(row scale), one rounding.
+struct StreamDeqArgs {
+    const unsigned char* stream;
+    const uint16_t* table;
+    const uint16_t* row_scale;
+    const uint8_t* row_mask;
+    const int32_t* perms;
+    void* out;
+    int64_t ld_out;
+    int R, C, NS, NV, PC, NG, r0, r1, raw, vec;
+    uint32_t off_slots, off_rows, off_steps;
+};
+
+template <int DT>
+__global__ __launch_bounds__(256) void stream_dequant_kernel(StreamDeqArgs a) {
+    typedef typename store_as<DT>::type T;
+    const int lane = threadIdx.x & 63;
+    const int w = (int)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (w >= a.NV * a.NG) return;
+    const int v = w / a.NG, g = w - v * a.NG, s = v % a.NS, kp = v / a.NS;
+    const uint32_t slot = reinterpret_cast<const uint32_t*>(a.stream + a.off_slots)[(size_t)w * 64 + lane];
+    const uint32_t place = slot & STREAM_NO_ROW;
+    const int cnt = (int)(slot >> STREAM_ROW_BITS);
+    uint32_t row = STREAM_NO_ROW;
+    if (place != STREAM_NO_ROW) row = a.perms ? reinterpret_cast<const uint32_t*>(a.stream + a.off_rows)[place] : place;
+    const bool mine = row != STREAM_NO_ROW && (int)row >= a.r0 && (int)row < a.r1 && cnt > 0;
+    if (__ballot(mine) == 0) return;                             // (wave-uniform) none of this group's rows is wanted
+    const uint32_t* goff = reinterpret_cast<const uint32_t*>(a.stream) + w;
+    const uint32_t st0 = goff[0];
+    const int nst = (int)(goff[1] - st0);
+    const float sc = (mine && !a.raw) ? h2f(a.row_scale[row]) : 1.f;
+    const int32_t* pm = (mine && a.perms) ? a.perms + (size_t)(a.row_mask ? a.row_mask[row] : 0) * a.C : nullptr;
+    T* orow = reinterpret_cast<T*>(a.out) + (mine ? (int64_t)((int)row - a.r0) * a.ld_out : 0);
+    const unsigned char* rec = a.stream + a.off_steps + (size_t)st0 * 768 + lane * 12;
+    for (int t = 0; t < nst; ++t) {
+        const u32x3 r = *reinterpret_cast<const u32x3*>(rec + (size_t)t * 768);
+        const uint32_t e[4] = {r.x, (r.x >> 24) | (r.y << 8), (r.y >> 16) | (r.z << 16), r.z >> 8};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (!mine || 4 * t + j >= cnt) continue;
+            const uint32_t tag = (e[j] & 0xFFFu) + ((uint32_t)s << STREAM_SLICE_BITS);
+            const int c0 = ((int)((e[j] >> STREAM_SLICE_BITS) & 0xFFFu) + kp * a.PC) * 8;
+            const u32x4 cw = *reinterpret_cast<const u32x4*>(a.table + (size_t)tag * 8);
+            T o[8];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t pair = cw[k];
+                o[2 * k] = store_as<DT>::cvt(h2f((uint16_t)(pair & 0xFFFFu)) * sc);
+                o[2 * k + 1] = store_as<DT>::cvt(h2f((uint16_t)(pair >> 16)) * sc);
+            }
+            if (pm) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) orow[pm[c0 + k]] = o[k];
+            } else if (a.vec) {
+                constexpr int PER = 16 / (int)sizeof(T);         // elements per 16-byte store
+#pragma unroll
+                for (int q = 0; q < 8 / PER; ++q) {
+                    u32x4 pk;
+                    __builtin_memcpy(&pk, o + q * PER, 16);
+                    *reinterpret_cast<u32x4*>(orow + c0 + q * PER) = pk;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) orow[c0 + k] = o[k];
+            }
+        }
+    }
+}
+
+int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s, bool raw) {
+    if (!stream_shape(m)) return fail(SQ_EINVAL, "sq_dequant: a matrix without tags needs its tag stream");
+    const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m));
+    StreamDeqArgs a;
+    a.stream = (const unsigned char*)m.stream; a.table = m.table; a.row_scale = m.row_scale; a.row_mask = m.row_mask; a.perms = m.perms;
+    a.out = out; a.ld_out = ld_out; a.R = m.R; a.C = m.C; a.NS = g.NS; a.NV = g.NV; a.PC = g.PC; a.NG = g.NG; a.r0 = r0; a.r1 = r1;
+    a.raw = raw ? 1 : 0;
+    a.off_slots = (uint32_t)g.off_slots; a.off_rows = (uint32_t)g.off_rows; a.off_steps = (uint32_t)g.off_steps;
+    const size_t es = out_dtype == SQ_F32 ? 4 : 2;
+    a.vec = ((uintptr_t)out & 15) == 0 && (ld_out * es) % 16 == 0;
+    const unsigned grid = (unsigned)(((int64_t)g.NV * g.NG + 3) / 4);
+    switch (out_dtype) {
+        case SQ_F32: hipLaunchKernelGGL((stream_dequant_kernel<SQ_F32>), dim3(grid), dim3(256), 0, s, a); break;
+        case SQ_F16: hipLaunchKernelGGL((stream_dequant_kernel<SQ_F16>), dim3(grid), dim3(256), 0, s, a); break;
+        case SQ_BF16: hipLaunchKernelGGL((stream_dequant_kernel<SQ_BF16>), dim3(grid), dim3(256), 0, s, a); break;
+        default: return fail(SQ_EINVAL, "sq_dequant: out_dtype %d", out_dtype);
+    }
+    return check_launch("sq_dequant(stream)");
+}
+
 bool stream_shape(const sq_matrix& m) {
     return m.stream && stream_runs_of(m) > 0 && m.stream_groups > 0 && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
            (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0;

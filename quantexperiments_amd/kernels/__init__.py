@@ -100,6 +100,8 @@ class PackedLinear(torch.nn.Module):
     def build_stream(self, runs: int = 0) -> None:
         """(Re)build the bucketed tag stream cut into about `runs` row runs (0 = suited to a launch of this
         matrix alone; prepare_stack picks the runs of pieces that are launched together)."""
+        if self.words is None:
+            raise RuntimeError("the packed tags of this matrix were dropped (compact): its stream cannot be rebuilt")
         self.stream, self.stream_runs, self.stream_groups = build_stream(
             self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs)
         self.stream_asked = runs
@@ -119,7 +121,7 @@ class PackedLinear(torch.nn.Module):
 
     @property
     def device(self):
-        return self.words.device
+        return self.table.device
 
     def descriptor(self, y_off: int = 0) -> SqMatrix:
         p = lambda t: None if t is None else t.data_ptr()
@@ -167,8 +169,22 @@ class PackedLinear(torch.nn.Module):
         return y if self.bias is None else y + self.bias
 
     def stored_bytes(self) -> int:
-        """Bytes the product must stream from HBM: tags + table + scales (as the reference counts)."""
-        return sum(t.numel() * t.element_size() for t in (self.words, self.table, self.row_scale))
+        """Bytes the product must stream from HBM: tags + table + scales (as the reference counts); the tag stream
+        in place of the tags once they have been dropped."""
+        tags = self.words if self.words is not None else self.stream
+        return sum(t.numel() * t.element_size() for t in (tags, self.table, self.row_scale))
+
+    def make_compact(self) -> None:
+        """Keep one copy of the tags (the reference's `compact`, shapequant/vllm_ext/core.py:215-253): a matrix with
+        a slice stream drops the packed tags and serves every row count, decode and prefill from the stream (the
+        decode-time speed stays; more than a few rows and dense decoding get slower); a matrix whose stream is the
+        tile-major copy of its tags drops that copy instead.  The stream can no longer be re-cut afterwards."""
+        if self.stream is None:
+            return
+        if self.stream_tiled:
+            self.stream, self.stream_tiled = None, False
+        else:
+            self.words = None
 
 
 def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, runs: int = 0):
@@ -208,7 +224,7 @@ def prepare_stack(pieces, workgroups: int | None = None) -> None:
     for p in ps:
         buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // STREAM_PART_MAX)
         runs = max(1, round(workgroups * p.R / rows / buckets))
-        if p.stream is None or (runs != p.stream_asked and not (len(ps) == 1 and p.stream_asked == 0)):
+        if p.words is not None and (p.stream is None or (runs != p.stream_asked and not (len(ps) == 1 and p.stream_asked == 0))):
             p.build_stream(runs)
 
 

@@ -72,43 +72,37 @@ def neutral_defaults():
 
 
 _TUNED: dict = {}
-_TIME_STREAM: dict = {}
 
 
-def _time(fn, reps: int, n: int = 10) -> float:
-    """GPU ms per call: HIP-graph replay of n calls, median of reps
-    (reference shapequant/vllm_ext/core.py:168-195)."""
-    dev = torch.cuda.current_device()
-    s = _TIME_STREAM.setdefault(dev, torch.cuda.Stream())
-    s.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(s):
-        fn()
-        fn()
-    torch.cuda.current_stream().wait_stream(s)
+def _graph_ms(fn, calls: int = 10, reps: int = 5) -> float:
+    """Milliseconds per fn() on the GPU: `calls` of them recorded into one HIP graph, the graph replayed `reps`
+    times between events, median replay (the measure behind PackedShards.tune; the reference times the same way,
+    shapequant/vllm_ext/core.py:168-195)."""
+    import statistics
+    fn()                                                # buffers grow here, never under capture
     torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        for _ in range(n):
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(calls):
             fn()
-    ts = []
-    for _ in range(reps):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        g.replay()
-        b.record()
-        torch.cuda.synchronize()
-        ts.append(a.elapsed_time(b) / n)
-    del g
-    return sorted(ts)[len(ts) // 2]
+    graph.replay()
+    torch.cuda.synchronize()
+    marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for begin, end in marks:
+        begin.record()
+        graph.replay()
+        end.record()
+    torch.cuda.synchronize()
+    return statistics.median(b.elapsed_time(e) for b, e in marks) / calls
 
 
 class PackedShards:
     def __init__(self, rls: list, *, bmax: int = BMAX, layout: str = "file", warps: int = 8, bps: int = 2,
                  xs: bool = False, max_split: int = 8, large: str = "fused", chunk_bytes: int = 24 << 20,
                  dequant_from: int = 1 << 30, compact: bool = False):
-        # layout / warps / bps / xs / max_split / compact tune the reference's CUDA launchers; the HIP
-        # library plans its own launches and reads the file layout in place (one copy of the tags, which
-        # is what `compact` asks for), so they are accepted and ignored.
+        # layout / warps / bps / xs / max_split tune the reference's CUDA launchers; the HIP library plans its
+        # own launches, so they are accepted and ignored.  compact: one copy of every matrix' tags instead of two
+        # (packed tags + the load-time layout the decode kernels read), see PackedLinear.make_compact.
         if large not in ("dequant", "chunked", "fused"):
             raise ValueError(f"large={large!r}: dequant | chunked | fused")
         if not rls:
@@ -135,8 +129,10 @@ class PackedShards:
         self.cross = bmax            # M <= cross: small path, else the large-M path (tune() moves it)
         self.device = rls[0].device
         self.sq_name = ""            # set by the vLLM plugin (layer prefix)
-        if len(rls) > 1:
-            prepare_stack(self.rls)  # tag streams cut for a joint launch of these pieces
+        prepare_stack(self.rls)      # tag streams cut for a joint launch of these pieces (built here if they were not)
+        if compact:
+            for rl in self.rls:
+                rl.make_compact()
 
     @classmethod
     def from_packed(cls, pf, names: list, dev="cuda", **kw) -> "PackedShards":
@@ -162,30 +158,28 @@ class PackedShards:
         return torch.cat([rl.dense(torch.float16) for rl in self.rls])
 
     def tune_launch(self, reps: int = 3) -> list:
-        """Launch geometry is planned inside the library per shape; nothing to search here."""
-        return []
+        """The reference searches warps x blocks x split-K per shape here (shapequant/vllm_ext/core.py:259-296).
+        The library plans its launches from the shape and the device's compute units; the one choice left to the
+        caller, how many runs the pieces' tag streams are cut into, is made in prepare_stack from the same CU count.
+        Returns the run counts in use."""
+        return [rl.stream_runs & 0xFFFF for rl in self.rls]
 
     @torch.no_grad()
     def tune(self, Ms=(8, 16, 24, 32), reps: int = 5) -> int:
-        """Measure the small path against the large-M path at each M <= bmax and set cross = the
-        largest M before the large path first wins; cached per shape
+        """Where the large-M route starts to win: both routes are timed at each M <= bmax, `cross` becomes the last
+        M before the large route is the faster one, and the answer is remembered per shape
         (reference shapequant/vllm_ext/core.py:308-328)."""
-        k = self.key()
-        if k in _TUNED:
-            self.cross = _TUNED[k]
-            return self.cross
-        cross = 0
-        for M in Ms:
-            if M > self.bmax:
-                break
-            x = torch.randn(M, self.C, device=self.device, dtype=torch.bfloat16)
-            t_small = _time(lambda: self._small(x, M), reps)
-            t_large = _time(lambda: self._large(x), reps)
-            if t_large < t_small:
-                break
-            cross = M
-        self.cross = _TUNED[k] = cross
-        return cross
+        shape = self.key()
+        if shape not in _TUNED:
+            last_small = 0
+            for M in (m for m in Ms if m <= self.bmax):
+                x = torch.randn(M, self.C, device=self.device, dtype=torch.bfloat16)
+                if _graph_ms(lambda: self._large(x), reps=reps) < _graph_ms(lambda: self._small(x, M), reps=reps):
+                    break
+                last_small = M
+            _TUNED[shape] = last_small
+        self.cross = _TUNED[shape]
+        return self.cross
 
     # ------------------------------------------------------------------ forward
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -341,9 +335,11 @@ def register(ps) -> int:
 
 
 def pool_tile_words() -> int:
-    """The reference pools its per-matrix tile-word copies here (reference
-    shapequant/vllm_ext/core.py:630-670).  The HIP kernels read the file layout in place and keep
-    no second copy, so there is nothing to pool: returns 0 bytes."""
+    """The reference moves its per-matrix tile-word copies into one pooled buffer here (reference
+    shapequant/vllm_ext/core.py:630-670) to defragment after loading.  This library's load-time layouts (the slice
+    stream, the tile-major copy of d = 4 tags) are ordinary torch tensors allocated once at their final size, so
+    there is nothing to move: returns 0 bytes.  What they cost is reported by PackedShards.nbytes(); compact = True
+    keeps one copy per matrix."""
     return 0
 
 

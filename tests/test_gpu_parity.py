@@ -516,6 +516,68 @@ def test_custom_op_compiles_and_graph_captures(large):
             assert torch.equal(y, f(x))
 
 
+# ------------------------------------------------------------------ one copy of the tags (the reference's `compact`)
+@pytest.mark.parametrize("case", [(300, 1024, 16, 1), (257, 3584, 16, 1), (140, 5120, 16, 16), (700, 1024, 14, 3), (65, 18944, 16, 1)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_one_copy_residency_serves_everything_from_the_stream(case):
+    """A matrix that has dropped its packed tags and kept only the slice stream (reference
+    shapequant/vllm_ext/core.py:215-253: one resident copy): decoded weights stay bit-exact (every dtype, row
+    ranges), batch 1 gives the same bits as the two-copy matrix, and more rows and prefill stay within tolerance."""
+    from quantexperiments_amd.kernels import linear_gemm, linear_small
+    R, C, bits, M = case
+    s = synth(R, C, 8, bits, 1, M, seed=sum(case))
+    full, one = to_device(s), to_device(s)
+    one.make_compact()
+    assert one.words is None and one.stream is not None and one.descriptor().tags is None
+    with pytest.raises(RuntimeError, match="dropped"):
+        one.build_stream(2)
+    ref = s.decode()
+    assert torch.equal(one.dense(torch.float32).cpu(), torch.from_numpy(ref))
+    assert np.array_equal(one.dense(torch.float16).float().cpu().numpy(), O.round_fp16(ref))
+    assert np.array_equal(one.dense(torch.bfloat16).float().cpu().numpy(), O.round_bf16(ref))
+    r0, r1 = R // 3, min(R, R // 3 + 70)
+    assert torch.equal(one.dense(torch.float32, rows=(r0, r1)).cpu(), torch.from_numpy(ref[r0:r1]))
+    x = rand_x(1, C, torch.bfloat16, seed=1)
+    ya, yb = torch.empty(1, R, dtype=torch.float32, device="cuda"), torch.empty(1, R, dtype=torch.float32, device="cuda")
+    linear_small([full], x.cuda(), ya)
+    linear_small([one], x.cuda(), yb)
+    assert torch.equal(ya, yb) and rel_max_err(yb.cpu().numpy(), _ref(s, x)) < TOL
+    for B in (3, 9, 32):
+        xb = rand_x(B, C, torch.bfloat16, seed=B)
+        y = torch.empty(B, R, dtype=torch.float32, device="cuda")
+        linear_small([one], xb.cuda(), y)
+        assert rel_max_err(y.cpu().numpy(), _ref(s, xb)) < TOL, B
+    for T in (40, 300):
+        xt = rand_x(T, C, torch.bfloat16, seed=T)
+        y = torch.empty(T, R, dtype=torch.float32, device="cuda")
+        linear_gemm([one], xt.cuda(), y)
+        assert rel_max_err(y.cpu().numpy(), _ref(s, xt)) < TOL, T
+
+
+def test_packed_shards_compact_keeps_one_copy():
+    from quantexperiments_amd.vllm_ext.core import PackedShards
+    ss = [synth(260, 1024, 8, 16, seed=1), synth(70, 1024, 8, 16, seed=2)]
+    two = PackedShards([to_device(s) for s in ss])
+    one = PackedShards([to_device(s) for s in ss], compact=True)
+    tags = sum(s.words.nbytes for s in ss)
+    assert one.nbytes() == two.nbytes() - tags and all(rl.words is None for rl in one.rls)
+    for M in (1, 5, 33, 300):
+        x = rand_x(M, 1024, torch.bfloat16, seed=M).cuda()
+        a, b = two.forward(x), one.forward(x)
+        assert a.shape == b.shape == (M, 330) and b.dtype == torch.bfloat16
+        ref = np.concatenate([_ref(s, x.cpu()) for s in ss], axis=1)
+        _check_lowp(b, ref, slack=TOL)
+        if M == 1:
+            assert torch.equal(a, b)
+    assert torch.equal(one.dense(), two.dense())
+    # a format whose load-time layout is the tile-major copy of its tags (d = 4): compact drops that copy
+    s4 = synth(200, 3584, 4, 12, seed=3)
+    p4 = PackedShards([to_device(s4)], compact=True)
+    assert p4.rls[0].stream is None and p4.rls[0].words is not None
+    x = rand_x(2, 3584, torch.bfloat16, seed=7).cuda()
+    _check_lowp(p4.forward(x), _ref(s4, x.cpu()), slack=TOL)
+
+
 # ------------------------------------------------------------------ full-size matrices
 @pytest.mark.parametrize("shape", [(18944, 3584, 8, 16, 1), (3584, 18944, 8, 16, 1), (5120, 5120, 8, 16, 16), (3584, 3584, 4, 12, 1)],
                          ids=lambda c: "x".join(map(str, c)))
