@@ -54,11 +54,10 @@ constexpr int MMA_TT = 4;     // 16-row tiles multiplied between two workgroup b
 #define SQ_TRACE_POINT(k)
 #endif
 
-// two packed bf16 -> two packed fp16 (round toward zero: exact for every fp16-normal value)
-__device__ __forceinline__ uint32_t bf2h_pk(uint32_t v) {
-    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(__builtin_bit_cast(float, v << 16),
-                                                                  __builtin_bit_cast(float, v & 0xFFFF0000u)));
-}
+// two packed bf16 -> two packed fp16: round to nearest even like every other kernel of the library (exact for every
+// fp16-normal value, +-inf beyond 65,504; a round-toward-zero conversion would clamp to 65,504 instead and make this
+// kernel differ from the batch-1 one on the same input)
+__device__ __forceinline__ uint32_t bf2h_pk(uint32_t v) { return bf2h_x2(v); }
 
 template <int BITS, int D, int RW, int NT, bool LDS_TAB>
 __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {

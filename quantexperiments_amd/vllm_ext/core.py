@@ -343,9 +343,49 @@ def pool_tile_words() -> int:
     return 0
 
 
+class _Trace:
+    """SHAPEQUANT_DEBUG=1: a line on stdout whenever a layer's output is not finite or its input leaves the fp16
+    range (the kernels multiply activations as fp16: a bf16 value beyond 65,504 becomes inf there), plus one summary
+    line per layer at its first call with more than one row.  Eager calls only: it reads values back, which a stream
+    under capture cannot do.  At most LIMIT alarm lines per process (the reference's trace,
+    shapequant/vllm_ext/core.py:673-690)."""
+    FP16_MAX = 65504.0
+    LIMIT = 64
+
+    def __init__(self):
+        import os
+        self.enabled = os.environ.get("SHAPEQUANT_DEBUG") == "1"
+        self.alarms = 0
+        self.summarised: set = set()
+
+    def __call__(self, op: str, handle: int, x: torch.Tensor, y: torch.Tensor) -> None:
+        if not self.enabled or x.numel() == 0 or y.numel() == 0 or torch.cuda.is_current_stream_capturing():
+            return
+        rows = x.reshape(-1, x.shape[-1]).shape[0]
+        x_top = float(x.float().abs().max()) if x.is_floating_point() else 0.0
+        y_ok = bool(torch.isfinite(y).all())
+        if rows > 1 and handle not in self.summarised:
+            self.summarised.add(handle)
+            rms = lambda t: float(t.float().square().mean().sqrt())
+            print(f"[sqhip trace] {op} layer {handle} ({getattr(_REGISTRY[handle], 'sq_name', '') or type(_REGISTRY[handle]).__name__}): "
+                  f"{rows} rows, |x| max {x_top:.4g} rms {rms(x) if x.is_floating_point() else 0.0:.4g}, y rms {rms(y):.4g}, finite {y_ok}",
+                  flush=True)
+        bad_x = not (x_top <= self.FP16_MAX)             # also true for NaN
+        if (bad_x or not y_ok) and self.alarms < self.LIMIT:
+            self.alarms += 1
+            why = "input beyond the fp16 range" if bad_x else "output not finite"
+            print(f"[sqhip alarm] {op} layer {handle}: {why}; x {tuple(x.shape)} {x.dtype} |x| max {x_top:.4g}, "
+                  f"y finite {y_ok}", flush=True)
+
+
+_trace = _Trace()
+
+
 @torch.library.custom_op("shapequant::linear", mutates_args=())
 def linear_op(x: torch.Tensor, handle: int) -> torch.Tensor:
-    return _REGISTRY[handle].forward(x)
+    y = _REGISTRY[handle].forward(x)
+    _trace("linear", handle, x, y)
+    return y
 
 
 @linear_op.register_fake
@@ -355,7 +395,9 @@ def _(x: torch.Tensor, handle: int) -> torch.Tensor:
 
 @torch.library.custom_op("shapequant::embed", mutates_args=())
 def embed_op(ids: torch.Tensor, handle: int) -> torch.Tensor:
-    return _REGISTRY[handle].forward(ids)
+    y = _REGISTRY[handle].forward(ids)
+    _trace("embed", handle, ids, y)
+    return y
 
 
 @embed_op.register_fake

@@ -516,6 +516,66 @@ def test_custom_op_compiles_and_graph_captures(large):
             assert torch.equal(y, f(x))
 
 
+def test_bf16_activations_beyond_the_fp16_range_saturate_and_are_reported(capsys, monkeypatch):
+    """Activations are multiplied as fp16: a bf16 value beyond 65,504 turns into inf inside the kernels (documented
+    behaviour, pinned here), every output row that meets it with a nonzero weight is inf or nan, rows of finite
+    activations in the same call are untouched, and SHAPEQUANT_DEBUG=1 reports the layer (reference
+    shapequant/vllm_ext/core.py:673-690)."""
+    from quantexperiments_amd.vllm_ext import core
+    s = synth(96, 512, 8, 16, seed=9)
+    ps = core.PackedShards([to_device(s)])
+    h = core.register(ps)
+    x = rand_x(2, 512, torch.bfloat16, seed=2)
+    x[0, 7] = 70000.0                                            # bf16 holds it (70144), fp16 does not
+    monkeypatch.setattr(core, "_trace", core._Trace())
+    core._trace.enabled = True
+    y = torch.ops.shapequant.linear(x.cuda(), h)
+    assert not torch.isfinite(y[0]).any()                        # every row has a nonzero weight in column 7
+    ref = _ref(s, x[1:2])
+    _check_lowp(y[1:2], ref)
+    # the same on every route: one row (tag-stream kernel), a few rows (matrix-core kernel), prefill (tile GEMM)
+    for rows in (1, 9, 40, 300):
+        xr = rand_x(rows, 512, torch.bfloat16, seed=rows)
+        xr[0, 7] = -70000.0
+        yr = ps.forward(xr.cuda())
+        assert not torch.isfinite(yr[0]).any() and torch.isfinite(yr[1:]).all(), rows
+    out = capsys.readouterr().out
+    assert "[sqhip alarm] linear layer %d: input beyond the fp16 range" % h in out and "[sqhip trace]" in out
+    core._trace.enabled = False
+    torch.ops.shapequant.linear(x.cuda(), h)
+    assert capsys.readouterr().out == ""
+    # the largest fp16 value itself is fine
+    x[0, 7] = 65280.0
+    y = torch.ops.shapequant.linear(x.cuda(), h)
+    assert torch.isfinite(y).all()
+
+
+def test_launcher_refuses_stream_counts_the_builder_did_not_make():
+    """sq_matrix.stream_runs / stream_groups come from the caller: values that do not describe the buffer (a run count
+    that leaves the last run empty, runs longer than stated, too few groups) are refused before anything is launched."""
+    import ctypes
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    lin = to_device(synth(700, 512, 8, 16, seed=4))
+    lin.build_stream(4)
+    runs, run_max = lin.stream_runs & 0xFFFF, lin.stream_runs >> 16
+    x = torch.zeros(1, 512, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros(1, 700, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(1 << 22, dtype=torch.uint8, device="cuda")
+
+    def call(stream_runs, groups):
+        m = lin.descriptor(0)
+        m.stream_runs, m.stream_groups = stream_runs, groups
+        return L.sq_linear_small(_lib.matrix_array([m]), 1, x.data_ptr(), _lib.SQ_BF16, 512, y.data_ptr(), _lib.SQ_BF16, 700, 1,
+                                 ws.data_ptr(), ws.numel(), _lib.stream_ptr(x.device))
+    assert call(lin.stream_runs, lin.stream_groups) == 0
+    assert call(runs | ((run_max + 1) << 16), lin.stream_groups) == _lib.SQ_EINVAL       # longer runs than the cut gives
+    assert call((runs + 7) | (run_max << 16), lin.stream_groups) == _lib.SQ_EINVAL       # an empty last run
+    assert call(lin.stream_runs, lin.stream_groups - 1) == _lib.SQ_EINVAL                # fewer groups than rows need
+    assert call(runs, lin.stream_groups) in (_lib.SQ_EINVAL, _lib.SQ_EUNSUPPORTED, 0)    # no run length: not a stream -> row kernel
+    torch.cuda.synchronize()
+
+
 # ------------------------------------------------------------------ one copy of the tags (the reference's `compact`)
 @pytest.mark.parametrize("case", [(300, 1024, 16, 1), (257, 3584, 16, 1), (140, 5120, 16, 16), (700, 1024, 14, 3), (65, 18944, 16, 1)],
                          ids=lambda c: "x".join(map(str, c)))

@@ -289,6 +289,83 @@ def test_stream_builder_keeps_every_tag(R, C, bits, runs, M):
     assert np.array_equal(_walk_stream(buf, R, C, 8, bits, eff, NG, row_mask), tags)
 
 
+def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask, PF=3, NW=16):
+    """Every byte range of the stream buffer that stream_kernel (csrc/sq_stream.hip) forms an address for, replayed on
+    the host: the run table, the group heads (with the kernel's clamp of the group index), the first steps a wave
+    requests before it knows whether it has any (the prologue reads step 0 for a group without steps), the steps
+    fetched ahead inside the loop (clamped to the group's last step), the shares of a group that several waves walk,
+    and the row list of the finishing workgroup.  Yields (what, first byte, end byte)."""
+    runs, run_max = runs_out & 0xFFFF, runs_out >> 16
+    U, NS = C // 8, 1 << (bits - 12)
+    KP = -(-U // PART_MAX)
+    NV = NS * KP
+    off_slots = ((NV * NG + 1) * 4 + 255) & ~255
+    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
+    off_rows = (off_runs + runs * 16 + 255) & ~255
+    off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
+    goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0).astype(np.int64)
+    rt = np.frombuffer(buf, np.int32, runs * 4, off_runs).reshape(runs, 4)
+    gr = -(-NG // runs)
+    for v in range(NV):
+        for wi in range(runs):
+            if row_mask is not None:
+                yield "run table", off_runs + wi * 16, off_runs + wi * 16 + 12
+                g0, ng = int(rt[wi, 0]), int(rt[wi, 1])
+            else:
+                g0, ng = wi * gr, min(gr, NG - wi * gr)
+            ng = min(ng, run_max)                       # the kernel never walks more groups than its LDS holds sums for
+            assert ng >= 1, (v, wi, g0, ng)
+            split = NW // ng if ng * 2 <= NW else 1
+            yield "row list", off_rows + g0 * 256, off_rows + (g0 + ng) * 256
+            # head(k) for every k a wave can ask for: its own groups and, one ahead, the index behind the last one
+            for k in range(ng + 1):
+                kc = min(k, ng - 1)
+                i = v * NG + g0 + kc
+                yield "group offsets", i * 4, i * 4 + 8
+                yield "slots", off_slots + i * 256, off_slots + i * 256 + 256
+                if k >= ng:
+                    continue
+                st0, nst = int(goff[i]), int(goff[i + 1] - goff[i])
+                for sub in range(split):
+                    s0, s1 = nst * sub // split, nst * (sub + 1) // split
+                    a, n = st0 + s0, s1 - s0
+                    # prologue (first_steps_always): a wave without steps reads step 0 of the stream
+                    steps = [a + min(q, max(n - 1, 0)) if n > 0 else 0 for q in range(PF)]
+                    # the loop: PF steps ahead, clamped to the share's last step
+                    steps += [a + min(t0 + PF + q, n - 1) for t0 in range(0, n, PF) for q in range(PF) if t0 + PF < n]
+                    for st in set(steps):
+                        yield "steps", off_steps + st * 768, off_steps + st * 768 + 768
+
+
+@pytest.mark.parametrize("R,C,bits,runs,M", [(1, 8, 16, 0, 1), (1, 8, 14, 6, 1), (65, 8, 16, 6, 1), (64, 8, 16, 3, 1), (63, 64, 16, 2, 1),
+                                              (130, 64, 14, 5, 1), (257, 64, 15, 4, 1), (130, 3584, 16, 1, 1), (700, 512, 16, 16, 1),
+                                              (5, 64, 16, 0, 3), (300, 512, 16, 3, 4), (1000, 256, 14, 2, 16),
+                                              (12900, 64, 14, 1, 1), (70, 32800, 16, 0, 1)])
+def test_kernel_addresses_stay_inside_the_stream(R, C, bits, runs, M):
+    """The batch-1 kernel once read past the end of the stream for a last group without steps (a single row with one
+    chunk leaves 15 of its 16 buckets empty, and their groups begin where the stream ends).  Every address the kernel
+    can form is replayed here against the builder's buffer; degenerate shapes included."""
+    rng = np.random.default_rng(R * 7 + C + bits + M)
+    tags = rng.integers(0, 1 << bits, (R, C // 8))
+    row_mask = rng.integers(0, M, R).astype(np.uint8) if M > 1 else None
+    words = np.ascontiguousarray(O.pack_bits(tags, bits))
+    import ctypes
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    ptr = words.ctypes.data_as(ctypes.c_void_p)
+    mp = None if row_mask is None else row_mask.ctypes.data_as(ctypes.c_void_p)
+    n = L.sq_stream_bytes(ptr, R, words.shape[1], C, 8, bits, mp, runs)
+    out = np.zeros(n, np.uint8)
+    r, g = ctypes.c_int32(0), ctypes.c_int32(0)
+    assert L.sq_stream_build(ptr, R, words.shape[1], C, 8, bits, mp, runs, out.ctypes.data_as(ctypes.c_void_p), n, ctypes.byref(r), ctypes.byref(g)) == 0
+    assert 1 <= (r.value >> 16) <= 96 and 1 <= (r.value & 0xFFFF) <= g.value
+    count = 0
+    for what, a, b in _stream_reads(out.tobytes(), R, C, bits, r.value, g.value, row_mask):
+        assert 0 <= a < b <= n, (what, a, b, n)
+        count += 1
+    assert count > 0
+
+
 # the lanes one clock of a ds_read_b128 serves on gfx950 (measured: see LDS_CLOCK_LANES in csrc/sq_stream.hip)
 LDS_CLOCK_LANES = [[0, 1, 2, 3, 12, 13, 14, 15, 20, 21, 22, 23, 24, 25, 26, 27],
                    [4, 5, 6, 7, 8, 9, 10, 11, 16, 17, 18, 19, 28, 29, 30, 31]]

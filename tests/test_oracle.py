@@ -378,3 +378,40 @@ def test_silu_mul_fixed_points():
     assert np.all(np.abs(O.silu_mul(np.full((1, 4), -20.0), one)[0, 0]) < 1e-7)
     assert np.array_equal(O.silu_mul(np.full((1, 4), 1.0), one)[0, 0],
                           np.full(4, np.float16(1.0 / (1.0 + math.exp(-1.0))), dtype=np.float32))
+
+
+def test_chunk_rows_closed_form():
+    """chunk_rows (reference shapequant/codebook.py:212-218) against what it must produce for w[r, c] = 100 r + c: chunk
+    k of row r is row r * ceil(C / d) + k of the result and holds 100 r + d k + j at position j, zeros beyond column
+    C; pad = the zeros added per row."""
+    for R, C, d in ((3, 8, 4), (2, 10, 4), (4, 5, 8), (1, 1, 3), (5, 12, 1)):
+        w = (100.0 * np.arange(R)[:, None] + np.arange(C)[None, :]).astype(np.float32)
+        chunks, pad = O.chunk_rows(w, d)
+        per = -(-C // d)
+        assert pad == per * d - C and chunks.shape == (R * per, d)
+        for r in range(R):
+            for k in range(per):
+                for j in range(d):
+                    c = k * d + j
+                    assert chunks[r * per + k, j] == (100.0 * r + c if c < C else 0.0)
+
+
+def test_torch_cpu_layer_is_decode_then_matmul():
+    """The CPU baseline that bench.py times (torch gather + scale + scatter + fp32 matmul + bf16 round) gives the
+    product of the oracle's own decode, rounded to bf16: with and without column orders."""
+    import torch
+    for M in (1, 4):
+        g = torch.Generator().manual_seed(11 + M)
+        R, C, d, bits = 24, 64, 8, 14
+        tags = torch.randint(0, 1 << bits, (R, C // d), generator=g).numpy()
+        table = (torch.randn(1 << bits, d, generator=g) * 0.5).half()
+        rs = (torch.rand(R, generator=g) * 0.02 + 0.01).half()
+        rm = torch.randint(0, M, (R,), generator=g).to(torch.uint8) if M > 1 else None
+        perms = torch.from_numpy(O.seeded_perms(C, M, 5))
+        x = torch.randn(3, C, generator=g).to(torch.bfloat16)
+        words = torch.from_numpy(O.pack_bits(tags, bits))
+        y, _, _ = O.torch_cpu_layer(words, table, rs, rm, perms if M > 1 else None, bits, x)
+        w = O.decode_tensors(tags, table.numpy(), rs.numpy(), None, None if rm is None else rm.numpy(), perms.numpy(), 1 << bits)
+        ref = O.linear(x.float().numpy(), w)
+        got = y.float().numpy().astype(np.float64)
+        assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -8 + 1e-6 * np.abs(ref).max())    # one bf16 rounding of an fp32 sum
