@@ -24,16 +24,21 @@ class _Workspace:
     shape once eagerly first, as with the reference's shared buffers (reference
     shapequant/vllm_ext/core.py:198-209, shapequant/kernels/batched_runs.py:628-640)."""
     bufs: dict = {}
+    retired: list = []          # outgrown buffers: a HIP graph captured earlier still launches kernels on them
 
     @classmethod
     def get(cls, nbytes: int, dev, kind: str = "kernels") -> torch.Tensor:
         """kind "kernels": the buffer handed to the library (its first 4096 bytes are the library's counters
-        and stay zero between calls); any other kind names a separate buffer the caller may overwrite."""
+        and stay zero between calls); any other kind names a separate buffer the caller may overwrite.
+        A buffer that has to grow is replaced, never freed: graphs captured with the old one stay valid (the
+        reference keeps a reference per launcher for the same reason, shapequant/kernels/batched_runs.py:741-743)."""
         key = (str(dev), kind)
         b = cls.bufs.get(key)
         if b is None or b.numel() < nbytes:
             if torch.cuda.is_current_stream_capturing():
                 raise RuntimeError("sqhip workspace must grow outside graph capture: run this shape once eagerly first")
+            if b is not None:
+                cls.retired.append(b)
             b = cls.bufs[key] = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)   # counters start at zero
         return b
 
