@@ -76,13 +76,13 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
 
 /* sq_linear_small without a workspace argument, for callers that cannot allocate device memory (code under HIP graph
  * capture that has not grown a workspace beforehand, tight serving loops, harnesses that forbid hipMalloc): same
- * arguments, same kernels and bit-identical results, with the partial sums and arrival counters kept in a device array
+ * arguments, same kernels and bit-identical results, with the workspace (header included) kept in a device array
  * of SQ_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on until the process ends.  It has no
  * counterpart in the reference (whose launchers grow torch buffers on demand).  Pieces and row counts whose workspace
  * (sq_workspace_bytes(mats, n_mats, B, 0)) exceeds the array are refused with SQ_EWORKSPACE; nothing is allocated or freed,
  * here or in anything it calls.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
  * (two streams, two threads) race; calls on one stream are safe. */
-#define SQ_NOALLOC_SCRATCH_BYTES (16u << 20)
+#define SQ_NOALLOC_SCRATCH_BYTES (48u << 20)
 int sq_linear_small_noalloc(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx,
                             void* y, int y_dtype, int64_t ldy, int32_t B, void* stream);
 
@@ -118,9 +118,14 @@ size_t sq_gemm_dense_workspace_bytes(int32_t R, int32_t C, int32_t T);
 /* Bytes of workspace sq_linear_small (which = 0) or sq_linear_gemm (which = 1) needs for these
  * pieces at `rows` activation rows; the caller grows its buffer before any graph capture
  * (the reference grows its buffers the same way: batched_runs.py:628-640, runs_gemm.py:396-404).
- * A workspace must be 256-byte aligned and its first 4096 bytes must be ZERO when it is first handed
- * to the library (they hold arrival counters that every call leaves at zero again); one workspace
- * serves one stream at a time. */
+ * A workspace must be 256-byte aligned and its first SQ_WS_HEADER_BYTES must be ZERO when it is first
+ * handed to the library, and nobody else may write there afterwards: the header holds the partial sums that
+ * the workgroups of the decode-time kernel for large codebooks exchange.  A partial sum is its own arrival
+ * flag (a word is zero until its sum has been written, and the workgroup that adds a word up puts zero back),
+ * so every call leaves the header zeroed again and no call ever clears it.  Everything else a call needs lies
+ * behind the header and may hold anything.  One workspace serves one stream at a time; a call that is
+ * abandoned half way (a device reset) leaves a header that must be zeroed before it is used again. */
+#define SQ_WS_HEADER_BYTES (32u << 20)
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which);
 
 /* Load-time regrouping of a matrix' tags for codebooks that do not fit LDS (d = 8, K = 8192..65,536, one

@@ -13,7 +13,8 @@ LIB_PATH = _HERE / "libsqhip.so"
 SQ_F32, SQ_F16, SQ_BF16 = 0, 1, 2
 SQ_OK, SQ_EINVAL, SQ_EUNSUPPORTED, SQ_EWORKSPACE, SQ_ELAUNCH = 0, -1, -2, -3, -4
 SMALL_BMAX = 32
-NOALLOC_SCRATCH_BYTES = 16 << 20
+WS_HEADER = 32 << 20            # SQ_WS_HEADER_BYTES: zero when a workspace is first handed over
+NOALLOC_SCRATCH_BYTES = 48 << 20
 
 DTYPES = {torch.float32: SQ_F32, torch.float16: SQ_F16, torch.bfloat16: SQ_BF16}
 

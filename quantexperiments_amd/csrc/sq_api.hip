@@ -98,14 +98,15 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
     const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
     if (small_takes_gemm_route(mats, n_mats, B, x, ldx))
         return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
-                           has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
+                           has_ws ? ws_bytes - SQ_WS_HEADER : 0, has_ws ? workspace : nullptr, (hipStream_t)stream);
     return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
-                        has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
+                        has_ws ? ws_bytes - SQ_WS_HEADER : 0, has_ws ? workspace : nullptr, (hipStream_t)stream);
 }
 
 // ---- sq_linear_small for callers that cannot allocate: the workspace is a device array of this library.
 // In host code `g_static_scratch` is only a handle for hipGetSymbolAddress: the device address it stands for is looked
 // up once per device and kept; kernels are handed that address, never the symbol.
+static_assert(sq::SQ_WS_HEADER == SQ_WS_HEADER_BYTES, "the header size is part of the ABI");
 static __device__ __align__(256) unsigned char g_static_scratch[SQ_NOALLOC_SCRATCH_BYTES];
 static void* g_static_scratch_ptr[64];
 
@@ -122,8 +123,8 @@ static void* static_scratch(hipStream_t s) {
         void* ptr = nullptr;
         const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
         if (e != hipSuccess || !ptr) { fail(SQ_ELAUNCH, "sq_linear_small_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e)); return nullptr; }
-        // the arrival counters at the head must be zero before the first call (a fill kernel, not a memset node, so
-        // that this is also safe as the first thing a graph capture records)
+        // the header (the tag-stream kernel's partial sums) must be zero before the first call (a fill kernel, not a
+        // memset node, so that this is also safe as the first thing a graph capture records)
         hipLaunchKernelGGL(noalloc_clear_kernel, dim3((unsigned)(SQ_WS_HEADER / 4 / 256)), dim3(256), 0, s, (unsigned*)ptr, (int)(SQ_WS_HEADER / 4));
         if (check_launch("sq_linear_small_noalloc(clear)")) return nullptr;
         g_static_scratch_ptr[dev] = ptr;
@@ -145,8 +146,8 @@ int sq_linear_small_noalloc(const sq_matrix* mats, int32_t n_mats, const void* x
     if (!ws) return SQ_ELAUNCH;
     const size_t inner = (size_t)SQ_NOALLOC_SCRATCH_BYTES - SQ_WS_HEADER;
     if (small_takes_gemm_route(mats, n_mats, B, x, ldx))
-        return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, ws + SQ_WS_HEADER, inner, (unsigned*)ws, (hipStream_t)stream);
-    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, ws + SQ_WS_HEADER, inner, (unsigned*)ws, (hipStream_t)stream);
+        return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, ws + SQ_WS_HEADER, inner, ws, (hipStream_t)stream);
+    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, ws + SQ_WS_HEADER, inner, ws, (hipStream_t)stream);
 }
 
 int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_producer* from, int x_dtype, void* y, int y_dtype,
@@ -184,14 +185,14 @@ int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_produce
     const size_t wsb = has_ws ? ws_bytes - SQ_WS_HEADER : 0;
     const bool aligned = (((uintptr_t)from->h_in | (uintptr_t)from->h_out | (uintptr_t)from->add | (uintptr_t)from->up | (uintptr_t)from->w) & 15) == 0;
     if (aligned && small_fuses_producer(mats, n_mats, B))
-        return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, (unsigned*)workspace, s, from);
+        return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, has_ws ? workspace : nullptr, s, from);
     rc = addnorm ? launch_addnorm(from->h_in, from->h_out, from->ld_h, from->add, x_dtype, from->ld_in, from->w, x_dtype, nullptr, 1, B,
                                   C, from->eps, from->x_out, x_dtype, s)
                  : launch_silu_mul(from->add, from->up, x_dtype, from->ld_in, nullptr, 1, B, C, from->x_out, s);
     if (rc) return rc;
     if (small_takes_gemm_route(mats, n_mats, B, from->x_out, C))
-        return launch_gemm(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, (unsigned*)workspace, s);
-    return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, (unsigned*)workspace, s);
+        return launch_gemm(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, has_ws ? workspace : nullptr, s);
+    return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, has_ws ? workspace : nullptr, s);
 }
 
 int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
@@ -201,7 +202,7 @@ int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_d
     if (T == 0 || n_mats == 0) return SQ_OK;
     const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
     return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
-                       has_ws ? ws_bytes - SQ_WS_HEADER : 0, (unsigned*)workspace, (hipStream_t)stream);
+                       has_ws ? ws_bytes - SQ_WS_HEADER : 0, has_ws ? workspace : nullptr, (hipStream_t)stream);
 }
 
 int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype, int64_t ldx,
@@ -240,7 +241,7 @@ size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, i
     // which = 0 covers both kernels a stack with column orders may take (the caller's x decides, see sq_linear_small)
     const size_t inner = which == 0 ? std::max(small_workspace(mats, n_mats, rows), small_gemm_route_workspace(mats, n_mats, rows))
                                     : gemm_workspace(mats, n_mats, rows);
-    return inner ? inner + SQ_WS_HEADER : 0;
+    return (inner || small_uses_sums(mats, n_mats)) ? inner + SQ_WS_HEADER : 0;
 }
 
 size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,

@@ -94,10 +94,11 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// A caller's workspace starts with SQ_WS_HEADER bytes of arrival counters that are zero whenever no call is
-// running (kernels that use them put them back to zero); the launchers get the part behind the header.
-constexpr size_t SQ_WS_HEADER = 4096;
-constexpr int SQ_WS_COUNTERS = 1024;
+// A caller's workspace starts with SQ_WS_HEADER bytes that only the tag-stream kernel touches: the partial sums its
+// workgroups exchange.  Every word of them is zero whenever no call is running (a partial sum doubles as its own arrival
+// flag and whoever adds it up puts zero back), so they must be zero when the workspace is first handed over and nothing
+// else may ever be written there; the other launchers get the part behind the header.
+constexpr size_t SQ_WS_HEADER = (size_t)32 << 20;
 
 // error plumbing shared by the launchers (defined in sq_api.hip)
 int fail(int code, const char* fmt, ...);
@@ -108,13 +109,15 @@ int device_cus();       // compute units of the current device (cached)
 int launch_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s,
                    bool raw = false);
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s,
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, void* sums, hipStream_t s,
                  const sq_producer* from = nullptr);
 // one activation row of these pieces is a single launch of the tag-stream kernel, which can produce its own x
 bool small_fuses_producer(const sq_matrix* mats, int n, int B);
 size_t small_workspace(const sq_matrix* mats, int n, int B);
+// some piece runs the tag-stream kernel, whose partial sums live in the workspace header (`sums` above)
+bool small_uses_sums(const sq_matrix* mats, int n);
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                int64_t ldy, int T, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s);
+                int64_t ldy, int T, void* ws, size_t ws_bytes, void* sums, hipStream_t s);
 // stacks with column orders and more than a few activation rows: sq_linear_small runs the decode + tile GEMM route
 bool small_takes_gemm_route(const sq_matrix* mats, int n, int B, const void* x, int64_t ldx);
 size_t small_gemm_route_workspace(const sq_matrix* mats, int n, int B);

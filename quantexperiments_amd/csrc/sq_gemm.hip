@@ -285,9 +285,9 @@ int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, con
 }
 
 int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                int64_t ldy, int T, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s) {
+                int64_t ldy, int T, void* ws, size_t ws_bytes, void* sums, hipStream_t s) {
     if (T <= SQ_SMALL_BMAX && !small_takes_gemm_route(mats, n, T, x, ldx))
-        return launch_small(mats, n, x, x_dtype, ldx, y, y_dtype, ldy, T, ws, ws_bytes, counters, s);
+        return launch_small(mats, n, x, x_dtype, ldx, y, y_dtype, ldy, T, ws, ws_bytes, sums, s);
     if (T > SQ_SMALL_BMAX && T <= small_pass_limit(mats, n) && x_vec_ok(x, ldx, mats[0].C)) {
         // a few passes of the decode-time kernel read the packed tags a few times; decoding to fp16 first
         // (below) writes and reads 8 to 16 times as many bytes once
@@ -295,7 +295,7 @@ int launch_gemm(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_
         for (int t = 0; t < T; t += SQ_SMALL_BMAX) {
             const int nb = T - t < SQ_SMALL_BMAX ? T - t : SQ_SMALL_BMAX;
             int rc = launch_small(mats, n, (const char*)x + (size_t)t * ldx * 2, x_dtype, ldx, (char*)y + (size_t)t * ldy * ys,
-                                  y_dtype, ldy, nb, ws, ws_bytes, counters, s);
+                                  y_dtype, ldy, nb, ws, ws_bytes, sums, s);
             if (rc) return rc;
         }
         return SQ_OK;

@@ -184,11 +184,17 @@ static size_t mma_part_bytes(const sq_matrix& m, int B) {
 size_t small_workspace(const sq_matrix* mats, int n, int B) {
     size_t tot = 0;
     for (int i = 0; i < n; ++i) {
-        if (stream_rows(mats[i], B)) tot += stream_part_bytes(mats[i], B);
-        else if (mma_shape(mats[i])) tot += mma_part_bytes(mats[i], B);
+        if (stream_rows(mats[i], B)) continue;                   // its partial sums live in the workspace header
+        if (mma_shape(mats[i])) tot += mma_part_bytes(mats[i], B);
         else if (mats[i].perms && fast_shape(mats[i])) tot += xp_bytes(mats[i], B);
     }
     return tot;
+}
+
+bool small_uses_sums(const sq_matrix* mats, int n) {
+    for (int i = 0; i < n; ++i)
+        if (mats[i].R > 0 && stream_shape(mats[i])) return true;
+    return false;
 }
 
 // Pieces [0, cnt) share format and row length: one persistent launch (+ one reduction per piece if ks > 1).
@@ -263,24 +269,24 @@ bool small_fuses_producer(const sq_matrix* mats, int n, int B) {
 }
 
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                 int64_t ldy, int B, void* ws, size_t ws_bytes, unsigned* counters, hipStream_t s, const sq_producer* from) {
+                 int64_t ldy, int B, void* ws, size_t ws_bytes, void* sums, hipStream_t s, const sq_producer* from) {
     if (from && !small_fuses_producer(mats, n, B)) return fail(SQ_EUNSUPPORTED, "sq_linear_small_from: no fused kernel for this stack");
     if (small_workspace(mats, n, B) > ws_bytes)
         return fail(SQ_EWORKSPACE, "sq_linear_small: workspace %zu < %zu", ws_bytes, small_workspace(mats, n, B));
     const int cus = device_cus();
     const bool x_ok = (B == 1 || ldx % 8 == 0) && (((uintptr_t)x & 15) == 0);   // 16-byte activation loads
     size_t ws_off = 0;
-    int counters_used = 0;
     int i = 0;
     while (i < n) {
         const sq_matrix& m0 = mats[i];
         if (m0.R == 0) { ++i; continue; }
         const int ud = unit_dwords(m0.bits);
         if (stream_rows(m0, B) && (x_ok || from)) {
+            if (!sums) return fail(SQ_EWORKSPACE, "sq_linear_small: these pieces need a workspace (its header holds their partial sums)");
             int j = i + 1;
             while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_rows(mats[j], B) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
-            int rc = launch_stream_group(mats + i, j - i, x, x_dtype, ldx, y, y_dtype, ldy, B, (char*)ws, ws_off, counters,
-                                         counters_used, s, from);
+            j = i + stream_group_len(mats + i, j - i);
+            int rc = launch_stream_group(mats + i, j - i, x, x_dtype, ldx, y, y_dtype, ldy, B, (char*)sums, s, from);
             if (rc) return rc;
             i = j;
             continue;
@@ -301,7 +307,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         if (pl.TS == 0) {
             int rc = launch_small_generic(mats + i, 1, x, x_dtype, ldx, y, y_dtype, ldy, B, s);
             if (rc) return rc;
-            if (stream_rows(m0, B)) ws_off += stream_part_bytes(m0, B);
+            if (stream_rows(m0, B)) {}
             else if (mma_shape(m0)) ws_off += mma_part_bytes(m0, B);
             else if (m0.perms && fast_shape(m0)) ws_off += xp_bytes(m0, B);
             ++i;

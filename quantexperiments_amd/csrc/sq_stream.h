@@ -31,11 +31,12 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
 inline int stream_runs_of(const sq_matrix& m) { return m.stream_runs & 0xFFFF; }
 inline int stream_run_max_of(const sq_matrix& m) { return (int)((uint32_t)m.stream_runs >> 16); }
 bool stream_shape(const sq_matrix& m);
-size_t stream_part_bytes(const sq_matrix& m, int B);
+size_t stream_part_bytes(const sq_matrix& m, int rows);   // partial sums of one pass of `rows` activation rows
 // dense rows [r0, r1) of a matrix that is held as its tag stream only (sq_matrix.tags == NULL)
 int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s, bool raw);
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                        int64_t ldy, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
-                        hipStream_t s, const sq_producer* from = nullptr);
+                        int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from = nullptr);
+// pieces [0, n) a single launch can take: their partial sums of one activation row fit the workspace header together
+int stream_group_len(const sq_matrix* mats, int n);
 
 }  // namespace sq

@@ -11,15 +11,15 @@
 // Rows are first ordered by column order (row_mask, stable), so that consecutive rows share one; each column
 // order's rows are cut into groups of 64 (the last group of an order may be short) and into runs of at most GR
 // groups, one workgroup per (bucket, run); the caller picks the number of runs so that the pieces it launches
-// together make about two workgroups per CU.  Within a bucket the rows of a run are sorted by entry count
+// together make about one workgroup (of 16 waves) per CU.  Within a bucket the rows of a run are sorted by entry count
 // (descending, stable): one lane per row, one wave per group.  A group is stored as steps of 64 x 12 bytes
 // (4 entries per lane per step, lane-major, so a wave reads 768 contiguous bytes per step) padded to the longest
 // row of the group; sorting keeps that padding near 10 percent.  A workgroup stages its slice and its part of x
 // (gathered through the run's column order, if any) in LDS; each lane accumulates dot(codeword, x chunk) over
-// its entries in fp32 and writes one partial sum per (bucket, row).  The workgroups of all buckets that cover
-// the same run count themselves off on a counter in the workspace; the last one to arrive adds the NS * KP
-// partials of each row of the run in a fixed order (so results do not depend on scheduling), applies the row
-// scale and stores y.
+// its entries in fp32 and leaves one partial sum per (bucket, row) in the workspace header, whose words are zero
+// between launches: a partial sum is its own arrival flag.  The workgroups of all buckets that cover the same run
+// each take a share of the run's rows, read the NS * KP partials of a row until none is zero, add them in a fixed
+// order (so results do not depend on scheduling), apply the row scale, store y and put zero back.
 //
 // Stream buffer (one allocation; offsets follow from C/d, the tag width, the group and run counts):
 //   goff   uint32 [NV * NG + 1]   first step of every group, cumulative over buckets (NV = KP * NS buckets,
@@ -429,8 +429,7 @@ struct StreamPiece {
     const unsigned char* stream;
     const uint16_t* table;
     const uint16_t* row_scale;
-    float* part;                      // [NV][NB][NG * 64], indexed by place
-    unsigned* counters;               // one per run; zero before the launch, zero after it
+    float* part;                      // [NV][NB][NG * 64] words, indexed by place: zero before the launch, zero after it
     const int32_t* perms;             // [M, C] column orders or NULL
     int R, C, U, NS, NV, PC, NG, y_off;
     uint32_t off_slots, off_runs, off_rows, off_steps;
@@ -517,6 +516,8 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 constexpr int STREAM_TAB = 65536;     // the codebook slice
 constexpr int STREAM_PF = 3;          // steps fetched ahead (2 to 4 measure alike, 6 and 8 slower: the loop runs at the memory system's rate)
 constexpr int STREAM_NW = 16;         // waves per workgroup: one workgroup per CU
+constexpr uint32_t STREAM_ZERO_SUM = 0x7FFFFFFFu;  // how a partial sum with all bits zero is written (zero = not there yet)
+constexpr int STREAM_SPIN_MAX = 1 << 20;           // polls of an item's partial sums before it gives up
 
 // LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group)
 static inline int stream_xs(int pc) { return (pc + 16) * 16; }
@@ -557,8 +558,8 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     // Workgroups go to the 8 XCDs in turn (workgroup i to XCD i mod 8), each with an L2 of its own.  When the
     // bucket count is a multiple of 8 the bucket (and with it the slice) is made a function of the workgroup index
     // modulo 8, so an XCD only ever stages an eighth of the buckets' slices (one fetch from memory, then hits in
-    // its L2), and the workgroups of all buckets that share a run are neighbours in the grid and arrive together.
-    // Any other mapping is as correct.
+    // its L2).  Either way the NV workgroups of a run are consecutive in the grid: they wait for each other's partial
+    // sums at the end, and workgroups are dispatched in grid order, so whoever a workgroup waits for is running or done.
     const int local = (int)blockIdx.x - P.wg_begin;
     int v, wi;
     if ((P.NV & 7) == 0 && (P.wg_begin & 7) == 0) {
@@ -566,8 +567,8 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         v = (local & 7) + 8 * (rest % per);
         wi = rest / per;
     } else {
-        v = local / P.nwg;
-        wi = local - v * P.nwg;
+        wi = local / P.NV;
+        v = local - wi * P.NV;
     }
     const int s = v % P.NS, kp = v / P.NS;
     SQ_TRACE_POINT(0);
@@ -585,7 +586,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     const int xs = a.xs;
     const unsigned char* ldsx = lds + STREAM_TAB;
     float* psum = reinterpret_cast<float*>(lds + STREAM_TAB + NB * xs);          // [NB][a.nl_max], indexed by place - 64 g0
-    unsigned* flag = reinterpret_cast<unsigned*>(psum + (size_t)NB * a.nl_max);  // [0] arrival result, [1] next group
+    unsigned* flag = reinterpret_cast<unsigned*>(psum + (size_t)NB * a.nl_max);  // [1] next group
 
     // The groups of a run are sorted longest first.  Wave w starts with group w, then group 2 NW - 1 - w; after
     // that every wave draws the next unclaimed group from a counter in LDS, so all waves stay busy to the end.
@@ -889,103 +890,76 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     SQ_TRACE_POINT(2);
     __syncthreads();
     // The run's partial sums leave as whole lines (device-scope stores: written through to memory, so other XCDs'
-    // L2s never hold a stale copy and no cache-wide write-back is needed before the workgroup counts itself off).
-    // Places of a short last group hold no row: what is written there is never read.
+    // L2s never hold a stale copy).  A partial sum is its own arrival flag: the words of `part` are zero between
+    // launches, a sum whose bits are zero travels as STREAM_ZERO_SUM (a NaN pattern no sum can have), and whoever
+    // adds a word up puts zero back.  Nobody waits for a store to be acknowledged and there is no arrival counter.
     {
         const int nl = ng * 64;
+        uint32_t* pw = reinterpret_cast<uint32_t*>(part) + (size_t)g0 * 64;
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-            for (int i = tid; i < nl; i += NTH)
-                __hip_atomic_store(part + b * np + (size_t)g0 * 64 + i, psum[b * a.nl_max + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int b = 0; b < NB; ++b) {
+            if (b >= a.nb) break;
+            for (int i = tid; i < nl; i += NTH) {
+                const uint32_t u = __builtin_bit_cast(uint32_t, psum[b * a.nl_max + i]);
+                __hip_atomic_store(pw + b * np + i, u ? u : STREAM_ZERO_SUM, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
     }
-
-    // Count this workgroup off once all its partial sums have been acknowledged (the barrier waits for every
-    // wave's outstanding stores).  The workgroup that finds every other bucket's workgroup already counted
-    // reads all partial sums back with device-scope loads and finishes the rows.
-    __builtin_amdgcn_s_waitcnt(0);
     SQ_TRACE_POINT(3);
-    __syncthreads();
-    SQ_TRACE_POINT(4);
-    if (tid == 0) {
-        const unsigned old = atomicAdd(P.counters + wi, 1u);
-        if (old == (unsigned)P.NV - 1u) P.counters[wi] = 0u;    // everyone has arrived: leave the counter as found
-        flag[0] = old;
-    }
-    __syncthreads();
-    SQ_TRACE_POINT(5);
-    if (flag[0] != (unsigned)P.NV - 1u) return;
-    // places 64 g0 .. 64 (g0 + ng) - 1: consecutive partial sums; `rows` says which row each place is.  An item
-    // is one (activation row, place); 64 partial sums are in flight per thread: four items at a time when a row
-    // has 16 buckets, else one item's buckets 64 at a time; a row's partials are always added in bucket order
+    // Bucket v of the run's NV workgroups finishes share v of the run's (activation row, place) items: it reads the
+    // NV partial sums of an item with device-scope loads until none of them is zero, adds them in bucket order, writes
+    // y and zeroes the words.  The NV workgroups of a run are neighbours in the grid and workgroups are dispatched in
+    // grid order, so a workgroup only ever waits for workgroups that are already running or done; the wait is bounded
+    // all the same (an item that gives up is written as NaN).
     const uint32_t* rows0 = reinterpret_cast<const uint32_t*>(P.stream + P.off_rows) + (size_t)g0 * 64;
     const int nl = ng * 64, items = nl * a.nb;
-    const float* pp = P.part + (size_t)g0 * 64;
+    const int i_lo = (int)((int64_t)items * v / P.NV), i_hi = (int)((int64_t)items * (v + 1) / P.NV);
+    uint32_t* pp = reinterpret_cast<uint32_t*>(P.part) + (size_t)g0 * 64;
     const size_t ysz = a.y_dtype == SQ_F32 ? 4 : 2;
-    auto row_of = [&](int i) -> uint32_t {
-        return P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
-    };
-    if (P.NV <= 16) {
-        // Every load below is unconditional (indices are clamped, missing terms are dropped afterwards): a load the
-        // compiler must guard with a branch is waited for before the next one goes out, and the 64 partial sums
-        // of a thread would take four trips to memory instead of one.
-        for (int ib = tid; ib < items; ib += 4 * NTH) {
-            float t[4][16], rs[4];
-            uint32_t rr[4];
-            int bb[4];
-            bool live[4];
+    for (int it = i_lo + tid; it < i_hi; it += NTH) {
+        const int b = it / nl, i = it - b * nl;
+        const uint32_t r = P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
+        const float rs = h2f(P.row_scale[r != STREAM_NO_ROW ? r : 0u]);
+        uint32_t* q = pp + (size_t)b * np + i;
+        const size_t bs = (size_t)NB * np;                      // words from one bucket's partial sums to the next
+        float sum = 0.f;
+        bool ok = true;
+        if (P.NV <= 16) {
+            uint32_t u[16];
+            for (int spin = 0;; ++spin) {
+                // (unconditional loads from clamped indices: all of them are in flight together)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                live[q] = ib + q * NTH < items;
-                const int it = min(ib + q * NTH, items - 1);
-                bb[q] = it / nl;
-            }
-            if (P.perms) {                                      // the four row ids in one trip
+                for (int k = 0; k < 16; ++k) u[k] = __hip_atomic_load(q + (size_t)min(k, P.NV - 1) * bs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ok = true;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) rr[q] = rows0[min(ib + q * NTH, items - 1) - bb[q] * nl];
-            } else {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) rr[q] = row_of(min(ib + q * NTH, items - 1) - bb[q] * nl);
+                for (int k = 0; k < 16; ++k) ok = ok && u[k] != 0u;
+                if (ok || spin >= STREAM_SPIN_MAX) break;
+                __builtin_amdgcn_s_sleep(2);
             }
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (!live[q]) rr[q] = STREAM_NO_ROW;
+            for (int k = 0; k < 16; ++k)
+                if (k < P.NV) sum += u[k] == STREAM_ZERO_SUM ? 0.f : __builtin_bit_cast(float, u[k]);
+        } else {
+            for (int v0 = 0; v0 < P.NV; v0 += 32) {
+                uint32_t u[32];
+                for (int spin = 0;; ++spin) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) rs[q] = h2f(P.row_scale[rr[q] != STREAM_NO_ROW ? rr[q] : 0u]);
+                    for (int k = 0; k < 32; ++k) u[k] = __hip_atomic_load(q + (size_t)min(v0 + k, P.NV - 1) * bs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    bool all = true;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int it = min(ib + q * NTH, items - 1);
-                const uint32_t off = (uint32_t)(bb[q] * (int)np + (it - bb[q] * nl));  // uniform base + 32-bit lane offset
+                    for (int k = 0; k < 32; ++k) all = all && u[k] != 0u;
+                    if (all) break;
+                    if (spin >= STREAM_SPIN_MAX) { ok = false; break; }
+                    __builtin_amdgcn_s_sleep(2);
+                }
 #pragma unroll
-                for (int k = 0; k < 16; ++k)
-                    t[q][k] = __hip_atomic_load(pp + (size_t)min(k, P.NV - 1) * NB * np + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float sum = 0.f;
-#pragma unroll
-                for (int k = 0; k < 16; ++k) sum += k < P.NV ? t[q][k] : 0.f;
-                if (rr[q] != STREAM_NO_ROW)
-                    store_y((char*)a.y + (size_t)bb[q] * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + rr[q], sum * rs[q]);
+                for (int k = 0; k < 32; ++k)
+                    if (v0 + k < P.NV) sum += u[k] == STREAM_ZERO_SUM ? 0.f : __builtin_bit_cast(float, u[k]);
             }
         }
-    } else {
-        for (int it = tid; it < items; it += NTH) {
-            const int b = it / nl, i = it - b * nl;
-            const uint32_t r = row_of(i);
-            if (r == STREAM_NO_ROW) continue;
-            const uint32_t off = (uint32_t)(b * (int)np + i);
-            float sum = 0.f;
-            for (int v0 = 0; v0 < P.NV; v0 += 64) {
-                float t[64];
-#pragma unroll
-                for (int k = 0; k < 64; ++k)
-                    t[k] = v0 + k < P.NV
-                               ? __hip_atomic_load(pp + (size_t)(v0 + k) * NB * np + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
-#pragma unroll
-                for (int k = 0; k < 64; ++k) sum += t[k];
-            }
-            store_y((char*)a.y + (size_t)b * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
-        }
+        for (int k = 0; k < P.NV; ++k) __hip_atomic_store(q + (size_t)k * bs, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (r != STREAM_NO_ROW)
+            store_y((char*)a.y + (size_t)b * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + r, ok ? sum * rs : __builtin_nanf(""));
     }
     SQ_TRACE_POINT(6);
 }
@@ -1100,23 +1074,33 @@ int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t 
 
 bool stream_shape(const sq_matrix& m) {
     return m.stream && stream_runs_of(m) > 0 && m.stream_groups > 0 && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
-           (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0;
+           (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0 &&
+           stream_part_bytes(m, 1) <= SQ_WS_HEADER;
 }
 
 // rows of one pass: 1, 2, 4 or 8
 int stream_pass_rows(int B) { return B > 4 ? 8 : B > 2 ? 4 : B > 1 ? 2 : 1; }
 
-size_t stream_part_bytes(const sq_matrix& m, int B) {
+size_t stream_part_bytes(const sq_matrix& m, int rows) {
     const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m));
-    return (((size_t)g.NV * stream_pass_rows(B) * g.NG * 64 * 4) + 255) & ~(size_t)255;
+    return (((size_t)g.NV * rows * g.NG * 64 * 4) + 255) & ~(size_t)255;
+}
+
+int stream_group_len(const sq_matrix* mats, int n) {
+    size_t tot = 0;
+    int k = 0;
+    for (; k < n; ++k) {
+        tot += stream_part_bytes(mats[k], 1);
+        if (tot > SQ_WS_HEADER) break;
+    }
+    return k > 0 ? k : 1;
 }
 
 // Pieces [0, cnt) (same C), B activation rows in passes of up to 8 (fewer when the parts of x and the runs' partial
-// sums of that many rows do not fit LDS beside the slice): one launch per pass.  `counters` is the zeroed head of the
-// workspace; every pass uses the same partial sums and counters (one stream).
+// sums of that many rows do not fit LDS beside the slice, or the pieces' partial sums of that many rows the workspace
+// header): one launch per pass.  `sums` is the workspace header; every pass uses it from its start (a pass leaves it zeroed).
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                        int64_t ldy, int B, char* ws, size_t& ws_off, unsigned* counters, int& counters_used,
-                        hipStream_t s, const sq_producer* from) {
+                        int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from) {
     StreamArgs a;
     a.h_in = nullptr; a.h_out = nullptr; a.add = a.up = a.w = nullptr; a.x_out = nullptr; a.eps = 0.f;
     if (from) {
@@ -1128,7 +1112,15 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     a.ldy = ldy;
     a.x_dtype = x_dtype;
     a.y_dtype = y_dtype;
+    int rows = from ? 1 : stream_pass_rows(B);
+    for (;; rows >>= 1) {
+        size_t tot = 0;
+        for (int k = 0; k < cnt; ++k) tot += stream_part_bytes(mats[k], rows);
+        if (tot <= SQ_WS_HEADER) break;
+        if (rows == 1) return fail(SQ_EUNSUPPORTED, "sq_linear_small: the partial sums of these pieces (%zu bytes) do not fit the workspace header", tot);
+    }
     int wg = 0, pc = 0, nl_max = 64;
+    size_t sums_off = 0;
     for (int k = 0; k < cnt; ++k) {
         const sq_matrix& m = mats[k];
         const int runs = stream_runs_of(m), run_max = stream_run_max_of(m);
@@ -1144,16 +1136,13 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         P.stream = (const unsigned char*)m.stream;
         P.table = m.table;
         P.row_scale = m.row_scale;
-        P.part = (float*)(ws + ws_off);
-        ws_off += stream_part_bytes(m, B);
+        P.part = (float*)(sums + sums_off);
+        sums_off += stream_part_bytes(m, rows);
         P.perms = m.perms;
         P.R = m.R; P.C = m.C; P.U = g.U; P.NS = g.NS; P.NV = g.NV; P.PC = g.PC; P.NG = g.NG; P.y_off = m.y_off;
         P.off_slots = (uint32_t)g.off_slots; P.off_runs = (uint32_t)g.off_runs; P.off_rows = (uint32_t)g.off_rows;
         P.off_steps = (uint32_t)g.off_steps;
         const int nwg = g.runs;
-        if (counters_used + nwg > SQ_WS_COUNTERS) return fail(SQ_EUNSUPPORTED, "sq_linear_small: too many row-block runs");
-        P.counters = counters + counters_used;
-        counters_used += nwg;
         P.wg_begin = wg;
         P.nwg = nwg;
         wg += g.NV * nwg;
@@ -1172,7 +1161,6 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         if (from->mode == 1) return nx4 ? stream_launch<1, 4, 1>(a, wg, s) : stream_launch<1, 1, 1>(a, wg, s);
         return nx4 ? stream_launch<1, 4, 2>(a, wg, s) : stream_launch<1, 1, 2>(a, wg, s);
     }
-    int rows = stream_pass_rows(B);
     while (rows > 1 && stream_smem(rows, a.xs, a.nl_max) > 160 * 1024) rows >>= 1;
     const size_t ysz = y_dtype == SQ_F32 ? 4 : 2;
     for (int b0 = 0; b0 < B; b0 += rows) {

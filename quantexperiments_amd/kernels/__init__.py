@@ -28,8 +28,9 @@ class _Workspace:
 
     @classmethod
     def get(cls, nbytes: int, dev, kind: str = "kernels") -> torch.Tensor:
-        """kind "kernels": the buffer handed to the library (its first 4096 bytes are the library's counters
-        and stay zero between calls); any other kind names a separate buffer the caller may overwrite.
+        """kind "kernels": the buffer handed to the library (its header, the first _lib.WS_HEADER bytes, holds the
+        partial sums of the library's decode kernel, is zero between calls and must never be written by anyone
+        else); any other kind names a separate buffer the caller may overwrite.
         A buffer that has to grow is replaced, never freed: graphs captured with the old one stay valid (the
         reference keeps a reference per launcher for the same reason, shapequant/kernels/batched_runs.py:741-743)."""
         key = (str(dev), kind)
@@ -39,7 +40,7 @@ class _Workspace:
                 raise RuntimeError("sqhip workspace must grow outside graph capture: run this shape once eagerly first")
             if b is not None:
                 cls.retired.append(b)
-            b = cls.bufs[key] = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)   # counters start at zero
+            b = cls.bufs[key] = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)   # the header starts at zero
         return b
 
 

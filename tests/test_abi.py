@@ -77,12 +77,16 @@ def test_workspace_sizes_are_host_arithmetic():
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 64, 1) == 0
     lds = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 4, 12, 1, 1, 48, 0)
     assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 160, 1) == 0          # codebook in LDS: up to 160 rows
-    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 161, 1) == 4096 + 64 * 512 * 2 + 161 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 161, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 161 * 512 * 2
     # beyond: raw fp16 codewords of the largest piece + an fp16 copy of the activations
-    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == 4096 + 64 * 512 * 2 + 100 * 512 * 2
-    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == 4096 + 64 * 512 * 2 + 2048 * 512 * 2
-    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == 4096 + 16 * 2 * 512 * 2
-    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == 4096 + 64 * 512 * 2 + 100 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 100 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 2048 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == _lib.WS_HEADER + 16 * 2 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 100 * 512 * 2
+    # a matrix with a tag stream keeps its partial sums in the header and needs nothing behind it at decode time
+    streamed = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 8, 16, 1, 1, 32, 0, 0x8000, (1 << 16) | 1, 1)
+    assert L.sq_workspace_bytes(_lib.matrix_array([streamed]), 1, 1, 0) == _lib.WS_HEADER
+    assert L.sq_workspace_bytes(_lib.matrix_array([streamed]), 1, 8, 0) == _lib.WS_HEADER
 
 
 def test_block32_entry_points_check_arguments_on_the_host():
@@ -102,16 +106,16 @@ def test_block32_entry_points_check_arguments_on_the_host():
     # more than 32 activation rows need the workspace sq_q8_workspace_bytes names
     assert L.sq_q8_linear(q, sc, 64, 64, x, bf, 64, y, bf, 64, 40, None, 0, None) == _lib.SQ_EWORKSPACE
     assert L.sq_q8_workspace_bytes(64, 64, 32) == 0
-    assert L.sq_q8_workspace_bytes(64, 64, 40) == 4096 + 64 * 64 * 2 + 40 * 64 * 2      # decoded rows + fp16 x
+    assert L.sq_q8_workspace_bytes(64, 64, 40) == _lib.WS_HEADER + 64 * 64 * 2 + 40 * 64 * 2      # decoded rows + fp16 x
     assert L.sq_q8_workspace_bytes(64, 48, 40) == 0
     # 3 .. 320 rows with C % 256 == 0: an fp16 copy of the activations
     assert L.sq_q8_workspace_bytes(64, 256, 2) == 0
-    assert L.sq_q8_workspace_bytes(64, 256, 3) == 4096 + 3 * 256 * 2
-    assert L.sq_q8_workspace_bytes(64, 1024, 4) == 4096 + 4 * 1024 * 2
-    assert L.sq_q8_workspace_bytes(64, 256, 8) == 4096 + 8 * 256 * 2
-    assert L.sq_q8_workspace_bytes(64, 256, 128) == 4096 + 128 * 256 * 2
-    assert L.sq_q8_workspace_bytes(64, 256, 320) == 4096 + 320 * 256 * 2
-    assert L.sq_q8_workspace_bytes(64, 256, 321) == 4096 + 64 * 256 * 2 + 321 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 3) == _lib.WS_HEADER + 3 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 1024, 4) == _lib.WS_HEADER + 4 * 1024 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 8) == _lib.WS_HEADER + 8 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 128) == _lib.WS_HEADER + 128 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 320) == _lib.WS_HEADER + 320 * 256 * 2
+    assert L.sq_q8_workspace_bytes(64, 256, 321) == _lib.WS_HEADER + 64 * 256 * 2 + 321 * 256 * 2
     assert L.sq_q8_linear(q, sc, 64, 256, x, bf, 256, y, bf, 64, 8, None, 0, None) == _lib.SQ_EWORKSPACE
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 64, 3, 65, None) == _lib.SQ_EINVAL                    # rows outside
     assert L.sq_q8_dequant(q, sc, 64, 64, y, f32, 32, 0, 4, None) == _lib.SQ_EINVAL                     # ld_out < C

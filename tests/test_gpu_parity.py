@@ -252,6 +252,44 @@ def test_stream_gemv_matches_oracle_and_row_path(case, dtype):
         assert rel_max_err(y2.cpu().numpy(), y32.cpu().numpy().astype(np.float64)) < 1e-5
 
 
+def test_workspace_header_is_zero_after_every_stream_launch():
+    # The header of a workspace holds the partial sums the workgroups of the tag-stream kernel exchange; a word is its
+    # own arrival flag, so every launch must leave all of them zero, whatever runs between two launches writes behind
+    # the header only, and a repeated launch must give the same bits.  Raw C ABI, a workspace of this test's own.
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    H = _lib.WS_HEADER
+    cases = [synth(260, 3584, 8, 16, seed=1), synth(300, 5120, 8, 16, 1, 16, seed=2), synth(65, 18944, 8, 16, seed=3)]
+    lins = [to_device(s) for s in cases]
+    need = max(max(L.sq_workspace_bytes(_lib.matrix_array([l.descriptor(0)]), 1, B, w) for B in (1, 2, 8, 19, 300) for w in (0, 1)) for l in lins)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    ws[H:] = 0xA5                                         # behind the header anything may lie around
+
+    def small(lin, x, B):
+        y = torch.empty(B, lin.R, dtype=torch.float32, device="cuda")
+        _lib.check(L.sq_linear_small(_lib.matrix_array([lin.descriptor(0)]), 1, x.data_ptr(), _lib.DTYPES[x.dtype], x.shape[1],
+                                     y.data_ptr(), _lib.SQ_F32, lin.R, B, ws.data_ptr(), need, _lib.stream_ptr(x.device)))
+        torch.cuda.synchronize()
+        assert not ws[:H].any(), (lin.R, lin.C, B)
+        return y
+
+    for s, lin in zip(cases, lins):
+        first = {}
+        for B in (1, 2, 3, 8):
+            x = rand_x(B, s.C, torch.bfloat16, seed=B).cuda()
+            first[B] = small(lin, x, B)
+            assert rel_max_err(first[B].cpu().numpy(), _ref(s, x.cpu())) < TOL
+        # a prefill product through the same workspace (decoded weights and activations behind the header)
+        xt = rand_x(300, s.C, torch.bfloat16, seed=9).cuda()
+        yt = torch.empty(300, s.R, dtype=torch.float32, device="cuda")
+        _lib.check(L.sq_linear_gemm(_lib.matrix_array([lin.descriptor(0)]), 1, xt.data_ptr(), _lib.SQ_BF16, s.C, yt.data_ptr(),
+                                    _lib.SQ_F32, s.R, 300, ws.data_ptr(), need, _lib.stream_ptr(xt.device)))
+        torch.cuda.synchronize()
+        assert not ws[:H].any()
+        for B in (8, 1):
+            assert torch.equal(small(lin, rand_x(B, s.C, torch.bfloat16, seed=B).cuda(), B), first[B])
+
+
 def test_stream_padding_never_touches_the_codebook():
     # codeword 0 of every slice is inf and no tag names it: padded stream entries (tag 0) must not leak into a sum
     from quantexperiments_amd.kernels import linear_small
@@ -357,7 +395,7 @@ def test_gemm_dense_with_workspace_splits_the_last_round():
     from quantexperiments_amd.kernels import gemm_dense
     g = torch.Generator().manual_seed(6)
     R, C, T = 2048, 4096, 250
-    assert _lib.lib().sq_gemm_dense_workspace_bytes(R, C, T) == 4096 + 8 * 4 * 256 * 256 * 4
+    assert _lib.lib().sq_gemm_dense_workspace_bytes(R, C, T) == _lib.WS_HEADER + 8 * 4 * 256 * 256 * 4
     assert _lib.lib().sq_gemm_dense_workspace_bytes(R, C, 32) == 0 and _lib.lib().sq_gemm_dense_workspace_bytes(R, 4000, T) == 0
     w = (torch.randn(R, C, generator=g) * 0.05).half().cuda()
     x = torch.randn(T, C, generator=g).half().cuda()
@@ -424,7 +462,7 @@ def test_gemm_of_neighbouring_and_scattered_pieces():
             assert rel_max_err(y[:, o:o + s.R].cpu().numpy(), ref) < TOL
             covered[o:o + s.R] = True
         assert (y[:, ~covered.cuda()] == 3.0).all()
-        assert not ws[:4096].any()                      # the counter header is left at zero
+        assert not ws[:_lib.WS_HEADER].any()            # the header is left at zero
 
 
 # ------------------------------------------------------------------ the layer object and the op
@@ -561,7 +599,7 @@ def test_launcher_refuses_stream_counts_the_builder_did_not_make():
     runs, run_max = lin.stream_runs & 0xFFFF, lin.stream_runs >> 16
     x = torch.zeros(1, 512, dtype=torch.bfloat16, device="cuda")
     y = torch.zeros(1, 700, dtype=torch.bfloat16, device="cuda")
-    ws = torch.zeros(1 << 22, dtype=torch.uint8, device="cuda")
+    ws = torch.zeros(_lib.WS_HEADER + (1 << 20), dtype=torch.uint8, device="cuda")
 
     def call(stream_runs, groups):
         m = lin.descriptor(0)
