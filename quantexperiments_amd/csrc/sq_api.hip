@@ -184,7 +184,7 @@ int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_produce
     void* ws = has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr;
     const size_t wsb = has_ws ? ws_bytes - SQ_WS_HEADER : 0;
     const bool aligned = (((uintptr_t)from->h_in | (uintptr_t)from->h_out | (uintptr_t)from->add | (uintptr_t)from->up | (uintptr_t)from->w) & 15) == 0;
-    if (aligned && small_fuses_producer(mats, n_mats, B))
+    if (addnorm && aligned && small_fuses_producer(mats, n_mats, B))
         return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, has_ws ? workspace : nullptr, s, from);
     rc = addnorm ? launch_addnorm(from->h_in, from->h_out, from->ld_h, from->add, x_dtype, from->ld_in, from->w, x_dtype, nullptr, 1, B,
                                   C, from->eps, from->x_out, x_dtype, s)

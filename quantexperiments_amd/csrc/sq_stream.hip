@@ -446,29 +446,29 @@ struct StreamArgs {
     int xs;                           // LDS bytes of one activation row's part of x (its chunks + 16 zero chunks)
     int nl_max;                       // places of the longest run (64 per group): floats per row of the LDS partial sums
     int x_dtype, y_dtype;
-    // Producer of the activation row (stream_kernel<1, NW, PRO> with PRO != 0 only): the row is computed while it is
-    // staged instead of being read from x.  PRO 1: round(v * rsqrt(mean(v^2) + eps) * w) with v = h_in + add;
-    // PRO 2: silu(add) * up.  add / up / w / x_out hold x_dtype; x_out (and h_out) are written once per launch.
+    // Producer of the activation row (stream_kernel<1, NX, 1> only): the row is computed while it is staged instead
+    // of being read from x: round(v * rsqrt(mean(v^2) + eps) * w) with v = h_in + add.  add / w / x_out hold x_dtype;
+    // x_out (and h_out) are written once per launch.  (SiLU(gate) * up is not produced this way: every workgroup
+    // would evaluate the whole row's exponentials, several microseconds against a stand-alone launch of under four.)
     const float* h_in;
     float* h_out;
     const uint16_t* add;
-    const uint16_t* up;
     const uint16_t* w;
     uint16_t* x_out;
     float eps;
 };
 
 // The operands of one chunk (8 elements) of the produced row, fetched first and finished once the row's scale is known.
-// PRO 1: h, lo = add, hi = w.  PRO 2: lo = gate, hi = up.
+// h, lo = add, hi = w.
 struct ProRaw { float h[8]; uint32_t lo[4], hi[4]; };
 
 // chunk ci in natural order: 16-byte loads (every pointer 16-byte aligned)
 template <int PRO>
 __device__ __forceinline__ ProRaw pro_fetch(const StreamArgs& a, int ci) {
     ProRaw r;
-    const u32x4 hi = reinterpret_cast<const u32x4*>(PRO == 1 ? a.w : a.up)[ci];
+    const u32x4 hi = reinterpret_cast<const u32x4*>(a.w)[ci];
     u32x4 lo = u32x4{0u, 0u, 0u, 0u};
-    if (PRO == 2 || a.add) lo = reinterpret_cast<const u32x4*>(a.add)[ci];
+    if (a.add) lo = reinterpret_cast<const u32x4*>(a.add)[ci];
 #pragma unroll
     for (int k = 0; k < 4; ++k) { r.lo[k] = lo[k]; r.hi[k] = hi[k]; }
     if (PRO == 1) {
@@ -482,12 +482,12 @@ __device__ __forceinline__ ProRaw pro_fetch(const StreamArgs& a, int ci) {
 template <int PRO>
 __device__ __forceinline__ ProRaw pro_gather(const StreamArgs& a, const int32_t* idx) {
     ProRaw r;
-    const uint16_t* hp = PRO == 1 ? a.w : a.up;
+    const uint16_t* hp = a.w;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int i0 = idx[2 * k], i1 = idx[2 * k + 1];
         r.hi[k] = (uint32_t)hp[i0] | ((uint32_t)hp[i1] << 16);
-        r.lo[k] = (PRO == 2 || a.add) ? ((uint32_t)a.add[i0] | ((uint32_t)a.add[i1] << 16)) : 0u;
+        r.lo[k] = a.add ? ((uint32_t)a.add[i0] | ((uint32_t)a.add[i1] << 16)) : 0u;
         if (PRO == 1) { r.h[2 * k] = a.h_in[i0]; r.h[2 * k + 1] = a.h_in[i1]; }
     }
     return r;
@@ -505,10 +505,7 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
     uint32_t e[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-        if (PRO == 2)
-            e[k] = silu_mul_one((uint16_t)(r.lo[k >> 1] >> (16 * (k & 1))), (uint16_t)(r.hi[k >> 1] >> (16 * (k & 1))), a.x_dtype);
-        else
-            e[k] = round16(pro_v(a, r, k) * rstd * pro_f(r.hi[k >> 1], k, a.x_dtype), a.x_dtype);
+        e[k] = round16(pro_v(a, r, k) * rstd * pro_f(r.hi[k >> 1], k, a.x_dtype), a.x_dtype);
     }
     return u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
 }
@@ -545,7 +542,7 @@ typedef __attribute__((address_space(3))) void* stream_lptr_t;
 // [16 block sums (PRO 1)].
 template <int NB, int NX, int PRO = 0>
 __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
-    static_assert(PRO == 0 || NB == 1, "produced activations: one row");
+    static_assert(PRO == 0 || (PRO == 1 && NB == 1), "produced activations: add + norm, one row");
     constexpr int NW = STREAM_NW, NTH = NW * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1102,9 +1099,9 @@ int stream_group_len(const sq_matrix* mats, int n) {
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                         int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from) {
     StreamArgs a;
-    a.h_in = nullptr; a.h_out = nullptr; a.add = a.up = a.w = nullptr; a.x_out = nullptr; a.eps = 0.f;
+    a.h_in = nullptr; a.h_out = nullptr; a.add = a.w = nullptr; a.x_out = nullptr; a.eps = 0.f;
     if (from) {
-        a.h_in = from->h_in; a.h_out = from->h_out; a.add = (const uint16_t*)from->add; a.up = (const uint16_t*)from->up;
+        a.h_in = from->h_in; a.h_out = from->h_out; a.add = (const uint16_t*)from->add;
         a.w = (const uint16_t*)from->w; a.x_out = (uint16_t*)from->x_out; a.eps = from->eps;
     }
     a.n = cnt;
@@ -1158,8 +1155,8 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     if (from) {
         if (B != 1) return fail(SQ_EINVAL, "sq_linear_small_from: fused producers take one activation row");
         a.x = (const uint16_t*)x; a.y = y; a.nb = 1;
-        if (from->mode == 1) return nx4 ? stream_launch<1, 4, 1>(a, wg, s) : stream_launch<1, 1, 1>(a, wg, s);
-        return nx4 ? stream_launch<1, 4, 2>(a, wg, s) : stream_launch<1, 1, 2>(a, wg, s);
+        if (from->mode != SQ_FROM_ADDNORM) return fail(SQ_EINVAL, "sq_linear_small_from: only add + norm is produced inside the kernel");
+        return nx4 ? stream_launch<1, 4, 1>(a, wg, s) : stream_launch<1, 1, 1>(a, wg, s);
     }
     while (rows > 1 && stream_smem(rows, a.xs, a.nl_max) > 160 * 1024) rows >>= 1;
     const size_t ysz = y_dtype == SQ_F32 ? 4 : 2;
