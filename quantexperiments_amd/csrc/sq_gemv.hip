@@ -116,13 +116,15 @@ static Plan plan_for(int U, int bits, int d) {
 
 // The tag-stream kernel multiplies up to 8 activation rows per pass (every codeword gathered once, one x gather
 // per row).  With column orders (where the alternative is the VALU kernel) it is used for any B <= 32.  Without,
-// it wins over the matrix-core kernel's single L2 gather per tag for up to 4 rows of a large matrix (measured on
-// the two 18944 x 3584 pieces: 49 / 73 / 119 us at B = 2 / 4 / 8 against 85 us; on one 3584 x 3584: 21 / 26 us
-// against 14 us).
+// it wins over the matrix-core kernel's single L2 gather per tag up to 4 rows on every shape, and up to 8 rows
+// when a row's part of x is short enough for several rows per pass.  Measured on the 7B layer (microseconds,
+// stream / matrix-core kernel): q|k|v 13.8 / 26.7 at 2 rows, 14.5 / 27.1 at 4, 18.6 / 26.8 at 8; o 12.5 / 15.0, 13.7 /
+// 14.9, 17.6 / 15.4; gate|up 24.7 / (85 at any row count), 33.5, 62.8; down (rows of 2368 chunks) 18.3, 33.4 / (52 at
+// any row count), 63.2.
 static bool stream_rows(const sq_matrix& m, int B) {
     if (!stream_shape(m)) return false;
     if (!m.tags) return true;                                    // one-copy residency: the stream is all there is
-    return B == 1 || m.perms != nullptr || (B <= 4 && (int64_t)m.R * m.C >= (int64_t)32 << 20);
+    return B <= 4 || m.perms != nullptr || (B <= 8 && m.C / m.d <= 1024);
 }
 
 // ---- matrix-core path (pieces without column orders)

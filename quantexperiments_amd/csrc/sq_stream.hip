@@ -514,7 +514,7 @@ constexpr int STREAM_TAB = 65536;     // the codebook slice
 constexpr int STREAM_PF = 3;          // steps fetched ahead (2 to 4 measure alike, 6 and 8 slower: the loop runs at the memory system's rate)
 constexpr int STREAM_NW = 16;         // waves per workgroup: one workgroup per CU
 constexpr uint32_t STREAM_ZERO_SUM = 0x7FFFFFFFu;  // how a partial sum with all bits zero is written (zero = not there yet)
-constexpr int STREAM_SPIN_MAX = 1 << 20;           // polls of an item's partial sums before it gives up
+constexpr int STREAM_SPIN_MAX = 1 << 18;           // polls of an item's partial sums before it gives up
 
 // LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group)
 static inline int stream_xs(int pc) { return (pc + 16) * 16; }
