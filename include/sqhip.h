@@ -66,7 +66,8 @@ int sq_dequant(const sq_matrix* m, void* out, int out_dtype, int64_t ld_out, int
  * (elements).  x_dtype / y_dtype: SQ_F16 or SQ_BF16 (y may also be SQ_F32).
  * Replaces proto_runs.gemv (reference shapequant/kernels/proto_runs.py:505-571), cuda_gemv.gemv
  * (cuda_gemv.py:148-172), PackedLinear.gemv (gemv.py:142-156) and RunsBatch.run
- * (batched_runs.py:745-771).  Pieces with M > 1 need workspace (see sq_workspace_bytes); from 11 activation
+ * (batched_runs.py:745-771).  Pieces with M > 1 and pieces with a slice stream need a workspace (see
+ * sq_workspace_bytes; the latter keep their partial sums in its header); from 11 activation
  * rows on, a stack that has column orders (and C % 64 == 0, 16-byte aligned x, ldx % 8 == 0) is decoded to
  * fp16 in the workspace and multiplied by the tile GEMM, which is faster than its decode-time kernel there. */
 #define SQ_SMALL_BMAX 32
@@ -129,8 +130,8 @@ size_t sq_gemm_dense_workspace_bytes(int32_t R, int32_t C, int32_t T);
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which);
 
 /* Load-time regrouping of a matrix' tags for codebooks that do not fit LDS (d = 8, K = 8192..65,536, one
- * codebook): the decode-time product (batch 1, up to 4 rows of large matrices, any B <= 32 with column
- * orders) then gathers codewords from a 64 KB LDS slice instead of from L2.
+ * codebook): the decode-time product (up to 4 activation rows, up to 8 of rows with at most 1024 chunks, any
+ * B <= 32 with column orders) then gathers codewords from a 64 KB LDS slice instead of from L2.
  * HOST pointers: `tags_host` is the file's tag tensor in host memory, `row_mask_host` the file's row_mask
  * (NULL when the matrix has one column order), `out_host` receives sq_stream_bytes() bytes that the caller
  * copies to the device (16-byte aligned) and names in sq_matrix.stream, together with *runs_out and
