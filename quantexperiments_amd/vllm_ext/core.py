@@ -62,13 +62,13 @@ def neutral_defaults():
     """torch's stock defaults (CPU device, float32) while the layer's tensors are built: vLLM
     constructs models under a GPU default device and a bf16 default dtype
     (reference shapequant/vllm_ext/core.py:145-156)."""
-    dt = torch.get_default_dtype()
-    torch.set_default_dtype(torch.float32)
+    saved = torch.get_default_dtype()
     try:
+        torch.set_default_dtype(torch.float32)
         with torch.device("cpu"):
             yield
     finally:
-        torch.set_default_dtype(dt)
+        torch.set_default_dtype(saved)
 
 
 _TUNED: dict = {}
@@ -240,22 +240,20 @@ class Q8Head:
 
     def __init__(self, q: torch.Tensor, sc: torch.Tensor, R: int | None = None, small_max: int = 32,
                  chunk_rows: int = 8192, tiled: bool | None = None, keep: torch.Tensor | None = None):
-        self.V, self.C = q.shape
-        self.keep = None
-        if keep is not None:
-            if keep.shape != (self.V,) or R is None or int(keep.max()) >= R:
-                raise ValueError(f"q8 head: keep {tuple(keep.shape)} for {self.V} rows, R {R}")
-            self.keep = keep.to(device=q.device, dtype=torch.int64).contiguous()
-        if self.C % 32 or sc.shape != (self.V, self.C // 32):
+        if q.dim() != 2 or q.shape[1] % 32 or tuple(sc.shape) != (q.shape[0], q.shape[1] // 32):
             raise ValueError(f"q8 head: q {tuple(q.shape)}, scale {tuple(sc.shape)}")
         if q.device.type != "cuda":
             raise ValueError("Q8Head holds device tensors: pass cuda tensors")
-        self.R = self.V if R is None else R
+        self.V, self.C = int(q.shape[0]), int(q.shape[1])
+        self.R = self.V if R is None else int(R)
         if self.R < self.V:
             raise ValueError(f"q8 head has {self.V} rows, layer wants {self.R}")
-        self.small_max = min(small_max, BMAX)
-        self.tiled = False
-        self.chunk_rows = chunk_rows
+        self.keep = None
+        if keep is not None:                                # a pruned head: row i of q is token id keep[i] of an R-row head
+            if R is None or tuple(keep.shape) != (self.V,) or int(keep.max()) >= self.R:
+                raise ValueError(f"q8 head: keep {tuple(keep.shape)} for {self.V} rows, R {R}")
+            self.keep = keep.to(device=q.device, dtype=torch.int64).contiguous()
+        self.small_max, self.chunk_rows, self.tiled = min(small_max, BMAX), chunk_rows, False
         self.q, self.sc = q.contiguous(), sc.contiguous()
 
     def nbytes(self) -> int:
