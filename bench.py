@@ -66,16 +66,31 @@ def launch_bytes(shapes, names, d, bits, G=1, M=1, B=1):
     return n + B * C * 2
 
 
-def make_layer(torch, dev, gen, shapes, d, bits, G=1, M=1):
+def skewed_tags(torch, gen, R, n, bits, how):
+    """Tags whose codeword popularity follows a Zipf law (weight 1 / rank): "zipf" scatters the popular codewords over
+    the whole codebook (what k-means labels look like), "zipf-sorted" makes codeword 0 the most popular one, so the
+    first slice of 4096 codewords holds most of the tags (the worst case for a slice stream)."""
+    K = 1 << bits
+    w = 1.0 / torch.arange(1, K + 1, dtype=torch.float64)
+    cdf = torch.cumsum(w / w.sum(), 0)
+    rank = torch.searchsorted(cdf, torch.rand(R, n, generator=gen, dtype=torch.float64)).clamp_(max=K - 1)
+    return rank if how == "zipf-sorted" else torch.randperm(K, generator=gen)[rank]
+
+
+def make_layer(torch, dev, gen, shapes, d, bits, G=1, M=1, tags="uniform"):
     """One layer of PackedLinear pieces with synthetic contents drawn from the CPU generator `gen` (per matrix: tags,
     table, row scales, codebook ids, row orders); the pieces of each launch get their load-time tag streams cut for
     that launch (as PackedShards does at load)."""
     from quantexperiments_amd.kernels import PackedLinear, prepare_stack
     from quantexperiments_amd.masks import seeded_perms
+    from quantexperiments_amd.packed import pack_bits
     out = {}
     for i, (nm, (R, C)) in enumerate(shapes.items()):
         W = (C // d) * bits // 32
-        words = torch.randint(-2 ** 31, 2 ** 31, (R, W), dtype=torch.int64, generator=gen).to(torch.int32)
+        if tags == "uniform":
+            words = torch.randint(-2 ** 31, 2 ** 31, (R, W), dtype=torch.int64, generator=gen).to(torch.int32)
+        else:
+            words = pack_bits(skewed_tags(torch, gen, R, C // d, bits, tags), bits)
         table = torch.randn(G << bits, d, generator=gen).to(torch.float16)
         rs = (torch.randn(R, generator=gen) * 0.005 + 0.02).abs().to(torch.float16)
         rb = torch.randint(0, G, (R,), generator=gen).to(torch.uint8) if G > 1 else None
@@ -299,7 +314,7 @@ def resident_bytes(layer):
     return {**kinds, "total": total, "bits_per_weight": 8.0 * total / weights}
 
 
-def sweep(torch, dev, spec: str, rows: str, n_layers: int):
+def sweep(torch, dev, spec: str, rows: str, n_layers: int, tags: str = "uniform"):
     """Other formats and shapes than the headline's, one layer (4 launches) per activation-row count:
     spec = "<7b|27b>,d,bits,G,M", e.g. "7b,4,12,1,1" (cfg3), "27b,8,16,1,16" (cfg5), "27b,4,12,4,1" (the shipped 27B
     format).  Up to 32 rows through sq_linear_small, above through sq_linear_gemm; n_layers distinct layers rotated
@@ -309,14 +324,14 @@ def sweep(torch, dev, spec: str, rows: str, n_layers: int):
     d, bits, G, M = int(d), int(bits), int(G), int(M)
     shapes = SHAPES_7B if model == "7b" else SHAPES_27B
     gen = torch.Generator().manual_seed(0)
-    layers = [make_layer(torch, dev, gen, shapes, d, bits, G, M) for _ in range(n_layers)]
+    layers = [make_layer(torch, dev, gen, shapes, d, bits, G, M, tags) for _ in range(n_layers)]
     nbytes = sum(launch_bytes(shapes, l, d, bits, G, M) for l in LAUNCHES)
     res = {}
     for B in [int(b) for b in rows.split(",")]:
         tot, per = layer_times(torch, dev, layers, shapes, B, linear_small if B <= 32 else linear_gemm, gen)
         res[f"B{B}"] = {"us_per_layer": tot, "GBps_packed": nbytes / tot / 1e3,
                         "tflops": 2.0 * B * sum(R * C for R, C in shapes.values()) / tot / 1e6, "per_launch_us": per}
-    return {"sweep": spec, "layers_rotated": n_layers, "rows": res, "resident": resident_bytes(layers[0])}
+    return {"sweep": spec, "tags": tags, "layers_rotated": n_layers, "rows": res, "resident": resident_bytes(layers[0])}
 
 
 def main():
@@ -340,6 +355,8 @@ def main():
                     help="time one layer of another format / shape set instead of the headline workload and print only "
                          "that object, e.g. 7b,4,12,1,1 (cfg3), 27b,8,16,1,16 (cfg5); see --rows")
     ap.add_argument("--rows", default="1", help="activation-row counts for --sweep, comma separated")
+    ap.add_argument("--tags", default="uniform", choices=("uniform", "zipf", "zipf-sorted"),
+                    help="tag distribution of --sweep: uniform, or Zipf codeword popularity scattered over / sorted into the codebook")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic to scale rocprofv3 counters by)")
     args = ap.parse_args()
@@ -356,7 +373,7 @@ def main():
         print(json.dumps({"lm_head": lm_head(torch, dev)}))
         return
     if args.sweep:
-        print(json.dumps(sweep(torch, dev, args.sweep, args.rows, min(args.layers, 4 if args.sweep.startswith("27b") else 16))))
+        print(json.dumps(sweep(torch, dev, args.sweep, args.rows, min(args.layers, 4 if args.sweep.startswith("27b") else 16), args.tags)))
         return
     D, BITS = 8, 16
     gen = torch.Generator().manual_seed(0)

@@ -161,6 +161,21 @@ int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, i
                     const uint8_t* row_mask_host, int32_t runs, void* out_host, size_t out_bytes,
                     int32_t* runs_out, int32_t* groups_out);
 
+/* The same with the matrix' codebook at hand (`table_host`: fp16 [2^bits, d] in host memory; NULL = the two calls
+ * above).  A workgroup of the decode-time kernel gathers from one slice of 4096 codewords, so its work is the number of
+ * tags that point into its slice: tags that favour some codewords (a codebook whose first entries are its most used
+ * ones, a few very common shapes) would leave most workgroups waiting for a few.  With the codebook the builder
+ * relabels the codewords (most used first, each to the slice that carries the fewest tags so far), writes the
+ * relabelled codebook into the buffer and the kernels read their slices from there, so every slice carries the same
+ * share of the tags whatever their distribution; results are the same bits.  The buffer grows by the codebook and a
+ * 2-byte back map per codeword (1.1 MiB at K = 65,536).  Formats the slice stream does not cover ignore `table_host`.
+ * No counterpart in the reference, whose kernels gather from the whole codebook. */
+size_t sq_stream_bytes_balanced(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                                const uint8_t* row_mask_host, int32_t runs, const void* table_host);
+int sq_stream_build_balanced(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                             const uint8_t* row_mask_host, int32_t runs, const void* table_host, void* out_host,
+                             size_t out_bytes, int32_t* runs_out, int32_t* groups_out);
+
 /* ---- The packed file's block-32 side formats (reference shapequant/packed.py:30-40): the 8-bit output head
  * `aux.lm_head` (q int8 [V, C], scale fp16 [V, C/32], w = q * scale of the row's 32-column block) and the 4-bit
  * embedding `aux.embed` (q uint8 [V, C/2] with column 2k in the low and 2k+1 in the high nibble of byte k, each

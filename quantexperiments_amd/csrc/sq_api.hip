@@ -244,16 +244,16 @@ size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, i
     return (inner || small_uses_sums(mats, n_mats)) ? inner + SQ_WS_HEADER : 0;
 }
 
-size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
-                       const uint8_t* row_mask_host, int32_t runs) {
+size_t sq_stream_bytes_balanced(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                                const uint8_t* row_mask_host, int32_t runs, const void* table_host) {
     if (!tags_host || d <= 0 || (int64_t)W * 32 < (int64_t)(C / d) * bits) return 0;
     if (!stream_format_ok(R, C, d, bits)) return !row_mask_host && tiled_format_ok(R, W, C, d, bits) ? tiled_bytes(R, W) : 0;
-    return stream_bytes_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs);
+    return stream_bytes_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs, (const uint16_t*)table_host);
 }
 
-int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
-                    const uint8_t* row_mask_host, int32_t runs, void* out_host, size_t out_bytes, int32_t* runs_out,
-                    int32_t* groups_out) {
+int sq_stream_build_balanced(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                             const uint8_t* row_mask_host, int32_t runs, const void* table_host, void* out_host, size_t out_bytes,
+                             int32_t* runs_out, int32_t* groups_out) {
     if (!tags_host || !out_host || !runs_out || !groups_out) return fail(SQ_EINVAL, "sq_stream_build: null pointer");
     if (d > 0 && !stream_format_ok(R, C, d, bits) && !row_mask_host && tiled_format_ok(R, W, C, d, bits)) {
         if (out_bytes < tiled_bytes(R, W)) return fail(SQ_EINVAL, "sq_stream_build: out_bytes %zu < %zu", out_bytes, tiled_bytes(R, W));
@@ -265,7 +265,18 @@ int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, i
     if (d <= 0 || !stream_format_ok(R, C, d, bits)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: d %d bits %d R %d not covered", d, bits, R);
     if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_stream_build: W %d too small", W);
     return stream_build_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs, (unsigned char*)out_host,
-                             out_bytes, runs_out, groups_out);
+                             out_bytes, runs_out, groups_out, (const uint16_t*)table_host);
+}
+
+size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                       const uint8_t* row_mask_host, int32_t runs) {
+    return sq_stream_bytes_balanced(tags_host, R, W, C, d, bits, row_mask_host, runs, nullptr);
+}
+
+int sq_stream_build(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                    const uint8_t* row_mask_host, int32_t runs, void* out_host, size_t out_bytes, int32_t* runs_out,
+                    int32_t* groups_out) {
+    return sq_stream_build_balanced(tags_host, R, W, C, d, bits, row_mask_host, runs, nullptr, out_host, out_bytes, runs_out, groups_out);
 }
 
 static int check_q8(const char* who, const void* q, const void* scale, int32_t V, int32_t C) {

@@ -19,17 +19,28 @@ struct StreamGeom {
     int U, NS, KP, PC, NV, NG;               // chunks per row, slices, column parts, chunks per part, buckets, groups
     int runs;
     size_t off_slots, off_runs, off_rows, off_steps;   // byte offsets inside the stream buffer
+    size_t off_table, off_unmap;             // balanced streams: the relabelled codebook and uint16 new id -> file id (else 0)
     uint64_t total_steps;                    // filled by the builder only
 };
 
-StreamGeom stream_geom(int C, int d, int bits, int groups, int runs);
+StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced = false);
 bool stream_format_ok(int R, int C, int d, int bits);
-size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs);
+// table: the matrix' codebook (fp16 [2^bits, d], host memory) or NULL.  With it the codewords are relabelled so that
+// every slice of 4096 carries the same share of the tags whatever their distribution, and the buffer holds the
+// relabelled copy of the codebook that the kernels then read their slices from.
+size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
+                         const uint16_t* table = nullptr);
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out);
-// sq_matrix.stream_runs is sq_stream_build's runs_out: the run count in the low 16 bits, the groups of the longest run above
+                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table = nullptr);
+// sq_matrix.stream_runs is sq_stream_build's runs_out: the run count in the low 16 bits, the groups of the longest run
+// in the next 8, bit 30 = the stream carries a relabelled codebook
+constexpr int STREAM_BALANCED = 1 << 30;
 inline int stream_runs_of(const sq_matrix& m) { return m.stream_runs & 0xFFFF; }
-inline int stream_run_max_of(const sq_matrix& m) { return (int)((uint32_t)m.stream_runs >> 16); }
+inline int stream_run_max_of(const sq_matrix& m) { return (int)(((uint32_t)m.stream_runs >> 16) & 0xFFu); }
+inline bool stream_balanced_of(const sq_matrix& m) { return (m.stream_runs & STREAM_BALANCED) != 0; }
+inline StreamGeom stream_geom_of(const sq_matrix& m) {
+    return stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m), stream_balanced_of(m));
+}
 bool stream_shape(const sq_matrix& m);
 size_t stream_part_bytes(const sq_matrix& m, int rows);   // partial sums of one pass of `rows` activation rows
 // dense rows [r0, r1) of a matrix that is held as its tag stream only (sq_matrix.tags == NULL)

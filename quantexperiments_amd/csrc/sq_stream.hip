@@ -40,7 +40,7 @@ constexpr int STREAM_CLIMB = 1;      // hill-climbing passes of the entry orderi
 
 namespace sq {
 
-StreamGeom stream_geom(int C, int d, int bits, int groups, int runs) {
+StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced) {
     StreamGeom g;
     g.U = C / d;
     g.NS = 1 << (bits - STREAM_SLICE_BITS);
@@ -52,7 +52,14 @@ StreamGeom stream_geom(int C, int d, int bits, int groups, int runs) {
     g.off_slots = (((size_t)g.NV * g.NG + 1) * 4 + 255) & ~(size_t)255;
     g.off_runs = (g.off_slots + (size_t)g.NV * g.NG * 64 * 4 + 255) & ~(size_t)255;
     g.off_rows = (g.off_runs + (size_t)runs * 16 + 255) & ~(size_t)255;
-    g.off_steps = (g.off_rows + (size_t)g.NG * 64 * 4 + 255) & ~(size_t)255;
+    size_t end = (g.off_rows + (size_t)g.NG * 64 * 4 + 255) & ~(size_t)255;
+    g.off_table = g.off_unmap = 0;
+    if (balanced) {
+        g.off_table = end;
+        g.off_unmap = end + ((size_t)d * 2 << bits);
+        end = (g.off_unmap + ((size_t)2 << bits) + 255) & ~(size_t)255;
+    }
+    g.off_steps = end;
     g.total_steps = 0;
     return g;
 }
@@ -95,10 +102,41 @@ struct StreamPlan {
     std::vector<uint16_t> cnt;       // [NV][R]
     std::vector<uint32_t> pos;       // [NV][R]: lane position (group * 64 + lane) of row r in bucket v
     std::vector<uint32_t> goff;      // [NV * NG + 1]
+    std::vector<uint16_t> remap;     // balanced streams: file id -> new id (empty: identity)
 };
 
+// Relabelling of the codewords for a stream with a codebook of its own: the codewords are dealt, most used first, to
+// whichever slice of 4096 carries the fewest tags so far and still has room, so every slice ends up with the same
+// share of the tags (a slice is one workgroup's work) whatever the distribution of the tags is, and a slice's popular
+// codewords get consecutive places, i.e. different LDS bank groups.
+static void balance_codewords(const uint32_t* tags, int R, int W, int U, int bits, std::vector<uint16_t>& remap) {
+    const int K = 1 << bits, NS = K >> STREAM_SLICE_BITS, SL = 1 << STREAM_SLICE_BITS;
+    std::vector<uint64_t> count(K, 0);
+    for (int r = 0; r < R; ++r) {
+        const uint32_t* row = tags + (size_t)r * W;
+        for (int j = 0; j < U; ++j) ++count[host_tag(row, W, bits, j)];
+    }
+    std::vector<uint32_t> ids(K);
+    for (int k = 0; k < K; ++k) ids[k] = (uint32_t)k;
+    std::stable_sort(ids.begin(), ids.end(), [&count](uint32_t a, uint32_t b) { return count[a] > count[b]; });
+    std::vector<uint64_t> load(NS, 0);
+    std::vector<int> fill(NS, 0);
+    remap.assign(K, 0);
+    for (int k = 0; k < K; ++k) {
+        int best = -1;
+        for (int sl = 0; sl < NS; ++sl)
+            if (fill[sl] < SL && (best < 0 || load[sl] < load[best])) best = sl;
+        remap[ids[k]] = (uint16_t)(best * SL + fill[best]);
+        ++fill[best];
+        load[best] += count[ids[k]];
+    }
+}
+
 static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                        StreamPlan& P) {
+                        StreamPlan& P, bool balanced) {
+    P.remap.clear();
+    if (balanced) balance_codewords(tags, R, W, C / d, bits, P.remap);
+    const uint16_t* remap = balanced ? P.remap.data() : nullptr;
     // rows by column order, groups and runs
     std::vector<uint32_t> order(R);
     for (int r = 0; r < R; ++r) order[r] = (uint32_t)r;
@@ -148,7 +186,7 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
             P.GR = std::max(P.GR, std::min(GR, ngm[i] - q));
         }
     }
-    P.g = stream_geom(C, d, bits, (int)(P.base.size() / 64), (int)P.runs.size());
+    P.g = stream_geom(C, d, bits, (int)(P.base.size() / 64), (int)P.runs.size(), balanced);
     const StreamGeom& g = P.g;
     P.cnt.assign((size_t)g.NV * R, 0);
     P.pos.assign((size_t)g.NV * R, 0);
@@ -157,7 +195,8 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
         for (int r = a; r < b; ++r) {
             const uint32_t* row = tags + (size_t)r * W;
             for (int j = 0; j < g.U; ++j) {
-                const uint32_t t = host_tag(row, W, bits, j);
+                uint32_t t = host_tag(row, W, bits, j);
+                if (remap) t = remap[t];
                 const int v = (j / g.PC) * g.NS + (int)(t >> STREAM_SLICE_BITS);
                 ++P.cnt[(size_t)v * R + r];
             }
@@ -185,9 +224,10 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     P.g.total_steps = tot;
 }
 
-size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs) {
+size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
+                         const uint16_t* table) {
     StreamPlan P;
-    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P);
+    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr);
     return P.g.off_steps + (size_t)P.g.total_steps * 768;
 }
 
@@ -351,9 +391,10 @@ struct BankMatch {
 };
 
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out) {
+                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table) {
     StreamPlan P;
-    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P);
+    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr);
+    const uint16_t* remap = table ? P.remap.data() : nullptr;
     const StreamGeom& g = P.g;
     const size_t need = g.off_steps + (size_t)g.total_steps * 768;
     if (g.total_steps >= ((uint64_t)1 << 32) || g.runs >= (1 << 16)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: matrix too large");
@@ -362,6 +403,14 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
     memcpy(out, P.goff.data(), P.goff.size() * 4);
     memcpy(out + g.off_runs, P.runs.data(), P.runs.size() * sizeof(StreamRun));
     memcpy(out + g.off_rows, P.base.data(), P.base.size() * 4);
+    if (table) {
+        uint16_t* tab = (uint16_t*)(out + g.off_table);
+        uint16_t* unmap = (uint16_t*)(out + g.off_unmap);
+        for (int k = 0; k < (1 << bits); ++k) {
+            memcpy(tab + (size_t)remap[k] * d, table + (size_t)k * d, (size_t)d * 2);
+            unmap[remap[k]] = (uint16_t)k;
+        }
+    }
     std::vector<uint32_t> place(R);
     for (size_t k = 0; k < P.base.size(); ++k)
         if (P.base[k] != STREAM_NO_ROW) place[P.base[k]] = (uint32_t)k;
@@ -379,7 +428,8 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
                 slots[(size_t)v * g.NG * 64 + k] = place[r] | ((uint32_t)P.cnt[(size_t)v * R + r] << STREAM_ROW_BITS);
             }
             for (int j = 0; j < g.U; ++j) {
-                const uint32_t t = host_tag(row, W, bits, j);
+                uint32_t t = host_tag(row, W, bits, j);
+                if (remap) t = remap[t];
                 const int kp = j / g.PC, v = kp * g.NS + (int)(t >> STREAM_SLICE_BITS);
                 const uint32_t k = P.pos[(size_t)v * R + r], n = q[v]++;
                 const uint32_t e = (t & ((1u << STREAM_SLICE_BITS) - 1u)) | ((uint32_t)(j - kp * g.PC) << STREAM_SLICE_BITS);
@@ -418,7 +468,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             for (int q = 0; q < 4; ++q) bm.order_lanes(base, sl, LDS_CLOCK_LANES[q], ns, (uint32_t)g.PC);
         }
     });
-    if (runs_out) *runs_out = g.runs | (P.GR << 16);
+    if (runs_out) *runs_out = g.runs | (P.GR << 16) | (table ? STREAM_BALANCED : 0);
     if (groups_out) *groups_out = g.NG;
     return SQ_OK;
 }
@@ -1051,9 +1101,10 @@ __global__ __launch_bounds__(256) void stream_dequant_kernel(StreamDeqArgs a) {
 
 int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s, bool raw) {
     if (!stream_shape(m)) return fail(SQ_EINVAL, "sq_dequant: a matrix without tags needs its tag stream");
-    const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m));
+    const StreamGeom g = stream_geom_of(m);
     StreamDeqArgs a;
-    a.stream = (const unsigned char*)m.stream; a.table = m.table; a.row_scale = m.row_scale; a.row_mask = m.row_mask; a.perms = m.perms;
+    a.stream = (const unsigned char*)m.stream;
+    a.table = g.off_table ? (const uint16_t*)((const unsigned char*)m.stream + g.off_table) : m.table; a.row_scale = m.row_scale; a.row_mask = m.row_mask; a.perms = m.perms;
     a.out = out; a.ld_out = ld_out; a.R = m.R; a.C = m.C; a.NS = g.NS; a.NV = g.NV; a.PC = g.PC; a.NG = g.NG; a.r0 = r0; a.r1 = r1;
     a.raw = raw ? 1 : 0;
     a.off_slots = (uint32_t)g.off_slots; a.off_rows = (uint32_t)g.off_rows; a.off_steps = (uint32_t)g.off_steps;
@@ -1079,7 +1130,7 @@ bool stream_shape(const sq_matrix& m) {
 int stream_pass_rows(int B) { return B > 4 ? 8 : B > 2 ? 4 : B > 1 ? 2 : 1; }
 
 size_t stream_part_bytes(const sq_matrix& m, int rows) {
-    const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m));
+    const StreamGeom g = stream_geom_of(m);
     return (((size_t)g.NV * rows * g.NG * 64 * 4) + 255) & ~(size_t)255;
 }
 
@@ -1121,7 +1172,7 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     for (int k = 0; k < cnt; ++k) {
         const sq_matrix& m = mats[k];
         const int runs = stream_runs_of(m), run_max = stream_run_max_of(m);
-        const StreamGeom g = stream_geom(m.C, m.d, m.bits, m.stream_groups, runs);
+        const StreamGeom g = stream_geom_of(m);
         if (m.stream_groups < (m.R + 63) / 64 || runs > m.stream_groups || runs < 1 || run_max < 1 || run_max > STREAM_RUN_MAX)
             return fail(SQ_EINVAL, "sq_linear_small: stream_runs 0x%x / stream_groups %d do not fit %d rows", m.stream_runs, m.stream_groups, m.R);
         // Without column orders the kernel cuts the groups into runs of ceil(groups / runs) itself: a run count that
@@ -1131,7 +1182,7 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
             return fail(SQ_EINVAL, "sq_linear_small: stream_runs 0x%x does not cut %d groups the way the builder does", m.stream_runs, m.stream_groups);
         StreamPiece& P = a.p[k];
         P.stream = (const unsigned char*)m.stream;
-        P.table = m.table;
+        P.table = g.off_table ? (const uint16_t*)((const unsigned char*)m.stream + g.off_table) : m.table;
         P.row_scale = m.row_scale;
         P.part = (float*)(sums + sums_off);
         sums_off += stream_part_bytes(m, rows);

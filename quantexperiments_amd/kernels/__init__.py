@@ -91,6 +91,7 @@ class PackedLinear(torch.nn.Module):
         self.stream_runs = self.stream_groups = 0
         self.stream_asked = None
         self.stream_tiled = False
+        self.balance = True         # slice streams carry a relabelled codebook whose slices share the tags evenly
         # stream: True builds now, cut for a launch of this matrix alone; "later" leaves the build to prepare_stack
         # (pieces that will be launched together are cut for the joint launch, and built once); False: never
         self.wants_stream = bool(stream) and self.G == 1 and table.numel() * 2 > 128 * 1024 and d == 8 and 12 < self.bits <= 16
@@ -109,7 +110,8 @@ class PackedLinear(torch.nn.Module):
         if self.words is None:
             raise RuntimeError("the packed tags of this matrix were dropped (compact): its stream cannot be rebuilt")
         self.stream, self.stream_runs, self.stream_groups = build_stream(
-            self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs)
+            self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs,
+            table=self.table if self.balance and self.G == 1 and self.d == 8 else None)
         self.stream_asked = runs
         if self.stream is None:
             self.wants_stream = False
@@ -193,23 +195,29 @@ class PackedLinear(torch.nn.Module):
             self.words = None
 
 
-def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, runs: int = 0):
+def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, runs: int = 0, table=None):
     """(stream, runs, groups): the bucketed tag stream of one matrix (sq_stream_build) as a uint8 tensor on
-    words' device with the library's runs_out (run count and longest run, packed) and group count, to be handed
-    back in sq_matrix, or (None, 0, 0) when the format is not covered.  The regrouping itself is the library's host routine; the tags make one trip to host memory at
-    load time."""
+    words' device with the library's runs_out (opaque: run count, longest run, flags) and group count, to be handed
+    back in sq_matrix, or (None, 0, 0) when the format is not covered.  The regrouping itself is the library's host
+    routine; the tags make one trip to host memory at load time.  With `table` (the matrix' fp16 codebook) the library
+    relabels the codewords so that every slice of the codebook carries the same share of the tags, whatever their
+    distribution, and the stream holds the relabelled codebook (sq_stream_build_balanced)."""
     L = _lib.lib()
     host = words.detach().to("cpu", torch.int32).contiguous()
     mask = None if row_mask is None else row_mask.detach().to("cpu", torch.uint8).contiguous()
     mp = None if mask is None else mask.data_ptr()
+    tab = None if table is None else table.detach().to("cpu", torch.float16).contiguous()
+    if tab is not None and tab.numel() != (d << bits):
+        raise ValueError(f"codebook of {tab.numel()} values for {bits}-bit tags of {d}")
+    tp = None if tab is None else tab.data_ptr()
     R, W = host.shape
-    n = L.sq_stream_bytes(host.data_ptr(), R, W, C, d, bits, mp, runs)
+    n = L.sq_stream_bytes_balanced(host.data_ptr(), R, W, C, d, bits, mp, runs, tp)
     if n == 0:
         return None, 0, 0
     out = torch.empty(n, dtype=torch.uint8)
     r, g = ctypes.c_int32(0), ctypes.c_int32(0)
-    _lib.check(L.sq_stream_build(host.data_ptr(), R, W, C, d, bits, mp, runs, out.data_ptr(), n, ctypes.byref(r),
-                                 ctypes.byref(g)))
+    _lib.check(L.sq_stream_build_balanced(host.data_ptr(), R, W, C, d, bits, mp, runs, tp, out.data_ptr(), n, ctypes.byref(r),
+                                          ctypes.byref(g)))
     return out.to(words.device), r.value, g.value
 
 

@@ -596,7 +596,7 @@ def test_launcher_refuses_stream_counts_the_builder_did_not_make():
     L = _lib.lib()
     lin = to_device(synth(700, 512, 8, 16, seed=4))
     lin.build_stream(4)
-    runs, run_max = lin.stream_runs & 0xFFFF, lin.stream_runs >> 16
+    runs, run_max, flags = lin.stream_runs & 0xFFFF, (lin.stream_runs >> 16) & 0xFF, lin.stream_runs & ~0xFFFFFF
     x = torch.zeros(1, 512, dtype=torch.bfloat16, device="cuda")
     y = torch.zeros(1, 700, dtype=torch.bfloat16, device="cuda")
     ws = torch.zeros(_lib.WS_HEADER + (1 << 20), dtype=torch.uint8, device="cuda")
@@ -607,8 +607,8 @@ def test_launcher_refuses_stream_counts_the_builder_did_not_make():
         return L.sq_linear_small(_lib.matrix_array([m]), 1, x.data_ptr(), _lib.SQ_BF16, 512, y.data_ptr(), _lib.SQ_BF16, 700, 1,
                                  ws.data_ptr(), ws.numel(), _lib.stream_ptr(x.device))
     assert call(lin.stream_runs, lin.stream_groups) == 0
-    assert call(runs | ((run_max + 1) << 16), lin.stream_groups) == _lib.SQ_EINVAL       # longer runs than the cut gives
-    assert call((runs + 7) | (run_max << 16), lin.stream_groups) == _lib.SQ_EINVAL       # an empty last run
+    assert call(flags | runs | ((run_max + 1) << 16), lin.stream_groups) == _lib.SQ_EINVAL   # longer runs than the cut gives
+    assert call(flags | (runs + 7) | (run_max << 16), lin.stream_groups) == _lib.SQ_EINVAL   # an empty last run
     assert call(lin.stream_runs, lin.stream_groups - 1) == _lib.SQ_EINVAL                # fewer groups than rows need
     assert call(runs, lin.stream_groups) in (_lib.SQ_EINVAL, _lib.SQ_EUNSUPPORTED, 0)    # no run length: not a stream -> row kernel
     torch.cuda.synchronize()

@@ -178,29 +178,42 @@ def test_neutral_defaults_and_registry():
 
 # ---------------------------------------------------------------------------- bucketed tag stream (host builder)
 
-def _build_stream(words, R, C, bits, row_mask, runs):
+def _build_stream(words, R, C, bits, row_mask, runs, table=None):
+    """Bytes of the stream, its run count and its group count; with `table` (fp16 [2^bits, 8]) the balanced form."""
     import ctypes
     from quantexperiments_amd import _lib
     L = _lib.lib()
     W = words.shape[1]
     ptr = words.ctypes.data_as(ctypes.c_void_p)
     mp = None if row_mask is None else row_mask.ctypes.data_as(ctypes.c_void_p)
-    n = L.sq_stream_bytes(ptr, R, W, C, 8, bits, mp, runs)
-    assert n > 0
-    out = np.zeros(n, np.uint8)
     r, g = ctypes.c_int32(0), ctypes.c_int32(0)
-    args = (ptr, R, W, C, 8, bits, mp, runs, out.ctypes.data_as(ctypes.c_void_p))
-    assert L.sq_stream_build(*args, n, ctypes.byref(r), ctypes.byref(g)) == 0
-    assert L.sq_stream_build(*args, n - 1, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EINVAL
-    # runs_out: the run count in the low 16 bits, the groups of the longest run above
+    if table is None:
+        n = L.sq_stream_bytes(ptr, R, W, C, 8, bits, mp, runs)
+        assert n > 0
+        out = np.zeros(n, np.uint8)
+        args = (ptr, R, W, C, 8, bits, mp, runs, out.ctypes.data_as(ctypes.c_void_p))
+        assert L.sq_stream_build(*args, n, ctypes.byref(r), ctypes.byref(g)) == 0
+        assert L.sq_stream_build(*args, n - 1, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EINVAL
+        assert not r.value & (1 << 30)
+    else:
+        tp = table.ctypes.data_as(ctypes.c_void_p)
+        n = L.sq_stream_bytes_balanced(ptr, R, W, C, 8, bits, mp, runs, tp)
+        assert n > (18 << bits)                            # the relabelled codebook and the back map are inside
+        out = np.zeros(n, np.uint8)
+        assert L.sq_stream_build_balanced(ptr, R, W, C, 8, bits, mp, runs, tp, out.ctypes.data_as(ctypes.c_void_p), n,
+                                          ctypes.byref(r), ctypes.byref(g)) == 0
+        assert r.value & (1 << 30)
+    # runs_out: the run count in the low 16 bits, the groups of the longest run in the next 8, bit 30 = balanced
+    _build_stream.runs_out = r.value
     return out.tobytes(), r.value & 0xFFFF, g.value
 
 
 PART_MAX = 4064     # chunks per column part (sq_stream.h)
 
 
-def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
-    """Rebuild the [R, C/d] tag matrix from a stream buffer, checking its structure on the way."""
+def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
+    """Rebuild the [R, C/d] tag matrix from a stream buffer, checking its structure on the way.  A balanced stream
+    (built with `table`) stores relabelled tags, its relabelled codebook and the map back to the file's labels."""
     U, NS = C // d, 1 << (bits - 12)
     KP = -(-U // PART_MAX)
     PC = -(-U // KP)
@@ -209,6 +222,15 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
     off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
     off_rows = (off_runs + runs * 16 + 255) & ~255
     off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
+    unmap = None
+    if table is not None:
+        K = 1 << bits
+        off_table, off_unmap = off_steps, off_steps + K * d * 2
+        off_steps = (off_unmap + K * 2 + 255) & ~255
+        unmap = np.frombuffer(buf, np.uint16, K, off_unmap).astype(np.int64)
+        assert sorted(unmap.tolist()) == list(range(K))                        # a permutation of the labels
+        moved = np.frombuffer(buf, np.uint16, K * d, off_table).reshape(K, d)
+        assert np.array_equal(moved, table.view(np.uint16).reshape(K, d)[unmap])   # codeword `new` is the file's unmap[new]
     goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
     slots = np.frombuffer(buf, np.uint32, NV * NG * 64, off_slots).reshape(NV, NG * 64)
     rt = np.frombuffer(buf, np.int32, runs * 4, off_runs).reshape(runs, 4)
@@ -268,7 +290,7 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask):
                 assert len(set(chunk.tolist())) == c and (chunk >= kp * PC).all() and (chunk < min(U, (kp + 1) * PC)).all()
                 assert (tags[rows[k], chunk] == -1).all()
                 tags[rows[k], chunk] = (e[lane, :c] & 0xFFF) + (s << 12)
-    return tags
+    return tags if unmap is None else unmap[tags]
 
 
 @pytest.mark.parametrize("R,C,bits,runs,M", [(70, 512, 16, 0, 1), (130, 5376, 16, 2, 1), (64, 1024, 13, 5, 1), (1, 8, 14, 0, 1),
@@ -289,13 +311,46 @@ def test_stream_builder_keeps_every_tag(R, C, bits, runs, M):
     assert np.array_equal(_walk_stream(buf, R, C, 8, bits, eff, NG, row_mask), tags)
 
 
+@pytest.mark.parametrize("R,C,bits,runs,M", [(300, 512, 16, 3, 1), (130, 3584, 14, 2, 1), (200, 256, 16, 0, 4)])
+def test_balanced_stream_relabels_codewords_and_evens_out_the_slices(R, C, bits, runs, M):
+    """sq_stream_build_balanced: tags drawn with a Zipf popularity whose most popular codewords all sit in the first
+    slice of the codebook.  The stream must still hold every tag (through its map back to the file's labels), carry
+    the relabelled codebook, and give every slice of 4096 codewords the same share of the entries (the plain stream
+    puts most of them into slice 0)."""
+    rng = np.random.default_rng(R + bits)
+    K, U = 1 << bits, C // 8
+    w = 1.0 / np.arange(1, K + 1)
+    tags = rng.choice(K, size=(R, U), p=w / w.sum())
+    row_mask = rng.integers(0, M, R).astype(np.uint8) if M > 1 else None
+    table = rng.standard_normal((K, 8)).astype(np.float16)
+    words = np.ascontiguousarray(O.pack_bits(tags, bits))
+    buf, eff, NG = _build_stream(words, R, C, bits, row_mask, runs, table)
+    assert np.array_equal(_walk_stream(buf, R, C, 8, bits, eff, NG, row_mask, table), tags)
+    for what, a, b in _stream_reads(buf, R, C, bits, _build_stream.runs_out, NG, row_mask):   # (defined below)
+        assert 0 <= a < b <= len(buf), (what, a, b)
+    NS = K >> 12
+    def slice_loads(b, balanced):
+        NV = NS * -(-U // PART_MAX)
+        off_slots = ((NV * NG + 1) * 4 + 255) & ~255
+        cnt = np.frombuffer(b, np.uint32, NV * NG * 64, off_slots).reshape(NV, -1) >> 19
+        return cnt.sum(1).reshape(-1, NS).sum(0)
+    plain, _, NG2 = _build_stream(words, R, C, bits, row_mask, runs)
+    assert NG2 == NG
+    lb, lp = slice_loads(buf, True), slice_loads(plain, False)
+    assert lb.sum() == lp.sum() == R * U
+    assert lp.max() > 2.5 * lp.mean()                     # slice 0 of the plain stream: most of the tags
+    # the most popular codeword alone may outweigh a slice's fair share; nothing else may
+    top = int(np.bincount(tags.ravel(), minlength=K).max())
+    assert lb.max() <= max(1.02 * lb.mean() + 1, top)
+
+
 def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask, PF=3, NW=16):
     """Every byte range of the stream buffer that stream_kernel (csrc/sq_stream.hip) forms an address for, replayed on
     the host: the run table, the group heads (with the kernel's clamp of the group index), the first steps a wave
     requests before it knows whether it has any (the prologue reads step 0 for a group without steps), the steps
     fetched ahead inside the loop (clamped to the group's last step), the shares of a group that several waves walk,
     and the row list of the finishing workgroup.  Yields (what, first byte, end byte)."""
-    runs, run_max = runs_out & 0xFFFF, runs_out >> 16
+    runs, run_max, balanced = runs_out & 0xFFFF, (runs_out >> 16) & 0xFF, bool(runs_out & (1 << 30))
     U, NS = C // 8, 1 << (bits - 12)
     KP = -(-U // PART_MAX)
     NV = NS * KP
@@ -303,6 +358,9 @@ def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask, PF=3, NW=16):
     off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
     off_rows = (off_runs + runs * 16 + 255) & ~255
     off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
+    if balanced:                                        # relabelled codebook and back map sit in front of the steps
+        yield "codebook slices", off_steps, off_steps + (16 << bits)
+        off_steps = (off_steps + (18 << bits) + 255) & ~255
     goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0).astype(np.int64)
     rt = np.frombuffer(buf, np.int32, runs * 4, off_runs).reshape(runs, 4)
     gr = -(-NG // runs)
@@ -358,7 +416,7 @@ def test_kernel_addresses_stay_inside_the_stream(R, C, bits, runs, M):
     out = np.zeros(n, np.uint8)
     r, g = ctypes.c_int32(0), ctypes.c_int32(0)
     assert L.sq_stream_build(ptr, R, words.shape[1], C, 8, bits, mp, runs, out.ctypes.data_as(ctypes.c_void_p), n, ctypes.byref(r), ctypes.byref(g)) == 0
-    assert 1 <= (r.value >> 16) <= 96 and 1 <= (r.value & 0xFFFF) <= g.value
+    assert 1 <= ((r.value >> 16) & 0xFF) <= 96 and 1 <= (r.value & 0xFFFF) <= g.value
     count = 0
     for what, a, b in _stream_reads(out.tobytes(), R, C, bits, r.value, g.value, row_mask):
         assert 0 <= a < b <= n, (what, a, b, n)
