@@ -44,7 +44,7 @@ typedef struct sq_matrix {
     int32_t R, C, d, bits, G, M, W;
     int32_t y_off;              /* first output column of this piece in the stacked Y */
     const void*     stream;     /* optional: device copy of the buffer sq_stream_build wrote for `tags`; NULL = none */
-    int32_t stream_runs;        /* runs_out of sq_stream_build for that buffer (opaque: run count and longest run, packed) */
+    int32_t stream_runs;        /* runs_out of sq_stream_build for that buffer (opaque: run count, longest run, column orders per run, flags) */
     int32_t stream_groups;      /* groups_out of sq_stream_build for that buffer */
 } sq_matrix;
 

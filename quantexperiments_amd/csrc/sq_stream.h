@@ -12,6 +12,7 @@ constexpr int STREAM_RUN_MAX = 96;           // most groups of 64 rows in one ru
 constexpr int STREAM_ROW_BITS = 19;          // slot = row | count << 19
 constexpr uint32_t STREAM_NO_ROW = (1u << STREAM_ROW_BITS) - 1u;
 constexpr int GEMV_MAX_PIECES_STREAM = 4;
+constexpr int STREAM_RUN_ORDERS = 8;         // most column orders whose rows may share a run (one gathered copy of x in LDS each)
 
 constexpr int STREAM_DEFAULT_WGS = 256;      // workgroups a matrix launched alone should make (one per CU on 256 CUs)
 
@@ -33,10 +34,11 @@ size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int b
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                       unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table = nullptr);
 // sq_matrix.stream_runs is sq_stream_build's runs_out: the run count in the low 16 bits, the groups of the longest run
-// in the next 8, bit 30 = the stream carries a relabelled codebook
+// in the next 8, the most column orders in one run (less one) in bits 24-26, bit 30 = the stream carries a relabelled codebook
 constexpr int STREAM_BALANCED = 1 << 30;
 inline int stream_runs_of(const sq_matrix& m) { return m.stream_runs & 0xFFFF; }
 inline int stream_run_max_of(const sq_matrix& m) { return (int)(((uint32_t)m.stream_runs >> 16) & 0xFFu); }
+inline int stream_run_orders_of(const sq_matrix& m) { return (int)(((uint32_t)m.stream_runs >> 24) & 7u) + 1; }
 inline bool stream_balanced_of(const sq_matrix& m) { return (m.stream_runs & STREAM_BALANCED) != 0; }
 inline StreamGeom stream_geom_of(const sq_matrix& m) {
     return stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m), stream_balanced_of(m));

@@ -26,7 +26,8 @@
 //                                 NG groups per bucket, bucket v = kp * NS + s)
 //   slots  uint32 [NV * NG * 64]  place | count << 19 per lane; place = the row's index in `rows` (below),
 //                                 0x7FFFF marks a lane without a row; lanes 64 g .. 64 g + 63 of a bucket are group g
-//   runs   int32 [runs][4]        first group, group count, column order, 0
+//   runs   [runs] x 32 bytes       first group, group count, column orders of the run, 0; first group (within the run) and
+//                                 id of each of up to 8 column orders (one byte each)
 //   rows   uint32 [NG * 64]       the rows ordered by column order, 64 per group (0x7FFFF where a group is short):
 //                                 places 64 g0 .. 64 (g0 + ng) - 1 are a run's rows, and partial sums are indexed by place
 //   steps  [total][64][3] uint32  entries
@@ -40,6 +41,12 @@ constexpr int STREAM_CLIMB = 1;      // hill-climbing passes of the entry orderi
 
 namespace sq {
 
+// A run: groups g0 .. g0 + ng - 1 of every bucket.  Its rows belong to `norders` column orders (one without row orders);
+// the groups of order[i] begin at group bound[i] of the run (bound[0] = 0), and the kernel keeps copy i of x, gathered
+// through that order, in LDS for them.
+struct StreamRun { int32_t g0, ng, norders, zero; uint8_t bound[STREAM_RUN_ORDERS]; uint8_t order[STREAM_RUN_ORDERS]; };
+static_assert(sizeof(StreamRun) == 32, "run records are read as 8 dwords");
+
 StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced) {
     StreamGeom g;
     g.U = C / d;
@@ -51,7 +58,7 @@ StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanc
     g.runs = runs;
     g.off_slots = (((size_t)g.NV * g.NG + 1) * 4 + 255) & ~(size_t)255;
     g.off_runs = (g.off_slots + (size_t)g.NV * g.NG * 64 * 4 + 255) & ~(size_t)255;
-    g.off_rows = (g.off_runs + (size_t)runs * 16 + 255) & ~(size_t)255;
+    g.off_rows = (g.off_runs + (size_t)runs * sizeof(StreamRun) + 255) & ~(size_t)255;
     size_t end = (g.off_rows + (size_t)g.NG * 64 * 4 + 255) & ~(size_t)255;
     g.off_table = g.off_unmap = 0;
     if (balanced) {
@@ -92,11 +99,11 @@ static void parallel_rows(int R, const std::function<void(int, int)>& fn) {
     for (auto& t : th) t.join();
 }
 
-struct StreamRun { int32_t g0, ng, order, zero; };
 
 struct StreamPlan {
     StreamGeom g;
     int GR;                          // groups in the longest run
+    int orders_max;                  // most column orders in one run
     std::vector<StreamRun> runs;
     std::vector<uint32_t> base;      // [NG * 64]: rows ordered by column order, STREAM_NO_ROW where a group is short
     std::vector<uint16_t> cnt;       // [NV][R]
@@ -145,8 +152,10 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     StreamGeom g0 = stream_geom(C, d, bits, 0, 0);
     if (runs <= 0) runs = (STREAM_DEFAULT_WGS + g0.NV / 2) / g0.NV;
     if (runs < 1) runs = 1;
-    // groups per column order; GR = the fewest groups per run that keep the run count within the request (or
-    // at one run per column order when there are more orders than that)
+    // Groups per column order.  A run takes the groups of one order, GR at a time, or, when orders are small, the whole
+    // groups of up to `cap` orders that follow each other (a masked k projection has 64 rows per order: one run per order
+    // would be 16 workgroups of one group each per bucket).  cap: as many gathered copies of x as fit LDS beside the slice
+    // and the run's partial sums, and as the staging loop covers with four chunks per thread.
     std::vector<int> first, ngm;
     for (int a = 0; a < R;) {
         int b = a;
@@ -157,34 +166,64 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
         a = b;
     }
     first.push_back(R);
-    int GR = 1;
-    for (;; ++GR) {
+    int total_groups = 0;
+    for (int q : ngm) total_groups += q;
+    const int xs_bytes = (g0.PC + 16) * 16;
+    int cap = (160 * 1024 - 65536 - STREAM_RUN_MAX * 256 - 1024) / xs_bytes;
+    cap = std::min(cap, std::min(4, 4096 / g0.PC));            // (4: two activation rows per pass still fit LDS at C = 5120)
+    if (cap < 1 || !row_mask) cap = 1;
+    // the runs for a run length GR (into `out` if given): returns their number
+    auto pack = [&](int GR, std::vector<StreamRun>* out, int* longest) {
         int64_t n = 0;
-        bool whole = true;
-        for (int q : ngm) { n += (q + GR - 1) / GR; whole = whole && q <= GR; }
-        if (n <= runs || whole) break;
-    }
-    // A run's partial sums are staged in LDS: no run longer than STREAM_RUN_MAX groups (more runs than asked for then).
+        StreamRun cur{0, 0, 0, 0, {0}, {0}};
+        int gbase = 0, lg = 1;
+        auto flush = [&]() {
+            if (cur.ng > 0) { ++n; lg = std::max(lg, cur.ng); if (out) out->push_back(cur); }
+            cur = StreamRun{0, 0, 0, 0, {0}, {0}};
+        };
+        for (size_t i = 0; i < ngm.size(); ++i) {
+            const int q = ngm[i], m = row_mask ? row_mask[order[first[i]]] : 0;
+            if (q > GR) {                                        // an order longer than a run: runs of its own
+                flush();
+                for (int p0 = 0; p0 < q; p0 += GR) {
+                    cur = StreamRun{gbase + p0, std::min(GR, q - p0), 1, 0, {0}, {(uint8_t)m}};
+                    flush();
+                }
+            } else if (cur.ng > 0 && cur.ng + q <= GR && cur.norders < cap) {
+                cur.bound[cur.norders] = (uint8_t)cur.ng;
+                cur.order[cur.norders] = (uint8_t)m;
+                ++cur.norders;
+                cur.ng += q;
+            } else {
+                flush();
+                cur = StreamRun{gbase, q, 1, 0, {0}, {(uint8_t)m}};
+            }
+            gbase += q;
+        }
+        flush();
+        if (longest) *longest = lg;
+        return n;
+    };
+    // GR = the fewest groups per run that keep the run count within the request.  A run's partial sums are staged in
+    // LDS: no run longer than STREAM_RUN_MAX groups (more runs than asked for then).
+    int GR = 1;
+    while (GR < STREAM_RUN_MAX && GR < total_groups && pack(GR, nullptr, nullptr) > runs) ++GR;
     // With one column order the kernel derives the cut from the run count alone, as ceil(groups / runs) per run: settle
     // on a run length that this formula gives back.
-    if (GR > STREAM_RUN_MAX) GR = STREAM_RUN_MAX;
     if (ngm.size() == 1)
         for (;;) {
             const int n = (ngm[0] + GR - 1) / GR, g2 = (ngm[0] + n - 1) / n;
             if (g2 == GR) break;
             GR = g2;
         }
-    P.GR = 1;
     P.runs.clear();
     P.base.clear();
+    pack(GR, &P.runs, &P.GR);
+    P.orders_max = 1;
+    for (const StreamRun& run : P.runs) P.orders_max = std::max(P.orders_max, (int)run.norders);
     for (size_t i = 0; i < ngm.size(); ++i) {
-        const int a = first[i], b = first[i + 1], gbase = (int)(P.base.size() / 64);
-        const int m = row_mask ? row_mask[order[a]] : 0;
+        const int a = first[i], b = first[i + 1];
         for (int k = 0; k < ngm[i] * 64; ++k) P.base.push_back(a + k < b ? order[a + k] : STREAM_NO_ROW);
-        for (int q = 0; q < ngm[i]; q += GR) {
-            P.runs.push_back(StreamRun{gbase + q, std::min(GR, ngm[i] - q), m, 0});
-            P.GR = std::max(P.GR, std::min(GR, ngm[i] - q));
-        }
     }
     P.g = stream_geom(C, d, bits, (int)(P.base.size() / 64), (int)P.runs.size(), balanced);
     const StreamGeom& g = P.g;
@@ -208,13 +247,17 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
         for (int v = a; v < b; ++v) {
             const uint16_t* c = &P.cnt[(size_t)v * R];
             for (const StreamRun& run : P.runs) {
-                rows.clear();
-                for (int k = run.g0 * 64; k < (run.g0 + run.ng) * 64; ++k)
-                    if (P.base[k] != STREAM_NO_ROW) rows.push_back(P.base[k]);
-                std::stable_sort(rows.begin(), rows.end(), [c](uint32_t x, uint32_t y) { return c[x] > c[y]; });
-                for (size_t k = 0; k < rows.size(); ++k) P.pos[(size_t)v * R + rows[k]] = (uint32_t)(run.g0 * 64 + k);
-                for (size_t k = 0; k < rows.size(); k += 64)
-                    steps[(size_t)v * g.NG + run.g0 + k / 64] = (c[rows[k]] + 3u) / 4u;
+                // rows move between the groups of one column order only: a group reads one copy of x
+                for (int oi = 0; oi < run.norders; ++oi) {
+                    const int ga = run.g0 + run.bound[oi], gb = run.g0 + (oi + 1 < run.norders ? run.bound[oi + 1] : run.ng);
+                    rows.clear();
+                    for (int k = ga * 64; k < gb * 64; ++k)
+                        if (P.base[k] != STREAM_NO_ROW) rows.push_back(P.base[k]);
+                    std::stable_sort(rows.begin(), rows.end(), [c](uint32_t x, uint32_t y) { return c[x] > c[y]; });
+                    for (size_t k = 0; k < rows.size(); ++k) P.pos[(size_t)v * R + rows[k]] = (uint32_t)(ga * 64 + k);
+                    for (size_t k = 0; k < rows.size(); k += 64)
+                        steps[(size_t)v * g.NG + ga + k / 64] = (c[rows[k]] + 3u) / 4u;
+                }
             }
         }
     });
@@ -468,7 +511,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             for (int q = 0; q < 4; ++q) bm.order_lanes(base, sl, LDS_CLOCK_LANES[q], ns, (uint32_t)g.PC);
         }
     });
-    if (runs_out) *runs_out = g.runs | (P.GR << 16) | (table ? STREAM_BALANCED : 0);
+    if (runs_out) *runs_out = g.runs | (P.GR << 16) | ((P.orders_max - 1) << 24) | (table ? STREAM_BALANCED : 0);
     if (groups_out) *groups_out = g.NG;
     return SQ_OK;
 }
@@ -494,6 +537,11 @@ struct StreamArgs {
     int64_t ldx, ldy;
     int nb;                           // activation rows of this pass (<= NB)
     int xs;                           // LDS bytes of one activation row's part of x (its chunks + 16 zero chunks)
+    int xcopies;                      // copies of x per activation row in LDS: the most column orders in one run of the launch
+    int xtmp;                         // bytes per activation row of its copy in natural order in LDS (column orders are then
+                                      // applied from LDS), 0: gathered from memory
+    int orders;                       // 1: some piece has column orders
+    int xtmp_own;                     // 1: those copies have LDS of their own behind everything else, 0: they sit where the slice goes
     int nl_max;                       // places of the longest run (64 per group): floats per row of the LDS partial sums
     int x_dtype, y_dtype;
     // Producer of the activation row (stream_kernel<1, NX, 1> only): the row is computed while it is staged instead
@@ -590,7 +638,7 @@ typedef __attribute__((address_space(3))) void* stream_lptr_t;
 // a row's part of x per thread (1: parts of up to 1024 chunks, 4: up to 4096).  One workgroup of 16 waves per CU.
 // LDS: [codebook slice 64 KB][NB x parts of a.xs bytes][partial sums of the run: NB x a.nl_max floats][two words of flags]
 // [16 block sums (PRO 1)].
-template <int NB, int NX, int PRO = 0>
+template <int NB, int NX, int PRO = 0, int ORD = 1>
 __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     static_assert(PRO == 0 || (PRO == 1 && NB == 1), "produced activations: add + norm, one row");
     constexpr int NW = STREAM_NW, NTH = NW * 64;
@@ -601,6 +649,8 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     for (int k = 1; k < GEMV_MAX_PIECES_STREAM; ++k)
         if (k < a.n && (int)blockIdx.x >= a.p[k].wg_begin) pi = k;
     const StreamPiece P = a.p[pi];                             // by value: the piece's fields arrive in one batch of scalar loads
+    // ORD 0: no piece of the launch has column orders (everything that serves them compiles away)
+    const int32_t* const perms = ORD ? P.perms : nullptr;
     SQ_TRACE_DEP(7, "s", P.NV);
     // Workgroups go to the 8 XCDs in turn (workgroup i to XCD i mod 8), each with an L2 of its own.  When the
     // bucket count is a multiple of 8 the bucket (and with it the slice) is made a function of the workgroup index
@@ -621,9 +671,15 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     SQ_TRACE_POINT(0);
     // this workgroup's run: groups g0 .. g0 + ng - 1 of the bucket, all of one column order
     // (without column orders every run but the last has ceil(NG / runs) groups: no need to wait for the table)
-    const int32_t* run = reinterpret_cast<const int32_t*>(P.stream + P.off_runs) + wi * 4;
+    const int32_t* run = reinterpret_cast<const int32_t*>(P.stream + P.off_runs) + wi * 8;
     const int gr = (P.NG + P.nwg - 1) / P.nwg;
-    const int g0 = P.perms ? run[0] : wi * gr, ng = min(P.perms ? run[1] : min(gr, P.NG - g0), a.nl_max >> 6);
+    const int g0 = perms ? run[0] : wi * gr, ng = min(perms ? run[1] : min(gr, P.NG - g0), a.nl_max >> 6);
+    // the run's column orders (with row orders only): copy i of x, gathered through order i, serves the groups from
+    // bound i on
+    const int no = perms ? min(max(run[2], 1), a.xcopies) : 1;
+    const uint32_t bnd_lo = perms ? (uint32_t)run[4] : 0u, bnd_hi = perms ? (uint32_t)run[5] : 0u;
+    const uint32_t ord_lo = perms ? (uint32_t)run[6] : 0u, ord_hi = perms ? (uint32_t)run[7] : 0u;
+    auto byte_of = [](uint32_t lo, uint32_t hi, int i) { return (int)(((i < 4 ? lo >> (8 * i) : hi >> (8 * (i - 4)))) & 0xFFu); };
 
     const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG + g0;
     const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
@@ -632,7 +688,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     float* part = P.part + (size_t)v * NB * np;
     const int xs = a.xs;
     const unsigned char* ldsx = lds + STREAM_TAB;
-    float* psum = reinterpret_cast<float*>(lds + STREAM_TAB + NB * xs);          // [NB][a.nl_max], indexed by place - 64 g0
+    float* psum = reinterpret_cast<float*>(lds + STREAM_TAB + a.xcopies * NB * xs);   // [NB][a.nl_max], indexed by place - 64 g0
     unsigned* flag = reinterpret_cast<unsigned*>(psum + (size_t)NB * a.nl_max);  // [1] next group
 
     // The groups of a run are sorted longest first.  Wave w starts with group w, then group 2 NW - 1 - w; after
@@ -683,6 +739,10 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         kcur = wave < ng * split ? wave / split : ng;
         knext = ng;
     }
+    // Column orders through LDS (a.xtmp > 0): the activation rows first sit in natural order where the slice goes, and
+    // the kd 16 KB blocks of the slice that they cover are copied once the rows have been read from there.
+    const bool via_lds = PRO == 0 && perms != nullptr && a.xtmp > 0;   // uniform in the workgroup
+    const int kd = via_lds && !a.xtmp_own ? (NB * a.xtmp + NTH * 16 - 1) / (NTH * 16) : 0;
     // The codebook slice is copied global -> LDS without passing through registers (a wave instruction moves 1 KB, lane l
     // to the wave's base + 16 l).  It goes out first: loads are accounted for in the order they were issued, and the
     // small scattered reads of the group heads below come back later than this bulk copy does.
@@ -690,8 +750,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table) + (size_t)s * STREAM_TAB;
 #pragma unroll
         for (int k = 0; k < STREAM_TAB / (NTH * 16); ++k)
-            __builtin_amdgcn_global_load_lds((stream_gptr_t)(src + ((size_t)k * NTH + tid) * 16),
-                                             (stream_lptr_t)(lds + (k * NTH + wave * 64) * 16), 16, 0, 0);
+            if (k >= kd)
+                __builtin_amdgcn_global_load_lds((stream_gptr_t)(src + ((size_t)k * NTH + tid) * 16),
+                                                 (stream_lptr_t)(lds + (k * NTH + wave * 64) * 16), 16, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     // the first head's words are requested here and used only after the staging loads have gone out
@@ -708,15 +769,24 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     {
         u32x4 xq[NB][NX];
         const int c0 = kp * P.PC, nc = min(P.PC, P.U - c0);
+        // this thread's items of the staged x: item it = (copy, chunk) = (it / nc, it % nc), it = tid + k * NTH
+        const int total = no * nc;
+        int it_o[NX], it_c[NX];
+#pragma unroll
+        for (int k = 0; k < NX; ++k) {
+            const int it = min(tid + k * NTH, total - 1);
+            it_o[k] = no > 1 ? it / nc : 0;
+            it_c[k] = it - it_o[k] * nc;
+        }
         if (PRO != 0) {
             // every operand of the produced row is requested before anything waits: this thread's chunks, then
             // (PRO 1) its share of the whole row for the mean square
-            const int32_t* pm = P.perms ? P.perms + (size_t)run[2] * P.C : nullptr;
+            const bool pm = perms != nullptr;
             ProRaw raw[NX];
 #pragma unroll
             for (int k = 0; k < NX; ++k) {
-                const int ci = c0 + min(tid + k * NTH, nc - 1);
-                raw[k] = pm ? pro_gather<PRO>(a, pm + (size_t)ci * 8) : pro_fetch<PRO>(a, ci);
+                const int ci = c0 + it_c[k];
+                raw[k] = pm ? pro_gather<PRO>(a, perms + (size_t)byte_of(ord_lo, ord_hi, it_o[k]) * P.C + (size_t)ci * 8) : pro_fetch<PRO>(a, ci);
             }
             float rstd = 0.f;
             if (PRO == 1) {
@@ -727,7 +797,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                 static_assert(NTH == 1024, "one slot per thread");
                 float* red = reinterpret_cast<float*>(flag + 4);
                 float ps = 0.f;
-                if (pm == nullptr && nc == P.U && P.U <= NX * NTH) {
+                if (!pm && nc == P.U && P.U <= NX * NTH) {
                     // one column part, natural order: this thread's chunks are its slot's chunks, already fetched
 #pragma unroll
                     for (int k = 0; k < NX; ++k)
@@ -760,7 +830,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
             for (int k = 0; k < NX; ++k) xq[0][k] = pro_finish<PRO>(a, raw[k], rstd);
             if (pi == 0 && s == 0 && wi == 0) {
                 // one workgroup per column part leaves the produced row (and the updated residual) in memory
-                if (pm == nullptr) {
+                if (!pm) {
 #pragma unroll
                     for (int k = 0; k < NX; ++k) {
                         const int c = tid + k * NTH;
@@ -791,21 +861,39 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
             const uint16_t* xr = a.x + (int64_t)min(b, a.nb - 1) * a.ldx;
             if (PRO != 0) {
                 // filled above
-            } else if (P.perms == nullptr) {
+            } else if (perms == nullptr) {
                 const u32x4* xsrc = reinterpret_cast<const u32x4*>(xr) + c0;
 #pragma unroll
                 for (int k = 0; k < NX; ++k) xq[b][k] = xsrc[min(tid + k * NTH, nc - 1)];
+            } else if (a.xtmp > 0) {
+                // column orders, the row in natural order first: its chunks go to LDS below and the copies are
+                // gathered from there (one part per row here, so the row has at most NX * NTH chunks)
+                const u32x4* xsrc = reinterpret_cast<const u32x4*>(xr);
+#pragma unroll
+                for (int k = 0; k < NX; ++k) xq[b][k] = xsrc[min(tid + k * NTH, P.U - 1)];
             } else {
                 // chunk j of a row with column order m multiplies x[perm_m[8 j .. 8 j + 7]]
-                const int32_t* pm = P.perms + (size_t)run[2] * P.C + (size_t)c0 * 8;
 #pragma unroll
                 for (int k = 0; k < NX; ++k) {
-                    const int32_t* pk = pm + (size_t)min(tid + k * NTH, nc - 1) * 8;
+                    if (k > 0 && tid + k * NTH >= total) { xq[b][k] = xq[b][0]; continue; }
+                    const int32_t* pk = perms + (size_t)byte_of(ord_lo, ord_hi, it_o[k]) * P.C + (size_t)(c0 + it_c[k]) * 8;
                     const u32x4 i0 = *reinterpret_cast<const u32x4*>(pk), i1 = *reinterpret_cast<const u32x4*>(pk + 4);
                     const uint32_t e0 = xr[i0.x], e1 = xr[i0.y], e2 = xr[i0.z], e3 = xr[i0.w];
                     const uint32_t e4 = xr[i1.x], e5 = xr[i1.y], e6 = xr[i1.z], e7 = xr[i1.w];
                     xq[b][k] = u32x4{e0 | (e1 << 16), e2 | (e3 << 16), e4 | (e5 << 16), e6 | (e7 << 16)};
                 }
+            }
+        }
+        // Column orders through LDS: a scattered 2-byte read from memory occupies the address unit for a clock per lane
+        // (8 reads per chunk and copy: microseconds once a run has several orders), the same read from LDS costs a few
+        // clocks per wave.  The positions come from memory meanwhile.
+        u32x4 ix[NX][2];
+        if (via_lds) {
+#pragma unroll
+            for (int k = 0; k < NX; ++k) {
+                const int32_t* pk = perms + (size_t)byte_of(ord_lo, ord_hi, it_o[k]) * P.C + (size_t)(c0 + it_c[k]) * 8;
+                ix[k][0] = *reinterpret_cast<const u32x4*>(pk);
+                ix[k][1] = *reinterpret_cast<const u32x4*>(pk + 4);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -814,21 +902,51 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         first_steps_always(hn, nx);
         __builtin_amdgcn_sched_barrier(0);
         SQ_TRACE_DEP(9, "v", xq[0][0].x);
+        if (via_lds) {
+            unsigned char* tmp = a.xtmp_own ? reinterpret_cast<unsigned char*>(flag + 20) : lds;   // [NB][a.xtmp]
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+#pragma unroll
+                for (int k = 0; k < NX; ++k)
+                    if (tid + k * NTH < P.U) reinterpret_cast<u32x4*>(tmp + b * a.xtmp)[tid + k * NTH] = xq[b][k];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint16_t* xt = reinterpret_cast<const uint16_t*>(tmp + b * a.xtmp);
+#pragma unroll
+                for (int k = 0; k < NX; ++k) {
+                    if (tid + k * NTH >= total) continue;
+                    const u32x4 i0 = ix[k][0], i1 = ix[k][1];
+                    const uint32_t e0 = xt[i0.x], e1 = xt[i0.y], e2 = xt[i0.z], e3 = xt[i0.w];
+                    const uint32_t e4 = xt[i1.x], e5 = xt[i1.y], e6 = xt[i1.z], e7 = xt[i1.w];
+                    xq[b][k] = u32x4{e0 | (e1 << 16), e2 | (e3 << 16), e4 | (e5 << 16), e6 | (e7 << 16)};
+                }
+            }
+            if (kd > 0) __syncthreads();                        // every wave has what it reads of the rows: the slice may land
+            const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table) + (size_t)s * STREAM_TAB;
+#pragma unroll
+            for (int k = 0; k < STREAM_TAB / (NTH * 16); ++k)
+                if (k < kd)
+                    __builtin_amdgcn_global_load_lds((stream_gptr_t)(src + ((size_t)k * NTH + tid) * 16),
+                                                     (stream_lptr_t)(lds + (k * NTH + wave * 64) * 16), 16, 0, 0);
+        }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            u32x4* xd = reinterpret_cast<u32x4*>(lds + STREAM_TAB + b * xs);
 #pragma unroll
             for (int k = 0; k < NX; ++k) {
                 u32x4 q = xq[b][k];
                 if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
-                if (tid + k * NTH < nc) xd[tid + k * NTH] = q;
+                // copy o of activation row b lives at [o][b]
+                if (tid + k * NTH < total) reinterpret_cast<u32x4*>(lds + STREAM_TAB + (it_o[k] * NB + b) * xs)[it_c[k]] = q;
             }
         }
-        if (tid < NB * 16)                                       // the chunks that padding entries multiply with
+        if (tid < no * NB * 16)                                  // the chunks that padding entries multiply with, in every copy
             reinterpret_cast<u32x4*>(lds + STREAM_TAB + (tid >> 4) * xs)[P.PC + (tid & 15)] = u32x4{0u, 0u, 0u, 0u};
         if (tid == 0) flag[1] = 2 * NW;
-        // the slice copies were issued before everything except the STREAM_PF loads of the first steps
-        __builtin_amdgcn_s_waitcnt(stream_vmcnt_only(STREAM_PF));
+        // the slice copies were issued before everything except the STREAM_PF loads of the first steps (or last of all)
+        if (kd > 0) __builtin_amdgcn_s_waitcnt(stream_vmcnt_only(0));
+        else __builtin_amdgcn_s_waitcnt(stream_vmcnt_only(STREAM_PF));
         SQ_TRACE_POINT(10);
     }
     __syncthreads();
@@ -851,6 +969,11 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         const int cnt = (int)(h.slot >> STREAM_ROW_BITS);
         const uint32_t row = h.slot & STREAM_NO_ROW;
         const unsigned char* eb = steps + (size_t)h.st0 * 768;
+        // the copy of x for this group's column order
+        int xc = 0;
+#pragma unroll
+        for (int oi = 1; oi < STREAM_RUN_ORDERS; ++oi) xc += (oi < no && kcur >= byte_of(bnd_lo, bnd_hi, oi)) ? 1 : 0;
+        const unsigned char* ldsx_u = ldsx + (size_t)xc * NB * xs;
         float acc[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) acc[b] = 0.f;
@@ -881,7 +1004,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                         const uint32_t ta = (e[j0 + jj] & 0xFFFu) << 4, xa = ((e[j0 + jj] >> 12) & 0xFFFu) << 4;
                         cw[jj] = *reinterpret_cast<const u32x4*>(lds + ta);
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx + b * xs + xa);
+                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx_u + b * xs + xa);
                     }
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
@@ -965,7 +1088,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     const size_t ysz = a.y_dtype == SQ_F32 ? 4 : 2;
     for (int it = i_lo + tid; it < i_hi; it += NTH) {
         const int b = it / nl, i = it - b * nl;
-        const uint32_t r = P.perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
+        const uint32_t r = perms ? rows0[i] : (g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW);
         const float rs = h2f(P.row_scale[r != STREAM_NO_ROW ? r : 0u]);
         uint32_t* q = pp + (size_t)b * np + i;
         const size_t bs = (size_t)NB * np;                      // words from one bucket's partial sums to the next
@@ -1012,20 +1135,25 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 }
 
 // LDS bytes of a launch: slice, NB parts of x, NB partial-sum vectors of the longest run, flags, block sums
-static size_t stream_smem(int nb_t, int xs, int nl_max) {
-    return (size_t)STREAM_TAB + (size_t)nb_t * xs + (size_t)nb_t * nl_max * 4 + 16 + 64;
+static size_t stream_smem(int nb_t, int xs, int nl_max, int xcopies = 1, int xtmp = 0) {
+    return (size_t)STREAM_TAB + (size_t)xcopies * nb_t * xs + (size_t)nb_t * nl_max * 4 + 16 + 64 + (size_t)nb_t * xtmp;
 }
 
-template <int NB, int NX, int PRO = 0>
-static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
+template <int NB, int NX, int PRO, int ORD>
+static int stream_launch_as(const StreamArgs& a, int grid, hipStream_t s) {
     static bool raised = false;
     if (!raised) {
-        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NX, PRO>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NX, PRO, ORD>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         (void)hipGetLastError();
         raised = true;
     }
-    hipLaunchKernelGGL((stream_kernel<NB, NX, PRO>), dim3((unsigned)grid), dim3(STREAM_NW * 64), stream_smem(NB, a.xs, a.nl_max), s, a);
+    hipLaunchKernelGGL((stream_kernel<NB, NX, PRO, ORD>), dim3((unsigned)grid), dim3(STREAM_NW * 64), stream_smem(NB, a.xs, a.nl_max, a.xcopies, a.xtmp_own ? a.xtmp : 0), s, a);
     return check_launch("sq_linear_small(stream)");
+}
+// (a.orders: some piece of the launch has column orders)
+template <int NB, int NX, int PRO = 0>
+static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
+    return a.orders ? stream_launch_as<NB, NX, PRO, 1>(a, grid, s) : stream_launch_as<NB, NX, PRO, 0>(a, grid, s);
 }
 
 // ---- dense rows from the tag stream alone (a matrix held in one copy: sq_matrix.tags == NULL).  One wave per (bucket,
@@ -1167,7 +1295,9 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         if (tot <= SQ_WS_HEADER) break;
         if (rows == 1) return fail(SQ_EUNSUPPORTED, "sq_linear_small: the partial sums of these pieces (%zu bytes) do not fit the workspace header", tot);
     }
-    int wg = 0, pc = 0, nl_max = 64;
+    int wg = 0, pc = 0, nl_max = 64, xcopies = 1, xtmp = 0;
+    a.orders = 0;
+    bool one_part = true;                                       // every piece with column orders has one column part
     size_t sums_off = 0;
     for (int k = 0; k < cnt; ++k) {
         const sq_matrix& m = mats[k];
@@ -1196,20 +1326,33 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         wg += g.NV * nwg;
         pc = g.PC;                                               // (pieces of one launch share C)
         nl_max = std::max(nl_max, run_max * 64);
+        if (m.perms) {
+            a.orders = 1;
+            xcopies = std::max(xcopies, stream_run_orders_of(m));
+            xtmp = std::max(xtmp, (m.C * 2 + 15) & ~15);
+            one_part = one_part && g.U == g.PC;
+        }
     }
     for (int k = cnt; k < GEMV_MAX_PIECES_STREAM; ++k) a.p[k] = a.p[0];
     a.xs = stream_xs(pc);
     a.nl_max = nl_max;
-    if (stream_smem(1, a.xs, a.nl_max) > 160 * 1024)
-        return fail(SQ_EUNSUPPORTED, "sq_linear_small: rows of %d chunks per column part do not fit LDS", pc);
-    const bool nx4 = pc > STREAM_NW * 64;
+    a.xcopies = xcopies;
+    a.xtmp = a.xtmp_own = 0;
+    if (from || !one_part) xtmp = 0;                            // (produced rows and rows of several parts: gathered from memory)
+    if (stream_smem(1, a.xs, a.nl_max, xcopies) > 160 * 1024 || pc * xcopies > 4 * STREAM_NW * 64)
+        return fail(SQ_EUNSUPPORTED, "sq_linear_small: %d copies of a row part of %d chunks do not fit LDS", xcopies, pc);
+    const bool nx4 = pc * xcopies > STREAM_NW * 64;             // chunks of x (over all its copies) per thread: 1 or 4
     if (from) {
         if (B != 1) return fail(SQ_EINVAL, "sq_linear_small_from: fused producers take one activation row");
         a.x = (const uint16_t*)x; a.y = y; a.nb = 1;
         if (from->mode != SQ_FROM_ADDNORM) return fail(SQ_EINVAL, "sq_linear_small_from: only add + norm is produced inside the kernel");
         return nx4 ? stream_launch<1, 4, 1>(a, wg, s) : stream_launch<1, 1, 1>(a, wg, s);
     }
-    while (rows > 1 && stream_smem(rows, a.xs, a.nl_max) > 160 * 1024) rows >>= 1;
+    while (rows > 1 && stream_smem(rows, a.xs, a.nl_max, xcopies) > 160 * 1024) rows >>= 1;
+    // Column orders are applied from copies of the rows in LDS: in LDS of their own where that is left, else where
+    // the slice lands afterwards (that part of the slice is then copied a round trip later), if they fit there.
+    a.xtmp_own = xtmp > 0 && stream_smem(rows, a.xs, a.nl_max, xcopies, xtmp) <= 160 * 1024;
+    a.xtmp = a.xtmp_own || rows * xtmp <= STREAM_TAB ? xtmp : 0;
     const size_t ysz = y_dtype == SQ_F32 ? 4 : 2;
     for (int b0 = 0; b0 < B; b0 += rows) {
         a.x = (const uint16_t*)((const char*)x + (size_t)b0 * ldx * 2);

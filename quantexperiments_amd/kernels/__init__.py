@@ -234,12 +234,17 @@ def prepare_stack(pieces, workgroups: int | None = None) -> None:
         return
     if workgroups is None:
         workgroups = torch.cuda.get_device_properties(ps[0].device).multi_processor_count
+    # Smallest piece first: a piece with column orders can need more runs than its share (a run holds the whole
+    # groups of a few orders), and what it takes beyond its share comes off the larger pieces' runs, so the launch
+    # still fits the device in one round of workgroups.
     rows = sum(p.R for p in ps)
-    for p in ps:
+    for p in sorted(ps, key=lambda q: q.R):
         buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // STREAM_PART_MAX)
         runs = max(1, round(workgroups * p.R / rows / buckets))
         if p.words is not None and (p.stream is None or (runs != p.stream_asked and not (len(ps) == 1 and p.stream_asked == 0))):
             p.build_stream(runs)
+        workgroups = max(workgroups - (p.stream_runs & 0xFFFF) * buckets, buckets)
+        rows -= p.R
 
 
 def _prep(pieces, x: torch.Tensor, y: torch.Tensor):

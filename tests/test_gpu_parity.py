@@ -246,10 +246,19 @@ def test_stream_gemv_matches_oracle_and_row_path(case, dtype):
                 linear_small([lin], xb[b:b + 1].cuda(), y2)
                 assert torch.equal(y2[0], yb[b, :R]), (B, b)
     # another cut into row runs: same sums up to the order of fp32 additions within a row
+    # (with column orders a run then holds the groups of up to four orders, each reading its own gathered copy of x,
+    # and the copies are made from the rows held in LDS: beside the slice at 1 row, in its place at more)
     for runs in (1, 3):
         lin.build_stream(runs)
         linear_small([lin], x.cuda(), y2)
         assert rel_max_err(y2.cpu().numpy(), y32.cpu().numpy().astype(np.float64)) < 1e-5
+        if M > 1:
+            assert runs > 1 or C > 16384 or (lin.stream_runs >> 24) & 7 >= 1   # several orders per run
+            for B in (2, 4, 7):
+                xb = rand_x(B, C, dtype, seed=R + B + runs)
+                yb = torch.full((B, R + 3), 5.0, dtype=torch.float32, device="cuda")
+                linear_small([lin], xb.cuda(), yb[:, :R])
+                assert rel_max_err(yb[:, :R].cpu().numpy(), _ref(s, xb)) < TOL and (yb[:, R:] == 5.0).all()
 
 
 def test_workspace_header_is_zero_after_every_stream_launch():

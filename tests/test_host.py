@@ -220,7 +220,7 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
     NV = NS * KP
     off_slots = ((NV * NG + 1) * 4 + 255) & ~255
     off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
-    off_rows = (off_runs + runs * 16 + 255) & ~255
+    off_rows = (off_runs + runs * 32 + 255) & ~255
     off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
     unmap = None
     if table is not None:
@@ -233,7 +233,9 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
         assert np.array_equal(moved, table.view(np.uint16).reshape(K, d)[unmap])   # codeword `new` is the file's unmap[new]
     goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
     slots = np.frombuffer(buf, np.uint32, NV * NG * 64, off_slots).reshape(NV, NG * 64)
-    rt = np.frombuffer(buf, np.int32, runs * 4, off_runs).reshape(runs, 4)
+    rt = np.frombuffer(buf, np.int32, runs * 8, off_runs).reshape(runs, 8)[:, :4]       # g0, ng, column orders, 0
+    rb = np.frombuffer(buf, np.uint8, runs * 32, off_runs).reshape(runs, 32)
+    bounds, orders = rb[:, 16:24], rb[:, 24:32]                               # first group (in the run) and id of each order
     base = np.frombuffer(buf, np.uint32, NG * 64, off_rows)                   # place -> row
     assert sorted(base[base != 0x7FFFF].tolist()) == list(range(R))
     if row_mask is None:
@@ -242,7 +244,8 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
     assert len(buf) == off_steps + int(goff[-1]) * 768
     # runs tile the groups in order; every run has one column order
     assert rt[0, 0] == 0 and (rt[1:, 0] == rt[:-1, 0] + rt[:-1, 1]).all() and rt[-1, 0] + rt[-1, 1] == NG
-    assert (rt[:, 1] >= 1).all() and (rt[:, 3] == 0).all() and (np.diff(rt[:, 2]) >= 0).all()
+    assert (rt[:, 1] >= 1).all() and (rt[:, 3] == 0).all() and (rt[:, 2] >= 1).all() and (rt[:, 2] <= 4).all()
+    assert (bounds[:, 0] == 0).all() and (rt[:, 2] == 1).all() or row_mask is not None
     if row_mask is None:                                                      # the cut the kernel derives from the run count
         gr = -(-NG // runs)
         assert (rt[:, 0] == np.arange(runs) * gr).all() and (rt[:, 1] == np.minimum(gr, NG - rt[:, 0])).all()
@@ -259,14 +262,21 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
         assert (rows[real] != 0x7FFFF).all()
         assert sorted(rows[real].tolist()) == list(range(R))                  # every row once per bucket
         sets = []
-        for g0, ng, order, _ in rt:                                           # sorted by count within each run
+        for ri, (g0, ng, no, _) in enumerate(rt):
             sl = slice(g0 * 64, (g0 + ng) * 64)
-            assert (np.diff(cnts[sl][real[sl]].astype(np.int64)) <= 0).all()
-            assert real[sl][:int(real[sl].sum())].all()                       # rows first, empty lanes last
             sets.append(frozenset(rows[sl][real[sl]].tolist()))
             assert ((places[sl][real[sl]] >= g0 * 64) & (places[sl][real[sl]] < (g0 + ng) * 64)).all()
-            if row_mask is not None:
-                assert (row_mask[rows[sl][real[sl]]] == order).all()
+            # the run's column orders: groups bound[i] .. bound[i + 1] - 1 of the run hold rows of order[i] only, in
+            # every bucket (a group reads one copy of x), sorted by count, rows first and empty lanes last
+            bnd = [int(b) for b in bounds[ri, :no]] + [int(ng)]
+            assert bnd[0] == 0 and all(a < b for a, b in zip(bnd, bnd[1:]))
+            for oi in range(no):
+                so = slice((g0 + bnd[oi]) * 64, (g0 + bnd[oi + 1]) * 64)
+                assert (np.diff(cnts[so][real[so]].astype(np.int64)) <= 0).all()
+                assert real[so][:int(real[so].sum())].all() and real[so].any()
+                assert sorted(rows[so][real[so]].tolist()) == sorted(base[so][base[so] != 0x7FFFF].tolist())
+                if row_mask is not None:
+                    assert (row_mask[rows[so][real[so]]] == orders[ri, oi]).all()
         run_rows = run_rows or sets
         assert sets == run_rows                                               # the same rows in every bucket's run
         for g in range(NG):
@@ -356,18 +366,18 @@ def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask, PF=3, NW=16):
     NV = NS * KP
     off_slots = ((NV * NG + 1) * 4 + 255) & ~255
     off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
-    off_rows = (off_runs + runs * 16 + 255) & ~255
+    off_rows = (off_runs + runs * 32 + 255) & ~255
     off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
     if balanced:                                        # relabelled codebook and back map sit in front of the steps
         yield "codebook slices", off_steps, off_steps + (16 << bits)
         off_steps = (off_steps + (18 << bits) + 255) & ~255
     goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0).astype(np.int64)
-    rt = np.frombuffer(buf, np.int32, runs * 4, off_runs).reshape(runs, 4)
+    rt = np.frombuffer(buf, np.int32, runs * 8, off_runs).reshape(runs, 8)
     gr = -(-NG // runs)
     for v in range(NV):
         for wi in range(runs):
             if row_mask is not None:
-                yield "run table", off_runs + wi * 16, off_runs + wi * 16 + 12
+                yield "run table", off_runs + wi * 32, off_runs + wi * 32 + 32
                 g0, ng = int(rt[wi, 0]), int(rt[wi, 1])
             else:
                 g0, ng = wi * gr, min(gr, NG - wi * gr)
@@ -454,7 +464,7 @@ def test_stream_builder_orders_entries_for_the_lds_banks():
     NV = 16
     off_slots = ((NV * NG + 1) * 4 + 255) & ~255
     off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
-    off_rows = (off_runs + runs * 16 + 255) & ~255
+    off_rows = (off_runs + runs * 32 + 255) & ~255
     off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
     goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
     steps = np.frombuffer(buf, np.uint8, int(goff[-1]) * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.int64)
