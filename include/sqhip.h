@@ -234,12 +234,13 @@ int sq_silu_mul(const void* gate, const void* up, int dtype, int64_t ld, const i
 
 /* sq_linear_small whose activations X [B, C] are produced by one of the two neighbours above instead of being read:
  * the same results, bit for bit, as sq_addnorm / sq_silu_mul (perms = NULL) into x_out followed by sq_linear_small
- * on x_out.  For one activation row of pieces that run on the tag-stream kernel (codebooks beyond LDS, or column
- * orders) the add + norm producer is fused into that kernel: every workgroup computes its part of the row while it
- * stages it (the mean square of the whole row included, in the stand-alone kernel's summation order), so no launch
- * and no dependency bubble sit between the two; otherwise, and always for SiLU * up (whose exponentials every
- * workgroup would have to repeat for the whole row: measured slower than the extra launch), the library launches
- * the stand-alone kernel first.  This is the
+ * on x_out.  For one activation row of pieces that run on the tag-stream kernel (codebooks beyond LDS) and have no
+ * column orders the add + norm producer is fused into that kernel: every workgroup computes its part of the row while
+ * it stages it (the mean square of the whole row included, in the stand-alone kernel's summation order), so no launch
+ * and no dependency bubble sit between the two; otherwise (with column orders every workgroup would gather the
+ * producer's operands through each order of its run), and always for SiLU * up (whose exponentials every workgroup
+ * would have to repeat for the whole row), both measured slower than the extra launch, the library launches the
+ * stand-alone kernel first.  This is the
  * counterpart of the reference's epi argument (reference shapequant/kernels/proto_runs.py:505-571, EPI 1 / EPI 2 at
  * :223-287), turned round: there the producing kernel's last blocks write the next product's input, here the
  * consuming kernel's workgroups compute it, which needs no launch-wide ticket and no cross-die visibility.

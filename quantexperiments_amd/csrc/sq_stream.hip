@@ -576,20 +576,6 @@ __device__ __forceinline__ ProRaw pro_fetch(const StreamArgs& a, int ci) {
     }
     return r;
 }
-// the 8 elements idx[0..7] (a chunk of a column order)
-template <int PRO>
-__device__ __forceinline__ ProRaw pro_gather(const StreamArgs& a, const int32_t* idx) {
-    ProRaw r;
-    const uint16_t* hp = a.w;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const int i0 = idx[2 * k], i1 = idx[2 * k + 1];
-        r.hi[k] = (uint32_t)hp[i0] | ((uint32_t)hp[i1] << 16);
-        r.lo[k] = a.add ? ((uint32_t)a.add[i0] | ((uint32_t)a.add[i1] << 16)) : 0u;
-        if (PRO == 1) { r.h[2 * k] = a.h_in[i0]; r.h[2 * k + 1] = a.h_in[i1]; }
-    }
-    return r;
-}
 __device__ __forceinline__ float pro_f(uint32_t pair, int k, int dtype) {
     const uint16_t b = (uint16_t)(pair >> (16 * (k & 1)));
     return dtype == SQ_BF16 ? bf2f(b) : h2f(b);
@@ -640,7 +626,7 @@ typedef __attribute__((address_space(3))) void* stream_lptr_t;
 // [16 block sums (PRO 1)].
 template <int NB, int NX, int PRO = 0, int ORD = 1>
 __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
-    static_assert(PRO == 0 || (PRO == 1 && NB == 1), "produced activations: add + norm, one row");
+    static_assert(PRO == 0 || (PRO == 1 && NB == 1 && ORD == 0), "produced activations: add + norm, one row, no column orders");
     constexpr int NW = STREAM_NW, NTH = NW * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -781,13 +767,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         if (PRO != 0) {
             // every operand of the produced row is requested before anything waits: this thread's chunks, then
             // (PRO 1) its share of the whole row for the mean square
-            const bool pm = perms != nullptr;
             ProRaw raw[NX];
 #pragma unroll
-            for (int k = 0; k < NX; ++k) {
-                const int ci = c0 + it_c[k];
-                raw[k] = pm ? pro_gather<PRO>(a, perms + (size_t)byte_of(ord_lo, ord_hi, it_o[k]) * P.C + (size_t)ci * 8) : pro_fetch<PRO>(a, ci);
-            }
+            for (int k = 0; k < NX; ++k) raw[k] = pro_fetch<PRO>(a, c0 + it_c[k]);
             float rstd = 0.f;
             if (PRO == 1) {
                 // Mean square of the whole row in the stand-alone kernel's order, so both give the same bits: slot j
@@ -797,7 +779,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                 static_assert(NTH == 1024, "one slot per thread");
                 float* red = reinterpret_cast<float*>(flag + 4);
                 float ps = 0.f;
-                if (!pm && nc == P.U && P.U <= NX * NTH) {
+                if (nc == P.U && P.U <= NX * NTH) {
                     // one column part, natural order: this thread's chunks are its slot's chunks, already fetched
 #pragma unroll
                     for (int k = 0; k < NX; ++k)
@@ -830,28 +812,17 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
             for (int k = 0; k < NX; ++k) xq[0][k] = pro_finish<PRO>(a, raw[k], rstd);
             if (pi == 0 && s == 0 && wi == 0) {
                 // one workgroup per column part leaves the produced row (and the updated residual) in memory
-                if (!pm) {
 #pragma unroll
-                    for (int k = 0; k < NX; ++k) {
-                        const int c = tid + k * NTH;
-                        if (c >= nc) continue;
-                        reinterpret_cast<u32x4*>(a.x_out)[c0 + c] = xq[0][k];
-                        if (PRO == 1 && a.h_out) {
-                            float4v o0, o1;
+                for (int k = 0; k < NX; ++k) {
+                    const int c = tid + k * NTH;
+                    if (c >= nc) continue;
+                    reinterpret_cast<u32x4*>(a.x_out)[c0 + c] = xq[0][k];
+                    if (PRO == 1 && a.h_out) {
+                        float4v o0, o1;
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) { o0[e] = pro_v(a, raw[k], e); o1[e] = pro_v(a, raw[k], 4 + e); }
-                            reinterpret_cast<float4v*>(a.h_out)[2 * (c0 + c)] = o0;
-                            reinterpret_cast<float4v*>(a.h_out)[2 * (c0 + c) + 1] = o1;
-                        }
-                    }
-                } else {
-                    for (int c = tid; c < nc; c += NTH) {
-                        const ProRaw r = pro_fetch<PRO>(a, c0 + c);
-                        reinterpret_cast<u32x4*>(a.x_out)[c0 + c] = pro_finish<PRO>(a, r, rstd);
-                        if (PRO == 1 && a.h_out) {
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) a.h_out[(c0 + c) * 8 + e] = pro_v(a, r, e);
-                        }
+                        for (int e = 0; e < 4; ++e) { o0[e] = pro_v(a, raw[k], e); o1[e] = pro_v(a, raw[k], 4 + e); }
+                        reinterpret_cast<float4v*>(a.h_out)[2 * (c0 + c)] = o0;
+                        reinterpret_cast<float4v*>(a.h_out)[2 * (c0 + c) + 1] = o1;
                     }
                 }
             }
@@ -1153,7 +1124,11 @@ static int stream_launch_as(const StreamArgs& a, int grid, hipStream_t s) {
 // (a.orders: some piece of the launch has column orders)
 template <int NB, int NX, int PRO = 0>
 static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
-    return a.orders ? stream_launch_as<NB, NX, PRO, 1>(a, grid, s) : stream_launch_as<NB, NX, PRO, 0>(a, grid, s);
+    if (PRO != 0) {
+        if (a.orders) return fail(SQ_EUNSUPPORTED, "sq_linear_small_from: no fused kernel for pieces with column orders");
+        return stream_launch_as<NB, NX, PRO, 0>(a, grid, s);
+    }
+    return a.orders ? stream_launch_as<NB, NX, 0, 1>(a, grid, s) : stream_launch_as<NB, NX, 0, 0>(a, grid, s);
 }
 
 // ---- dense rows from the tag stream alone (a matrix held in one copy: sq_matrix.tags == NULL).  One wave per (bucket,
