@@ -744,6 +744,35 @@ def test_full_7b_layer_stacked_launches_against_c_oracle(launch):
     assert torch.equal(yb, y.to(torch.bfloat16))              # the 16-bit output is the fp32 one rounded once
 
 
+@pytest.mark.parametrize("B", [1, 2, 5])
+def test_full_27b_masked_qkv_stack_against_oracle(B):
+    """The q|k|v launch of the masked 27B-shaped layer the benchmark times (5120 + 1024 + 1024 rows of 5120 columns,
+    16 column orders each, d = 8, 16-bit tags), stacked and cut for the joint launch: the small pieces' runs hold the
+    groups of four column orders (four gathered copies of x, four chunks per thread), the large piece's of two, and
+    with more than one activation row the rows' natural-order copies sit where the slice lands."""
+    from quantexperiments_amd.kernels import linear_small, prepare_stack
+    C = 5120
+    x = rand_x(B, C, torch.bfloat16, seed=B)
+    pieces, refs = [], []
+    for k, R in enumerate((5120, 1024, 1024)):
+        s = synth(R, C, 8, 16, 1, 16, seed=40 + k)
+        pieces.append(to_device(s, stream="later"))
+        refs.append(_ref(s, x))
+    prepare_stack(pieces)
+    assert all(p.stream is not None for p in pieces)
+    orders = [((p.stream_runs >> 24) & 7) + 1 for p in pieces]
+    assert orders[0] >= 2 and orders[1] == 4 and orders[2] == 4
+    # one round of workgroups: 16 buckets per run, one workgroup per compute unit
+    assert sum(p.stream_runs & 0xFFFF for p in pieces) * 16 <= torch.cuda.get_device_properties(0).multi_processor_count
+    ref = np.concatenate(refs, axis=1)
+    y = torch.full((B, ref.shape[1]), 7.0, dtype=torch.float32, device="cuda")
+    linear_small(pieces, x.cuda(), y)
+    assert rel_max_err(y.cpu().numpy(), ref) < TOL
+    yb = torch.empty(B, ref.shape[1], dtype=torch.bfloat16, device="cuda")
+    linear_small(pieces, x.cuda(), yb)
+    _check_lowp(yb, ref)
+
+
 @pytest.mark.parametrize("shape", [(18944, 3584, 1), (3584, 18944, 1), (5120, 5120, 16)], ids=lambda c: "x".join(map(str, c)))
 def test_full_size_gemm_rows_against_gemv(shape):
     """M = 2048 prefill at the 7B gate/up and down sizes and at a 27B-class matrix with 16 column orders: every
