@@ -15,6 +15,23 @@ constexpr int GEMV_MAX_PIECES_STREAM = 4;
 constexpr int STREAM_RUN_ORDERS = 8;         // most column orders whose rows may share a run (one gathered copy of x in LDS each)
 
 constexpr int STREAM_DEFAULT_WGS = 256;      // workgroups a matrix launched alone should make (one per CU on 256 CUs)
+constexpr int STREAM_NW = 16;                // waves per workgroup of the kernel: one workgroup per CU
+constexpr int STREAM_PF = 3;                 // steps the kernel fetches ahead (2 to 4 measure alike, 6 and 8 slower), and the steps
+                                             // of every unit that the buffer keeps in its first-steps region
+
+// A unit is what one wave walks without a break: a group of a run, or, in a run of at most STREAM_NW / 2 groups, one of
+// the STREAM_NW / groups contiguous shares of a group's steps (share j of `split`: steps [nst j / split, nst (j + 1) / split)).
+__host__ __device__ inline int stream_split_of(int ng) { return ng * 2 <= STREAM_NW ? STREAM_NW / ng : 1; }
+
+// Where the steps are (all positions in 768-byte steps from off_steps).  The first STREAM_PF steps of every unit sit in a
+// region of their own, at a place that follows from the unit's index alone: ((unit * NV + bucket) * STREAM_PF), so a
+// wave can ask for them before it has read anything else of the buffer; a launch then starts with one round trip to
+// memory instead of two (offsets, then steps).  The remaining steps of a group follow each other in the rest region,
+// share after share.  Per (bucket, group) the buffer holds four words: {rest, nst, unit0, split} = the place of the
+// group's first remaining step, its step count, the index of its first unit and its share count; when every share has
+// at least STREAM_PF steps (nst / split >= STREAM_PF), step t of share j (t counted within the group) is at
+// rest + t - STREAM_PF (j + 1) once it is past the share's first STREAM_PF; otherwise the first-steps region holds
+// the whole group.
 
 struct StreamGeom {
     int U, NS, KP, PC, NV, NG;               // chunks per row, slices, column parts, chunks per part, buckets, groups

@@ -22,15 +22,15 @@
 // order (so results do not depend on scheduling), apply the row scale, store y and put zero back.
 //
 // Stream buffer (one allocation; offsets follow from C/d, the tag width, the group and run counts):
-//   goff   uint32 [NV * NG + 1]   first step of every group, cumulative over buckets (NV = KP * NS buckets,
-//                                 NG groups per bucket, bucket v = kp * NS + s)
+//   heads  uint32 [NV * NG][4]    {rest, nst, unit0, split} of every group (NV = KP * NS buckets, NG groups per bucket,
+//                                 bucket v = kp * NS + s): where its steps are, see sq_stream.h
 //   slots  uint32 [NV * NG * 64]  place | count << 19 per lane; place = the row's index in `rows` (below),
 //                                 0x7FFFF marks a lane without a row; lanes 64 g .. 64 g + 63 of a bucket are group g
-//   runs   [runs] x 32 bytes       first group, group count, column orders of the run, 0; first group (within the run) and
-//                                 id of each of up to 8 column orders (one byte each)
+//   runs   [runs] x 32 bytes       first group, group count, column orders of the run, index of its first unit; first
+//                                 group (within the run) and id of each of up to 8 column orders (one byte each)
 //   rows   uint32 [NG * 64]       the rows ordered by column order, 64 per group (0x7FFFF where a group is short):
 //                                 places 64 g0 .. 64 (g0 + ng) - 1 are a run's rows, and partial sums are indexed by place
-//   steps  [total][64][3] uint32  entries
+//   steps  [total][64][3] uint32  entries: the first-steps region (STREAM_PF steps per unit and bucket), then the rest
 #include <algorithm>
 #include <string.h>
 #include <thread>
@@ -44,7 +44,8 @@ namespace sq {
 // A run: groups g0 .. g0 + ng - 1 of every bucket.  Its rows belong to `norders` column orders (one without row orders);
 // the groups of order[i] begin at group bound[i] of the run (bound[0] = 0), and the kernel keeps copy i of x, gathered
 // through that order, in LDS for them.
-struct StreamRun { int32_t g0, ng, norders, zero; uint8_t bound[STREAM_RUN_ORDERS]; uint8_t order[STREAM_RUN_ORDERS]; };
+// u0: the index of the run's first unit (units are counted run after run).
+struct StreamRun { int32_t g0, ng, norders, u0; uint8_t bound[STREAM_RUN_ORDERS]; uint8_t order[STREAM_RUN_ORDERS]; };
 static_assert(sizeof(StreamRun) == 32, "run records are read as 8 dwords");
 
 StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced) {
@@ -56,7 +57,7 @@ StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanc
     g.NV = g.NS * g.KP;
     g.NG = groups;
     g.runs = runs;
-    g.off_slots = (((size_t)g.NV * g.NG + 1) * 4 + 255) & ~(size_t)255;
+    g.off_slots = ((size_t)g.NV * g.NG * 16 + 255) & ~(size_t)255;          // four words per (bucket, group)
     g.off_runs = (g.off_slots + (size_t)g.NV * g.NG * 64 * 4 + 255) & ~(size_t)255;
     g.off_rows = (g.off_runs + (size_t)runs * sizeof(StreamRun) + 255) & ~(size_t)255;
     size_t end = (g.off_rows + (size_t)g.NG * 64 * 4 + 255) & ~(size_t)255;
@@ -108,7 +109,12 @@ struct StreamPlan {
     std::vector<uint32_t> base;      // [NG * 64]: rows ordered by column order, STREAM_NO_ROW where a group is short
     std::vector<uint16_t> cnt;       // [NV][R]
     std::vector<uint32_t> pos;       // [NV][R]: lane position (group * 64 + lane) of row r in bucket v
-    std::vector<uint32_t> goff;      // [NV * NG + 1]
+    std::vector<uint32_t> goff;      // [NV * NG + 1]: the groups' steps counted bucket after bucket, group after group (how the
+                                     // builder lays them out before they move to their places)
+    uint64_t logical_steps;          // goff[NV * NG]
+    int NU;                          // units of one bucket
+    std::vector<uint32_t> run_of;    // [NG]: the run of a group
+    std::vector<uint32_t> head4;     // [NV * NG][4]: {rest, nst, unit0, split}, what the buffer holds per (bucket, group)
     std::vector<uint16_t> remap;     // balanced streams: file id -> new id (empty: identity)
 };
 
@@ -264,7 +270,31 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     uint64_t tot = 0;
     for (size_t k = 0; k < steps.size(); ++k) { P.goff[k] = (uint32_t)tot; tot += steps[k]; }
     P.goff[steps.size()] = (uint32_t)tot;
-    P.g.total_steps = tot;
+    P.logical_steps = tot;
+    // Units and places: the first-steps region (NU units x NV buckets x STREAM_PF steps) comes first, the groups'
+    // remaining steps follow bucket after bucket, group after group.
+    P.NU = 0;
+    P.run_of.assign(g.NG, 0);
+    for (size_t ri = 0; ri < P.runs.size(); ++ri) {
+        StreamRun& run = P.runs[ri];
+        run.u0 = P.NU;
+        P.NU += run.ng * stream_split_of(run.ng);
+        for (int k = 0; k < run.ng; ++k) P.run_of[run.g0 + k] = (uint32_t)ri;
+    }
+    P.head4.assign((size_t)g.NV * g.NG * 4, 0);
+    uint64_t at = (uint64_t)P.NU * g.NV * STREAM_PF;
+    for (int v = 0; v < g.NV; ++v)
+        for (int gi = 0; gi < g.NG; ++gi) {
+            const StreamRun& run = P.runs[P.run_of[gi]];
+            const uint32_t split = (uint32_t)stream_split_of(run.ng), nst = steps[(size_t)v * g.NG + gi];
+            uint32_t* h = &P.head4[((size_t)v * g.NG + gi) * 4];
+            h[0] = (uint32_t)at;
+            h[1] = nst;
+            h[2] = (uint32_t)run.u0 + (uint32_t)(gi - run.g0) * split;
+            h[3] = split;
+            if (nst / split >= (uint32_t)STREAM_PF) at += nst - split * STREAM_PF;
+        }
+    P.g.total_steps = at;
 }
 
 size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
@@ -443,7 +473,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
     if (g.total_steps >= ((uint64_t)1 << 32) || g.runs >= (1 << 16)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: matrix too large");
     if (bytes < need) return fail(SQ_EINVAL, "sq_stream_build: buffer %zu < %zu", bytes, need);
     memset(out, 0, need);
-    memcpy(out, P.goff.data(), P.goff.size() * 4);
+    memcpy(out, P.head4.data(), P.head4.size() * 4);
     memcpy(out + g.off_runs, P.runs.data(), P.runs.size() * sizeof(StreamRun));
     memcpy(out + g.off_rows, P.base.data(), P.base.size() * 4);
     if (table) {
@@ -459,7 +489,9 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
         if (P.base[k] != STREAM_NO_ROW) place[P.base[k]] = (uint32_t)k;
     uint32_t* slots = (uint32_t*)(out + g.off_slots);
     for (size_t k = 0; k < (size_t)g.NV * g.NG * 64; ++k) slots[k] = STREAM_NO_ROW;
-    unsigned char* steps = out + g.off_steps;
+    // the steps are made group after group (P.goff) in a buffer of their own and moved to their places at the end
+    std::vector<unsigned char> laid((size_t)P.logical_steps * 768, 0);
+    unsigned char* steps = laid.data();
     parallel_rows(R, [&](int a, int b) {
         std::vector<uint32_t> q(g.NV), last(g.NV);
         for (int r = a; r < b; ++r) {
@@ -509,6 +541,22 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             const uint32_t* sl = slots + (size_t)vg * 64;
             unsigned char* base = steps + (size_t)st0 * 768;
             for (int q = 0; q < 4; ++q) bm.order_lanes(base, sl, LDS_CLOCK_LANES[q], ns, (uint32_t)g.PC);
+        }
+    });
+    // to their places: the first STREAM_PF steps of every unit into the first-steps region, the rest behind each other
+    parallel_rows(g.NV * g.NG, [&](int a, int b) {
+        for (int vg = a; vg < b; ++vg) {
+            const uint32_t* h = &P.head4[(size_t)vg * 4];
+            const int v = vg / g.NG, nst = (int)h[1], split = (int)h[3];
+            const unsigned char* src = steps + (size_t)P.goff[vg] * 768;
+            for (int j = 0; j < split; ++j) {
+                const int s0 = nst * j / split, s1 = nst * (j + 1) / split;
+                for (int t = s0; t < s1; ++t) {
+                    const uint64_t to = t - s0 < STREAM_PF ? ((uint64_t)(h[2] + j) * g.NV + v) * STREAM_PF + (t - s0)
+                                                           : (uint64_t)h[0] + t - (uint64_t)STREAM_PF * (j + 1);
+                    memcpy(out + g.off_steps + to * 768, src + (size_t)t * 768, 768);
+                }
+            }
         }
     });
     if (runs_out) *runs_out = g.runs | (P.GR << 16) | ((P.orders_max - 1) << 24) | (table ? STREAM_BALANCED : 0);
@@ -595,15 +643,17 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 }
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
-constexpr int STREAM_PF = 3;          // steps fetched ahead (2 to 4 measure alike, 6 and 8 slower: the loop runs at the memory system's rate)
-constexpr int STREAM_NW = 16;         // waves per workgroup: one workgroup per CU
 constexpr uint32_t STREAM_ZERO_SUM = 0x7FFFFFFFu;  // how a partial sum with all bits zero is written (zero = not there yet)
 constexpr int STREAM_SPIN_MAX = 1 << 18;           // polls of an item's partial sums before it gives up
 
 // LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group)
 static inline int stream_xs(int pc) { return (pc + 16) * 16; }
 
-struct StreamHead { uint32_t st0; int nst; uint32_t slot; };
+// what a wave walks of a group: nst steps, of which step t >= STREAM_PF is step rb + t of the buffer (the first STREAM_PF
+// are in the first-steps region), and this lane's slot
+struct StreamHead { uint32_t rb; int nst; uint32_t slot; };
+// a group's words as loaded ({rest, nst, unit0, split} and this lane's slot) and its index in the run
+struct StreamHeadRaw { uint32_t rest, nst, sl; int k; };
 
 // Optional per-wave timeline (debug builds define SQ_TRACE_POINT).
 #ifndef SQ_TRACE_POINT
@@ -667,7 +717,8 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     const uint32_t ord_lo = perms ? (uint32_t)run[6] : 0u, ord_hi = perms ? (uint32_t)run[7] : 0u;
     auto byte_of = [](uint32_t lo, uint32_t hi, int i) { return (int)(((i < 4 ? lo >> (8 * i) : hi >> (8 * (i - 4)))) & 0xFFu); };
 
-    const uint32_t* goff = reinterpret_cast<const uint32_t*>(P.stream) + (size_t)v * P.NG + g0;
+    const u32x4* gw = reinterpret_cast<const u32x4*>(P.stream) + (size_t)v * P.NG + g0;   // {rest, nst, unit0, split} per group
+    const int u0 = perms ? run[3] : wi * gr * stream_split_of(gr);   // this run's first unit
     const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
     const unsigned char* steps = P.stream + P.off_steps + lane * 12;
     const size_t np = (size_t)P.NG * 64;
@@ -687,38 +738,46 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     // row's sums are formed in the same order whatever NB, NX and PRO are.
     const int split = ng * 2 <= NW ? NW / ng : 1;
     const int sub = wave % split;
-    // The head of group k from its three loaded words (first step, end step, this lane's slot).
-    auto head_from = [&](int k, uint32_t ga, uint32_t gb, uint32_t sl) {
-        StreamHead h{ga, (int)(gb - ga), sl};
+    // What this wave walks of group k, from the group's loaded words: the whole group, or its share of the steps.
+    auto head_from = [&](int k, uint32_t rest, uint32_t nst_g, uint32_t sl) {
+        StreamHead h{rest - (uint32_t)STREAM_PF, (int)nst_g, sl};
         if (k >= ng) h = StreamHead{0u, 0, STREAM_NO_ROW};
         else if (split > 1) {                                   // uniform in the workgroup
             const int s0 = h.nst * sub / split, s1 = h.nst * (sub + 1) / split;
             const int cnt = max((int)(h.slot >> STREAM_ROW_BITS) - 4 * s0, 0);
-            h.st0 += (uint32_t)s0;
+            h.rb = rest + (uint32_t)s0 - (uint32_t)(STREAM_PF * (sub + 1));
             h.nst = s1 - s0;
             h.slot = (h.slot & STREAM_NO_ROW) | ((uint32_t)cnt << STREAM_ROW_BITS);
         }
         return h;
     };
     // (loads without a branch around them, from a clamped index: the compiler then knows how many loads are in
-    // flight and later waits do not have to cover these)
-    auto head = [&](int k) {
-        const int kc = min(k, ng - 1);
-        return head_from(k, goff[kc], goff[kc + 1], slots[(size_t)kc * 64 + lane]);
+    // flight and later waits do not have to cover these.)  The group's words are the same in every lane; loaded
+    // through an index the compiler takes for a per-lane value they stay in vector registers, and they are kept as
+    // loaded (`head_raw`) until the group is started (`resolve`): nothing waits for them where they are requested.
+    // A load the compiler knows to be uniform, or whose result is used at once, is followed by a wait there: one
+    // memory round trip of standstill per group.
+    auto uni = [](int v) { return (int)__builtin_amdgcn_readfirstlane(v); };
+    auto head_raw = [&](int k) {
+        int kc = min(k, ng - 1);
+        asm volatile("" : "+v"(kc));
+        const u32x2 w = *reinterpret_cast<const u32x2*>(gw + kc);       // (only the first two of the four words: every register
+                                                                        // a load writes must stay in use until it has landed)
+        return StreamHeadRaw{w.x, w.y, slots[(size_t)kc * 64 + lane], k};
     };
-    auto first_steps = [&](const StreamHead& h, u32x3* nx) {
-        if (h.nst > 0) {                                        // wave-uniform
-            const unsigned char* en = steps + (size_t)h.st0 * 768;
-#pragma unroll
-            for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, h.nst - 1) * 768);
-        }
+    // (the empty asm pins the arithmetic to the place of the call: hoisted to where the words are loaded it would bring
+    // the wait along)
+    auto resolve = [&](StreamHeadRaw r) {
+        asm volatile("" : "+v"(r.rest), "+v"(r.nst), "+v"(r.sl));
+        return head_from(r.k, r.rest, r.nst, r.sl);
     };
-    // the same without a branch, for the prologue: a wave without steps reads step 0 of the stream and ignores it
-    // (a group without steps may begin where the stream ends: it must not read from its own first step)
-    auto first_steps_always = [&](const StreamHead& h, u32x3* nx) {
-        const unsigned char* en = steps + (size_t)(h.nst > 0 ? h.st0 : 0u) * 768;
+    // The first STREAM_PF steps of this wave's unit of group k: their place follows from indices alone, so they are
+    // requested without having read anything (every unit has STREAM_PF steps there, used or not).
+    auto first_steps = [&](int k, u32x3* nx) {
+        const int unit = u0 + min(k, ng - 1) * split + sub;
+        const unsigned char* en = steps + ((size_t)unit * P.NV + v) * (STREAM_PF * 768);
 #pragma unroll
-        for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)min(q, max(h.nst - 1, 0)) * 768);
+        for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)q * 768);
     };
     int kcur = wave, knext = 2 * NW - 1 - wave;
     if (split > 1) {                                            // one share of one group per wave, or nothing
@@ -729,9 +788,17 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     // the kd 16 KB blocks of the slice that they cover are copied once the rows have been read from there.
     const bool via_lds = PRO == 0 && perms != nullptr && a.xtmp > 0;   // uniform in the workgroup
     const int kd = via_lds && !a.xtmp_own ? (NB * a.xtmp + NTH * 16 - 1) / (NTH * 16) : 0;
+    // The first head's words are requested first of all (through a vector index, see `head`): vector loads come back in
+    // the order they were issued, and behind the 64 KB of slice these three words would arrive a bulk copy later, with
+    // the first steps, whose addresses they give, another round trip behind.  They are used once the slice copy and
+    // the loads of x have gone out.
+    int kc0 = min(kcur, ng - 1);
+    asm volatile("" : "+v"(kc0));
+    const u32x2 head_w = *reinterpret_cast<const u32x2*>(gw + kc0);
+    const uint32_t head_s = slots[(size_t)kc0 * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
     // The codebook slice is copied global -> LDS without passing through registers (a wave instruction moves 1 KB, lane l
-    // to the wave's base + 16 l).  It goes out first: loads are accounted for in the order they were issued, and the
-    // small scattered reads of the group heads below come back later than this bulk copy does.
+    // to the wave's base + 16 l).
     {
         const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table) + (size_t)s * STREAM_TAB;
 #pragma unroll
@@ -741,11 +808,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                                                  (stream_lptr_t)(lds + (k * NTH + wave * 64) * 16), 16, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    // the first head's words are requested here and used only after the staging loads have gone out
-    const int kc0 = min(kcur, ng - 1);
-    const uint32_t head_a = goff[kc0], head_b = goff[kc0 + 1], head_s = slots[(size_t)kc0 * 64 + lane];
-    __builtin_amdgcn_sched_barrier(0);
-    StreamHead hn;
+    StreamHeadRaw hn;
     u32x3 nx[STREAM_PF];
 #pragma unroll
     for (int q = 0; q < STREAM_PF; ++q) nx[q] = u32x3{0u, 0u, 0u};
@@ -869,8 +932,8 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         }
         __builtin_amdgcn_sched_barrier(0);
         SQ_TRACE_DEP(8, "v", head_s);
-        hn = head_from(kcur, head_a, head_b, head_s);
-        first_steps_always(hn, nx);
+        hn = StreamHeadRaw{head_w.x, head_w.y, head_s, kcur};
+        first_steps(kcur, nx);
         __builtin_amdgcn_sched_barrier(0);
         SQ_TRACE_DEP(9, "v", xq[0][0].x);
         if (via_lds) {
@@ -928,18 +991,18 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
     for (int b = 0; b < NB; ++b) acc_share[b] = 0.f;
     while (kcur < ng) {
-        const StreamHead h = hn;
-        hn = head(knext);
+        const StreamHead h = resolve(hn);
+        hn = head_raw(knext);
         int kafter = ng;
         if (knext < ng) {
             unsigned tk = 0;
             if (lane == 0) tk = __hip_atomic_fetch_add(flag + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             kafter = (int)__builtin_amdgcn_readfirstlane(tk);
         }
-        const int nst = h.nst;
+        const int nst = uni(h.nst);
         const int cnt = (int)(h.slot >> STREAM_ROW_BITS);
         const uint32_t row = h.slot & STREAM_NO_ROW;
-        const unsigned char* eb = steps + (size_t)h.st0 * 768;
+        const unsigned char* eb = steps + (size_t)(uint32_t)uni((int)h.rb) * 768;
         // the copy of x for this group's column order
         int xc = 0;
 #pragma unroll
@@ -957,7 +1020,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                 for (int q = 0; q < STREAM_PF; ++q)
                     nx[q] = *reinterpret_cast<const u32x3*>(eb + (size_t)min(t0 + STREAM_PF + q, nst - 1) * 768);
             } else {
-                first_steps(hn, nx);                            // the next group's first steps
+                if (knext < ng) first_steps(knext, nx);         // the next group's first steps
             }
 #pragma unroll
             for (int q = 0; q < STREAM_PF; ++q) {
@@ -995,7 +1058,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
             for (int b = 0; b < NB; ++b) acc[b] = 0.f;
         }
-        if (nst == 0) first_steps(hn, nx);                      // a group without steps fetched nothing for its successor
+        if (nst == 0 && knext < ng) first_steps(knext, nx);    // a group without steps fetched nothing for its successor
         // A row's partial sum goes to its place in the run's partial-sum vector in LDS (rows sit at different lanes in
         // different buckets, so straight from here the 64 lanes would write 64 scattered 4-byte pieces to memory)
         if (split > 1) {
@@ -1160,15 +1223,18 @@ __global__ __launch_bounds__(256) void stream_dequant_kernel(StreamDeqArgs a) {
     if (place != STREAM_NO_ROW) row = a.perms ? reinterpret_cast<const uint32_t*>(a.stream + a.off_rows)[place] : place;
     const bool mine = row != STREAM_NO_ROW && (int)row >= a.r0 && (int)row < a.r1 && cnt > 0;
     if (__ballot(mine) == 0) return;                             // (wave-uniform) none of this group's rows is wanted
-    const uint32_t* goff = reinterpret_cast<const uint32_t*>(a.stream) + w;
-    const uint32_t st0 = goff[0];
-    const int nst = (int)(goff[1] - st0);
+    const u32x4 hw = reinterpret_cast<const u32x4*>(a.stream)[w];             // {rest, nst, unit0, split}
+    const int nst = (int)hw.y, split = (int)hw.w;
     const float sc = (mine && !a.raw) ? h2f(a.row_scale[row]) : 1.f;
     const int32_t* pm = (mine && a.perms) ? a.perms + (size_t)(a.row_mask ? a.row_mask[row] : 0) * a.C : nullptr;
     T* orow = reinterpret_cast<T*>(a.out) + (mine ? (int64_t)((int)row - a.r0) * a.ld_out : 0);
-    const unsigned char* rec = a.stream + a.off_steps + (size_t)st0 * 768 + lane * 12;
+    const unsigned char* rec = a.stream + a.off_steps + lane * 12;
+    int j = 0, s0 = 0, s1 = nst / split;                          // the share step t belongs to, its first and end step
     for (int t = 0; t < nst; ++t) {
-        const u32x3 r = *reinterpret_cast<const u32x3*>(rec + (size_t)t * 768);
+        while (t >= s1) { ++j; s0 = s1; s1 = nst * (j + 1) / split; }
+        const size_t at = t - s0 < STREAM_PF ? ((size_t)(hw.z + (uint32_t)j) * a.NV + v) * STREAM_PF + (size_t)(t - s0)
+                                             : (size_t)hw.x + (size_t)t - (size_t)STREAM_PF * (j + 1);
+        const u32x3 r = *reinterpret_cast<const u32x3*>(rec + at * 768);
         const uint32_t e[4] = {r.x, (r.x >> 24) | (r.y << 8), (r.y >> 16) | (r.z << 16), r.z >> 8};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {

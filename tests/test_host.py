@@ -209,6 +209,33 @@ def _build_stream(words, R, C, bits, row_mask, runs, table=None):
 
 
 PART_MAX = 4064     # chunks per column part (sq_stream.h)
+PF, NW = 3, 16      # steps of a unit in the first-steps region (= the kernel's prefetch depth); waves per workgroup
+
+
+def _step_places(head, v, NV):
+    """Places (in 768-byte steps from the start of the step area) of steps 0 .. nst - 1 of a group with head words
+    {rest, nst, unit0, split} in bucket v (sq_stream.h): the first PF steps of every share sit in the first-steps region
+    at ((unit0 + share) * NV + v) * PF, the others follow each other from `rest` on."""
+    rest, nst, unit0, split = (int(x) for x in head)
+    out = []
+    for j in range(split):
+        s0, s1 = nst * j // split, nst * (j + 1) // split
+        for t in range(s0, s1):
+            out.append(((unit0 + j) * NV + v) * PF + (t - s0) if t - s0 < PF else rest + t - PF * (j + 1))
+    return out
+
+
+def _stream_offsets(NV, NG, runs, bits, d, balanced):
+    off_slots = (NV * NG * 16 + 255) & ~255
+    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
+    off_rows = (off_runs + runs * 32 + 255) & ~255
+    off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
+    off_table = off_unmap = 0
+    if balanced:
+        K = 1 << bits
+        off_table, off_unmap = off_steps, off_steps + K * d * 2
+        off_steps = (off_unmap + K * 2 + 255) & ~255
+    return off_slots, off_runs, off_rows, off_table, off_unmap, off_steps
 
 
 def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
@@ -218,39 +245,45 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
     KP = -(-U // PART_MAX)
     PC = -(-U // KP)
     NV = NS * KP
-    off_slots = ((NV * NG + 1) * 4 + 255) & ~255
-    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
-    off_rows = (off_runs + runs * 32 + 255) & ~255
-    off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
+    off_slots, off_runs, off_rows, off_table, off_unmap, off_steps = _stream_offsets(NV, NG, runs, bits, d, table is not None)
     unmap = None
     if table is not None:
         K = 1 << bits
-        off_table, off_unmap = off_steps, off_steps + K * d * 2
-        off_steps = (off_unmap + K * 2 + 255) & ~255
         unmap = np.frombuffer(buf, np.uint16, K, off_unmap).astype(np.int64)
         assert sorted(unmap.tolist()) == list(range(K))                        # a permutation of the labels
         moved = np.frombuffer(buf, np.uint16, K * d, off_table).reshape(K, d)
         assert np.array_equal(moved, table.view(np.uint16).reshape(K, d)[unmap])   # codeword `new` is the file's unmap[new]
-    goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
+    heads = np.frombuffer(buf, np.uint32, NV * NG * 4, 0).reshape(NV, NG, 4).astype(np.int64)   # {rest, nst, unit0, split}
     slots = np.frombuffer(buf, np.uint32, NV * NG * 64, off_slots).reshape(NV, NG * 64)
-    rt = np.frombuffer(buf, np.int32, runs * 8, off_runs).reshape(runs, 8)[:, :4]       # g0, ng, column orders, 0
+    rt = np.frombuffer(buf, np.int32, runs * 8, off_runs).reshape(runs, 8)[:, :4]       # g0, ng, column orders, first unit
     rb = np.frombuffer(buf, np.uint8, runs * 32, off_runs).reshape(runs, 32)
     bounds, orders = rb[:, 16:24], rb[:, 24:32]                               # first group (in the run) and id of each order
     base = np.frombuffer(buf, np.uint32, NG * 64, off_rows)                   # place -> row
     assert sorted(base[base != 0x7FFFF].tolist()) == list(range(R))
     if row_mask is None:
         assert (base[:R] == np.arange(R)).all()
-    assert goff[0] == 0 and (np.diff(goff.astype(np.int64)) >= 0).all()
-    assert len(buf) == off_steps + int(goff[-1]) * 768
+    total = (len(buf) - off_steps) // 768
+    assert len(buf) == off_steps + total * 768
     # runs tile the groups in order; every run has one column order
     assert rt[0, 0] == 0 and (rt[1:, 0] == rt[:-1, 0] + rt[:-1, 1]).all() and rt[-1, 0] + rt[-1, 1] == NG
-    assert (rt[:, 1] >= 1).all() and (rt[:, 3] == 0).all() and (rt[:, 2] >= 1).all() and (rt[:, 2] <= 4).all()
+    assert (rt[:, 1] >= 1).all() and (rt[:, 2] >= 1).all() and (rt[:, 2] <= 4).all()
     assert (bounds[:, 0] == 0).all() and (rt[:, 2] == 1).all() or row_mask is not None
     if row_mask is None:                                                      # the cut the kernel derives from the run count
         gr = -(-NG // runs)
         assert (rt[:, 0] == np.arange(runs) * gr).all() and (rt[:, 1] == np.minimum(gr, NG - rt[:, 0])).all()
-    steps = np.frombuffer(buf, np.uint8, int(goff[-1]) * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.uint32)
+    steps = np.frombuffer(buf, np.uint8, total * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.uint32)
     ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
+    # units: run after run, a group of a run of at most NW / 2 groups has NW // groups of them (its waves' shares);
+    # every step of the buffer belongs to exactly one group
+    u0 = 0
+    for g0, ng, _, ru0 in rt:
+        split = NW // ng if ng * 2 <= NW else 1
+        assert ru0 == u0
+        assert (heads[:, g0:g0 + ng, 3] == split).all()
+        assert (heads[:, g0:g0 + ng, 2] == u0 + np.arange(ng) * split).all()
+        u0 += ng * split
+    NU, used = u0, np.zeros(total, bool)
+    assert total >= NU * NV * PF
     tags = np.full((R, U), -1, np.int64)
     run_rows = None
     for v in range(NV):
@@ -280,9 +313,13 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
         run_rows = run_rows or sets
         assert sets == run_rows                                               # the same rows in every bucket's run
         for g in range(NG):
-            n = int(goff[v * NG + g + 1]) - int(goff[v * NG + g])
+            n = int(heads[v, g, 1])
             assert n == -(-int(cnts[g * 64]) // 4)                            # padded to the group's longest row
-            e = ent[int(goff[v * NG + g]):int(goff[v * NG + g + 1])]          # [n, 64, 4]
+            at = _step_places(heads[v, g], v, NV)
+            assert len(at) == n and not used[at].any()
+            assert all((a < NU * NV * PF) == (k_ < PF) for a, k_ in zip(at, _share_pos(n, int(heads[v, g, 3]))))
+            used[at] = True
+            e = ent[at]                                                        # [n, 64, 4]
             e = e.transpose(1, 0, 2).reshape(64, n * 4)
             for lane in range(64):
                 k = g * 64 + lane
@@ -300,7 +337,16 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
                 assert len(set(chunk.tolist())) == c and (chunk >= kp * PC).all() and (chunk < min(U, (kp + 1) * PC)).all()
                 assert (tags[rows[k], chunk] == -1).all()
                 tags[rows[k], chunk] = (e[lane, :c] & 0xFFF) + (s << 12)
+    assert used[NU * NV * PF:].all()                                          # the rest region has no holes
     return tags if unmap is None else unmap[tags]
+
+
+def _share_pos(nst, split):
+    """Position of every step of a group within its share."""
+    out = []
+    for j in range(split):
+        out += list(range(nst * (j + 1) // split - nst * j // split))
+    return out
 
 
 @pytest.mark.parametrize("R,C,bits,runs,M", [(70, 512, 16, 0, 1), (130, 5376, 16, 2, 1), (64, 1024, 13, 5, 1), (1, 8, 14, 0, 1),
@@ -341,7 +387,7 @@ def test_balanced_stream_relabels_codewords_and_evens_out_the_slices(R, C, bits,
     NS = K >> 12
     def slice_loads(b, balanced):
         NV = NS * -(-U // PART_MAX)
-        off_slots = ((NV * NG + 1) * 4 + 255) & ~255
+        off_slots = (NV * NG * 16 + 255) & ~255
         cnt = np.frombuffer(b, np.uint32, NV * NG * 64, off_slots).reshape(NV, -1) >> 19
         return cnt.sum(1).reshape(-1, NS).sum(0)
     plain, _, NG2 = _build_stream(words, R, C, bits, row_mask, runs)
@@ -354,54 +400,53 @@ def test_balanced_stream_relabels_codewords_and_evens_out_the_slices(R, C, bits,
     assert lb.max() <= max(1.02 * lb.mean() + 1, top)
 
 
-def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask, PF=3, NW=16):
+def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask):
     """Every byte range of the stream buffer that stream_kernel (csrc/sq_stream.hip) forms an address for, replayed on
-    the host: the run table, the group heads (with the kernel's clamp of the group index), the first steps a wave
-    requests before it knows whether it has any (the prologue reads step 0 for a group without steps), the steps
-    fetched ahead inside the loop (clamped to the group's last step), the shares of a group that several waves walk,
-    and the row list of the finishing workgroup.  Yields (what, first byte, end byte)."""
+    the host: the run table, the group heads (with the kernel's clamp of the group index), the first steps of a wave's
+    unit, which it requests before it knows whether the unit has any, the steps fetched ahead inside the loop (clamped
+    to the share's last step), the shares of a group that several waves walk, and the row list of the finishing
+    workgroup.  Yields (what, first byte, end byte)."""
     runs, run_max, balanced = runs_out & 0xFFFF, (runs_out >> 16) & 0xFF, bool(runs_out & (1 << 30))
     U, NS = C // 8, 1 << (bits - 12)
     KP = -(-U // PART_MAX)
     NV = NS * KP
-    off_slots = ((NV * NG + 1) * 4 + 255) & ~255
-    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
-    off_rows = (off_runs + runs * 32 + 255) & ~255
-    off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
+    off_slots, off_runs, off_rows, off_table, _, off_steps = _stream_offsets(NV, NG, runs, bits, 8, balanced)
     if balanced:                                        # relabelled codebook and back map sit in front of the steps
-        yield "codebook slices", off_steps, off_steps + (16 << bits)
-        off_steps = (off_steps + (18 << bits) + 255) & ~255
-    goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0).astype(np.int64)
+        yield "codebook slices", off_table, off_table + (16 << bits)
+    heads = np.frombuffer(buf, np.uint32, NV * NG * 4, 0).reshape(NV * NG, 4).astype(np.int64)
     rt = np.frombuffer(buf, np.int32, runs * 8, off_runs).reshape(runs, 8)
     gr = -(-NG // runs)
     for v in range(NV):
         for wi in range(runs):
             if row_mask is not None:
                 yield "run table", off_runs + wi * 32, off_runs + wi * 32 + 32
-                g0, ng = int(rt[wi, 0]), int(rt[wi, 1])
+                g0, ng, u0 = int(rt[wi, 0]), int(rt[wi, 1]), int(rt[wi, 3])
             else:
                 g0, ng = wi * gr, min(gr, NG - wi * gr)
+                u0 = wi * gr * (NW // gr if gr * 2 <= NW else 1)    # every run before this one has gr groups
             ng = min(ng, run_max)                       # the kernel never walks more groups than its LDS holds sums for
             assert ng >= 1, (v, wi, g0, ng)
             split = NW // ng if ng * 2 <= NW else 1
             yield "row list", off_rows + g0 * 256, off_rows + (g0 + ng) * 256
-            # head(k) for every k a wave can ask for: its own groups and, one ahead, the index behind the last one
+            # head_raw(k) for every k a wave can ask for: its own groups and, one ahead, the index behind the last one;
+            # first_steps(k): the PF steps of the wave's unit in the first-steps region, whether the unit has that many or not
             for k in range(ng + 1):
                 kc = min(k, ng - 1)
                 i = v * NG + g0 + kc
-                yield "group offsets", i * 4, i * 4 + 8
+                yield "group words", i * 16, i * 16 + 16
                 yield "slots", off_slots + i * 256, off_slots + i * 256 + 256
+                for sub in range(split):
+                    first = ((u0 + kc * split + sub) * NV + v) * PF
+                    yield "first steps", off_steps + first * 768, off_steps + (first + PF) * 768
                 if k >= ng:
                     continue
-                st0, nst = int(goff[i]), int(goff[i + 1] - goff[i])
+                rest, nst = int(heads[i, 0]), int(heads[i, 1])
+                assert int(heads[i, 2]) == u0 + kc * split and int(heads[i, 3]) == split
                 for sub in range(split):
                     s0, s1 = nst * sub // split, nst * (sub + 1) // split
-                    a, n = st0 + s0, s1 - s0
-                    # prologue (first_steps_always): a wave without steps reads step 0 of the stream
-                    steps = [a + min(q, max(n - 1, 0)) if n > 0 else 0 for q in range(PF)]
+                    rb, n = rest + s0 - PF * (sub + 1), s1 - s0
                     # the loop: PF steps ahead, clamped to the share's last step
-                    steps += [a + min(t0 + PF + q, n - 1) for t0 in range(0, n, PF) for q in range(PF) if t0 + PF < n]
-                    for st in set(steps):
+                    for st in {rb + min(t0 + PF + q, n - 1) for t0 in range(0, n, PF) for q in range(PF) if t0 + PF < n}:
                         yield "steps", off_steps + st * 768, off_steps + st * 768 + 768
 
 
@@ -462,13 +507,11 @@ def test_stream_builder_orders_entries_for_the_lds_banks():
     tags = rng.integers(0, 1 << bits, size=(R, C // 8))
     buf, runs, NG = _build_stream(O.pack_bits(tags, bits), R, C, bits, None, 1)
     NV = 16
-    off_slots = ((NV * NG + 1) * 4 + 255) & ~255
-    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
-    off_rows = (off_runs + runs * 32 + 255) & ~255
-    off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
-    goff = np.frombuffer(buf, np.uint32, NV * NG + 1, 0)
-    steps = np.frombuffer(buf, np.uint8, int(goff[-1]) * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.int64)
+    off_steps = _stream_offsets(NV, NG, runs, bits, 8, False)[-1]
+    heads = np.frombuffer(buf, np.uint32, NV * NG * 4, 0).reshape(NV, NG, 4)
+    steps = np.frombuffer(buf, np.uint8, len(buf) - off_steps, off_steps).reshape(-1, 64, 4, 3).astype(np.int64)
     ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
+    ent = ent[[a for v in range(NV) for g in range(NG) for a in _step_places(heads[v, g], v, NV)]]   # the groups' steps only
     cw, xc = [], []
     for lanes in LDS_CLOCK_LANES:
         e = ent[:, lanes, :].transpose(0, 2, 1).reshape(-1, 16)               # [slot, lane of the clock]
