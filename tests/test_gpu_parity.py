@@ -624,16 +624,21 @@ def test_launcher_refuses_stream_counts_the_builder_did_not_make():
 
 
 # ------------------------------------------------------------------ one copy of the tags (the reference's `compact`)
-@pytest.mark.parametrize("case", [(300, 1024, 16, 1), (257, 3584, 16, 1), (140, 5120, 16, 16), (700, 1024, 14, 3), (65, 18944, 16, 1)],
-                         ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("case", [(300, 1024, 16, 1), (257, 3584, 16, 1), (140, 5120, 16, 16), (700, 1024, 14, 3), (65, 18944, 16, 1),
+                                  (140, 5120, 16, 16, 1), (700, 1024, 14, 3, 1), (2368, 512, 14, 1, 1)],   # cut into one run: several
+                         ids=lambda c: "x".join(map(str, c)))                                         # column orders per run, 37 groups
 def test_one_copy_residency_serves_everything_from_the_stream(case):
     """A matrix that has dropped its packed tags and kept only the slice stream (reference
     shapequant/vllm_ext/core.py:215-253: one resident copy): decoded weights stay bit-exact (every dtype, row
     ranges), batch 1 gives the same bits as the two-copy matrix, and more rows and prefill stay within tolerance."""
     from quantexperiments_amd.kernels import linear_gemm, linear_small
-    R, C, bits, M = case
-    s = synth(R, C, 8, bits, 1, M, seed=sum(case))
+    R, C, bits, M = case[:4]
+    s = synth(R, C, 8, bits, 1, M, seed=sum(case[:4]))
     full, one = to_device(s), to_device(s)
+    if len(case) > 4:
+        full.build_stream(case[4])
+        one.build_stream(case[4])
+        assert M == 1 or (one.stream_runs >> 24) & 7 >= 1
     one.make_compact()
     assert one.words is None and one.stream is not None and one.descriptor().tags is None
     with pytest.raises(RuntimeError, match="dropped"):
