@@ -9,39 +9,57 @@ constexpr int STREAM_SLICE_BITS = 12;        // 4096 codewords of 16 bytes per L
 constexpr int STREAM_PART_MAX = 4064;        // most chunks in one column part: its chunks and the 16 zero chunks that padding
                                              // entries multiply with (chunks PC .. PC + 15 of the part) fit 12 bits of an entry
 constexpr int STREAM_RUN_MAX = 96;           // most groups of 64 rows in one run (a run's partial sums are staged in LDS)
-constexpr int STREAM_ROW_BITS = 19;          // slot = row | count << 19
+constexpr int STREAM_ROW_BITS = 19;          // places (indices into the row list) stay below 2^19
 constexpr uint32_t STREAM_NO_ROW = (1u << STREAM_ROW_BITS) - 1u;
+// Slot of a lane (16 bits per lane, group and bucket): the lane's row as its place counted from the run's first place
+// (a run has at most STREAM_RUN_MAX * 64 = 6144 places), STREAM_SLOT_NONE for a lane without a row, and
+// STREAM_SLOT_HAS when the row has entries in the bucket (a lane without any walks a neighbour's entries and its sum is
+// dropped).
+constexpr uint32_t STREAM_SLOT_NONE = 0x1FFFu;
+constexpr uint32_t STREAM_SLOT_HAS = 0x2000u;
+// Entry formats.  Wide: 24 bits (12-bit tag within the slice, 12-bit chunk within the column part), four per lane and
+// step in 12 bytes, steps of 768 bytes.  Narrow, for column parts of at most STREAM_NARROW_MAX chunks (9 bits name the
+// part's chunks and the 16 zero chunks behind them): 21 bits (12 + 9), three per lane and step in 8 bytes (entry i at
+// bits 21 i of the lane's 64), steps of 512 bytes.  Either way a prefetch batch is 12 entries per lane.
+constexpr int STREAM_NARROW_MAX = 496;
+struct StreamFmt { int narrow, eps, lane_bytes, step_bytes, pf, chunk_bits; };
+__host__ __device__ inline StreamFmt stream_fmt(int PC) {
+    return PC <= STREAM_NARROW_MAX ? StreamFmt{1, 3, 8, 512, 4, 9} : StreamFmt{0, 4, 12, 768, 3, 12};
+}
 constexpr int GEMV_MAX_PIECES_STREAM = 4;
 constexpr int STREAM_RUN_ORDERS = 8;         // most column orders whose rows may share a run (one gathered copy of x in LDS each)
 
 constexpr int STREAM_DEFAULT_WGS = 256;      // workgroups a matrix launched alone should make (one per CU on 256 CUs)
 constexpr int STREAM_NW = 16;                // waves per workgroup of the kernel: one workgroup per CU
-constexpr int STREAM_PF = 3;                 // steps the kernel fetches ahead (2 to 4 measure alike, 6 and 8 slower), and the steps
-                                             // of every unit that the buffer keeps in its first-steps region
+// Steps the kernel fetches ahead = StreamFmt.pf (12 entries per lane; 2 to 4 wide steps measure alike, 6 and 8 slower);
+// the first of every unit's steps are kept in the first-steps region.
 
 // A unit is what one wave walks without a break: a group of a run, or, in a run of at most STREAM_NW / 2 groups, one of
 // the STREAM_NW / groups contiguous shares of a group's steps (share j of `split`: steps [nst j / split, nst (j + 1) / split)).
 __host__ __device__ inline int stream_split_of(int ng) { return ng * 2 <= STREAM_NW ? STREAM_NW / ng : 1; }
 
-// Where the steps are (all positions in 768-byte steps from off_steps).  The first STREAM_PF steps of every unit sit in a
-// region of their own, at a place that follows from the unit's index alone: ((unit * NV + bucket) * STREAM_PF), so a
+// Where the steps are (all positions in steps from off_steps; PF = StreamFmt.pf).  The first FS steps of every unit sit
+// in a region of their own, at a place that follows from the unit's index alone: ((unit * NV + bucket) * FS), so a
 // wave can ask for them before it has read anything else of the buffer; a launch then starts with one round trip to
-// memory instead of two (offsets, then steps).  The remaining steps of a group follow each other in the rest region,
-// share after share.  Per (bucket, group) the buffer holds four words: {rest, nst, unit0, split} = the place of the
-// group's first remaining step, its step count, the index of its first unit and its share count; when every share has
-// at least STREAM_PF steps (nst / split >= STREAM_PF), step t of share j (t counted within the group) is at
-// rest + t - STREAM_PF (j + 1) once it is past the share's first STREAM_PF; otherwise the first-steps region holds
-// the whole group.
+// memory instead of two (offsets, then steps).  FS is PF, or, in a matrix none of whose units has that many steps (short
+// shares of small matrices), the longest unit's step count.  The remaining steps of a group follow each other in the
+// rest region, share after share.  Per (bucket, group) the buffer holds four words: {rest, nst, unit0, split | g0 << 8}
+// = the place of the group's first remaining step, its step count, the index of its first unit, its share count and the
+// first group of its run; when every share has at least PF steps (nst / split >= PF), step t of share j (t counted
+// within the group) is at rest + t - PF (j + 1) once it is past the share's first PF; otherwise the first-steps region
+// holds the whole group.
 
 struct StreamGeom {
     int U, NS, KP, PC, NV, NG;               // chunks per row, slices, column parts, chunks per part, buckets, groups
     int runs;
+    int fs;                                  // steps per unit in the first-steps region (1 .. fmt.pf)
+    StreamFmt fmt;
     size_t off_slots, off_runs, off_rows, off_steps;   // byte offsets inside the stream buffer
     size_t off_table, off_unmap;             // balanced streams: the relabelled codebook and uint16 new id -> file id (else 0)
     uint64_t total_steps;                    // filled by the builder only
 };
 
-StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced = false);
+StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced = false, int fs = 0);
 bool stream_format_ok(int R, int C, int d, int bits);
 // table: the matrix' codebook (fp16 [2^bits, d], host memory) or NULL.  With it the codewords are relabelled so that
 // every slice of 4096 carries the same share of the tags whatever their distribution, and the buffer holds the
@@ -51,14 +69,16 @@ size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int b
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                       unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table = nullptr);
 // sq_matrix.stream_runs is sq_stream_build's runs_out: the run count in the low 16 bits, the groups of the longest run
-// in the next 8, the most column orders in one run (less one) in bits 24-26, bit 30 = the stream carries a relabelled codebook
+// in the next 8, the most column orders in one run (less one) in bits 24-26, the steps per unit of the first-steps region
+// (less one) in bits 27-28, bit 30 = the stream carries a relabelled codebook
 constexpr int STREAM_BALANCED = 1 << 30;
+inline int stream_fs_of(const sq_matrix& m) { return (int)(((uint32_t)m.stream_runs >> 27) & 3u) + 1; }
 inline int stream_runs_of(const sq_matrix& m) { return m.stream_runs & 0xFFFF; }
 inline int stream_run_max_of(const sq_matrix& m) { return (int)(((uint32_t)m.stream_runs >> 16) & 0xFFu); }
 inline int stream_run_orders_of(const sq_matrix& m) { return (int)(((uint32_t)m.stream_runs >> 24) & 7u) + 1; }
 inline bool stream_balanced_of(const sq_matrix& m) { return (m.stream_runs & STREAM_BALANCED) != 0; }
 inline StreamGeom stream_geom_of(const sq_matrix& m) {
-    return stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m), stream_balanced_of(m));
+    return stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m), stream_balanced_of(m), stream_fs_of(m));
 }
 bool stream_shape(const sq_matrix& m);
 size_t stream_part_bytes(const sq_matrix& m, int rows);   // partial sums of one pass of `rows` activation rows

@@ -5,7 +5,7 @@
 // codebook they point into, so that every workgroup gathers from a 64 KB slice held in LDS:
 //
 //   bucket (kp, s)   column part kp (PC chunks of d columns each) x codebook slice s (tags s*4096 .. +4095)
-//   entry            24 bits: tag & 4095 | (chunk - kp * PC) << 12
+//   entry            tag & 4095 | (chunk - kp * PC) << 12: 24 bits, or 21 when the part has at most 496 chunks
 //   lane task        the entries of one row in one bucket (about C/d / (KP * NS) of them)
 //
 // Rows are first ordered by column order (row_mask, stable), so that consecutive rows share one; each column
@@ -13,8 +13,9 @@
 // groups, one workgroup per (bucket, run); the caller picks the number of runs so that the pieces it launches
 // together make about one workgroup (of 16 waves) per CU.  Within a bucket the rows of a run are sorted by entry count
 // (descending, stable): one lane per row, one wave per group.  A group is stored as steps of 64 x 12 bytes
-// (4 entries per lane per step, lane-major, so a wave reads 768 contiguous bytes per step) padded to the longest
-// row of the group; sorting keeps that padding near 10 percent.  A workgroup stages its slice and its part of x
+// (4 entries of 24 bits per lane and step, lane-major, so a wave reads 768 contiguous bytes per step) or of 64 x 8
+// bytes (3 entries of 21 bits), padded to the longest row of the group; sorting keeps that padding at 5 to 7 percent
+// of a large matrix.  A workgroup stages its slice and its part of x
 // (gathered through the run's column order, if any) in LDS; each lane accumulates dot(codeword, x chunk) over
 // its entries in fp32 and leaves one partial sum per (bucket, row) in the workspace header, whose words are zero
 // between launches: a partial sum is its own arrival flag.  The workgroups of all buckets that cover the same run
@@ -22,16 +23,18 @@
 // order (so results do not depend on scheduling), apply the row scale, store y and put zero back.
 //
 // Stream buffer (one allocation; offsets follow from C/d, the tag width, the group and run counts):
-//   heads  uint32 [NV * NG][4]    {rest, nst, unit0, split} of every group (NV = KP * NS buckets, NG groups per bucket,
-//                                 bucket v = kp * NS + s): where its steps are, see sq_stream.h
-//   slots  uint32 [NV * NG * 64]  place | count << 19 per lane; place = the row's index in `rows` (below),
-//                                 0x7FFFF marks a lane without a row; lanes 64 g .. 64 g + 63 of a bucket are group g
+//   heads  uint32 [NV * NG][4]    {rest, nst, unit0, split | g0 << 8} of every group (NV = KP * NS buckets, NG groups per
+//                                 bucket, bucket v = kp * NS + s): where its steps are, see sq_stream.h
+//   slots  uint16 [NV * NG * 64]  the lane's place counted from its run's first place (place = the row's index in `rows`
+//                                 below; 0x1FFF: a lane without a row) | 0x2000 when the row has entries in the bucket;
+//                                 lanes 64 g .. 64 g + 63 of a bucket are group g
 //   runs   [runs] x 32 bytes       first group, group count, column orders of the run, index of its first unit; first
 //                                 group (within the run) and id of each of up to 8 column orders (one byte each)
 //   rows   uint32 [NG * 64]       the rows ordered by column order, 64 per group (0x7FFFF where a group is short):
 //                                 places 64 g0 .. 64 (g0 + ng) - 1 are a run's rows, and partial sums are indexed by place
-//   steps  [total][64][3] uint32  entries: the first-steps region (STREAM_PF steps per unit and bucket), then the rest
+//   steps  [total][64][12 | 8]    entries: the first-steps region (FS steps per unit and bucket), then the rest
 #include <algorithm>
+#include <atomic>
 #include <string.h>
 #include <thread>
 #include <vector>
@@ -48,7 +51,7 @@ namespace sq {
 struct StreamRun { int32_t g0, ng, norders, u0; uint8_t bound[STREAM_RUN_ORDERS]; uint8_t order[STREAM_RUN_ORDERS]; };
 static_assert(sizeof(StreamRun) == 32, "run records are read as 8 dwords");
 
-StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced) {
+StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced, int fs) {
     StreamGeom g;
     g.U = C / d;
     g.NS = 1 << (bits - STREAM_SLICE_BITS);
@@ -57,8 +60,10 @@ StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanc
     g.NV = g.NS * g.KP;
     g.NG = groups;
     g.runs = runs;
+    g.fmt = stream_fmt(g.PC);
+    g.fs = fs < 1 ? g.fmt.pf : fs < g.fmt.pf ? fs : g.fmt.pf;
     g.off_slots = ((size_t)g.NV * g.NG * 16 + 255) & ~(size_t)255;          // four words per (bucket, group)
-    g.off_runs = (g.off_slots + (size_t)g.NV * g.NG * 64 * 4 + 255) & ~(size_t)255;
+    g.off_runs = (g.off_slots + (size_t)g.NV * g.NG * 64 * 2 + 255) & ~(size_t)255;
     g.off_rows = (g.off_runs + (size_t)runs * sizeof(StreamRun) + 255) & ~(size_t)255;
     size_t end = (g.off_rows + (size_t)g.NG * 64 * 4 + 255) & ~(size_t)255;
     g.off_table = g.off_unmap = 0;
@@ -113,6 +118,8 @@ struct StreamPlan {
                                      // builder lays them out before they move to their places)
     uint64_t logical_steps;          // goff[NV * NG]
     int NU;                          // units of one bucket
+    std::vector<uint32_t> slot32;    // [NV * NG * 64]: place | count << STREAM_ROW_BITS per lane (STREAM_NO_ROW: no row), the
+                                     // builder's own form of the slots
     std::vector<uint32_t> run_of;    // [NG]: the run of a group
     std::vector<uint32_t> head4;     // [NV * NG][4]: {rest, nst, unit0, split}, what the buffer holds per (bucket, group)
     std::vector<uint16_t> remap;     // balanced streams: file id -> new id (empty: identity)
@@ -174,7 +181,7 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     first.push_back(R);
     int total_groups = 0;
     for (int q : ngm) total_groups += q;
-    const int xs_bytes = (g0.PC + 16) * 16;
+    const int xs_bytes = g0.fmt.narrow ? 8192 : (g0.PC + 16) * 16;     // (stream_xs)
     int cap = (160 * 1024 - 65536 - STREAM_RUN_MAX * 256 - 1024) / xs_bytes;
     cap = std::min(cap, std::min(4, 4096 / g0.PC));            // (4: two activation rows per pass still fit LDS at C = 5120)
     if (cap < 1 || !row_mask) cap = 1;
@@ -262,7 +269,7 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
                     std::stable_sort(rows.begin(), rows.end(), [c](uint32_t x, uint32_t y) { return c[x] > c[y]; });
                     for (size_t k = 0; k < rows.size(); ++k) P.pos[(size_t)v * R + rows[k]] = (uint32_t)(ga * 64 + k);
                     for (size_t k = 0; k < rows.size(); k += 64)
-                        steps[(size_t)v * g.NG + ga + k / 64] = (c[rows[k]] + 3u) / 4u;
+                        steps[(size_t)v * g.NG + ga + k / 64] = (c[rows[k]] + (uint32_t)g.fmt.eps - 1u) / (uint32_t)g.fmt.eps;
                 }
             }
         }
@@ -271,7 +278,7 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     for (size_t k = 0; k < steps.size(); ++k) { P.goff[k] = (uint32_t)tot; tot += steps[k]; }
     P.goff[steps.size()] = (uint32_t)tot;
     P.logical_steps = tot;
-    // Units and places: the first-steps region (NU units x NV buckets x STREAM_PF steps) comes first, the groups'
+    // Units and places: the first-steps region (NU units x NV buckets x FS steps) comes first, the groups'
     // remaining steps follow bucket after bucket, group after group.
     P.NU = 0;
     P.run_of.assign(g.NG, 0);
@@ -281,8 +288,17 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
         P.NU += run.ng * stream_split_of(run.ng);
         for (int k = 0; k < run.ng; ++k) P.run_of[run.g0 + k] = (uint32_t)ri;
     }
+    // FS: the longest unit's step count, at most the prefetch depth
+    const uint32_t PF = (uint32_t)g.fmt.pf;
+    uint32_t fs = 1;
+    for (int v = 0; v < g.NV; ++v)
+        for (int gi = 0; gi < g.NG; ++gi) {
+            const uint32_t split = (uint32_t)stream_split_of(P.runs[P.run_of[gi]].ng), nst = steps[(size_t)v * g.NG + gi];
+            fs = std::max(fs, std::min(PF, (nst + split - 1) / split));
+        }
+    P.g.fs = (int)fs;
     P.head4.assign((size_t)g.NV * g.NG * 4, 0);
-    uint64_t at = (uint64_t)P.NU * g.NV * STREAM_PF;
+    uint64_t at = (uint64_t)P.NU * g.NV * fs;
     for (int v = 0; v < g.NV; ++v)
         for (int gi = 0; gi < g.NG; ++gi) {
             const StreamRun& run = P.runs[P.run_of[gi]];
@@ -291,8 +307,8 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
             h[0] = (uint32_t)at;
             h[1] = nst;
             h[2] = (uint32_t)run.u0 + (uint32_t)(gi - run.g0) * split;
-            h[3] = split;
-            if (nst / split >= (uint32_t)STREAM_PF) at += nst - split * STREAM_PF;
+            h[3] = split | ((uint32_t)run.g0 << 8);
+            if (nst / split >= PF) at += nst - split * PF;
         }
     P.g.total_steps = at;
 }
@@ -301,7 +317,7 @@ size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int b
                          const uint16_t* table) {
     StreamPlan P;
     plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr);
-    return P.g.off_steps + (size_t)P.g.total_steps * 768;
+    return P.g.off_steps + (size_t)P.g.total_steps * P.g.fmt.step_bytes;
 }
 
 // The lanes of a wave that one clock of a 16-byte LDS read serves.  A ds_read_b128 takes four clocks; measured on
@@ -325,26 +341,23 @@ struct BankMatch {
     std::vector<uint8_t> ha, hb;             // [slot][16]: lanes per codeword / x bank group
     std::vector<uint8_t> mx;                 // [slot][4]: fullest codeword group, groups that full; the same for x
     uint32_t cnt[16];
+    uint32_t eps = 4;                        // entries per lane and step (StreamFmt.eps)
 
-    static unsigned char* rec_of(unsigned char* base, int lane, uint32_t n) {
-        return base + (size_t)(n >> 2) * 768 + lane * 12 + (n & 3) * 3;
-    }
-    static void put(unsigned char* r, uint32_t e) { r[0] = (unsigned char)e; r[1] = (unsigned char)(e >> 8); r[2] = (unsigned char)(e >> 16); }
+    // entry n of a lane in a group whose steps begin at base: entries are kept one per word, [step][lane][eps], until
+    // they are moved to their places
+    uint32_t* rec_of(uint32_t* base, int lane, uint32_t n) const { return base + ((size_t)(n / eps) * 64 + lane) * eps + n % eps; }
     static int ga(uint32_t e) { return (int)(e & 15u); }
     static int gb(uint32_t e) { return (int)((e >> STREAM_SLICE_BITS) & 15u); }
     void add(uint32_t n, uint32_t e, int d) { ha[n * 16 + ga(e)] += d; hb[n * 16 + gb(e)] += d; }
 
     // zero_chunk: the first of the 16 chunks of x that the kernel keeps at zero
-    void order_lanes(unsigned char* base, const uint32_t* sl, const int* lanes, uint32_t ns, uint32_t zero_chunk) {
+    void order_lanes(uint32_t* base, const uint32_t* sl, const int* lanes, uint32_t ns, uint32_t zero_chunk) {
         uint32_t most = 0;
         for (int l = 0; l < 16; ++l) {
             const uint32_t s0 = sl[lanes[l]];
             cnt[l] = (s0 & STREAM_NO_ROW) == STREAM_NO_ROW ? 0u : s0 >> STREAM_ROW_BITS;
             ent[l].resize(cnt[l]);
-            for (uint32_t n = 0; n < cnt[l]; ++n) {
-                const unsigned char* r = rec_of(base, lanes[l], n);
-                ent[l][n] = r[0] | (uint32_t)r[1] << 8 | (uint32_t)r[2] << 16;
-            }
+            for (uint32_t n = 0; n < cnt[l]; ++n) ent[l][n] = *rec_of(base, lanes[l], n);
             most = std::max(most, cnt[l]);
         }
         if (most == 0) return;
@@ -457,11 +470,26 @@ struct BankMatch {
             }
             for (int l = 0; l < 16; ++l) {
                 if (cnt[l] == 0) chosen[l] = donor >= 0 ? chosen[donor] : 0u;
-                put(rec_of(base, lanes[l], n), chosen[l]);
+                *rec_of(base, lanes[l], n) = chosen[l];
             }
         }
     }
 };
+
+// One step of 64 lanes x eps entries (one per word) into its bytes: 3 bytes per entry (wide), or the three 21-bit
+// entries of a lane in one 64-bit word (narrow).
+static void encode_step(const uint32_t* e, const StreamFmt& f, unsigned char* out) {
+    for (int lane = 0; lane < 64; ++lane) {
+        const uint32_t* r = e + (size_t)lane * f.eps;
+        unsigned char* o = out + (size_t)lane * f.lane_bytes;
+        if (f.narrow) {
+            const uint64_t w = (uint64_t)r[0] | (uint64_t)r[1] << 21 | (uint64_t)r[2] << 42;
+            for (int b = 0; b < 8; ++b) o[b] = (unsigned char)(w >> (8 * b));
+        } else {
+            for (int k = 0; k < 4; ++k) { o[3 * k] = (unsigned char)r[k]; o[3 * k + 1] = (unsigned char)(r[k] >> 8); o[3 * k + 2] = (unsigned char)(r[k] >> 16); }
+        }
+    }
+}
 
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                       unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table) {
@@ -469,7 +497,9 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
     plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr);
     const uint16_t* remap = table ? P.remap.data() : nullptr;
     const StreamGeom& g = P.g;
-    const size_t need = g.off_steps + (size_t)g.total_steps * 768;
+    const StreamFmt f = g.fmt;
+    const uint32_t EPS = (uint32_t)f.eps, PF = (uint32_t)f.pf, FS = (uint32_t)g.fs;
+    const size_t need = g.off_steps + (size_t)g.total_steps * f.step_bytes;
     if (g.total_steps >= ((uint64_t)1 << 32) || g.runs >= (1 << 16)) return fail(SQ_EUNSUPPORTED, "sq_stream_build: matrix too large");
     if (bytes < need) return fail(SQ_EINVAL, "sq_stream_build: buffer %zu < %zu", bytes, need);
     memset(out, 0, need);
@@ -487,11 +517,12 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
     std::vector<uint32_t> place(R);
     for (size_t k = 0; k < P.base.size(); ++k)
         if (P.base[k] != STREAM_NO_ROW) place[P.base[k]] = (uint32_t)k;
-    uint32_t* slots = (uint32_t*)(out + g.off_slots);
-    for (size_t k = 0; k < (size_t)g.NV * g.NG * 64; ++k) slots[k] = STREAM_NO_ROW;
-    // the steps are made group after group (P.goff) in a buffer of their own and moved to their places at the end
-    std::vector<unsigned char> laid((size_t)P.logical_steps * 768, 0);
-    unsigned char* steps = laid.data();
+    P.slot32.assign((size_t)g.NV * g.NG * 64, STREAM_NO_ROW);
+    uint32_t* slots = P.slot32.data();
+    // the steps are made group after group (P.goff), one entry per word, and moved to their places at the end
+    std::vector<uint32_t> laid((size_t)P.logical_steps * 64 * EPS, 0);
+    uint32_t* steps = laid.data();
+    auto rec = [&](size_t step0, uint32_t lane, uint32_t n) { return steps + ((step0 + n / EPS) * 64 + lane) * EPS + n % EPS; };
     parallel_rows(R, [&](int a, int b) {
         std::vector<uint32_t> q(g.NV), last(g.NV);
         for (int r = a; r < b; ++r) {
@@ -508,24 +539,19 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
                 const int kp = j / g.PC, v = kp * g.NS + (int)(t >> STREAM_SLICE_BITS);
                 const uint32_t k = P.pos[(size_t)v * R + r], n = q[v]++;
                 const uint32_t e = (t & ((1u << STREAM_SLICE_BITS) - 1u)) | ((uint32_t)(j - kp * g.PC) << STREAM_SLICE_BITS);
-                unsigned char* rec = steps + ((size_t)P.goff[(size_t)v * g.NG + (k >> 6)] + (n >> 2)) * 768 + (k & 63) * 12 +
-                                     (n & 3) * 3;
-                rec[0] = (unsigned char)e; rec[1] = (unsigned char)(e >> 8); rec[2] = (unsigned char)(e >> 16);
+                *rec(P.goff[(size_t)v * g.NG + (k >> 6)], k & 63, n) = e;
                 last[v] = e & ((1u << STREAM_SLICE_BITS) - 1u);
             }
             // Padding up to the group's longest row: the row's last codeword of the bucket again, at the chunk of x
             // that the kernel keeps at zero, so padding adds exactly nothing and needs no test in the inner loop
             // (a codeword that is not finite is already part of the row's sum; a row without entries in the
-            // bucket is dropped by its count).
+            // bucket is dropped by its slot).
             for (int v = 0; v < g.NV; ++v) {
                 const uint32_t k = P.pos[(size_t)v * R + r];
                 const size_t gi = (size_t)v * g.NG + (k >> 6);
-                const uint32_t cap = (P.goff[gi + 1] - P.goff[gi]) * 4u;
+                const uint32_t cap = (P.goff[gi + 1] - P.goff[gi]) * EPS;
                 const uint32_t e = last[v] | ((uint32_t)g.PC << STREAM_SLICE_BITS);
-                for (uint32_t n = q[v]; n < cap; ++n) {
-                    unsigned char* rec = steps + ((size_t)P.goff[gi] + (n >> 2)) * 768 + (k & 63) * 12 + (n & 3) * 3;
-                    rec[0] = (unsigned char)e; rec[1] = (unsigned char)(e >> 8); rec[2] = (unsigned char)(e >> 16);
-                }
+                for (uint32_t n = q[v]; n < cap; ++n) *rec(P.goff[gi], k & 63, n) = e;
             }
         }
     });
@@ -535,31 +561,41 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
     // of four banks (address / 16 mod 16): BankMatch arranges the entries of each clock's lanes.
     parallel_rows(g.NV * g.NG, [&](int a, int b) {
         BankMatch bm;
+        bm.eps = EPS;
         for (int vg = a; vg < b; ++vg) {
-            const uint32_t st0 = P.goff[vg], ns = (P.goff[vg + 1] - st0) * 4;
+            const uint32_t st0 = P.goff[vg], ns = (P.goff[vg + 1] - st0) * EPS;
             if (ns == 0) continue;
             const uint32_t* sl = slots + (size_t)vg * 64;
-            unsigned char* base = steps + (size_t)st0 * 768;
+            uint32_t* base = steps + (size_t)st0 * 64 * EPS;
             for (int q = 0; q < 4; ++q) bm.order_lanes(base, sl, LDS_CLOCK_LANES[q], ns, (uint32_t)g.PC);
         }
     });
-    // to their places: the first STREAM_PF steps of every unit into the first-steps region, the rest behind each other
+    // to their places: the first FS steps of every unit into the first-steps region, the rest behind each other; and
+    // the slots in their 16-bit form (place counted from the run's first place, entries or none)
+    uint16_t* slot16 = (uint16_t*)(out + g.off_slots);
     parallel_rows(g.NV * g.NG, [&](int a, int b) {
         for (int vg = a; vg < b; ++vg) {
             const uint32_t* h = &P.head4[(size_t)vg * 4];
-            const int v = vg / g.NG, nst = (int)h[1], split = (int)h[3];
-            const unsigned char* src = steps + (size_t)P.goff[vg] * 768;
+            const int v = vg / g.NG, nst = (int)h[1], split = (int)(h[3] & 0xFFu);
+            const uint32_t p0 = (h[3] >> 8) * 64u;
+            for (int lane = 0; lane < 64; ++lane) {
+                const uint32_t s32 = slots[(size_t)vg * 64 + lane];
+                slot16[(size_t)vg * 64 + lane] = (s32 & STREAM_NO_ROW) == STREAM_NO_ROW
+                    ? (uint16_t)STREAM_SLOT_NONE
+                    : (uint16_t)(((s32 & STREAM_NO_ROW) - p0) | ((s32 >> STREAM_ROW_BITS) ? STREAM_SLOT_HAS : 0u));
+            }
+            const uint32_t* src = steps + (size_t)P.goff[vg] * 64 * EPS;
             for (int j = 0; j < split; ++j) {
                 const int s0 = nst * j / split, s1 = nst * (j + 1) / split;
                 for (int t = s0; t < s1; ++t) {
-                    const uint64_t to = t - s0 < STREAM_PF ? ((uint64_t)(h[2] + j) * g.NV + v) * STREAM_PF + (t - s0)
-                                                           : (uint64_t)h[0] + t - (uint64_t)STREAM_PF * (j + 1);
-                    memcpy(out + g.off_steps + to * 768, src + (size_t)t * 768, 768);
+                    const uint64_t to = (uint32_t)(t - s0) < PF ? ((uint64_t)(h[2] + j) * g.NV + v) * FS + (t - s0)
+                                                                 : (uint64_t)h[0] + t - (uint64_t)PF * (j + 1);
+                    encode_step(src + (size_t)t * 64 * EPS, f, out + g.off_steps + to * f.step_bytes);
                 }
             }
         }
     });
-    if (runs_out) *runs_out = g.runs | (P.GR << 16) | ((P.orders_max - 1) << 24) | (table ? STREAM_BALANCED : 0);
+    if (runs_out) *runs_out = g.runs | (P.GR << 16) | ((P.orders_max - 1) << 24) | ((g.fs - 1) << 27) | (table ? STREAM_BALANCED : 0);
     if (groups_out) *groups_out = g.NG;
     return SQ_OK;
 }
@@ -573,6 +609,7 @@ struct StreamPiece {
     float* part;                      // [NV][NB][NG * 64] words, indexed by place: zero before the launch, zero after it
     const int32_t* perms;             // [M, C] column orders or NULL
     int R, C, U, NS, NV, PC, NG, y_off;
+    int fs;                           // steps per unit in the first-steps region
     uint32_t off_slots, off_runs, off_rows, off_steps;
     int wg_begin, nwg;                // first workgroup of the piece; workgroups (= runs) per bucket
 };
@@ -589,6 +626,7 @@ struct StreamArgs {
     int xtmp;                         // bytes per activation row of its copy in natural order in LDS (column orders are then
                                       // applied from LDS), 0: gathered from memory
     int orders;                       // 1: some piece has column orders
+    int narrow;                       // 1: the pieces' entries are 21 bits wide (StreamF<1>)
     int xtmp_own;                     // 1: those copies have LDS of their own behind everything else, 0: they sit where the slice goes
     int nl_max;                       // places of the longest run (64 per group): floats per row of the LDS partial sums
     int x_dtype, y_dtype;
@@ -646,14 +684,61 @@ constexpr int STREAM_TAB = 65536;     // the codebook slice
 constexpr uint32_t STREAM_ZERO_SUM = 0x7FFFFFFFu;  // how a partial sum with all bits zero is written (zero = not there yet)
 constexpr int STREAM_SPIN_MAX = 1 << 18;           // polls of an item's partial sums before it gives up
 
-// LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group)
-static inline int stream_xs(int pc) { return (pc + 16) * 16; }
+// LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group); the narrow format
+// gives every copy 8 KB, so the address of a chunk is its offset OR-ed into the copy's base
+static inline int stream_xs(int pc) { return stream_fmt(pc).narrow ? 8192 : (pc + 16) * 16; }
 
-// what a wave walks of a group: nst steps, of which step t >= STREAM_PF is step rb + t of the buffer (the first STREAM_PF
-// are in the first-steps region), and this lane's slot
+// what a wave walks of a group: nst steps, of which step t >= PF is step rb + t of the buffer (the first PF are in the
+// first-steps region), and this lane's slot
 struct StreamHead { uint32_t rb; int nst; uint32_t slot; };
-// a group's words as loaded ({rest, nst, unit0, split} and this lane's slot) and its index in the run
+// a group's words as loaded ({rest, nst, unit0, split | g0 << 8} and this lane's slot) and its index in the run
 struct StreamHeadRaw { uint32_t rest, nst, sl; int k; };
+
+// Bit field [OFF, OFF + W) of v times 16, plus base: the LDS address of a chunk of x from the word that holds its
+// index, in two instructions (v_bfe_u32, v_lshl_add_u32).  Written as a shift, a mask and an addition the compiler
+// makes three of it.
+template <int OFF, int W>
+__device__ __forceinline__ uint32_t stream_field16(uint32_t v, uint32_t base) {
+    uint32_t f, r;
+    asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(f) : "v"(v), "n"(OFF), "n"(W));
+    asm("v_lshl_add_u32 %0, %1, 4, %2" : "=v"(r) : "v"(f), "v"(base));
+    return r;
+}
+
+// The entry format as the kernels see it (sq_stream.h: StreamFmt).  addrs(): the LDS byte addresses of every entry's
+// codeword (its tag times 16: the slice begins at LDS address 0) and of its chunk of x (times 16, plus xbase), four
+// instructions per entry (five for one of the wide ones).
+template <int NAR> struct StreamF;
+template <> struct StreamF<0> {
+    static constexpr int EPS = 4, LB = 12, SB = 768, PF = 3;
+    static constexpr uint32_t CMASK = 0xFFFu;
+    typedef u32x3 vec;
+    // (bits above an entry's 24 are left in place: the address fields are cut out where they are used)
+    static __device__ __forceinline__ void entries(const vec& c, uint32_t* e) {
+        e[0] = c.x; e[1] = (c.x >> 24) | (c.y << 8); e[2] = (c.y >> 16) | (c.z << 16); e[3] = c.z >> 8;
+    }
+    static __device__ __forceinline__ void addrs(const vec& c, uint32_t xbase, uint32_t* ta, uint32_t* xa) {
+        ta[0] = (c.x << 4) & 0xFFF0u;                               xa[0] = stream_field16<12, 12>(c.x, xbase);
+        ta[1] = __builtin_amdgcn_alignbit(c.y, c.x, 20) & 0xFFF0u;  xa[1] = stream_field16<4, 12>(c.y, xbase);
+        ta[2] = (c.y >> 12) & 0xFFF0u;                              xa[2] = stream_field16<0, 12>(__builtin_amdgcn_alignbit(c.z, c.y, 28), xbase);
+        ta[3] = (c.z >> 4) & 0xFFF0u;                               xa[3] = stream_field16<20, 12>(c.z, xbase);
+    }
+    static __device__ __forceinline__ vec zero() { return vec{0u, 0u, 0u}; }
+};
+template <> struct StreamF<1> {
+    static constexpr int EPS = 3, LB = 8, SB = 512, PF = 4;
+    static constexpr uint32_t CMASK = 0x1FFu;
+    typedef u32x2 vec;
+    static __device__ __forceinline__ void entries(const vec& c, uint32_t* e) {
+        e[0] = c.x; e[1] = (c.x >> 21) | (c.y << 11); e[2] = c.y >> 10;
+    }
+    static __device__ __forceinline__ void addrs(const vec& c, uint32_t xbase, uint32_t* ta, uint32_t* xa) {
+        ta[0] = (c.x << 4) & 0xFFF0u;                               xa[0] = stream_field16<12, 9>(c.x, xbase);
+        ta[1] = __builtin_amdgcn_alignbit(c.y, c.x, 17) & 0xFFF0u;  xa[1] = stream_field16<1, 9>(c.y, xbase);
+        ta[2] = (c.y >> 6) & 0xFFF0u;                               xa[2] = stream_field16<22, 9>(c.y, xbase);
+    }
+    static __device__ __forceinline__ vec zero() { return vec{0u, 0u}; }
+};
 
 // Optional per-wave timeline (debug builds define SQ_TRACE_POINT).
 #ifndef SQ_TRACE_POINT
@@ -669,14 +754,19 @@ constexpr int stream_vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7
 
 typedef const __attribute__((address_space(1))) void* stream_gptr_t;
 typedef __attribute__((address_space(3))) void* stream_lptr_t;
+typedef __attribute__((address_space(3))) u32x4 stream_lds_u32x4;
 
 // NB activation rows per pass (every entry's codeword is gathered once and multiplied with NB x chunks), NX chunks of
-// a row's part of x per thread (1: parts of up to 1024 chunks, 4: up to 4096).  One workgroup of 16 waves per CU.
+// a row's part of x per thread (1: parts of up to 1024 chunks, 4: up to 4096), NAR: the entry format (1: 21-bit entries,
+// parts of at most 496 chunks).  One workgroup of 16 waves per CU.
 // LDS: [codebook slice 64 KB][NB x parts of a.xs bytes][partial sums of the run: NB x a.nl_max floats][two words of flags]
 // [16 block sums (PRO 1)].
-template <int NB, int NX, int PRO = 0, int ORD = 1>
+template <int NB, int NX, int PRO = 0, int ORD = 1, int NAR = 0>
 __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     static_assert(PRO == 0 || (PRO == 1 && NB == 1 && ORD == 0), "produced activations: add + norm, one row, no column orders");
+    typedef StreamF<NAR> F;
+    typedef typename F::vec evec;
+    constexpr int STREAM_PF = F::PF;
     constexpr int NW = STREAM_NW, NTH = NW * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -719,13 +809,15 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 
     const u32x4* gw = reinterpret_cast<const u32x4*>(P.stream) + (size_t)v * P.NG + g0;   // {rest, nst, unit0, split} per group
     const int u0 = perms ? run[3] : wi * gr * stream_split_of(gr);   // this run's first unit
-    const uint32_t* slots = reinterpret_cast<const uint32_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
-    const unsigned char* steps = P.stream + P.off_steps + lane * 12;
+    const uint16_t* slots = reinterpret_cast<const uint16_t*>(P.stream + P.off_slots) + ((size_t)v * P.NG + g0) * 64;
+    const unsigned char* steps = P.stream + P.off_steps + lane * F::LB;
     const size_t np = (size_t)P.NG * 64;
     float* part = P.part + (size_t)v * NB * np;
     const int xs = a.xs;
-    const unsigned char* ldsx = lds + STREAM_TAB;
-    float* psum = reinterpret_cast<float*>(lds + STREAM_TAB + a.xcopies * NB * xs);   // [NB][a.nl_max], indexed by place - 64 g0
+    // (the inner loop forms LDS addresses as numbers counted from the start of the dynamic LDS: that is address 0 in a
+    // kernel without static LDS; a build in which it is not leaves y unwritten, which no test survives)
+    if ((uint32_t)(uintptr_t)(stream_lptr_t)lds != 0u) return;
+    float* psum = reinterpret_cast<float*>(lds + STREAM_TAB + a.xcopies * NB * xs);   // [NB][a.nl_max], indexed by place in the run
     unsigned* flag = reinterpret_cast<unsigned*>(psum + (size_t)NB * a.nl_max);  // [1] next group
 
     // The groups of a run are sorted longest first.  Wave w starts with group w, then group 2 NW - 1 - w; after
@@ -741,13 +833,12 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     // What this wave walks of group k, from the group's loaded words: the whole group, or its share of the steps.
     auto head_from = [&](int k, uint32_t rest, uint32_t nst_g, uint32_t sl) {
         StreamHead h{rest - (uint32_t)STREAM_PF, (int)nst_g, sl};
-        if (k >= ng) h = StreamHead{0u, 0, STREAM_NO_ROW};
+        if (k >= ng) h = StreamHead{0u, 0, STREAM_SLOT_NONE};
         else if (split > 1) {                                   // uniform in the workgroup
+            // (a share that holds only padding of a row adds exactly nothing, like padding anywhere else)
             const int s0 = h.nst * sub / split, s1 = h.nst * (sub + 1) / split;
-            const int cnt = max((int)(h.slot >> STREAM_ROW_BITS) - 4 * s0, 0);
             h.rb = rest + (uint32_t)s0 - (uint32_t)(STREAM_PF * (sub + 1));
             h.nst = s1 - s0;
-            h.slot = (h.slot & STREAM_NO_ROW) | ((uint32_t)cnt << STREAM_ROW_BITS);
         }
         return h;
     };
@@ -763,7 +854,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         asm volatile("" : "+v"(kc));
         const u32x2 w = *reinterpret_cast<const u32x2*>(gw + kc);       // (only the first two of the four words: every register
                                                                         // a load writes must stay in use until it has landed)
-        return StreamHeadRaw{w.x, w.y, slots[(size_t)kc * 64 + lane], k};
+        return StreamHeadRaw{w.x, w.y, (uint32_t)slots[(size_t)kc * 64 + lane], k};
     };
     // (the empty asm pins the arithmetic to the place of the call: hoisted to where the words are loaded it would bring
     // the wait along)
@@ -773,11 +864,12 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     };
     // The first STREAM_PF steps of this wave's unit of group k: their place follows from indices alone, so they are
     // requested without having read anything (every unit has STREAM_PF steps there, used or not).
-    auto first_steps = [&](int k, u32x3* nx) {
+    const int fs = P.fs;
+    auto first_steps = [&](int k, evec* nx) {
         const int unit = u0 + min(k, ng - 1) * split + sub;
-        const unsigned char* en = steps + ((size_t)unit * P.NV + v) * (STREAM_PF * 768);
+        const unsigned char* en = steps + ((size_t)unit * P.NV + v) * (size_t)(fs * F::SB);
 #pragma unroll
-        for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const u32x3*>(en + (size_t)q * 768);
+        for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const evec*>(en + (size_t)min(q, fs - 1) * F::SB);
     };
     int kcur = wave, knext = 2 * NW - 1 - wave;
     if (split > 1) {                                            // one share of one group per wave, or nothing
@@ -809,9 +901,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
     StreamHeadRaw hn;
-    u32x3 nx[STREAM_PF];
+    evec nx[STREAM_PF];
 #pragma unroll
-    for (int q = 0; q < STREAM_PF; ++q) nx[q] = u32x3{0u, 0u, 0u};
+    for (int q = 0; q < STREAM_PF; ++q) nx[q] = F::zero();
 
     // Stage this part of the NB activation rows (as fp16); the first group's steps are requested before anything waits
     // for the staging loads.
@@ -1000,45 +1092,50 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
             kafter = (int)__builtin_amdgcn_readfirstlane(tk);
         }
         const int nst = uni(h.nst);
-        const int cnt = (int)(h.slot >> STREAM_ROW_BITS);
-        const uint32_t row = h.slot & STREAM_NO_ROW;
-        const unsigned char* eb = steps + (size_t)(uint32_t)uni((int)h.rb) * 768;
+        const bool has = (h.slot & STREAM_SLOT_HAS) != 0u;
+        const uint32_t row = h.slot & STREAM_SLOT_NONE;        // place in the run
+        const unsigned char* eb = steps + (size_t)(uint32_t)uni((int)h.rb) * F::SB;
         // the copy of x for this group's column order
         int xc = 0;
 #pragma unroll
         for (int oi = 1; oi < STREAM_RUN_ORDERS; ++oi) xc += (oi < no && kcur >= byte_of(bnd_lo, bnd_hi, oi)) ? 1 : 0;
-        const unsigned char* ldsx_u = ldsx + (size_t)xc * NB * xs;
+        // LDS byte address of this group's copy of x, kept in a vector register: a chunk's address is then one
+        // shift-and-add (the instruction takes one scalar or constant operand, and the shift count is one already)
+        uint32_t xbase = (uint32_t)STREAM_TAB + (uint32_t)(xc * NB * xs);
+        asm volatile("" : "+v"(xbase));
         float acc[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) acc[b] = 0.f;
         for (int t0 = 0; t0 < nst; t0 += STREAM_PF) {
-            u32x3 cur[STREAM_PF];
+            evec cur[STREAM_PF];
 #pragma unroll
             for (int q = 0; q < STREAM_PF; ++q) cur[q] = nx[q];
             if (t0 + STREAM_PF < nst) {                         // wave-uniform
 #pragma unroll
                 for (int q = 0; q < STREAM_PF; ++q)
-                    nx[q] = *reinterpret_cast<const u32x3*>(eb + (size_t)min(t0 + STREAM_PF + q, nst - 1) * 768);
+                    nx[q] = *reinterpret_cast<const evec*>(eb + (size_t)min(t0 + STREAM_PF + q, nst - 1) * F::SB);
             } else {
                 if (knext < ng) first_steps(knext, nx);         // the next group's first steps
             }
 #pragma unroll
             for (int q = 0; q < STREAM_PF; ++q) {
                 if (t0 + q >= nst) break;                       // wave-uniform
-                // (bits above an entry's 24 are left in place: the address fields are cut out below)
-                const uint32_t e[4] = {cur[q].x, (cur[q].x >> 24) | (cur[q].y << 8), (cur[q].y >> 16) | (cur[q].z << 16), cur[q].z >> 8};
+                uint32_t ta[F::EPS], xa[F::EPS];
+                F::addrs(cur[q], xbase, ta, xa);
                 // the LDS reads of EB entries go out together, then their products: a wave does not sit out one
                 // LDS round trip per entry
-                constexpr int EB = NB == 1 ? 4 : NB == 2 ? 2 : 1;
+                constexpr int EB = NB == 1 ? F::EPS : NB == 2 ? (NAR ? 3 : 2) : 1;
 #pragma unroll
-                for (int j0 = 0; j0 < 4; j0 += EB) {
+                for (int j0 = 0; j0 < F::EPS; j0 += EB) {
                     u32x4 cw[EB], xv[EB][NB];
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
-                        const uint32_t ta = (e[j0 + jj] & 0xFFFu) << 4, xa = ((e[j0 + jj] >> 12) & 0xFFFu) << 4;
-                        cw[jj] = *reinterpret_cast<const u32x4*>(lds + ta);
+                        // (LDS addresses as plain numbers: the kernel's dynamic LDS begins at address 0, checked at its
+                        // start, and `lds + offset` would cost an addition of that zero per read)
+                        cw[jj] = *reinterpret_cast<const stream_lds_u32x4*>((uintptr_t)ta[j0 + jj]);
 #pragma unroll
-                        for (int b = 0; b < NB; ++b) xv[jj][b] = *reinterpret_cast<const u32x4*>(ldsx_u + b * xs + xa);
+                        for (int b = 0; b < NB; ++b)
+                            xv[jj][b] = *reinterpret_cast<const stream_lds_u32x4*>((uintptr_t)(xa[j0 + jj] + (uint32_t)(b * (NAR ? 8192 : xs))));
                     }
 #pragma unroll
                     for (int jj = 0; jj < EB; ++jj) {
@@ -1054,7 +1151,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                 }
             }
         }
-        if (cnt == 0) {                                         // a row without entries in this bucket (or share)
+        if (!has) {                                             // no row, or a row without entries in this bucket
 #pragma unroll
             for (int b = 0; b < NB; ++b) acc[b] = 0.f;
         }
@@ -1065,9 +1162,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
             k_share = kcur;
 #pragma unroll
             for (int b = 0; b < NB; ++b) acc_share[b] = acc[b];
-        } else if (row != STREAM_NO_ROW) {
+        } else if (row != STREAM_SLOT_NONE) {
 #pragma unroll
-            for (int b = 0; b < NB; ++b) psum[b * a.nl_max + (int)row - g0 * 64] = acc[b];
+            for (int b = 0; b < NB; ++b) psum[b * a.nl_max + (int)row] = acc[b];
         }
         kcur = knext;
         knext = kafter;
@@ -1080,13 +1177,13 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         for (int b = 0; b < NB; ++b) share[(wave * NB + b) * 64 + lane] = acc_share[b];
         __syncthreads();
         if (sub == 0 && k_share >= 0) {
-            const uint32_t row = slots[(size_t)k_share * 64 + lane] & STREAM_NO_ROW;
-            if (row != STREAM_NO_ROW) {
+            const uint32_t row = slots[(size_t)k_share * 64 + lane] & STREAM_SLOT_NONE;
+            if (row != STREAM_SLOT_NONE) {
 #pragma unroll
                 for (int b = 0; b < NB; ++b) {
                     float sum = 0.f;
                     for (int j = 0; j < split; ++j) sum += share[((wave + j) * NB + b) * 64 + lane];
-                    psum[b * a.nl_max + (int)row - g0 * 64] = sum;
+                    psum[b * a.nl_max + (int)row] = sum;
                 }
             }
         }
@@ -1173,25 +1270,27 @@ static size_t stream_smem(int nb_t, int xs, int nl_max, int xcopies = 1, int xtm
     return (size_t)STREAM_TAB + (size_t)xcopies * nb_t * xs + (size_t)nb_t * nl_max * 4 + 16 + 64 + (size_t)nb_t * xtmp;
 }
 
-template <int NB, int NX, int PRO, int ORD>
+template <int NB, int NX, int PRO, int ORD, int NAR>
 static int stream_launch_as(const StreamArgs& a, int grid, hipStream_t s) {
-    static bool raised = false;
-    if (!raised) {
-        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NX, PRO, ORD>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    // (the attribute is a property of the function, the same on every device; setting it twice from two threads is harmless)
+    static std::atomic<bool> raised{false};
+    if (!raised.load(std::memory_order_acquire)) {
+        (void)hipFuncSetAttribute((const void*)stream_kernel<NB, NX, PRO, ORD, NAR>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         (void)hipGetLastError();
-        raised = true;
+        raised.store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((stream_kernel<NB, NX, PRO, ORD>), dim3((unsigned)grid), dim3(STREAM_NW * 64), stream_smem(NB, a.xs, a.nl_max, a.xcopies, a.xtmp_own ? a.xtmp : 0), s, a);
+    hipLaunchKernelGGL((stream_kernel<NB, NX, PRO, ORD, NAR>), dim3((unsigned)grid), dim3(STREAM_NW * 64), stream_smem(NB, a.xs, a.nl_max, a.xcopies, a.xtmp_own ? a.xtmp : 0), s, a);
     return check_launch("sq_linear_small(stream)");
 }
-// (a.orders: some piece of the launch has column orders)
+// (a.orders: some piece of the launch has column orders; a.narrow: the pieces' entry format)
 template <int NB, int NX, int PRO = 0>
 static int stream_launch(const StreamArgs& a, int grid, hipStream_t s) {
     if (PRO != 0) {
         if (a.orders) return fail(SQ_EUNSUPPORTED, "sq_linear_small_from: no fused kernel for pieces with column orders");
-        return stream_launch_as<NB, NX, PRO, 0>(a, grid, s);
+        return a.narrow ? stream_launch_as<NB, NX, PRO, 0, 1>(a, grid, s) : stream_launch_as<NB, NX, PRO, 0, 0>(a, grid, s);
     }
-    return a.orders ? stream_launch_as<NB, NX, 0, 1>(a, grid, s) : stream_launch_as<NB, NX, 0, 0>(a, grid, s);
+    if (a.narrow) return a.orders ? stream_launch_as<NB, NX, 0, 1, 1>(a, grid, s) : stream_launch_as<NB, NX, 0, 0, 1>(a, grid, s);
+    return a.orders ? stream_launch_as<NB, NX, 0, 1, 0>(a, grid, s) : stream_launch_as<NB, NX, 0, 0, 0>(a, grid, s);
 }
 
 // ---- dense rows from the tag stream alone (a matrix held in one copy: sq_matrix.tags == NULL).  One wave per (bucket,
@@ -1205,42 +1304,47 @@ struct StreamDeqArgs {
     const int32_t* perms;
     void* out;
     int64_t ld_out;
-    int R, C, NS, NV, PC, NG, r0, r1, raw, vec;
+    int R, C, NS, NV, PC, NG, fs, r0, r1, raw, vec;
     uint32_t off_slots, off_rows, off_steps;
 };
 
-template <int DT>
+template <int DT, int NAR>
 __global__ __launch_bounds__(256) void stream_dequant_kernel(StreamDeqArgs a) {
     typedef typename store_as<DT>::type T;
+    typedef StreamF<NAR> F;
+    constexpr int STREAM_PF = F::PF;
     const int lane = threadIdx.x & 63;
     const int w = (int)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     if (w >= a.NV * a.NG) return;
-    const int v = w / a.NG, g = w - v * a.NG, s = v % a.NS, kp = v / a.NS;
-    const uint32_t slot = reinterpret_cast<const uint32_t*>(a.stream + a.off_slots)[(size_t)w * 64 + lane];
-    const uint32_t place = slot & STREAM_NO_ROW;
-    const int cnt = (int)(slot >> STREAM_ROW_BITS);
+    const int v = w / a.NG, s = v % a.NS, kp = v / a.NS;
+    const u32x4 hw = reinterpret_cast<const u32x4*>(a.stream)[w];             // {rest, nst, unit0, split | g0 << 8}
+    const int nst = (int)hw.y, split = (int)(hw.w & 0xFFu);
+    const uint32_t slot = reinterpret_cast<const uint16_t*>(a.stream + a.off_slots)[(size_t)w * 64 + lane];
     uint32_t row = STREAM_NO_ROW;
-    if (place != STREAM_NO_ROW) row = a.perms ? reinterpret_cast<const uint32_t*>(a.stream + a.off_rows)[place] : place;
-    const bool mine = row != STREAM_NO_ROW && (int)row >= a.r0 && (int)row < a.r1 && cnt > 0;
+    if ((slot & STREAM_SLOT_NONE) != STREAM_SLOT_NONE) {
+        const uint32_t place = (slot & STREAM_SLOT_NONE) + (hw.w >> 8) * 64u;
+        row = a.perms ? reinterpret_cast<const uint32_t*>(a.stream + a.off_rows)[place] : place;
+    }
+    const bool mine = row != STREAM_NO_ROW && (int)row >= a.r0 && (int)row < a.r1 && (slot & STREAM_SLOT_HAS) != 0u;
     if (__ballot(mine) == 0) return;                             // (wave-uniform) none of this group's rows is wanted
-    const u32x4 hw = reinterpret_cast<const u32x4*>(a.stream)[w];             // {rest, nst, unit0, split}
-    const int nst = (int)hw.y, split = (int)hw.w;
     const float sc = (mine && !a.raw) ? h2f(a.row_scale[row]) : 1.f;
     const int32_t* pm = (mine && a.perms) ? a.perms + (size_t)(a.row_mask ? a.row_mask[row] : 0) * a.C : nullptr;
     T* orow = reinterpret_cast<T*>(a.out) + (mine ? (int64_t)((int)row - a.r0) * a.ld_out : 0);
-    const unsigned char* rec = a.stream + a.off_steps + lane * 12;
+    const unsigned char* rec = a.stream + a.off_steps + lane * F::LB;
     int j = 0, s0 = 0, s1 = nst / split;                          // the share step t belongs to, its first and end step
     for (int t = 0; t < nst; ++t) {
         while (t >= s1) { ++j; s0 = s1; s1 = nst * (j + 1) / split; }
-        const size_t at = t - s0 < STREAM_PF ? ((size_t)(hw.z + (uint32_t)j) * a.NV + v) * STREAM_PF + (size_t)(t - s0)
+        const size_t at = t - s0 < STREAM_PF ? ((size_t)(hw.z + (uint32_t)j) * a.NV + v) * a.fs + (size_t)(t - s0)
                                              : (size_t)hw.x + (size_t)t - (size_t)STREAM_PF * (j + 1);
-        const u32x3 r = *reinterpret_cast<const u32x3*>(rec + at * 768);
-        const uint32_t e[4] = {r.x, (r.x >> 24) | (r.y << 8), (r.y >> 16) | (r.z << 16), r.z >> 8};
+        uint32_t e[F::EPS];
+        F::entries(*reinterpret_cast<const typename F::vec*>(rec + at * F::SB), e);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (!mine || 4 * t + j >= cnt) continue;
+        for (int j = 0; j < F::EPS; ++j) {
+            // (padding entries name one of the zero chunks behind the part's own)
+            const int cj = (int)((e[j] >> STREAM_SLICE_BITS) & F::CMASK);
+            if (!mine || cj >= a.PC) continue;
             const uint32_t tag = (e[j] & 0xFFFu) + ((uint32_t)s << STREAM_SLICE_BITS);
-            const int c0 = ((int)((e[j] >> STREAM_SLICE_BITS) & 0xFFFu) + kp * a.PC) * 8;
+            const int c0 = (cj + kp * a.PC) * 8;
             const u32x4 cw = *reinterpret_cast<const u32x4*>(a.table + (size_t)tag * 8);
             T o[8];
 #pragma unroll
@@ -1274,18 +1378,21 @@ int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t 
     StreamDeqArgs a;
     a.stream = (const unsigned char*)m.stream;
     a.table = g.off_table ? (const uint16_t*)((const unsigned char*)m.stream + g.off_table) : m.table; a.row_scale = m.row_scale; a.row_mask = m.row_mask; a.perms = m.perms;
-    a.out = out; a.ld_out = ld_out; a.R = m.R; a.C = m.C; a.NS = g.NS; a.NV = g.NV; a.PC = g.PC; a.NG = g.NG; a.r0 = r0; a.r1 = r1;
+    a.out = out; a.ld_out = ld_out; a.R = m.R; a.C = m.C; a.NS = g.NS; a.NV = g.NV; a.PC = g.PC; a.NG = g.NG; a.fs = g.fs; a.r0 = r0; a.r1 = r1;
     a.raw = raw ? 1 : 0;
     a.off_slots = (uint32_t)g.off_slots; a.off_rows = (uint32_t)g.off_rows; a.off_steps = (uint32_t)g.off_steps;
     const size_t es = out_dtype == SQ_F32 ? 4 : 2;
     a.vec = ((uintptr_t)out & 15) == 0 && (ld_out * es) % 16 == 0;
     const unsigned grid = (unsigned)(((int64_t)g.NV * g.NG + 3) / 4);
+#define SQ_DEQ(DT) do { if (g.fmt.narrow) hipLaunchKernelGGL((stream_dequant_kernel<DT, 1>), dim3(grid), dim3(256), 0, s, a); \
+                        else hipLaunchKernelGGL((stream_dequant_kernel<DT, 0>), dim3(grid), dim3(256), 0, s, a); } while (0)
     switch (out_dtype) {
-        case SQ_F32: hipLaunchKernelGGL((stream_dequant_kernel<SQ_F32>), dim3(grid), dim3(256), 0, s, a); break;
-        case SQ_F16: hipLaunchKernelGGL((stream_dequant_kernel<SQ_F16>), dim3(grid), dim3(256), 0, s, a); break;
-        case SQ_BF16: hipLaunchKernelGGL((stream_dequant_kernel<SQ_BF16>), dim3(grid), dim3(256), 0, s, a); break;
+        case SQ_F32: SQ_DEQ(SQ_F32); break;
+        case SQ_F16: SQ_DEQ(SQ_F16); break;
+        case SQ_BF16: SQ_DEQ(SQ_BF16); break;
         default: return fail(SQ_EINVAL, "sq_dequant: out_dtype %d", out_dtype);
     }
+#undef SQ_DEQ
     return check_launch("sq_dequant(stream)");
 }
 
@@ -1359,6 +1466,7 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         sums_off += stream_part_bytes(m, rows);
         P.perms = m.perms;
         P.R = m.R; P.C = m.C; P.U = g.U; P.NS = g.NS; P.NV = g.NV; P.PC = g.PC; P.NG = g.NG; P.y_off = m.y_off;
+        P.fs = g.fs;
         P.off_slots = (uint32_t)g.off_slots; P.off_runs = (uint32_t)g.off_runs; P.off_rows = (uint32_t)g.off_rows;
         P.off_steps = (uint32_t)g.off_steps;
         const int nwg = g.runs;
@@ -1376,6 +1484,7 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     }
     for (int k = cnt; k < GEMV_MAX_PIECES_STREAM; ++k) a.p[k] = a.p[0];
     a.xs = stream_xs(pc);
+    a.narrow = stream_fmt(pc).narrow;
     a.nl_max = nl_max;
     a.xcopies = xcopies;
     a.xtmp = a.xtmp_own = 0;

@@ -122,33 +122,28 @@ def pack_tensors(local_tags: torch.Tensor, table: torch.Tensor, row_scale: torch
         if int(row_mask.min()) < 0 or int(row_mask.max()) >= M:
             raise ValueError("row_mask out of range")
         t["row_mask"] = row_mask.cpu().to(torch.uint8)
-    perms = mk.seeded_perms(C, M, torch.Generator(device="cpu").manual_seed(seed))
-    meta = {"R": R, "C": C, "d": d, "K": K, "G": G, "M": M, "seed": seed, "perm_crc": perm_crc(perms),
-            "bits": storage_bits(t)}
-    return t, meta
+    meta = MatrixMeta(R=R, C=C, d=d, K=K, G=G, M=M, seed=seed, perm_crc=0, bits=storage_bits(t))
+    meta.perm_crc = perm_crc(meta.column_orders())
+    return t, meta.to_json()
 
 
 def pack_matrix(fit, *, d: int, K: int, G: int, M: int, seed: int) -> tuple[dict, dict]:
     """The reference's entry point (reference shapequant/packed.py:97-131): `fit` is a quantiser
     result with .tags (one stage of global tags), .row_scale, .perms, .row_mask and
     .stats["books"][0]; global tags are split into (row_book, local tag)."""
-    if fit.tags is None or len(fit.tags) != 1:
+    stages = fit.tags
+    if stages is None or len(stages) != 1:
         raise ValueError("pack_matrix needs single-stage global tags (keep_tags=True)")
-    if K & (K - 1):
-        raise ValueError(f"K={K} is not a power of two")
-    R = fit.row_scale.shape[0]
-    C = fit.perms.shape[1]
-    if C % d:
-        raise ValueError(f"C={C} not divisible by d={d}")
-    gt = fit.tags[0].to(torch.int64).view(R, C // d).cpu()
-    book = torch.div(gt, K, rounding_mode="floor")
-    if not bool((book == book[:, :1]).all()):
+    R, C = fit.row_scale.shape[0], fit.perms.shape[1]
+    if K & (K - 1) or C % d:
+        raise ValueError(f"K={K} is not a power of two" if K & (K - 1) else f"C={C} not divisible by d={d}")
+    global_tags = stages[0].to(torch.int64).view(R, C // d).cpu()
+    book, local = global_tags >> (K.bit_length() - 1), global_tags & (K - 1)
+    if bool((book != book[:, :1]).any()):
         raise ValueError("a row's tags span several codebooks")
-    t, meta = pack_tensors(gt - book[:, :1] * K, fit.stats["books"][0], fit.row_scale, d=d, K=K, G=G, M=M, seed=seed,
-                           row_book=book[:, 0] if G > 1 else None,
-                           row_mask=fit.row_mask if M > 1 else None)
-    perms = mk.seeded_perms(C, M, torch.Generator(device="cpu").manual_seed(seed))
-    if not torch.equal(perms, fit.perms.cpu()):
+    t, meta = pack_tensors(local, fit.stats["books"][0], fit.row_scale, d=d, K=K, G=G, M=M, seed=seed,
+                           row_book=book[:, 0] if G > 1 else None, row_mask=fit.row_mask if M > 1 else None)
+    if not torch.equal(MatrixMeta.from_json(meta).column_orders(), fit.perms.cpu()):
         raise ValueError("fit's column orders do not regenerate from its seed")
     return t, meta
 
@@ -202,102 +197,147 @@ def q8_rows(q: torch.Tensor, sc: torch.Tensor, s: int = 0, e: int | None = None)
     return q8_dense(q, sc, s, max(s, e), torch.float32)
 
 
+class MatrixMeta:
+    """What the file's "matrices" metadata says about one matrix (reference shapequant/packed.py:122-131 writes the same
+    keys): the one place that knows which tensors a matrix has and how wide its tags are."""
+    KEYS = ("R", "C", "d", "K", "G", "M", "seed", "perm_crc", "bits")
+
+    def __init__(self, **kw):
+        missing = [k for k in self.KEYS if k not in kw]
+        if missing:
+            raise ValueError(f"matrix metadata lacks {missing}")
+        self.extra = {k: v for k, v in kw.items() if k not in self.KEYS}     # keys of later writers are carried along
+        for k in self.KEYS:
+            setattr(self, k, int(kw[k]))
+
+    @classmethod
+    def from_json(cls, d: dict) -> "MatrixMeta":
+        return cls(**d)
+
+    def to_json(self) -> dict:
+        return {**{k: getattr(self, k) for k in self.KEYS}, **self.extra}
+
+    @property
+    def tag_bits(self) -> int:
+        return int(math.log2(self.K))
+
+    @property
+    def chunks(self) -> int:
+        return self.C // self.d
+
+    def tensor_keys(self) -> tuple:
+        return ("tags", "table", "row_scale") + (("row_book",) if self.G > 1 else ()) + (("row_mask",) if self.M > 1 else ())
+
+    def column_orders(self) -> torch.Tensor:
+        return mk.seeded_perms(self.C, self.M, torch.Generator(device="cpu").manual_seed(self.seed))
+
+
+class AuxSection:
+    """The optional self-contained part of a file (reference shapequant/packed.py:30-40,162-183): 4-bit embedding, 8-bit
+    output head and every other parameter as stored.  `tensors` carry their file names ("aux. ..."), `meta` is the
+    JSON the file keeps under "aux"."""
+    PER_WEIGHT = {"embed": 4 + 16 / 32, "lm_head": 8 + 16 / 32}               # level bits + one fp16 scale per 32 columns
+
+    def __init__(self, tensors: dict, meta: dict):
+        self.tensors, self.meta = tensors, meta
+
+    @classmethod
+    def from_model(cls, model, block_names) -> "AuxSection":
+        """From an HF causal LM whose block linears `block_names` are packed separately."""
+        embed, head = model.model.embed_tokens.weight.detach(), model.lm_head.weight.detach()
+        packed_elsewhere = {"lm_head.weight", "model.embed_tokens.weight", *(f"{n}.weight" for n in block_names)}
+        kept = {n: p.detach().cpu().contiguous() for n, p in model.named_parameters() if n not in packed_elsewhere}
+        tensors = {f"aux.dense.{n}": t for n, t in kept.items()}
+        (tensors["aux.embed.q"], tensors["aux.embed.scale"]) = (t.cpu() for t in q4_embed_pack(embed))
+        tensors["aux.lm_head.q"], tensors["aux.lm_head.scale"], _ = q8_pack(head.float().cpu())
+        meta = {"embed": "q4_b32", "lm_head": "q8_b32", "dense": sorted(kept), "config": model.config.to_dict(),
+                "vocab": embed.shape[0], "hidden": embed.shape[1],
+                "tied": bool(getattr(model.config, "tie_word_embeddings", False))}
+        return cls(tensors, meta)
+
+    @classmethod
+    def bits_of(cls, meta: dict) -> dict:
+        n = meta["vocab"] * meta["hidden"]
+        return {k: n * b for k, b in cls.PER_WEIGHT.items()}
+
+    def dense(self) -> list:
+        return [t for k, t in self.tensors.items() if k.startswith("aux.dense.")]
+
+    def weights(self) -> int:
+        return 2 * self.meta["vocab"] * self.meta["hidden"] + sum(t.numel() for t in self.dense())
+
+    def bits(self) -> float:
+        return sum(self.bits_of(self.meta).values()) + sum(8 * t.numel() * t.element_size() for t in self.dense())
+
+
 def aux_from_model(model, block_names) -> tuple[dict, dict]:
-    """The aux section of an HF causal LM: 4-bit embedding, 8-bit head and every parameter that is
-    neither of those nor one of the packed block linears `block_names`
-    (reference shapequant/packed.py:162-177)."""
-    E = model.model.embed_tokens.weight.detach()
-    H = model.lm_head.weight.detach()
-    eq, es = q4_embed_pack(E)
-    hq, hs, _ = q8_pack(H.float().cpu())
-    left_out = {f"{n}.weight" for n in block_names} | {"lm_head.weight", "model.embed_tokens.weight"}
-    t = {"aux.embed.q": eq.cpu(), "aux.embed.scale": es.cpu(), "aux.lm_head.q": hq, "aux.lm_head.scale": hs}
-    dense = []
-    for n, p in model.named_parameters():
-        if n not in left_out:
-            t[f"aux.dense.{n}"] = p.detach().cpu().contiguous()
-            dense.append(n)
-    meta = {"embed": "q4_b32", "lm_head": "q8_b32", "dense": sorted(dense), "config": model.config.to_dict(),
-            "vocab": E.shape[0], "hidden": E.shape[1],
-            "tied": bool(getattr(model.config, "tie_word_embeddings", False))}
-    return t, meta
+    """(tensors, meta) of the aux section of an HF causal LM (reference shapequant/packed.py:162-177)."""
+    a = AuxSection.from_model(model, block_names)
+    return a.tensors, a.meta
 
 
 def aux_bits(meta: dict) -> dict:
-    """Storage bits of the aux embedding (4 + 16/32 per weight) and head (8 + 16/32)
-    (reference shapequant/packed.py:180-183)."""
-    n = meta["vocab"] * meta["hidden"]
-    return {"embed": n * 4.5, "lm_head": n * 8.5}
+    """Storage bits of the aux embedding and head (reference shapequant/packed.py:180-183)."""
+    return AuxSection.bits_of(meta)
 
 
 def save(path, packed: dict, *, base_model: str, extra: dict | None = None, aux: tuple | None = None) -> dict:
-    """Write {name: (tensors, meta)} to one safetensors file; returns the summary
-    (reference shapequant/packed.py:186-214).  `aux` = (tensors, meta) from aux_from_model."""
+    """Write {name: (tensors, meta)} to one safetensors file and return its summary (reference
+    shapequant/packed.py:186-214).  `aux`: (tensors, meta) as aux_from_model gives them."""
     from safetensors.torch import save_file
-    tensors, metas = {}, {}
-    for name, (t, m) in packed.items():
-        for k, v in t.items():
-            tensors[f"{name}.{k}"] = v.contiguous()
-        metas[name] = m
-    bits = sum(m["bits"] for m in metas.values())
-    numel = sum(m["R"] * m["C"] for m in metas.values())
+    metas = {name: MatrixMeta.from_json(m) for name, (_, m) in packed.items()}
+    out = {f"{name}.{k}": t[k].contiguous() for name, (t, _) in packed.items() for k in t}
+    bits, numel = sum(m.bits for m in metas.values()), sum(m.R * m.C for m in metas.values())
     summary = {"format": FORMAT, "base_model": base_model, "matrices": len(metas), "bits": bits, "numel": numel,
-               "bpw": bits / numel if numel else 0.0, **(extra or {})}
-    md = {"matrices": json.dumps(metas)}
+               "bpw": bits / numel if numel else 0.0}
+    summary.update(extra or {})
+    header = {"matrices": json.dumps({name: m.to_json() for name, m in metas.items()})}
     if aux is not None:
-        at, am = aux
-        tensors.update(at)
-        md["aux"] = json.dumps(am, default=str)
-        dense = [v for k, v in at.items() if k.startswith("aux.dense.")]
-        ab = aux_bits(am)
-        all_bits = bits + ab["embed"] + ab["lm_head"] + sum(v.numel() * v.element_size() * 8 for v in dense)
-        summary["bpw_all"] = all_bits / (numel + 2 * am["vocab"] * am["hidden"] + sum(v.numel() for v in dense))
-        summary["aux"] = True
-    md["summary"] = json.dumps(summary)
+        section = AuxSection(*aux)
+        out.update(section.tensors)
+        header["aux"] = json.dumps(section.meta, default=str)
+        summary.update(bpw_all=(bits + section.bits()) / (numel + section.weights()), aux=True)
+    header["summary"] = json.dumps(summary)
     Path(path).parent.mkdir(parents=True, exist_ok=True)
-    save_file(tensors, str(path), metadata=md)
+    save_file(out, str(path), metadata=header)
     return summary
 
 
 class PackedFile:
-    """Read access to a packed file (reference shapequant/packed.py:217-256): metadata, raw
-    tensors, regenerated column orders, unpacked tags, and the dense decode (on the GPU)."""
+    """Read access to a packed file (reference shapequant/packed.py:217-256): `summary`, `meta` (the file's JSON per
+    matrix, as the reference exposes it), `matrices` (the same as MatrixMeta), `aux`; raw tensors, regenerated
+    column orders, unpacked tags, and the dense decode (on the GPU)."""
 
     def __init__(self, path):
         from safetensors import safe_open
         self.path = str(path)
         self.f = safe_open(self.path, framework="pt", device="cpu")
-        md = self.f.metadata() or {}
-        if "summary" not in md or "matrices" not in md:
-            raise ValueError(f"{path}: not a {FORMAT} file (no summary / matrices metadata)")
-        self.summary = json.loads(md["summary"])
+        header = self.f.metadata() or {}
+        need = [k for k in ("summary", "matrices") if k not in header]
+        if need:
+            raise ValueError(f"{path}: not a {FORMAT} file (no {' / '.join(need)} metadata)")
+        self.summary, self.meta = json.loads(header["summary"]), json.loads(header["matrices"])
         if self.summary.get("format") != FORMAT:
             raise ValueError(f"{path}: format {self.summary.get('format')!r} != {FORMAT}")
-        self.meta = json.loads(md["matrices"])
-        self.aux = json.loads(md["aux"]) if "aux" in md else None
+        self.matrices = {name: MatrixMeta.from_json(m) for name, m in self.meta.items()}
+        self.aux = json.loads(header["aux"]) if "aux" in header else None
 
     def aux_tensor(self, name: str) -> torch.Tensor:
         return self.f.get_tensor(f"aux.{name}")
 
     def tensors(self, name: str) -> dict:
-        m = self.meta[name]
-        keys = ["tags", "table", "row_scale"]
-        if m["G"] > 1:
-            keys.append("row_book")
-        if m["M"] > 1:
-            keys.append("row_mask")
-        return {k: self.f.get_tensor(f"{name}.{k}") for k in keys}
+        return {k: self.f.get_tensor(f"{name}.{k}") for k in self.matrices[name].tensor_keys()}
 
     def perms(self, name: str) -> torch.Tensor:
-        m = self.meta[name]
-        p = mk.seeded_perms(m["C"], m["M"], torch.Generator(device="cpu").manual_seed(m["seed"]))
-        if perm_crc(p) != m["perm_crc"]:
+        m = self.matrices[name]
+        orders = m.column_orders()
+        if perm_crc(orders) != m.perm_crc:
             raise RuntimeError(f"{name}: regenerated column orders do not match the file (torch RNG changed?)")
-        return p
+        return orders
 
     def local_tags(self, name: str, device="cpu") -> torch.Tensor:
-        m = self.meta[name]
-        return unpack_bits(self.f.get_tensor(f"{name}.tags").to(device), int(math.log2(m["K"])), m["C"] // m["d"])
+        m = self.matrices[name]
+        return unpack_bits(self.f.get_tensor(f"{name}.tags").to(device), m.tag_bits, m.chunks)
 
     def decode(self, name: str, device="cuda") -> torch.Tensor:
         """Dense float32 [R, C] weight in the original row and column order, decoded by the HIP

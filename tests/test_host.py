@@ -209,25 +209,59 @@ def _build_stream(words, R, C, bits, row_mask, runs, table=None):
 
 
 PART_MAX = 4064     # chunks per column part (sq_stream.h)
-PF, NW = 3, 16      # steps of a unit in the first-steps region (= the kernel's prefetch depth); waves per workgroup
+NW = 16             # waves per workgroup
+SLOT_NONE, SLOT_HAS = 0x1FFF, 0x2000    # a lane's slot: place in its run (0x1FFF: no row) | 0x2000 when the row has entries here
 
 
-def _step_places(head, v, NV):
-    """Places (in 768-byte steps from the start of the step area) of steps 0 .. nst - 1 of a group with head words
-    {rest, nst, unit0, split} in bucket v (sq_stream.h): the first PF steps of every share sit in the first-steps region
-    at ((unit0 + share) * NV + v) * PF, the others follow each other from `rest` on."""
+class _Fmt:
+    """The two entry formats (sq_stream.h, StreamFmt): parts of at most 496 chunks store 21-bit entries, three per lane
+    and step in 8 bytes; wider parts 24-bit entries, four per lane and step in 12 bytes.  pf: the kernel's prefetch
+    depth in steps (12 entries per lane either way)."""
+    def __init__(self, PC):
+        self.narrow = PC <= 496
+        self.eps, self.lane_bytes, self.pf, self.cmask = (3, 8, 4, 0x1FF) if self.narrow else (4, 12, 3, 0xFFF)
+        self.step_bytes = 64 * self.lane_bytes
+
+    def entries(self, buf, off_steps, total):
+        """[step, lane, eps] entries of `total` steps."""
+        if self.narrow:
+            w = np.frombuffer(buf, "<u8", total * 64, off_steps).reshape(total, 64)
+            assert not (w >> np.uint64(63)).any()
+            return np.stack([(w >> np.uint64(21 * i)) & np.uint64(0x1FFFFF) for i in range(3)], -1).astype(np.int64)
+        b = np.frombuffer(buf, np.uint8, total * 768, off_steps).reshape(total, 64, 4, 3).astype(np.int64)
+        return b[..., 0] | b[..., 1] << 8 | b[..., 2] << 16
+
+
+def _geom(C, bits):
+    U, NS = C // 8, 1 << (bits - 12)
+    KP = -(-U // PART_MAX)
+    PC = -(-U // KP)
+    return U, NS, KP, PC, NS * KP, _Fmt(PC)
+
+
+def _fs_of(runs_out):
+    """Steps per unit in the first-steps region (bits 27-28 of runs_out, less one)."""
+    return ((runs_out >> 27) & 3) + 1
+
+
+def _step_places(head, v, NV, PF, FS):
+    """Places (in steps from the start of the step area) of steps 0 .. nst - 1 of a group with head words
+    {rest, nst, unit0, split | g0 << 8} in bucket v (sq_stream.h): the first PF steps of every share sit in the
+    first-steps region at ((unit0 + share) * NV + v) * FS, the others follow each other from `rest` on."""
     rest, nst, unit0, split = (int(x) for x in head)
+    split &= 0xFF
     out = []
     for j in range(split):
         s0, s1 = nst * j // split, nst * (j + 1) // split
         for t in range(s0, s1):
-            out.append(((unit0 + j) * NV + v) * PF + (t - s0) if t - s0 < PF else rest + t - PF * (j + 1))
+            assert t - s0 < FS or FS == PF
+            out.append(((unit0 + j) * NV + v) * FS + (t - s0) if t - s0 < PF else rest + t - PF * (j + 1))
     return out
 
 
 def _stream_offsets(NV, NG, runs, bits, d, balanced):
     off_slots = (NV * NG * 16 + 255) & ~255
-    off_runs = (off_slots + NV * NG * 64 * 4 + 255) & ~255
+    off_runs = (off_slots + NV * NG * 64 * 2 + 255) & ~255
     off_rows = (off_runs + runs * 32 + 255) & ~255
     off_steps = (off_rows + NG * 64 * 4 + 255) & ~255
     off_table = off_unmap = 0
@@ -238,13 +272,12 @@ def _stream_offsets(NV, NG, runs, bits, d, balanced):
     return off_slots, off_runs, off_rows, off_table, off_unmap, off_steps
 
 
-def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
+def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None, runs_out=None):
     """Rebuild the [R, C/d] tag matrix from a stream buffer, checking its structure on the way.  A balanced stream
     (built with `table`) stores relabelled tags, its relabelled codebook and the map back to the file's labels."""
-    U, NS = C // d, 1 << (bits - 12)
-    KP = -(-U // PART_MAX)
-    PC = -(-U // KP)
-    NV = NS * KP
+    U, NS, KP, PC, NV, F = _geom(C, bits)
+    PF, FS = F.pf, _fs_of(_build_stream.runs_out if runs_out is None else runs_out)
+    assert 1 <= FS <= PF
     off_slots, off_runs, off_rows, off_table, off_unmap, off_steps = _stream_offsets(NV, NG, runs, bits, d, table is not None)
     unmap = None
     if table is not None:
@@ -253,8 +286,8 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
         assert sorted(unmap.tolist()) == list(range(K))                        # a permutation of the labels
         moved = np.frombuffer(buf, np.uint16, K * d, off_table).reshape(K, d)
         assert np.array_equal(moved, table.view(np.uint16).reshape(K, d)[unmap])   # codeword `new` is the file's unmap[new]
-    heads = np.frombuffer(buf, np.uint32, NV * NG * 4, 0).reshape(NV, NG, 4).astype(np.int64)   # {rest, nst, unit0, split}
-    slots = np.frombuffer(buf, np.uint32, NV * NG * 64, off_slots).reshape(NV, NG * 64)
+    heads = np.frombuffer(buf, np.uint32, NV * NG * 4, 0).reshape(NV, NG, 4).astype(np.int64)   # {rest, nst, unit0, split | g0 << 8}
+    slots = np.frombuffer(buf, np.uint16, NV * NG * 64, off_slots).reshape(NV, NG * 64).astype(np.int64)
     rt = np.frombuffer(buf, np.int32, runs * 8, off_runs).reshape(runs, 8)[:, :4]       # g0, ng, column orders, first unit
     rb = np.frombuffer(buf, np.uint8, runs * 32, off_runs).reshape(runs, 32)
     bounds, orders = rb[:, 16:24], rb[:, 24:32]                               # first group (in the run) and id of each order
@@ -262,8 +295,8 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
     assert sorted(base[base != 0x7FFFF].tolist()) == list(range(R))
     if row_mask is None:
         assert (base[:R] == np.arange(R)).all()
-    total = (len(buf) - off_steps) // 768
-    assert len(buf) == off_steps + total * 768
+    total = (len(buf) - off_steps) // F.step_bytes
+    assert len(buf) == off_steps + total * F.step_bytes
     # runs tile the groups in order; every run has one column order
     assert rt[0, 0] == 0 and (rt[1:, 0] == rt[:-1, 0] + rt[:-1, 1]).all() and rt[-1, 0] + rt[-1, 1] == NG
     assert (rt[:, 1] >= 1).all() and (rt[:, 2] >= 1).all() and (rt[:, 2] <= 4).all()
@@ -271,29 +304,48 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
     if row_mask is None:                                                      # the cut the kernel derives from the run count
         gr = -(-NG // runs)
         assert (rt[:, 0] == np.arange(runs) * gr).all() and (rt[:, 1] == np.minimum(gr, NG - rt[:, 0])).all()
-    steps = np.frombuffer(buf, np.uint8, total * 768, off_steps).reshape(-1, 64, 4, 3).astype(np.uint32)
-    ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
+    ent = F.entries(buf, off_steps, total)                                    # [step, lane, eps]
     # units: run after run, a group of a run of at most NW / 2 groups has NW // groups of them (its waves' shares);
     # every step of the buffer belongs to exactly one group
     u0 = 0
+    run_g0 = np.zeros(NG, np.int64)
     for g0, ng, _, ru0 in rt:
         split = NW // ng if ng * 2 <= NW else 1
         assert ru0 == u0
-        assert (heads[:, g0:g0 + ng, 3] == split).all()
+        assert (heads[:, g0:g0 + ng, 3] == split | (g0 << 8)).all()           # share count and the run's first group
         assert (heads[:, g0:g0 + ng, 2] == u0 + np.arange(ng) * split).all()
+        run_g0[g0:g0 + ng] = g0
         u0 += ng * split
     NU, used = u0, np.zeros(total, bool)
-    assert total >= NU * NV * PF
+    assert total >= NU * NV * FS
     tags = np.full((R, U), -1, np.int64)
     run_rows = None
+    longest = 0
     for v in range(NV):
         kp, s = divmod(v, NS)
-        places = slots[v] & 0x7FFFF
-        cnts = slots[v] >> 19
-        real = places != 0x7FFFF
+        real = (slots[v] & SLOT_NONE) != SLOT_NONE
+        has = (slots[v] & SLOT_HAS) != 0
+        assert not (has & ~real).any()
+        places = np.where(real, (slots[v] & SLOT_NONE) + np.repeat(run_g0, 64) * 64, 0x7FFFF)   # counted from the run's first place
         rows = np.where(real, base[np.where(real, places, 0)], 0x7FFFF)
         assert (rows[real] != 0x7FFFF).all()
         assert sorted(rows[real].tolist()) == list(range(R))                  # every row once per bucket
+        # the groups' entries, and per lane the number of real ones (padding names a zero chunk behind the part's own)
+        cnts = np.zeros(NG * 64, np.int64)
+        group_e = []
+        for g in range(NG):
+            n = int(heads[v, g, 1])
+            at = _step_places(heads[v, g], v, NV, PF, FS)
+            assert len(at) == n and not used[at].any()
+            assert all((a < NU * NV * FS) == (k_ < PF) for a, k_ in zip(at, _share_pos(n, int(heads[v, g, 3]) & 0xFF)))
+            used[at] = True
+            longest = max([longest] + _share_lens(n, int(heads[v, g, 3]) & 0xFF))
+            e = ent[at].transpose(1, 0, 2).reshape(64, n * F.eps)              # [lane, entry]
+            assert (((e >> 12) & F.cmask) < PC + 16).all() and (e >> (12 + (9 if F.narrow else 12)) == 0).all()
+            group_e.append(e)
+            c = ((e >> 12) < PC).sum(1)
+            cnts[g * 64:(g + 1) * 64] = np.where(has[g * 64:(g + 1) * 64], c, 0)
+            assert n == -(-int(cnts[g * 64:(g + 1) * 64].max()) // F.eps)     # padded to the group's longest row
         sets = []
         for ri, (g0, ng, no, _) in enumerate(rt):
             sl = slice(g0 * 64, (g0 + ng) * 64)
@@ -305,7 +357,7 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
             assert bnd[0] == 0 and all(a < b for a, b in zip(bnd, bnd[1:]))
             for oi in range(no):
                 so = slice((g0 + bnd[oi]) * 64, (g0 + bnd[oi + 1]) * 64)
-                assert (np.diff(cnts[so][real[so]].astype(np.int64)) <= 0).all()
+                assert (np.diff(cnts[so][real[so]]) <= 0).all()
                 assert real[so][:int(real[so].sum())].all() and real[so].any()
                 assert sorted(rows[so][real[so]].tolist()) == sorted(base[so][base[so] != 0x7FFFF].tolist())
                 if row_mask is not None:
@@ -313,32 +365,28 @@ def _walk_stream(buf, R, C, d, bits, runs, NG, row_mask, table=None):
         run_rows = run_rows or sets
         assert sets == run_rows                                               # the same rows in every bucket's run
         for g in range(NG):
-            n = int(heads[v, g, 1])
-            assert n == -(-int(cnts[g * 64]) // 4)                            # padded to the group's longest row
-            at = _step_places(heads[v, g], v, NV)
-            assert len(at) == n and not used[at].any()
-            assert all((a < NU * NV * PF) == (k_ < PF) for a, k_ in zip(at, _share_pos(n, int(heads[v, g, 3]))))
-            used[at] = True
-            e = ent[at]                                                        # [n, 64, 4]
-            e = e.transpose(1, 0, 2).reshape(64, n * 4)
+            e = group_e[g]
             for lane in range(64):
                 k = g * 64 + lane
-                if not real[k] or int(cnts[k]) == 0:
-                    # a lane without a row or without entries reads valid addresses (what a neighbour reads, or zeros);
-                    # the kernel drops its sum
-                    assert ((e[lane] >> 12) < PC + 16).all()
-                    continue
+                if not has[k]:
+                    continue        # a lane without a row or without entries reads valid addresses (checked above); its sum is dropped
                 c = int(cnts[k])
-                # padding: one of the row's codewords of the bucket again, at one of the 16 zero chunks of x
-                assert ((e[lane, c:] >> 12 >= PC) & (e[lane, c:] >> 12 < PC + 16)).all()
+                assert c > 0
+                # real entries first, then padding: one of the row's codewords of the bucket again, at one of the 16 zero chunks of x
+                assert ((e[lane, :c] >> 12) < PC).all() and ((e[lane, c:] >> 12) >= PC).all()
                 assert set((e[lane, c:] & 0xFFF).tolist()) <= set((e[lane, :c] & 0xFFF).tolist())
                 # the entries of a lane come in an order chosen for the LDS banks: every chunk once, any order
                 chunk = (e[lane, :c] >> 12) + kp * PC
                 assert len(set(chunk.tolist())) == c and (chunk >= kp * PC).all() and (chunk < min(U, (kp + 1) * PC)).all()
                 assert (tags[rows[k], chunk] == -1).all()
                 tags[rows[k], chunk] = (e[lane, :c] & 0xFFF) + (s << 12)
-    assert used[NU * NV * PF:].all()                                          # the rest region has no holes
+    assert used[NU * NV * FS:].all()                                          # the rest region has no holes
+    assert FS == max(1, min(PF, longest))                                     # no slot of the first-steps region that no unit can fill
     return tags if unmap is None else unmap[tags]
+
+
+def _share_lens(nst, split):
+    return [nst * (j + 1) // split - nst * j // split for j in range(split)]
 
 
 def _share_pos(nst, split):
@@ -350,6 +398,8 @@ def _share_pos(nst, split):
 
 
 @pytest.mark.parametrize("R,C,bits,runs,M", [(70, 512, 16, 0, 1), (130, 5376, 16, 2, 1), (64, 1024, 13, 5, 1), (1, 8, 14, 0, 1),
+                                              (200, 3968, 16, 3, 1), (200, 3976, 16, 3, 1),      # the widest narrow part, the narrowest wide one
+                                              (90, 5120, 16, 2, 16),
                                               (1100, 256, 15, 4, 1), (1100, 256, 15, 7, 1), (300, 512, 16, 3, 4),
                                               (1000, 256, 14, 2, 16), (5, 64, 16, 0, 3),
                                               (12900, 64, 14, 1, 1),          # a run longer than the cap: more runs than asked for
@@ -385,14 +435,14 @@ def test_balanced_stream_relabels_codewords_and_evens_out_the_slices(R, C, bits,
     for what, a, b in _stream_reads(buf, R, C, bits, _build_stream.runs_out, NG, row_mask):   # (defined below)
         assert 0 <= a < b <= len(buf), (what, a, b)
     NS = K >> 12
-    def slice_loads(b, balanced):
-        NV = NS * -(-U // PART_MAX)
-        off_slots = (NV * NG * 16 + 255) & ~255
-        cnt = np.frombuffer(b, np.uint32, NV * NG * 64, off_slots).reshape(NV, -1) >> 19
-        return cnt.sum(1).reshape(-1, NS).sum(0)
-    plain, _, NG2 = _build_stream(words, R, C, bits, row_mask, runs)
+    def slice_loads(t):                                   # tags per slice of 4096 codewords
+        return np.bincount((t >> 12).ravel(), minlength=NS)
+    plain, eff2, NG2 = _build_stream(words, R, C, bits, row_mask, runs)
     assert NG2 == NG
-    lb, lp = slice_loads(buf, True), slice_loads(plain, False)
+    new_label = np.empty(K, np.int64)
+    _, _, _, _, NV, _ = _geom(C, bits)
+    new_label[np.frombuffer(buf, np.uint16, K, _stream_offsets(NV, NG, eff, bits, 8, True)[4]).astype(np.int64)] = np.arange(K)
+    lb, lp = slice_loads(new_label[tags]), slice_loads(tags)
     assert lb.sum() == lp.sum() == R * U
     assert lp.max() > 2.5 * lp.mean()                     # slice 0 of the plain stream: most of the tags
     # the most popular codeword alone may outweigh a slice's fair share; nothing else may
@@ -407,9 +457,8 @@ def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask):
     to the share's last step), the shares of a group that several waves walk, and the row list of the finishing
     workgroup.  Yields (what, first byte, end byte)."""
     runs, run_max, balanced = runs_out & 0xFFFF, (runs_out >> 16) & 0xFF, bool(runs_out & (1 << 30))
-    U, NS = C // 8, 1 << (bits - 12)
-    KP = -(-U // PART_MAX)
-    NV = NS * KP
+    U, NS, KP, PC, NV, F = _geom(C, bits)
+    PF, FS, SB = F.pf, _fs_of(runs_out), F.step_bytes
     off_slots, off_runs, off_rows, off_table, _, off_steps = _stream_offsets(NV, NG, runs, bits, 8, balanced)
     if balanced:                                        # relabelled codebook and back map sit in front of the steps
         yield "codebook slices", off_table, off_table + (16 << bits)
@@ -434,20 +483,21 @@ def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask):
                 kc = min(k, ng - 1)
                 i = v * NG + g0 + kc
                 yield "group words", i * 16, i * 16 + 16
-                yield "slots", off_slots + i * 256, off_slots + i * 256 + 256
+                yield "slots", off_slots + i * 128, off_slots + i * 128 + 128
                 for sub in range(split):
-                    first = ((u0 + kc * split + sub) * NV + v) * PF
-                    yield "first steps", off_steps + first * 768, off_steps + (first + PF) * 768
+                    # PF loads, step q of them at slot min(q, FS - 1) of the unit's FS slots
+                    first = ((u0 + kc * split + sub) * NV + v) * FS
+                    yield "first steps", off_steps + first * SB, off_steps + (first + FS) * SB
                 if k >= ng:
                     continue
                 rest, nst = int(heads[i, 0]), int(heads[i, 1])
-                assert int(heads[i, 2]) == u0 + kc * split and int(heads[i, 3]) == split
+                assert int(heads[i, 2]) == u0 + kc * split and int(heads[i, 3]) == split | (g0 << 8)
                 for sub in range(split):
                     s0, s1 = nst * sub // split, nst * (sub + 1) // split
                     rb, n = rest + s0 - PF * (sub + 1), s1 - s0
                     # the loop: PF steps ahead, clamped to the share's last step
                     for st in {rb + min(t0 + PF + q, n - 1) for t0 in range(0, n, PF) for q in range(PF) if t0 + PF < n}:
-                        yield "steps", off_steps + st * 768, off_steps + st * 768 + 768
+                        yield "steps", off_steps + st * SB, off_steps + st * SB + SB
 
 
 @pytest.mark.parametrize("R,C,bits,runs,M", [(1, 8, 16, 0, 1), (1, 8, 14, 6, 1), (65, 8, 16, 6, 1), (64, 8, 16, 3, 1), (63, 64, 16, 2, 1),
@@ -506,12 +556,12 @@ def test_stream_builder_orders_entries_for_the_lds_banks():
     R, C, bits = 512, 3584, 16
     tags = rng.integers(0, 1 << bits, size=(R, C // 8))
     buf, runs, NG = _build_stream(O.pack_bits(tags, bits), R, C, bits, None, 1)
-    NV = 16
+    _, _, _, _, NV, F = _geom(C, bits)
+    FS = _fs_of(_build_stream.runs_out)
     off_steps = _stream_offsets(NV, NG, runs, bits, 8, False)[-1]
     heads = np.frombuffer(buf, np.uint32, NV * NG * 4, 0).reshape(NV, NG, 4)
-    steps = np.frombuffer(buf, np.uint8, len(buf) - off_steps, off_steps).reshape(-1, 64, 4, 3).astype(np.int64)
-    ent = steps[..., 0] | steps[..., 1] << 8 | steps[..., 2] << 16            # [step, lane, 4]
-    ent = ent[[a for v in range(NV) for g in range(NG) for a in _step_places(heads[v, g], v, NV)]]   # the groups' steps only
+    ent = F.entries(buf, off_steps, (len(buf) - off_steps) // F.step_bytes)   # [step, lane, eps]
+    ent = ent[[a for v in range(NV) for g in range(NG) for a in _step_places(heads[v, g], v, NV, F.pf, FS)]]   # the groups' steps only
     cw, xc = [], []
     for lanes in LDS_CLOCK_LANES:
         e = ent[:, lanes, :].transpose(0, 2, 1).reshape(-1, 16)               # [slot, lane of the clock]
