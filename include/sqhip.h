@@ -117,17 +117,40 @@ int sq_gemm_dense_ws(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t
 size_t sq_gemm_dense_workspace_bytes(int32_t R, int32_t C, int32_t T);
 
 /* Bytes of workspace sq_linear_small (which = 0) or sq_linear_gemm (which = 1) needs for these
- * pieces at `rows` activation rows; the caller grows its buffer before any graph capture
+ * pieces at `rows` activation rows (which = 2 / 3: the same for a workspace that serves these pieces only, see
+ * below); the caller grows its buffer before any graph capture
  * (the reference grows its buffers the same way: batched_runs.py:628-640, runs_gemm.py:396-404).
- * A workspace must be 256-byte aligned and its first SQ_WS_HEADER_BYTES must be ZERO when it is first
- * handed to the library, and nobody else may write there afterwards: the header holds the partial sums that
- * the workgroups of the decode-time kernel for large codebooks exchange.  A partial sum is its own arrival
- * flag (a word is zero until its sum has been written, and the workgroup that adds a word up puts zero back),
- * so every call leaves the header zeroed again and no call ever clears it.  Everything else a call needs lies
- * behind the header and may hold anything.  One workspace serves one stream at a time; a call that is
- * abandoned half way (a device reset) leaves a header that must be zeroed before it is used again. */
+ * A workspace must be 256-byte aligned.  One of at least SQ_WS_HEADER_BYTES begins with a header of that size,
+ * which must be ZERO when the workspace is first handed to the library and which nobody else may write
+ * afterwards: it holds the partial sums that the workgroups of the decode-time kernel for large codebooks
+ * exchange, and in its last page the error word of that exchange.  A partial sum is its own arrival flag (a word
+ * is zero until its sum has been written, each word is one atomic location, and the workgroup that adds a
+ * word up puts zero back), so every call leaves the header zeroed again and no call ever clears it.
+ * Everything else a call needs lies behind the header and may hold anything.  One workspace serves one stream
+ * at a time.  A workspace smaller than SQ_WS_HEADER_BYTES has no header and is used from its first byte: it
+ * serves pieces that keep no partial sums (which | 2 below asks for the size of such a private workspace;
+ * pieces with a slice stream always need the header).
+ *
+ * When the exchange fails.  A workgroup waits for the partial sums of its rows a bounded number of polls
+ * (2^18, about a third of a second; sq_stream_spin_limit changes it).  If it gives up, because the workgroups
+ * it waits for were held up that long or because a launch was abandoned (a device reset), it writes NaN
+ * for its rows and sets the error word; the missing sums may still arrive afterwards and stay in the header, so
+ * from then on EVERY launch on that workspace writes NaN for all its rows (a dirty header never yields
+ * finite numbers), and the next sq_linear_small* call on that device returns SQ_ELAUNCH without launching
+ * anything (the workgroup also sets a word in pinned host memory, one 64-byte allocation per device made
+ * by the first call that is given a workspace with a header, which calls read without synchronising).
+ * sq_workspace_status(workspace, ws_bytes, stream) SYNCHRONISES the stream and returns SQ_ELAUNCH if the error
+ * word of that workspace is set; sq_workspace_reset enqueues a kernel that zeroes the header and clears the
+ * error (the caller makes sure no product is still running on the workspace: same stream, or synchronise
+ * first); sq_noalloc_reset does the same for sq_linear_small_noalloc's built-in array. */
 #define SQ_WS_HEADER_BYTES (32u << 20)
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which);
+int sq_workspace_status(const void* workspace, size_t ws_bytes, void* stream);
+int sq_workspace_reset(void* workspace, size_t ws_bytes, void* stream);
+int sq_noalloc_reset(void* stream);
+/* Polls of a row's partial sums before a workgroup gives up (negative: the default, 2^18).  Process-wide; meant
+ * for tests of the failure path (0: give up at once where a sum is missing, every kernel still ends normally). */
+void sq_stream_spin_limit(int32_t polls);
 
 /* Load-time regrouping of a matrix' tags for codebooks that do not fit LDS (d = 8, K = 8192..65,536, one
  * codebook): the decode-time product (up to 4 activation rows, up to 8 of rows with at most 1024 chunks, any

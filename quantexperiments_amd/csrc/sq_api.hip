@@ -1,5 +1,6 @@
 // extern "C" surface of libsqhip.so: argument checks, error text, dispatch to the launchers.
 #include <algorithm>
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 #include "sq_stream.h"
@@ -75,7 +76,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 106; }
+int sq_version(void) { return 107; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -89,18 +90,38 @@ int sq_dequant(const sq_matrix* m, void* out, int out_dtype, int64_t ld_out, int
     return launch_dequant(*m, out, out_dtype, ld_out, r0, r1, (hipStream_t)stream);
 }
 
+// A workspace as the launchers see it: the header (partial sums of the tag-stream kernel) and what lies behind it.  A
+// buffer of at least SQ_WS_HEADER bytes always begins with the header; a smaller one has none and is used from its
+// first byte, which serves pieces that keep no partial sums (a private workspace of a few KB for a d = 4 matrix).
+struct WsParts { void* sums; char* inner; size_t inner_bytes; };
+static WsParts split_workspace(void* workspace, size_t ws_bytes) {
+    if (!workspace) return WsParts{nullptr, nullptr, 0};
+    if (ws_bytes >= SQ_WS_HEADER) return WsParts{workspace, (char*)workspace + SQ_WS_HEADER, ws_bytes - SQ_WS_HEADER};
+    return WsParts{nullptr, (char*)workspace, ws_bytes};
+}
+
+// The exchange of the tag-stream kernel gave up in an earlier launch on this device (its workgroups set a host-visible
+// word then): partial sums may have arrived late, the header is no longer known to be zero, and every launch on it
+// writes NaN until sq_workspace_reset has run.
+static int refuse_if_poisoned(const char* who, const sq_matrix* mats, int n) {
+    if (small_uses_sums(mats, n) && stream_host_flag_set())
+        return fail(SQ_ELAUNCH, "%s: an earlier launch on this device gave up waiting for a partial sum; its workspace header may be "
+                                "dirty: call sq_workspace_reset on the workspace before using it again", who);
+    return SQ_OK;
+}
+
 int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                     int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream) {
     int rc = check_xy("sq_linear_small", mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B);
     if (rc) return rc;
     if (B > SQ_SMALL_BMAX) return fail(SQ_EINVAL, "sq_linear_small: B %d > %d", B, SQ_SMALL_BMAX);
     if (B == 0 || n_mats == 0) return SQ_OK;
-    const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
+    if ((rc = refuse_if_poisoned("sq_linear_small", mats, n_mats))) return rc;
+    const WsParts w = split_workspace(workspace, ws_bytes);
+    if (w.sums) (void)stream_host_flag((hipStream_t)stream, true);      // (one pinned host word per device, first call only)
     if (small_takes_gemm_route(mats, n_mats, B, x, ldx))
-        return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
-                           has_ws ? ws_bytes - SQ_WS_HEADER : 0, has_ws ? workspace : nullptr, (hipStream_t)stream);
-    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
-                        has_ws ? ws_bytes - SQ_WS_HEADER : 0, has_ws ? workspace : nullptr, (hipStream_t)stream);
+        return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, w.inner, w.inner_bytes, w.sums, (hipStream_t)stream);
+    return launch_small(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, B, w.inner, w.inner_bytes, w.sums, (hipStream_t)stream);
 }
 
 // ---- sq_linear_small for callers that cannot allocate: the workspace is a device array of this library.
@@ -108,28 +129,22 @@ int sq_linear_small(const sq_matrix* mats, int32_t n_mats, const void* x, int x_
 // up once per device and kept; kernels are handed that address, never the symbol.
 static_assert(sq::SQ_WS_HEADER == SQ_WS_HEADER_BYTES, "the header size is part of the ABI");
 static __device__ __align__(256) unsigned char g_static_scratch[SQ_NOALLOC_SCRATCH_BYTES];
-static void* g_static_scratch_ptr[64];
+static std::atomic<void*> g_static_scratch_ptr[64];
 
-__global__ void noalloc_clear_kernel(unsigned* p, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
-}
-
-// this device's copy of the scratch array (its address, looked up on first use with the device current), or nullptr + error
-static void* static_scratch(hipStream_t s) {
+// This device's copy of the scratch array (its address, looked up on first use with the device current), or nullptr +
+// error.  The array is zero when the code object is loaded, which is what the header must be before the first call:
+// nothing is launched here, so a first call under stream capture records only the product's own kernels.  (Two
+// threads that race to the first call look the same address up twice.)
+static void* static_scratch() {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { fail(SQ_ELAUNCH, "sq_linear_small_noalloc: no current device"); return nullptr; }
-    if (!g_static_scratch_ptr[dev]) {
-        void* ptr = nullptr;
+    void* ptr = g_static_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
         const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
         if (e != hipSuccess || !ptr) { fail(SQ_ELAUNCH, "sq_linear_small_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e)); return nullptr; }
-        // the header (the tag-stream kernel's partial sums) must be zero before the first call (a fill kernel, not a
-        // memset node, so that this is also safe as the first thing a graph capture records)
-        hipLaunchKernelGGL(noalloc_clear_kernel, dim3((unsigned)(SQ_WS_HEADER / 4 / 256)), dim3(256), 0, s, (unsigned*)ptr, (int)(SQ_WS_HEADER / 4));
-        if (check_launch("sq_linear_small_noalloc(clear)")) return nullptr;
-        g_static_scratch_ptr[dev] = ptr;
+        g_static_scratch_ptr[dev].store(ptr, std::memory_order_release);
     }
-    return g_static_scratch_ptr[dev];
+    return ptr;
 }
 
 int sq_linear_small_noalloc(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
@@ -142,7 +157,8 @@ int sq_linear_small_noalloc(const sq_matrix* mats, int32_t n_mats, const void* x
     if (need > (size_t)SQ_NOALLOC_SCRATCH_BYTES)
         return fail(SQ_EWORKSPACE, "sq_linear_small_noalloc: these pieces need %zu bytes of workspace at %d rows, the built-in scratch holds %u "
                                    "(use sq_linear_small with a workspace of the caller's)", need, B, (unsigned)SQ_NOALLOC_SCRATCH_BYTES);
-    char* ws = (char*)static_scratch((hipStream_t)stream);
+    if ((rc = refuse_if_poisoned("sq_linear_small_noalloc", mats, n_mats))) return rc;
+    char* ws = (char*)static_scratch();
     if (!ws) return SQ_ELAUNCH;
     const size_t inner = (size_t)SQ_NOALLOC_SCRATCH_BYTES - SQ_WS_HEADER;
     if (small_takes_gemm_route(mats, n_mats, B, x, ldx))
@@ -180,9 +196,12 @@ int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_produce
     if (B > 1 && ((addnorm && from->ld_h < C) || ((from->add || !addnorm) && from->ld_in < C)))
         return fail(SQ_EINVAL, "%s: ld_h %lld / ld_in %lld too small", who, (long long)from->ld_h, (long long)from->ld_in);
     hipStream_t s = (hipStream_t)stream;
-    const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
-    void* ws = has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr;
-    const size_t wsb = has_ws ? ws_bytes - SQ_WS_HEADER : 0;
+    if ((rc = refuse_if_poisoned(who, mats, n_mats))) return rc;
+    const WsParts wp = split_workspace(workspace, ws_bytes);
+    const bool has_ws = wp.sums != nullptr;
+    void* ws = wp.inner;
+    const size_t wsb = wp.inner_bytes;
+    if (has_ws) (void)stream_host_flag(s, true);
     const bool aligned = (((uintptr_t)from->h_in | (uintptr_t)from->h_out | (uintptr_t)from->add | (uintptr_t)from->up | (uintptr_t)from->w) & 15) == 0;
     if (addnorm && aligned && small_fuses_producer(mats, n_mats, B))
         return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, has_ws ? workspace : nullptr, s, from);
@@ -200,9 +219,9 @@ int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_d
     int rc = check_xy("sq_linear_gemm", mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T);
     if (rc) return rc;
     if (T == 0 || n_mats == 0) return SQ_OK;
-    const bool has_ws = workspace && ws_bytes >= SQ_WS_HEADER;
-    return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T, has_ws ? (char*)workspace + SQ_WS_HEADER : nullptr,
-                       has_ws ? ws_bytes - SQ_WS_HEADER : 0, has_ws ? workspace : nullptr, (hipStream_t)stream);
+    if (T <= SQ_SMALL_BMAX && (rc = refuse_if_poisoned("sq_linear_gemm", mats, n_mats))) return rc;
+    const WsParts w = split_workspace(workspace, ws_bytes);
+    return launch_gemm(mats, n_mats, x, x_dtype, ldx, y, y_dtype, ldy, T, w.inner, w.inner_bytes, w.sums, (hipStream_t)stream);
 }
 
 int sq_gemm_dense(const void* w, int w_dtype, int64_t ldw, int32_t R, int32_t C, const void* x, int x_dtype, int64_t ldx,
@@ -238,10 +257,50 @@ size_t sq_gemm_dense_workspace_bytes(int32_t R, int32_t C, int32_t T) {
 
 size_t sq_workspace_bytes(const sq_matrix* mats, int32_t n_mats, int32_t rows, int which) {
     if (!mats || n_mats <= 0 || rows <= 0) return 0;
-    // which = 0 covers both kernels a stack with column orders may take (the caller's x decides, see sq_linear_small)
-    const size_t inner = which == 0 ? std::max(small_workspace(mats, n_mats, rows), small_gemm_route_workspace(mats, n_mats, rows))
-                                    : gemm_workspace(mats, n_mats, rows);
-    return (inner || small_uses_sums(mats, n_mats)) ? inner + SQ_WS_HEADER : 0;
+    // which & 1 = 0 covers both kernels a stack with column orders may take (the caller's x decides, see sq_linear_small)
+    const size_t inner = (which & 1) == 0 ? std::max(small_workspace(mats, n_mats, rows), small_gemm_route_workspace(mats, n_mats, rows))
+                                          : gemm_workspace(mats, n_mats, rows);
+    const bool sums = small_uses_sums(mats, n_mats);
+    // which & 2: a workspace of the caller's own for these pieces alone: no header unless they keep partial sums in
+    // it (or need so much that the buffer would be taken for one that begins with a header)
+    if ((which & 2) && !sums && inner < SQ_WS_HEADER) return inner;
+    return (inner || sums) ? inner + SQ_WS_HEADER : 0;
+}
+
+__global__ void workspace_clear_kernel(uint32_t* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+int sq_workspace_reset(void* workspace, size_t ws_bytes, void* stream) {
+    if (!workspace || ((uintptr_t)workspace & 255)) return fail(SQ_EINVAL, "sq_workspace_reset: workspace %p", workspace);
+    if (ws_bytes < SQ_WS_HEADER) return SQ_OK;                  // no header, nothing to clear
+    const size_t n = SQ_WS_HEADER / 4;
+    hipLaunchKernelGGL(workspace_clear_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, (uint32_t*)workspace, n);
+    int rc = check_launch("sq_workspace_reset");
+    if (rc) return rc;
+    stream_host_flag_clear();
+    return SQ_OK;
+}
+
+int sq_workspace_status(const void* workspace, size_t ws_bytes, void* stream) {
+    if (!workspace) return fail(SQ_EINVAL, "sq_workspace_status: null workspace");
+    if (ws_bytes < SQ_WS_HEADER) return SQ_OK;
+    uint32_t word = 0;
+    hipError_t e = hipMemcpyAsync(&word, (const char*)workspace + SQ_WS_ERR_OFF, 4, hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return fail(SQ_ELAUNCH, "sq_workspace_status: %s", hipGetErrorString(e));
+    if (word) return fail(SQ_ELAUNCH, "sq_workspace_status: a launch on this workspace gave up waiting for a partial sum; results since "
+                                      "then are NaN: call sq_workspace_reset");
+    return SQ_OK;
+}
+
+void sq_stream_spin_limit(int32_t polls) { stream_set_spin(polls); }
+
+int sq_noalloc_reset(void* stream) {
+    char* ws = (char*)static_scratch();
+    if (!ws) return SQ_ELAUNCH;
+    return sq_workspace_reset(ws, (size_t)SQ_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 size_t sq_stream_bytes_balanced(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,

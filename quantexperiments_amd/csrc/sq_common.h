@@ -99,6 +99,12 @@ __device__ __forceinline__ float wave_sum(float v) {
 // flag and whoever adds it up puts zero back), so they must be zero when the workspace is first handed over and nothing
 // else may ever be written there; the other launchers get the part behind the header.
 constexpr size_t SQ_WS_HEADER = (size_t)32 << 20;
+// The partial sums fill at most the first SQ_WS_SUMS bytes of the header; its last page holds the error word of the
+// exchange (at SQ_WS_ERR_OFF): set by a workgroup that gave up waiting for a partial sum, read by every later launch
+// (which then writes NaN everywhere: partial sums that arrive late leave the header dirty, and a dirty header must
+// never yield finite numbers), cleared by sq_workspace_reset.
+constexpr size_t SQ_WS_SUMS = SQ_WS_HEADER - 4096;
+constexpr size_t SQ_WS_ERR_OFF = SQ_WS_HEADER - 256;
 
 // error plumbing shared by the launchers (defined in sq_api.hip)
 int fail(int code, const char* fmt, ...);

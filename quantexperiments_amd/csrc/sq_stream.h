@@ -88,5 +88,13 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
                         int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from = nullptr);
 // pieces [0, n) a single launch can take: their partial sums of one activation row fit the workspace header together
 int stream_group_len(const sq_matrix* mats, int n);
+// Polls of an item's partial sums before a workgroup gives up (sq_stream_spin_limit); and this device's host-visible
+// copy of the error word, which a workgroup that gives up also sets so that the next call can refuse without a
+// synchronisation: its device address (NULL when there is none and `may_allocate` is false, or under stream capture),
+// whether it is set, and its clearing.
+void stream_set_spin(int polls);
+uint32_t* stream_host_flag(hipStream_t s, bool may_allocate);
+bool stream_host_flag_set();
+void stream_host_flag_clear();
 
 }  // namespace sq

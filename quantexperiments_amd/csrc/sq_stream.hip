@@ -35,6 +35,7 @@
 //   steps  [total][64][12 | 8]    entries: the first-steps region (FS steps per unit and bucket), then the rest
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <string.h>
 #include <thread>
 #include <vector>
@@ -640,6 +641,9 @@ struct StreamArgs {
     const uint16_t* w;
     uint16_t* x_out;
     float eps;
+    uint32_t* err;                    // the workspace header's error word (SQ_WS_ERR_OFF)
+    uint32_t* host_err;               // its host-visible copy (pinned host memory) or NULL
+    int spin_max;                     // polls of an item's partial sums before it gives up
 };
 
 // The operands of one chunk (8 elements) of the produced row, fetched first and finished once the row's scale is known.
@@ -682,7 +686,7 @@ __device__ __forceinline__ u32x4 pro_finish(const StreamArgs& a, const ProRaw& r
 
 constexpr int STREAM_TAB = 65536;     // the codebook slice
 constexpr uint32_t STREAM_ZERO_SUM = 0x7FFFFFFFu;  // how a partial sum with all bits zero is written (zero = not there yet)
-constexpr int STREAM_SPIN_MAX = 1 << 18;           // polls of an item's partial sums before it gives up
+constexpr int STREAM_SPIN_MAX = 1 << 18;           // polls of an item's partial sums before it gives up (default)
 
 // LDS bytes of one activation row's part of x: pc chunks plus 16 zero chunks (one per bank group); the narrow format
 // gives every copy 8 KB, so the address of a chunk is its offset OR-ed into the copy's base
@@ -871,6 +875,10 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
         for (int q = 0; q < STREAM_PF; ++q) nx[q] = *reinterpret_cast<const evec*>(en + (size_t)min(q, fs - 1) * F::SB);
     };
+    // The error word of the exchange, requested now and looked at when y is written: once a launch on this workspace
+    // has given up waiting, partial sums may have arrived late and the header may be dirty; every launch then writes
+    // NaN until the host has reset the workspace.
+    const uint32_t err0 = __hip_atomic_load(a.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     int kcur = wave, knext = 2 * NW - 1 - wave;
     if (split > 1) {                                            // one share of one group per wave, or nothing
         kcur = wave < ng * split ? wave / split : ng;
@@ -1103,6 +1111,9 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
         // shift-and-add (the instruction takes one scalar or constant operand, and the shift count is one already)
         uint32_t xbase = (uint32_t)STREAM_TAB + (uint32_t)(xc * NB * xs);
         asm volatile("" : "+v"(xbase));
+        // (The same products on the matrix cores, which work beside the vector ALU - v_mfma_f32_4x4x4_16b_f16 gives lane j
+        // of every four the dot product of its own four halves of A and B as element j of its result - measured no
+        // faster on the large launches and slower on gate|up: 19.2-20.2 against 18.0-18.9 us on one machine.)
         float acc[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) acc[b] = 0.f;
@@ -1234,7 +1245,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
                 ok = true;
 #pragma unroll
                 for (int k = 0; k < 16; ++k) ok = ok && u[k] != 0u;
-                if (ok || spin >= STREAM_SPIN_MAX) break;
+                if (ok || spin >= a.spin_max) break;
                 __builtin_amdgcn_s_sleep(2);
             }
 #pragma unroll
@@ -1250,7 +1261,7 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
 #pragma unroll
                     for (int k = 0; k < 32; ++k) all = all && u[k] != 0u;
                     if (all) break;
-                    if (spin >= STREAM_SPIN_MAX) { ok = false; break; }
+                    if (spin >= a.spin_max) { ok = false; break; }
                     __builtin_amdgcn_s_sleep(2);
                 }
 #pragma unroll
@@ -1259,8 +1270,13 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
             }
         }
         for (int k = 0; k < P.NV; ++k) __hip_atomic_store(q + (size_t)k * bs, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!ok) {
+            // gave up: the missing sums may still arrive and stay in the header, so the workspace is marked unusable
+            __hip_atomic_store(a.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (a.host_err) __hip_atomic_store(a.host_err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
         if (r != STREAM_NO_ROW)
-            store_y((char*)a.y + (size_t)b * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + r, ok ? sum * rs : __builtin_nanf(""));
+            store_y((char*)a.y + (size_t)b * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + r, ok && err0 == 0u ? sum * rs : __builtin_nanf(""));
     }
     SQ_TRACE_POINT(6);
 }
@@ -1399,7 +1415,55 @@ int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t 
 bool stream_shape(const sq_matrix& m) {
     return m.stream && stream_runs_of(m) > 0 && m.stream_groups > 0 && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
            (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0 &&
-           stream_part_bytes(m, 1) <= SQ_WS_HEADER;
+           stream_part_bytes(m, 1) <= SQ_WS_SUMS;
+}
+
+// ---- the error word's host-visible copy and the spin limit
+static std::atomic<int> g_stream_spin{STREAM_SPIN_MAX};
+static std::atomic<uint32_t*> g_host_flag[64];          // per device: pinned host word
+static std::atomic<uint32_t*> g_host_flag_dev[64];      // its address as the device sees it
+
+void stream_set_spin(int polls) { g_stream_spin.store(polls < 0 ? STREAM_SPIN_MAX : polls, std::memory_order_relaxed); }
+
+static int current_device() {
+    int dev = 0;
+    return hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 ? dev : -1;
+}
+
+uint32_t* stream_host_flag(hipStream_t s, bool may_allocate) {
+    const int dev = current_device();
+    if (dev < 0) return nullptr;
+    uint32_t* d = g_host_flag_dev[dev].load(std::memory_order_acquire);
+    if (d || !may_allocate) return d;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone) { (void)hipGetLastError(); return nullptr; }
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    d = g_host_flag_dev[dev].load(std::memory_order_acquire);
+    if (d) return d;
+    void* h = nullptr;
+    void* hd = nullptr;
+    if (hipHostMalloc(&h, 64, hipHostMallocMapped) != hipSuccess || !h || hipHostGetDevicePointer(&hd, h, 0) != hipSuccess || !hd) {
+        (void)hipGetLastError();
+        if (h) (void)hipHostFree(h);
+        return nullptr;
+    }
+    *reinterpret_cast<volatile uint32_t*>(h) = 0u;
+    g_host_flag[dev].store(reinterpret_cast<uint32_t*>(h), std::memory_order_release);
+    g_host_flag_dev[dev].store(reinterpret_cast<uint32_t*>(hd), std::memory_order_release);
+    return reinterpret_cast<uint32_t*>(hd);
+}
+
+bool stream_host_flag_set() {
+    const int dev = current_device();
+    const uint32_t* h = dev < 0 ? nullptr : g_host_flag[dev].load(std::memory_order_acquire);
+    return h && *reinterpret_cast<const volatile uint32_t*>(h) != 0u;
+}
+
+void stream_host_flag_clear() {
+    const int dev = current_device();
+    uint32_t* h = dev < 0 ? nullptr : g_host_flag[dev].load(std::memory_order_acquire);
+    if (h) *reinterpret_cast<volatile uint32_t*>(h) = 0u;
 }
 
 // rows of one pass: 1, 2, 4 or 8
@@ -1415,7 +1479,7 @@ int stream_group_len(const sq_matrix* mats, int n) {
     int k = 0;
     for (; k < n; ++k) {
         tot += stream_part_bytes(mats[k], 1);
-        if (tot > SQ_WS_HEADER) break;
+        if (tot > SQ_WS_SUMS) break;
     }
     return k > 0 ? k : 1;
 }
@@ -1431,6 +1495,9 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
         a.h_in = from->h_in; a.h_out = from->h_out; a.add = (const uint16_t*)from->add;
         a.w = (const uint16_t*)from->w; a.x_out = (uint16_t*)from->x_out; a.eps = from->eps;
     }
+    a.err = reinterpret_cast<uint32_t*>(sums + SQ_WS_ERR_OFF);
+    a.host_err = stream_host_flag(s, false);
+    a.spin_max = g_stream_spin.load(std::memory_order_relaxed);
     a.n = cnt;
     a.ldx = ldx;
     a.ldy = ldy;
@@ -1440,7 +1507,7 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     for (;; rows >>= 1) {
         size_t tot = 0;
         for (int k = 0; k < cnt; ++k) tot += stream_part_bytes(mats[k], rows);
-        if (tot <= SQ_WS_HEADER) break;
+        if (tot <= SQ_WS_SUMS) break;
         if (rows == 1) return fail(SQ_EUNSUPPORTED, "sq_linear_small: the partial sums of these pieces (%zu bytes) do not fit the workspace header", tot);
     }
     int wg = 0, pc = 0, nl_max = 64, xcopies = 1, xtmp = 0;

@@ -24,24 +24,49 @@ class _Workspace:
     shape once eagerly first, as with the reference's shared buffers (reference
     shapequant/vllm_ext/core.py:198-209, shapequant/kernels/batched_runs.py:628-640)."""
     bufs: dict = {}
-    retired: list = []          # outgrown buffers: a HIP graph captured earlier still launches kernels on them
+    captured: set = set()       # keys of buffers that were handed out while a HIP graph was being captured
+    retired: list = []          # outgrown buffers that a captured graph still launches kernels on
 
     @classmethod
     def get(cls, nbytes: int, dev, kind: str = "kernels") -> torch.Tensor:
         """kind "kernels": the buffer handed to the library (its header, the first _lib.WS_HEADER bytes, holds the
         partial sums of the library's decode kernel, is zero between calls and must never be written by anyone
         else); any other kind names a separate buffer the caller may overwrite.
-        A buffer that has to grow is replaced, never freed: graphs captured with the old one stay valid (the
-        reference keeps a reference per launcher for the same reason, shapequant/kernels/batched_runs.py:741-743)."""
+        A buffer that has to grow is replaced; the old one is kept alive only if a graph was captured while it was
+        in use (such a graph still launches kernels on it; the reference keeps a reference per launcher for the
+        same reason, shapequant/kernels/batched_runs.py:741-743), otherwise it is freed.  Every buffer is at least
+        _lib.WS_HEADER bytes, so it always begins with the header, whichever pieces come first."""
         key = (str(dev), kind)
         b = cls.bufs.get(key)
+        capturing = torch.cuda.is_current_stream_capturing()
         if b is None or b.numel() < nbytes:
-            if torch.cuda.is_current_stream_capturing():
+            if capturing:
                 raise RuntimeError("sqhip workspace must grow outside graph capture: run this shape once eagerly first")
-            if b is not None:
+            if b is not None and key in cls.captured:
                 cls.retired.append(b)
-            b = cls.bufs[key] = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)   # the header starts at zero
+            cls.captured.discard(key)
+            floor = _lib.WS_HEADER + (1 << 20) if kind == "kernels" else 1 << 20
+            b = cls.bufs[key] = torch.zeros(max(nbytes, floor), dtype=torch.uint8, device=dev)   # the header starts at zero
+        if capturing:
+            cls.captured.add(key)
         return b
+
+    @classmethod
+    def status(cls, dev) -> None:
+        """Synchronise and raise if a launch on this device's workspace gave up waiting for a partial sum
+        (sq_workspace_status); every launch since then has written NaN."""
+        b = cls.bufs.get((str(dev), "kernels"))
+        if b is not None:
+            with torch.cuda.device(dev):
+                _lib.check(_lib.lib().sq_workspace_status(b.data_ptr(), b.numel(), _lib.stream_ptr(dev)))
+
+    @classmethod
+    def reset(cls, dev) -> None:
+        """Zero the header of this device's workspace and clear its error (sq_workspace_reset), on the current stream."""
+        b = cls.bufs.get((str(dev), "kernels"))
+        if b is not None:
+            with torch.cuda.device(dev):
+                _lib.check(_lib.lib().sq_workspace_reset(b.data_ptr(), b.numel(), _lib.stream_ptr(dev)))
 
 
 class PackedLinear(torch.nn.Module):

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     for name in _declared():
         assert getattr(L, name) is not None, name
-    assert L.sq_version() == 106
+    assert L.sq_version() == 107
 
 
 def test_struct_layout_matches_header():
@@ -82,6 +82,9 @@ def test_workspace_sizes_are_host_arithmetic():
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 100 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 2048 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 0) == _lib.WS_HEADER + 16 * 2 * 512 * 2
+    # which | 2: a workspace for these pieces alone has no header unless they keep partial sums there
+    assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 2, 2) == 16 * 2 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 3) == 64 * 512 * 2 + 100 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([masked]), 1, 100, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 100 * 512 * 2
     # a matrix with a tag stream keeps its partial sums in the header and needs nothing behind it at decode time
     streamed = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 8, 16, 1, 1, 32, 0, 0x8000, (1 << 16) | 1, 1)

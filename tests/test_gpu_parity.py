@@ -299,6 +299,100 @@ def test_workspace_header_is_zero_after_every_stream_launch():
             assert torch.equal(small(lin, rand_x(B, s.C, torch.bfloat16, seed=B).cuda(), B), first[B])
 
 
+def test_exchange_that_gives_up_is_sticky_and_reported():
+    """The partial-sum exchange of the tag-stream kernel waits a bounded number of polls.  With the limit at zero
+    (sq_stream_spin_limit; every kernel still ends normally) workgroups give up wherever a sum has not arrived yet: such
+    rows are NaN, never a finite wrong number, the error is reported, every later launch on that workspace writes NaN
+    until sq_workspace_reset, and after the reset results are right again.  Raw C ABI, workspaces of this test's own."""
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    H = _lib.WS_HEADER
+    s = synth(3584, 3584, 8, 16, seed=21)
+    # every tag in the first slice of the codebook, and a stream that does not even the slices out: the workgroups of
+    # the other fifteen slices have nothing to walk and ask for the first slice's sums long before they are there
+    s.tags %= 4096
+    s.words = O.pack_bits(s.tags, s.bits)
+    lin = to_device(s, stream="later")
+    lin.balance = False
+    lin.build_stream(0)
+    mats = _lib.matrix_array([lin.descriptor(0)])
+    need = L.sq_workspace_bytes(mats, 1, 1, 0)
+    x = rand_x(1, s.C, torch.bfloat16, seed=5).cuda()
+    ref = _ref(s, x.cpu())
+    st = _lib.stream_ptr(x.device)
+
+    def call(ws):
+        y = torch.full((1, s.R), 3.0, dtype=torch.float32, device="cuda")
+        rc = L.sq_linear_small(mats, 1, x.data_ptr(), _lib.SQ_BF16, s.C, y.data_ptr(), _lib.SQ_F32, s.R, 1, ws.data_ptr(), need, st)
+        torch.cuda.synchronize()
+        return rc, y.cpu().numpy()
+
+    try:
+        # a workspace whose error word is set (what a launch that gave up leaves behind): NaN everywhere, no finite value
+        ws2 = torch.zeros(need, dtype=torch.uint8, device="cuda")
+        ws2[H - 256] = 1
+        rc, y = call(ws2)
+        assert rc == 0 and np.isnan(y).all()
+        assert L.sq_workspace_status(ws2.data_ptr(), need, st) == _lib.SQ_ELAUNCH and b"gave up" in L.sq_last_error()
+        assert L.sq_workspace_reset(ws2.data_ptr(), need, st) == 0
+        assert L.sq_workspace_status(ws2.data_ptr(), need, st) == 0
+        rc, y = call(ws2)
+        assert rc == 0 and rel_max_err(y, ref) < TOL
+
+        # a launch whose workgroups give up at once
+        ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+        rc, y = call(ws)
+        assert rc == 0 and rel_max_err(y, ref) < TOL
+        L.sq_stream_spin_limit(0)
+        rc, y = call(ws)
+        L.sq_stream_spin_limit(-1)
+        assert rc == 0
+        bad = np.isnan(y)
+        assert bad.any(), "no workgroup had to wait: the launch was not a test of the failure path"
+        good = ~bad
+        assert np.abs(y[good] - ref[good]).max() <= TOL * np.abs(ref).max()          # what is not NaN is right
+        assert L.sq_workspace_status(ws.data_ptr(), need, st) == _lib.SQ_ELAUNCH
+        # the next call is refused on the host, without a synchronisation and without launching anything
+        rc, y = call(ws)
+        assert rc == _lib.SQ_ELAUNCH and b"sq_workspace_reset" in L.sq_last_error() and (y == 3.0).all()
+        assert L.sq_workspace_reset(ws.data_ptr(), need, st) == 0
+        torch.cuda.synchronize()
+        assert not ws[:H].any()
+        rc, y = call(ws)
+        assert rc == 0 and rel_max_err(y, ref) < TOL and not ws[:H].any()
+    finally:
+        L.sq_stream_spin_limit(-1)
+        L.sq_workspace_reset(ws2.data_ptr(), need, st)          # (also clears the device's host-visible error word)
+        torch.cuda.synchronize()
+
+
+def test_private_workspace_without_header_for_pieces_that_keep_no_sums():
+    """Pieces that keep no partial sums in the header (here d = 4 with column orders: permuted copies of x) run with a
+    workspace of sq_workspace_bytes(which = 2) bytes, a few KB with no header in front; pieces with a slice stream are
+    told to bring the header."""
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    s = synth(96, 256, 4, 10, 1, 4, seed=31)
+    lin = to_device(s)
+    mats = _lib.matrix_array([lin.descriptor(0)])
+    need = L.sq_workspace_bytes(mats, 1, 2, 2)
+    assert 0 < need < 1 << 20 and L.sq_workspace_bytes(mats, 1, 2, 0) == need + _lib.WS_HEADER
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device="cuda")
+    x = rand_x(2, s.C, torch.bfloat16, seed=6).cuda()
+    y = torch.empty(2, s.R, dtype=torch.float32, device="cuda")
+    _lib.check(L.sq_linear_small(mats, 1, x.data_ptr(), _lib.SQ_BF16, s.C, y.data_ptr(), _lib.SQ_F32, s.R, 2, ws.data_ptr(), need,
+                                 _lib.stream_ptr(x.device)))
+    torch.cuda.synchronize()
+    assert rel_max_err(y.cpu().numpy(), _ref(s, x.cpu())) < TOL
+    big = to_device(synth(70, 512, 8, 16, seed=32))
+    mb = _lib.matrix_array([big.descriptor(0)])
+    assert L.sq_workspace_bytes(mb, 1, 1, 2) == _lib.WS_HEADER
+    x = rand_x(1, 512, torch.bfloat16).cuda()
+    y = torch.empty(1, 70, dtype=torch.float32, device="cuda")
+    rc = L.sq_linear_small(mb, 1, x.data_ptr(), _lib.SQ_BF16, 512, y.data_ptr(), _lib.SQ_F32, 70, 1, ws.data_ptr(), need, _lib.stream_ptr(x.device))
+    assert rc == _lib.SQ_EWORKSPACE
+
+
 def test_stream_padding_never_touches_the_codebook():
     # codeword 0 of every slice is inf and no tag names it: padded stream entries (tag 0) must not leak into a sum
     from quantexperiments_amd.kernels import linear_small

@@ -69,3 +69,37 @@ def test_noalloc_refuses_what_does_not_fit():
     rc = L.sq_linear_small_noalloc(mats, 1, x.data_ptr(), _lib.SQ_BF16, C, y.data_ptr(), _lib.SQ_BF16, R, B, _lib.stream_ptr(x.device))
     assert rc == _lib.SQ_EWORKSPACE and b"built-in scratch" in L.sq_last_error()
     assert L.sq_linear_small_noalloc(mats, 1, x.data_ptr(), _lib.SQ_BF16, C, y.data_ptr(), _lib.SQ_BF16, R, 0, None) == 0
+
+
+def test_noalloc_under_graph_capture_allocates_nothing():
+    """A call recorded into a HIP graph (after one eager call, as any capture is warmed up): two replays with other work
+    between them give the bits of sq_linear_small, and the free device memory does not move across calls and replays."""
+    from quantexperiments_amd.kernels import prepare_stack
+    L = _lib.lib()
+    pieces = [to_device(synth(700, 3584, 8, 16, seed=13)), to_device(synth(300, 3584, 8, 16, seed=14))]
+    prepare_stack(pieces)
+    x = rand_x(1, 3584, torch.bfloat16, seed=4)
+    want, _ = _both(pieces, x)
+    R = sum(p.R for p in pieces)
+    mats = _lib.matrix_array([pieces[0].descriptor(0), pieces[1].descriptor(pieces[0].R)])
+    xd = x.cuda()
+    y = torch.zeros(1, R, dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    with torch.cuda.stream(side):
+        call = lambda: _lib.check(L.sq_linear_small_noalloc(mats, 2, xd.data_ptr(), _lib.SQ_BF16, 3584, y.data_ptr(), _lib.SQ_F32, R, 1,
+                                                            _lib.stream_ptr(xd.device)))
+        call()
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            call()
+        for k in range(2):
+            y.fill_(float(k))
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, want), k
+    assert torch.cuda.mem_get_info()[0] >= free0 - (8 << 20)      # (the graph object itself may take a little)
+    del g
