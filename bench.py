@@ -184,34 +184,42 @@ def layer_times(torch, dev, layers, shapes, B, fn, gen):
 
 
 def small_batch_crossover(torch, dev, gen, n_layers):
-    """cfg3: the 7B shapes in the d = 4, K = 4096, 12-bit format (3 bits per weight) at M = 2 .. 32 activation rows:
-    the decode-time kernel (sq_linear_small) against the large-M route (decode to fp16 + tile GEMM), with both
-    rooflines; crossover = the largest M at which the decode-time kernel is still the faster one."""
-    from quantexperiments_amd.kernels import linear_small
+    """cfg3: the 7B shapes in the d = 4, K = 4096, 12-bit format (3 bits per weight) from 1 to 256 activation rows, on
+    the two routes PackedShards.forward can take: "direct" = the library's own choice (sq_linear_small up to 32 rows;
+    sq_linear_gemm above: passes of 32 rows through the decode-time kernel up to 160 rows, then decode + 256 x 256
+    tile GEMM) and "dequant" = decode to fp16 + dense GEMM (the reference's large-M route).  Per M: both times, the
+    faster route and its fractions of the HBM roofline (packed bytes + x + y) and of the MFMA roofline (2 M R C).
+    crossover_M = the first M at which the MFMA fraction exceeds the HBM fraction: where the product stops being
+    bandwidth-bound on paper; route_change_M = the first M at which the dequant route is the faster one."""
+    from quantexperiments_amd.kernels import linear_gemm, linear_small
     from quantexperiments_amd.vllm_ext.core import PackedShards
     d, bits = 4, 12
     layers = [make_layer(torch, dev, gen, SHAPES_7B, d, bits) for _ in range(n_layers)]
-    shards = [{l: PackedShards([L[n] for n in l], large="dequant") for l in LAUNCHES} for L in layers[:1]]
-    nbytes = sum(launch_bytes(SHAPES_7B, l, d, bits) for l in LAUNCHES)
+    shards = {l: PackedShards([layers[0][n] for n in l], large="dequant") for l in LAUNCHES}
     flops1 = 2.0 * sum(R * C for R, C in SHAPES_7B.values())
-    res, cross, small_wins = {}, 0, True
-    for M in (1, 2, 4, 8, 16, 32):
-        small, per = layer_times(torch, dev, layers, SHAPES_7B, M, linear_small, gen)
-        r = {"small_us_per_layer": small, "per_launch_us": per, "GBps_packed": nbytes / small / 1e3,
-             "frac_hbm": nbytes / small / 1e3 / HBM_PEAK_GBS, "tflops": flops1 * M / small / 1e6,
-             "frac_mfma": flops1 * M / small / 1e6 / MFMA_PEAK_TFLOPS}
+    res, cross, change = {}, None, None
+    for M in (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256):
+        nbytes = sum(launch_bytes(SHAPES_7B, l, d, bits, B=M) for l in LAUNCHES)
+        direct, per = layer_times(torch, dev, layers if M <= 32 else layers[:2], SHAPES_7B, M, linear_small if M <= 32 else linear_gemm, gen)
+        r = {"direct_us_per_layer": direct, "per_launch_us": per}
+        best, route = direct, "direct"
         if M > 1:
             x = {C: torch.randn(M, C, generator=gen).to(torch.bfloat16).to(dev) for C in (3584, 18944)}
-            large = timed_graph(torch, lambda: [shards[0][l]._large(x[SHAPES_7B[l[0]][1]]) for l in LAUNCHES]) * 1e3
-            r["large_us_per_layer"] = large
-            small_wins = small_wins and small <= large
-            if small_wins:
-                cross = M
+            r["dequant_us_per_layer"] = timed_graph(torch, lambda: [shards[l]._large(x[SHAPES_7B[l[0]][1]]) for l in LAUNCHES]) * 1e3
+            if r["dequant_us_per_layer"] < best:
+                best, route = r["dequant_us_per_layer"], "dequant"
+        r.update(faster=route, us_per_layer=best, GBps=nbytes / best / 1e3, frac_hbm=nbytes / best / 1e3 / HBM_PEAK_GBS,
+                 tflops=flops1 * M / best / 1e6, frac_mfma=flops1 * M / best / 1e6 / MFMA_PEAK_TFLOPS)
+        if cross is None and r["frac_mfma"] > r["frac_hbm"]:
+            cross = M
+        if change is None and route == "dequant":
+            change = M
         res[f"M{M}"] = r
     return {"workload": "cfg3: 7B shapes, d=4, K=4096, 12-bit tags (3 bpw), bf16 rows", "layers_rotated": n_layers,
-            "bytes_per_layer": nbytes, "flops_per_row": flops1, "rows": res, "crossover_M": cross,
-            "note": "small = sq_linear_small; large = sq_dequant to fp16 + sq_gemm_dense (the reference's dequant route); "
-                    "crossover_M = largest M of the list up to which small is faster at every M"}
+            "flops_per_row": flops1, "rows": res, "crossover_M": cross, "route_change_M": change,
+            "note": "direct = sq_linear_small (M <= 32) / sq_linear_gemm (passes of 32 rows up to 160, then decode + tile GEMM); "
+                    "dequant = sq_dequant to fp16 + sq_gemm_dense; crossover_M = first M whose MFMA fraction exceeds its HBM "
+                    "fraction; route_change_M = first M at which the dequant route is faster (null: never up to 256)"}
 
 
 def masked_27b(torch, dev, gen, n_layers):

@@ -872,6 +872,78 @@ def test_full_27b_masked_qkv_stack_against_oracle(B):
     _check_lowp(yb, ref)
 
 
+def _stack(shapes, d, bits, M, seed0):
+    """Pieces of one launch built as bench.py and PackedShards build them (streams cut for the joint launch) and their
+    C-oracle weights."""
+    from quantexperiments_amd.kernels import prepare_stack
+    pieces, ws = [], []
+    for k, (R, C) in enumerate(shapes):
+        s = synth(R, C, d, bits, 1, M, seed=seed0 + k)
+        pieces.append(to_device(s, stream="later"))
+        ws.append(c_oracle.decode(s.words, bits, C, d, s.K, s.table, s.row_scale, None, s.row_mask, s.perms if M > 1 else None))
+    prepare_stack(pieces)
+    return pieces, ws
+
+
+@pytest.mark.parametrize("launch", ["gate|up", "down"])
+def test_full_27b_masked_mlp_launches_against_c_oracle(launch):
+    """The two large launches of the masked 27B-shaped layer the benchmark times (gate | up: 2 x 17408 x 5120, down:
+    5120 x 17408; 16 column orders each, d = 8, 16-bit tags), stacked and cut for the joint launch, at one and two
+    activation rows, every output against the float64 product of the C oracle's decode."""
+    from quantexperiments_amd.kernels import linear_small
+    shapes = [(17408, 5120), (17408, 5120)] if launch == "gate|up" else [(5120, 17408)]
+    pieces, ws = _stack(shapes, 8, 16, 16, 60 if launch == "down" else 61)
+    assert all(p.stream is not None for p in pieces)
+    C = shapes[0][1]
+    for B in (1, 2):
+        x = rand_x(B, C, torch.bfloat16, seed=B)
+        ref = np.concatenate([c_oracle.linear(_xf(x), w) for w in ws], axis=1)
+        y = torch.full((B, ref.shape[1]), 7.0, dtype=torch.float32, device="cuda")
+        linear_small(pieces, x.cuda(), y)
+        assert rel_max_err(y.cpu().numpy(), ref) < TOL, B
+        yb = torch.empty(B, ref.shape[1], dtype=torch.bfloat16, device="cuda")
+        linear_small(pieces, x.cuda(), yb)
+        _check_lowp(yb, ref)
+
+
+def test_full_27b_masked_down_at_2048_rows_against_c_oracle():
+    """cfg5 at M = 2048 on the down shape (5120 x 17408, 16 column orders): a sample of tokens against the float64
+    product of the C oracle's decode, and against the decode-time kernel's result for the same tokens."""
+    from quantexperiments_amd.kernels import linear_gemm, linear_small
+    (lin,), (w,) = _stack([(5120, 17408)], 8, 16, 16, 70)
+    x = rand_x(2048, 17408, torch.bfloat16, seed=3).cuda()
+    y = torch.empty(2048, 5120, dtype=torch.float32, device="cuda")
+    linear_gemm([lin], x, y)
+    toks = [0, 255, 256, 1023, 2047]
+    ref = c_oracle.linear(x[toks].float().cpu().numpy(), w)
+    assert rel_max_err(y[toks].cpu().numpy(), ref) < TOL
+    ys = torch.empty(len(toks), 5120, dtype=torch.float32, device="cuda")
+    linear_small([lin], x[toks].contiguous(), ys)
+    assert rel_max_err(ys.cpu().numpy(), ref) < TOL
+    yb = torch.empty(2048, 5120, dtype=torch.bfloat16, device="cuda")
+    linear_gemm([lin], x, yb)
+    _check_lowp(yb[toks], ref)
+
+
+@pytest.mark.parametrize("launch", ["q|k|v", "gate|up"])
+def test_full_7b_d4_stacks_at_small_batches_against_c_oracle(launch):
+    """cfg3 at full size: the q | k | v and gate | up launches of the 7B-shaped layer in the d = 4, K = 4096, 12-bit
+    format (tile-major copies of the tags, as the benchmark builds them) at 2, 16 and 32 activation rows."""
+    from quantexperiments_amd.kernels import linear_small
+    shapes = [(3584, 3584), (512, 3584), (512, 3584)] if launch == "q|k|v" else [(18944, 3584), (18944, 3584)]
+    pieces, ws = _stack(shapes, 4, 12, 1, 80 if launch == "q|k|v" else 85)
+    assert all(p.stream_tiled for p in pieces)
+    for B in (2, 16, 32):
+        x = rand_x(B, 3584, torch.bfloat16, seed=B)
+        ref = np.concatenate([c_oracle.linear(_xf(x), w) for w in ws], axis=1)
+        y = torch.full((B, ref.shape[1]), 7.0, dtype=torch.float32, device="cuda")
+        linear_small(pieces, x.cuda(), y)
+        assert rel_max_err(y.cpu().numpy(), ref) < TOL, B
+        yb = torch.empty(B, ref.shape[1], dtype=torch.bfloat16, device="cuda")
+        linear_small(pieces, x.cuda(), yb)
+        _check_lowp(yb, ref)
+
+
 @pytest.mark.parametrize("shape", [(18944, 3584, 1), (3584, 18944, 1), (5120, 5120, 16)], ids=lambda c: "x".join(map(str, c)))
 def test_full_size_gemm_rows_against_gemv(shape):
     """M = 2048 prefill at the 7B gate/up and down sizes and at a 27B-class matrix with 16 column orders: every
