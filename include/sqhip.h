@@ -199,6 +199,14 @@ int sq_stream_build_balanced(const int32_t* tags_host, int32_t R, int32_t W, int
                              const uint8_t* row_mask_host, int32_t runs, const void* table_host, void* out_host,
                              size_t out_bytes, int32_t* runs_out, int32_t* groups_out);
 
+/* The relabelling by itself, for callers that would rather keep ONE codebook: remap_out[k] (2^bits entries, host
+ * memory) is the new label of the file's codeword k.  A caller that rewrites its tags through remap_out and moves row k
+ * of its table to row remap_out[k] holds an equivalent packed matrix (every weight decodes to the same bits) whose
+ * slices carry equal shares of the tags; the plain sq_stream_build of those tags then needs no codebook copy of its
+ * own, and the relabelled table serves every other entry point too. */
+int sq_codebook_balance(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
+                        uint16_t* remap_out);
+
 /* ---- The packed file's block-32 side formats (reference shapequant/packed.py:30-40): the 8-bit output head
  * `aux.lm_head` (q int8 [V, C], scale fp16 [V, C/32], w = q * scale of the row's 32-column block) and the 4-bit
  * embedding `aux.embed` (q uint8 [V, C/2] with column 2k in the low and 2k+1 in the high nibble of byte k, each

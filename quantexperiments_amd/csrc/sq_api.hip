@@ -327,6 +327,14 @@ int sq_stream_build_balanced(const int32_t* tags_host, int32_t R, int32_t W, int
                              out_bytes, runs_out, groups_out, (const uint16_t*)table_host);
 }
 
+int sq_codebook_balance(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, uint16_t* remap_out) {
+    if (!tags_host || !remap_out) return fail(SQ_EINVAL, "sq_codebook_balance: null pointer");
+    if (d <= 0 || !stream_format_ok(R, C, d, bits)) return fail(SQ_EUNSUPPORTED, "sq_codebook_balance: d %d bits %d R %d not covered", d, bits, R);
+    if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_codebook_balance: W %d too small", W);
+    stream_balance_host((const uint32_t*)tags_host, R, W, C, d, bits, remap_out);
+    return SQ_OK;
+}
+
 size_t sq_stream_bytes(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
                        const uint8_t* row_mask_host, int32_t runs) {
     return sq_stream_bytes_balanced(tags_host, R, W, C, d, bits, row_mask_host, runs, nullptr);

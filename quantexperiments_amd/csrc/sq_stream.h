@@ -68,6 +68,8 @@ size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int b
                          const uint16_t* table = nullptr);
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                       unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table = nullptr);
+// remap_out[file label] = new label (2^bits entries): the relabelling a balanced stream applies, by itself
+void stream_balance_host(const uint32_t* tags, int R, int W, int C, int d, int bits, uint16_t* remap_out);
 // sq_matrix.stream_runs is sq_stream_build's runs_out: the run count in the low 16 bits, the groups of the longest run
 // in the next 8, the most column orders in one run (less one) in bits 24-26, the steps per unit of the first-steps region
 // (less one) in bits 27-28, bit 30 = the stream carries a relabelled codebook

@@ -314,6 +314,12 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     P.g.total_steps = at;
 }
 
+void stream_balance_host(const uint32_t* tags, int R, int W, int C, int d, int bits, uint16_t* remap_out) {
+    std::vector<uint16_t> remap;
+    balance_codewords(tags, R, W, C / d, bits, remap);
+    memcpy(remap_out, remap.data(), remap.size() * sizeof(uint16_t));
+}
+
 size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
                          const uint16_t* table) {
     StreamPlan P;

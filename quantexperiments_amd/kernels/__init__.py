@@ -116,7 +116,8 @@ class PackedLinear(torch.nn.Module):
         self.stream_runs = self.stream_groups = 0
         self.stream_asked = None
         self.stream_tiled = False
-        self.balance = True         # slice streams carry a relabelled codebook whose slices share the tags evenly
+        self.balance = True         # before its slice stream is built the matrix is relabelled so that the slices share the tags evenly
+        self.relabelled = False
         # stream: True builds now, cut for a launch of this matrix alone; "later" leaves the build to prepare_stack
         # (pieces that will be launched together are cut for the joint launch, and built once); False: never
         self.wants_stream = bool(stream) and self.G == 1 and table.numel() * 2 > 128 * 1024 and d == 8 and 12 < self.bits <= 16
@@ -134,12 +135,40 @@ class PackedLinear(torch.nn.Module):
         matrix alone; prepare_stack picks the runs of pieces that are launched together)."""
         if self.words is None:
             raise RuntimeError("the packed tags of this matrix were dropped (compact): its stream cannot be rebuilt")
+        if self.wants_stream and self.balance and not self.relabelled:
+            self._relabel()
         self.stream, self.stream_runs, self.stream_groups = build_stream(
-            self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs,
-            table=self.table if self.balance and self.G == 1 and self.d == 8 else None)
+            self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs)
         self.stream_asked = runs
         if self.stream is None:
             self.wants_stream = False
+
+    def _relabel(self) -> None:
+        """Give the codewords new labels so that every slice of 4096 carries the same share of this matrix' tags
+        (sq_codebook_balance: most used codewords first, each to the slice with the fewest tags so far), and keep the
+        relabelled pair: the tags are rewritten through the map and row k of the table moves to row map[k].  Every
+        weight decodes to the same bits as before, the tag-stream kernel's workgroups (one per slice) get equal work
+        whatever the distribution of the tags, and the matrix keeps ONE codebook (a stream that carries its own
+        relabelled copy, sq_stream_build_balanced, costs another 1.1 MiB per matrix)."""
+        from ..packed import pack_bits, unpack_bits
+        host = self.words.detach().to("cpu", torch.int32).contiguous()
+        remap = torch.empty(1 << self.bits, dtype=torch.int16)
+        rc = _lib.lib().sq_codebook_balance(host.data_ptr(), self.R, self.W, self.C, self.d, self.bits, remap.data_ptr())
+        if rc == _lib.SQ_EUNSUPPORTED:                  # a shape the slice stream does not cover: nothing to balance
+            self.relabelled = True
+            return
+        _lib.check(rc)
+        new_of = (remap.to(torch.int32) & 0xFFFF).to(torch.int64)            # file label -> new label
+        dev = self.words.device
+        if self.bits == 16:
+            old = (self.words.view(torch.int16).to(torch.int32) & 0xFFFF).to(torch.int64)
+            self.words = remap.to(dev)[old].view(torch.int32).reshape(self.R, self.W).contiguous()
+        else:
+            self.words = pack_bits(new_of[unpack_bits(host, self.bits, self.nch)], self.bits).to(dev)
+        table = torch.empty_like(self.table)
+        table[new_of.to(dev)] = self.table
+        self.table = table
+        self.relabelled = True
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -257,7 +286,8 @@ def prepare_stack(pieces, workgroups: int | None = None) -> None:
     ps = [p for p in pieces if p.wants_stream and not p.stream_tiled]
     if not ps:
         return
-    if workgroups is None:
+    default = workgroups is None
+    if default:
         workgroups = torch.cuda.get_device_properties(ps[0].device).multi_processor_count
     # Smallest piece first: a piece with column orders can need more runs than its share (a run holds the whole
     # groups of a few orders), and what it takes beyond its share comes off the larger pieces' runs, so the launch
@@ -266,7 +296,7 @@ def prepare_stack(pieces, workgroups: int | None = None) -> None:
     for p in sorted(ps, key=lambda q: q.R):
         buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // STREAM_PART_MAX)
         runs = max(1, round(workgroups * p.R / rows / buckets))
-        if p.words is not None and (p.stream is None or (runs != p.stream_asked and not (len(ps) == 1 and p.stream_asked == 0))):
+        if p.words is not None and (p.stream is None or (runs != p.stream_asked and not (default and len(ps) == 1 and p.stream_asked == 0))):
             p.build_stream(runs)
         workgroups = max(workgroups - (p.stream_runs & 0xFFFF) * buckets, buckets)
         rows -= p.R

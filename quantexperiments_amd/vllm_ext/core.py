@@ -157,11 +157,27 @@ class PackedShards:
         """fp16 [R, C] (testing)."""
         return torch.cat([rl.dense(torch.float16) for rl in self.rls])
 
-    def tune_launch(self, reps: int = 3) -> list:
-        """The reference searches warps x blocks x split-K per shape here (shapequant/vllm_ext/core.py:259-296).
-        The library plans its launches from the shape and the device's compute units; the one choice left to the
-        caller, how many runs the pieces' tag streams are cut into, is made in prepare_stack from the same CU count.
-        Returns the run counts in use."""
+    @torch.no_grad()
+    def tune_launch(self, reps: int = 3, factors=(1.0, 0.875, 1.125, 0.75)) -> list:
+        """Search the one launch parameter the caller owns, by measurement, per shape (the reference searches warps x
+        blocks x split-K here, shapequant/vllm_ext/core.py:259-296; the library plans everything else from the shape
+        and the device's compute units): into how many runs the pieces' tag streams are cut, i.e. how many workgroups
+        the batch-1 launch makes.  The streams are rebuilt for `factor` x one workgroup per compute unit, the batch-1
+        product is timed inside a HIP graph, the fastest cut is kept and remembered per shape.  Stacks without a
+        slice stream, or whose tags were dropped (compact), have nothing to search.  Returns the run counts in use."""
+        searchable = [rl for rl in self.rls if rl.wants_stream and not rl.stream_tiled and rl.words is not None]
+        if searchable and len(searchable) == len(self.rls):
+            shape = ("launch",) + self.key()
+            cus = torch.cuda.get_device_properties(self.device).multi_processor_count
+            if shape not in _TUNED:
+                x = torch.randn(1, self.C, device=self.device, dtype=torch.bfloat16)
+                timed = {}
+                for f in factors:
+                    prepare_stack(self.rls, workgroups=max(1, int(cus * f)))
+                    timed[f] = _graph_ms(lambda: self._small(x, 1), reps=reps)
+                _TUNED[shape] = min(timed, key=timed.get)
+                self.launch_search = timed               # milliseconds per product at every factor tried
+            prepare_stack(self.rls, workgroups=max(1, int(cus * _TUNED[shape])))
         return [rl.stream_runs & 0xFFFF for rl in self.rls]
 
     @torch.no_grad()

@@ -594,6 +594,28 @@ def test_packed_shards_forward(large, M):
         assert ps.forward(x.float().cuda()).dtype == torch.float32
 
 
+def test_tune_launch_searches_the_run_count_by_measurement():
+    """PackedShards.tune_launch (reference shapequant/vllm_ext/core.py:259-296): the streams of a stack are re-cut for
+    several workgroup counts, each cut is timed, the fastest one stays, is remembered per shape, and gives the
+    same numbers as before."""
+    from quantexperiments_amd.vllm_ext import core
+    a, b = synth(700, 3584, 8, 16, seed=91), synth(300, 3584, 8, 16, seed=92)
+    ps = core.PackedShards([to_device(a, stream="later"), to_device(b, stream="later")])
+    x = rand_x(1, 3584, torch.bfloat16, seed=2)
+    before = ps.forward(x.cuda()).float().cpu().numpy()
+    runs = ps.tune_launch(reps=2)
+    assert len(runs) == 2 and all(r >= 1 for r in runs) and len(ps.launch_search) == 4
+    assert min(ps.launch_search.values()) > 0
+    ref = np.concatenate([_ref(a, x), _ref(b, x)], axis=1)
+    after = ps.forward(x.cuda())
+    _check_lowp(after, ref)
+    assert np.abs(after.float().cpu().numpy() - before).max() <= 2.0 ** -7 * np.abs(ref).max()
+    ps2 = core.PackedShards([to_device(a, stream="later"), to_device(b, stream="later")])
+    assert ps2.tune_launch() == runs and not hasattr(ps2, "launch_search")          # remembered: nothing is timed again
+    d4 = core.PackedShards([to_device(synth(64, 256, 4, 12, seed=93))])
+    assert d4.tune_launch() == [0]                                                    # no slice stream, nothing to search
+
+
 def test_packed_shards_rejects_bad_pieces():
     from quantexperiments_amd.vllm_ext import core
     a, b = to_device(synth(8, 64, 4, 8)), to_device(synth(8, 128, 4, 8))

@@ -450,6 +450,39 @@ def test_balanced_stream_relabels_codewords_and_evens_out_the_slices(R, C, bits,
     assert lb.max() <= max(1.02 * lb.mean() + 1, top)
 
 
+def test_codebook_balance_gives_an_equivalent_matrix_with_even_slices():
+    """sq_codebook_balance: the relabelling by itself.  Tags rewritten through the map and the table's rows moved
+    with them decode to the same weights bit for bit, the map is a permutation, every slice of 4096 codewords carries
+    the same share of the tags, and the plain stream of the relabelled tags equals the tags."""
+    import ctypes
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(5)
+    R, C, bits = 300, 512, 15
+    K, U = 1 << bits, C // 8
+    w = 1.0 / np.arange(1, K + 1)
+    tags = rng.choice(K, size=(R, U), p=w / w.sum())                       # Zipf popularity, popular codewords first
+    table = rng.standard_normal((K, 8)).astype(np.float16)
+    rs = (rng.random(R) * 0.02 + 0.01).astype(np.float16)
+    words = np.ascontiguousarray(O.pack_bits(tags, bits))
+    remap = np.zeros(K, np.uint16)
+    assert L.sq_codebook_balance(words.ctypes.data_as(ctypes.c_void_p), R, words.shape[1], C, 8, bits,
+                                 remap.ctypes.data_as(ctypes.c_void_p)) == 0
+    new_of = remap.astype(np.int64)
+    assert sorted(new_of.tolist()) == list(range(K))
+    tags2 = new_of[tags]
+    table2 = np.empty_like(table)
+    table2[new_of] = table
+    perms = np.arange(C)[None]
+    assert np.array_equal(O.decode_tensors(tags2, table2, rs, None, None, perms, K), O.decode_tensors(tags, table, rs, None, None, perms, K))
+    load, load2 = np.bincount((tags >> 12).ravel(), minlength=K >> 12), np.bincount((tags2 >> 12).ravel(), minlength=K >> 12)
+    top = int(np.bincount(tags.ravel(), minlength=K).max())
+    assert load.max() > 2.5 * load.mean() and load2.max() <= max(1.02 * load2.mean() + 1, top)
+    buf, eff, NG = _build_stream(np.ascontiguousarray(O.pack_bits(tags2, bits)), R, C, bits, None, 2)
+    assert np.array_equal(_walk_stream(buf, R, C, 8, bits, eff, NG, None), tags2)
+    assert L.sq_codebook_balance(words.ctypes.data_as(ctypes.c_void_p), R, words.shape[1], C, 4, 12, remap.ctypes.data_as(ctypes.c_void_p)) == _lib.SQ_EUNSUPPORTED
+
+
 def _stream_reads(buf, R, C, bits, runs_out, NG, row_mask):
     """Every byte range of the stream buffer that stream_kernel (csrc/sq_stream.hip) forms an address for, replayed on
     the host: the run table, the group heads (with the kernel's clamp of the group index), the first steps of a wave's
