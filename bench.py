@@ -77,7 +77,7 @@ def skewed_tags(torch, gen, R, n, bits, how):
     return rank if how == "zipf-sorted" else torch.randperm(K, generator=gen)[rank]
 
 
-def make_layer(torch, dev, gen, shapes, d, bits, G=1, M=1, tags="uniform"):
+def make_layer(torch, dev, gen, shapes, d, bits, G=1, M=1, tags="uniform", stream="later"):
     """One layer of PackedLinear pieces with synthetic contents drawn from the CPU generator `gen` (per matrix: tags,
     table, row scales, codebook ids, row orders); the pieces of each launch get their load-time tag streams cut for
     that launch (as PackedShards does at load)."""
@@ -97,7 +97,7 @@ def make_layer(torch, dev, gen, shapes, d, bits, G=1, M=1, tags="uniform"):
         rm = torch.randint(0, M, (R,), generator=gen).to(torch.uint8) if M > 1 else None
         perms = seeded_perms(C, M, gen)
         t = lambda a: None if a is None else a.to(dev)
-        out[nm] = PackedLinear(t(words), t(table), t(rs), t(rb), t(rm), perms.to(dev), 1 << bits, d, stream="later")
+        out[nm] = PackedLinear(t(words), t(table), t(rs), t(rb), t(rm), perms.to(dev), 1 << bits, d, stream=stream)
     for l in LAUNCHES:
         prepare_stack([out[n] for n in l])
     return out
@@ -322,7 +322,7 @@ def resident_bytes(layer):
     return {**kinds, "total": total, "bits_per_weight": 8.0 * total / weights}
 
 
-def sweep(torch, dev, spec: str, rows: str, n_layers: int, tags: str = "uniform"):
+def sweep(torch, dev, spec: str, rows: str, n_layers: int, tags: str = "uniform", stream=True):
     """Other formats and shapes than the headline's, one layer (4 launches) per activation-row count:
     spec = "<7b|27b>,d,bits,G,M", e.g. "7b,4,12,1,1" (cfg3), "27b,8,16,1,16" (cfg5), "27b,4,12,4,1" (the shipped 27B
     format).  Up to 32 rows through sq_linear_small, above through sq_linear_gemm; n_layers distinct layers rotated
@@ -332,14 +332,15 @@ def sweep(torch, dev, spec: str, rows: str, n_layers: int, tags: str = "uniform"
     d, bits, G, M = int(d), int(bits), int(G), int(M)
     shapes = SHAPES_7B if model == "7b" else SHAPES_27B
     gen = torch.Generator().manual_seed(0)
-    layers = [make_layer(torch, dev, gen, shapes, d, bits, G, M, tags) for _ in range(n_layers)]
+    layers = [make_layer(torch, dev, gen, shapes, d, bits, G, M, tags, "later" if stream else False) for _ in range(n_layers)]
     nbytes = sum(launch_bytes(shapes, l, d, bits, G, M) for l in LAUNCHES)
     res = {}
     for B in [int(b) for b in rows.split(",")]:
         tot, per = layer_times(torch, dev, layers, shapes, B, linear_small if B <= 32 else linear_gemm, gen)
         res[f"B{B}"] = {"us_per_layer": tot, "GBps_packed": nbytes / tot / 1e3,
                         "tflops": 2.0 * B * sum(R * C for R, C in shapes.values()) / tot / 1e6, "per_launch_us": per}
-    return {"sweep": spec, "tags": tags, "layers_rotated": n_layers, "rows": res, "resident": resident_bytes(layers[0])}
+    return {"sweep": spec, "tags": tags, "load_time_layouts": bool(stream), "layers_rotated": n_layers, "rows": res,
+            "resident": resident_bytes(layers[0])}
 
 
 def main():
@@ -365,6 +366,9 @@ def main():
     ap.add_argument("--rows", default="1", help="activation-row counts for --sweep, comma separated")
     ap.add_argument("--tags", default="uniform", choices=("uniform", "zipf", "zipf-sorted"),
                     help="tag distribution of --sweep: uniform, or Zipf codeword popularity scattered over / sorted into the codebook")
+    ap.add_argument("--no-stream", action="store_true",
+                    help="--sweep without the load-time layouts (slice streams, tile-major copies): every row count then runs "
+                         "on the kernels that read the packed file's own layout")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 256 MiB device copies (a kernel of known traffic to scale rocprofv3 counters by)")
     args = ap.parse_args()
@@ -381,7 +385,8 @@ def main():
         print(json.dumps({"lm_head": lm_head(torch, dev)}))
         return
     if args.sweep:
-        print(json.dumps(sweep(torch, dev, args.sweep, args.rows, min(args.layers, 4 if args.sweep.startswith("27b") else 16), args.tags)))
+        print(json.dumps(sweep(torch, dev, args.sweep, args.rows, min(args.layers, 4 if args.sweep.startswith("27b") else 16), args.tags,
+                               not args.no_stream)))
         return
     D, BITS = 8, 16
     gen = torch.Generator().manual_seed(0)
