@@ -9,7 +9,7 @@ Steps rotate over enough distinct layers (>= 4x the 256 MB last-level cache) tha
 HBM.  K steps are captured in one HIP graph; the graph is replayed several times, each replay timed
 with HIP events on the launch stream, and the median replay counts.
 
-The batch-1 kernels read a load-time regrouping of the tags by codebook slice (about 3.4 bytes per
+The batch-1 kernels read a load-time regrouping of the tags by codebook slice (about 2.9 bytes per
 tag in HBM instead of the file's 2), built by the library when a layer is loaded; value still counts
 the packed file's bytes, which is what the metric is quoted on.
 
@@ -41,7 +41,7 @@ MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 / bf16
 # HBM bytes one gate|up launch of stream_kernel moves: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of
 # `bench.py --roofline-only --copy-probe`, scaled by the same counters' reading of a 256 MiB copy; the figures and
 # the commands are in the file named here.  It is a property of the kernel as profiled, not measured by this run.
-GATE_UP_TRAFFIC = {"bytes": 67_590_000, "source": "profiles/stream_kernel_gate_up_7b_bs1.md"}
+GATE_UP_TRAFFIC = {"bytes": 59_540_000, "source": "profiles/stream_kernel_gate_up_7b_bs1.md"}
 
 SHAPES_7B = {"q": (3584, 3584), "k": (512, 3584), "v": (512, 3584), "o": (3584, 3584),
              "gate": (18944, 3584), "up": (18944, 3584), "down": (3584, 18944)}
