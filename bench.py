@@ -154,8 +154,9 @@ def cpu_baseline(torch, layer, x, d, bits, shapes):
             "us_per_layer": total * 1e6, "decode_s": dec, "matmul_s": mm}
 
 
-def prefill(torch, dev, layer, shapes, names=("gate", "down"), T=2048):
-    """T-row prefill GEMM of single matrices: ms (median of REPS graph replays) and TFLOP/s."""
+def prefill(torch, dev, layer, shapes, names=("gate", "down"), T=2048, dense=True):
+    """T-row prefill GEMM of single matrices: ms (median of REPS graph replays) and TFLOP/s; with `dense`, also the
+    time of a dense bf16 GEMM of the same shape in PyTorch."""
     from quantexperiments_amd.kernels import linear_gemm
     res = {}
     for nm in names:
@@ -164,6 +165,13 @@ def prefill(torch, dev, layer, shapes, names=("gate", "down"), T=2048):
         y = torch.empty(T, R, device=dev, dtype=torch.bfloat16)
         ms = timed_graph(torch, lambda: linear_gemm([layer[nm]], x, y))
         res[nm] = {"ms": ms, "tflops": 2.0 * T * R * C / (ms * 1e-3) / 1e12}
+        if dense:
+            # for scale: the same product on a dense bf16 copy of the weights through PyTorch (the vendor GEMM library),
+            # timed the same way; it reads 4x the bytes and decodes nothing
+            w = (torch.randn(R, C, device=dev) * 0.02).to(torch.bfloat16)
+            lib = timed_graph(torch, lambda: torch.matmul(x, w.t(), out=y))
+            res[nm].update(library_dense_ms=lib, library_dense_tflops=2.0 * T * R * C / (lib * 1e-3) / 1e12, speed_vs_library_dense=lib / ms)
+            del w
     return res
 
 

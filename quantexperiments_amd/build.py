@@ -12,7 +12,7 @@ CSRC = HERE / "csrc"
 LIB = HERE / "libsqhip.so"
 SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_small_generic.hip", "sq_gemv.hip", "sq_gemv_b16d8.hip",
            "sq_gemv_b12d4.hip", "sq_gemv_b10d4.hip", "sq_gemv_b8d4.hip", "sq_gemm.hip", "sq_gemm256.hip", "sq_stream.hip",
-           "sq_q8.hip", "sq_neighbours.hip"]
+           "sq_q8.hip", "sq_neighbours.hip", "sq_segs.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

@@ -135,6 +135,12 @@ int launch_gemm_dense(const void* w, int w_dtype, int64_t ldw, int R, int C, con
                       void* y, int y_dtype, int64_t ldy, int T, hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
 size_t gemm_dense_workspace(int R, int C, int T);
 
+// d = 4 / 12-bit pieces at 1 or 2 activation rows, from the file's row-major tags (sq_segs.hip)
+bool segs_shape(const sq_matrix& m);
+bool segs_fits(const sq_matrix* mats, int cnt, int B, int cus);
+int launch_segs_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                      int64_t ldy, int B, int cus, hipStream_t s);
+
 // tile-major copy of the tags for the matrix-core decode kernel (host routines, sq_gemv.hip)
 bool tiled_format_ok(int R, int W, int C, int d, int bits);
 size_t tiled_bytes(int R, int W);

@@ -296,6 +296,19 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
             i = j;
             continue;
         }
+        if (B <= 2 && x_ok && segs_shape(m0)) {
+            // d = 4 / 12-bit rows of whole 128-tag segments at 1 or 2 activation rows: the row-segment kernel (7B-shaped
+            // layer: 45-46 us at one row, 56 at two, against 65-67 on the matrix-core kernel)
+            int j = i + 1;
+            while (j < n && j - i < 4 && segs_shape(mats[j]) && mats[j].W == m0.W) ++j;
+            if (segs_fits(mats + i, j - i, B, cus)) {
+                int rc = launch_segs_group(mats + i, j - i, x, x_dtype, ldx, y, y_dtype, ldy, B, cus, s);
+                if (rc) return rc;
+                for (int k = i; k < j; ++k) ws_off += mma_part_bytes(mats[k], B);   // (what small_workspace counted for them)
+                i = j;
+                continue;
+            }
+        }
         if (mma_shape(m0) && x_ok) {
             int j = i + 1;
             while (j < n && j - i < GEMV_MAX_PIECES && mma_shape(mats[j]) && mats[j].bits == m0.bits && mats[j].d == m0.d &&

@@ -1,0 +1,280 @@
+// Decode-time product of the d = 4 / 12-bit format (one codebook of 4096 entries, no column orders) at 1 or 2
+// activation rows, straight from the file's row-major tags.
+//
+// A row is cut into segments of 128 tags = 192 bytes = 512 columns; 16 lanes own a segment, lane j its tags
+// 8 j .. 8 j + 7 (three dwords).  A workgroup's 16-lane groups are bound to (row slot, segment) pairs for the whole
+// kernel: group g works on segment g mod nseg of row slot g / nseg, so the 32 activations a lane multiplies with never
+// change and stay in registers, and the four groups of a wave read 768 contiguous bytes of a row per step.  Step t
+// of a workgroup covers rows p0 + t rps .. + rps - 1 of its share [p0, p1) of the rows.  Per step a lane loads 12
+// bytes (eight steps are in flight per lane, requested before the codebook is staged), gathers eight 8-byte codewords
+// from the 32 KB codebook in LDS, adds 16 two-element dot products, and the 16 lanes of a group add up with four DPP
+// steps; the group's sum goes to its (row, segment) place in LDS.  No barrier inside the loop: after the last step one
+// barrier, then the rows' segments are added in segment order, scaled and stored.  A row's sum is formed in the same
+// order whatever the grid, the stack or the number of activation rows.
+//
+// Against the matrix-core kernel (sq_rows_mfma.h), which needs 196 registers per lane and therefore keeps 7 waves
+// per CU waiting on dependent loads, this one holds every byte it will read of a small matrix in flight at once.
+#include <atomic>
+#include "sq_gemv_kernel.h"
+
+namespace sq {
+
+constexpr int SEG_PF = 8;                // steps of tags in flight per lane
+constexpr int SEG_MAX_PIECES = 4;
+constexpr int SEG_MAX_WAVES = 16;
+// Activation rows per launch.  The products are vector-ALU dot instructions, 16 per lane, step and activation row:
+// measured on the 7B-shaped layer, two rows cost 56 us against 46 for one, four rows 85 (the matrix-core kernel: 67-69
+// at any of them).
+constexpr int SEG_MAX_ROWS = 2;
+constexpr int SEG_TABLE_BYTES = 4096 * 4 * 2;   // the codebook: 4096 entries of 4 fp16
+
+struct SegPiece {
+    const uint32_t* tags;
+    const uint16_t* table;
+    const uint16_t* row_scale;
+    int R, y_off, wg_begin, wg_count;
+};
+
+struct SegArgs {
+    SegPiece p[SEG_MAX_PIECES];
+    int n;
+    const uint16_t* x;                   // activation row b0
+    void* y;                             // output row b0
+    int64_t ldx, ldy;
+    int nb;                              // activation rows of this launch (<= NB)
+    int x_dtype, y_dtype;
+    int W;                               // dwords per row of tags
+    int nseg;                            // segments per row
+    int rps;                             // rows per step of a workgroup
+    int rows_max;                        // most rows in one workgroup's share: the LDS sums are [NB][rows_max][nseg]; the
+                                         // activation rows follow them as fp16 [NB][C]
+    int table_bytes;
+};
+
+typedef __attribute__((address_space(3))) void* seg_lptr_t;
+typedef const __attribute__((address_space(1))) void* seg_gptr_t;
+typedef __attribute__((address_space(3))) u32x2 seg_lds_u32x2;
+
+template <int NB>
+__global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = (int)blockDim.x >> 6;
+    int pi = 0;
+#pragma unroll
+    for (int k = 1; k < SEG_MAX_PIECES; ++k)
+        if (k < a.n && (int)blockIdx.x >= a.p[k].wg_begin) pi = k;
+    const SegPiece P = a.p[pi];
+    const int wg = (int)blockIdx.x - P.wg_begin;
+    const int p0 = (int)((int64_t)P.R * wg / P.wg_count), p1 = (int)((int64_t)P.R * (wg + 1) / P.wg_count);
+    const int nrows = p1 - p0;                                   // >= 1: the launcher makes no more workgroups than rows
+    const int nseg = a.nseg, rps = a.rps;
+    const int nsteps = (nrows + rps - 1) / rps;
+    // (the codeword gathers form LDS addresses as numbers counted from the start of the dynamic LDS, which is address 0
+    // in a kernel without static LDS; a build in which it is not leaves y unwritten, which no test survives)
+    if ((uint32_t)(uintptr_t)(seg_lptr_t)lds != 0u) return;
+
+    const int gidx = tid >> 4, j = tid & 15;
+    const bool active = gidx < nseg * rps;                       // groups past the last (row slot, segment) pair shadow group 0
+    const int g2 = active ? gidx : 0;
+    const int rsub = g2 / nseg, seg = g2 - rsub * nseg;
+    const uint32_t* tg = P.tags + seg * 48 + j * 3;
+    auto load_step = [&](int t) {
+        const int row = min(p0 + min(t, nsteps - 1) * rps + rsub, p1 - 1);
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x3*>(tg + (size_t)row * a.W));
+    };
+    // everything this workgroup needs from memory is requested before anything waits: the codebook (memory to LDS
+    // without passing through registers), the first steps of tags, the activation rows
+    {
+        const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table);
+        for (int c = wave; c < a.table_bytes / 1024; c += nwaves)
+            __builtin_amdgcn_global_load_lds((seg_gptr_t)(src + (size_t)c * 1024 + lane * 16), (seg_lptr_t)(lds + c * 1024), 16, 0, 0);
+    }
+    u32x3 ring[SEG_PF];
+#pragma unroll
+    for (int q = 0; q < SEG_PF; ++q) ring[q] = load_step(q);
+    // the activation rows go through LDS once per workgroup (every group of a segment needs the same 512 of them;
+    // fetched by each lane for itself they would cost as much cache traffic as the tags): 16 bytes per thread and turn
+    constexpr int XT = 4;                                        // turns requested together
+    const int xchunks = nseg * 64;                               // 16-byte pieces of a row
+    unsigned char* xs = lds + a.table_bytes + (((size_t)NB * a.rows_max * nseg * 4 + 15) & ~(size_t)15);   // [NB][C] fp16
+    for (int i0 = tid; i0 < NB * xchunks; i0 += XT * (int)blockDim.x) {
+        u32x4 v[XT];
+#pragma unroll
+        for (int k = 0; k < XT; ++k) {
+            const int i = min(i0 + k * (int)blockDim.x, NB * xchunks - 1), b = i / xchunks;
+            v[k] = reinterpret_cast<const u32x4*>(a.x + (int64_t)min(b, a.nb - 1) * a.ldx)[i - b * xchunks];
+        }
+#pragma unroll
+        for (int k = 0; k < XT; ++k) {
+            const int i = i0 + k * (int)blockDim.x;
+            u32x4 q = v[k];
+            if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
+            if (i < NB * xchunks) reinterpret_cast<u32x4*>(xs)[i] = q;
+        }
+    }
+    float* psum = reinterpret_cast<float*>(lds + a.table_bytes);   // [NB][rows_max][nseg]
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    uint32_t xr[NB][16];                                         // this lane's 32 activations per row, as fp16 pairs
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32x4 q = reinterpret_cast<const u32x4*>(xs + ((size_t)b * xchunks + seg * 64 + j * 4) * 16)[i];
+            xr[b][4 * i] = q.x; xr[b][4 * i + 1] = q.y; xr[b][4 * i + 2] = q.z; xr[b][4 * i + 3] = q.w;
+        }
+
+    // LDS byte addresses of the codewords of a lane's eight tags: tag k sits at bit 12 k of the lane's 96
+    auto addresses = [](const u32x3& w, uint32_t (&ad)[8]) {
+        ad[0] = (w.x << 3) & 0x7FF8u;
+        ad[1] = (w.x >> 9) & 0x7FF8u;
+        ad[2] = __builtin_amdgcn_alignbit(w.y, w.x, 21) & 0x7FF8u;
+        ad[3] = (w.y >> 1) & 0x7FF8u;
+        ad[4] = (w.y >> 13) & 0x7FF8u;
+        ad[5] = __builtin_amdgcn_alignbit(w.z, w.y, 25) & 0x7FF8u;
+        ad[6] = (w.z >> 5) & 0x7FF8u;
+        ad[7] = (w.z >> 17) & 0x7FF8u;
+    };
+    // the rest of a step: the eight codewords, their products, the group's sum to its place
+    auto finish = [&](int t, const uint32_t (&ad)[8]) {
+        u32x2 cw[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) cw[k] = *reinterpret_cast<const seg_lds_u32x2*>((uintptr_t)ad[k]);
+        float acc[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[b] = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t cwh = cw[k][h];                   // (bit_cast straight from a vector element misreads it)
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+                    acc[b] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, cwh), __builtin_bit_cast(half2v, xr[b][2 * k + h]), acc[b], false);
+            }
+        const int row = p0 + t * rps + rsub;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const float v = team_sum(acc[b], 16);                // every lane of the group holds the group's sum
+            if (j == 15 && active && row < p1) psum[((size_t)b * a.rows_max + (row - p0)) * nseg + seg] = v;
+        }
+    };
+    // Whole rounds of SEG_PF steps, then the rest.  Within a round a step's three registers are refilled for the next
+    // round once its addresses have been formed from them (the same registers: no copies at the end of a round, and
+    // no branch inside one, so the waits count loads exactly).
+    int t0 = 0;
+    for (; t0 + SEG_PF <= nsteps; t0 += SEG_PF) {
+#pragma unroll
+        for (int q = 0; q < SEG_PF; ++q) {
+            uint32_t ad[8];
+            addresses(ring[q], ad);
+            __builtin_amdgcn_sched_barrier(0);
+            ring[q] = load_step(t0 + q + SEG_PF);
+            __builtin_amdgcn_sched_barrier(0);
+            finish(t0 + q, ad);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < SEG_PF; ++q)
+        if (t0 + q < nsteps) {                                   // uniform in the workgroup
+            uint32_t ad[8];
+            addresses(ring[q], ad);
+            finish(t0 + q, ad);
+        }
+    __syncthreads();
+    const size_t ysz = a.y_dtype == SQ_F32 ? 4 : 2;
+    for (int idx = tid; idx < nrows * a.nb; idx += (int)blockDim.x) {
+        const int b = idx / nrows, rl = idx - b * nrows;
+        const float* ps = psum + ((size_t)b * a.rows_max + rl) * nseg;
+        float sum = 0.f;
+        for (int sgi = 0; sgi < nseg; ++sgi) sum += ps[sgi];
+        const int r = p0 + rl;
+        store_y((char*)a.y + (size_t)b * a.ldy * ysz, a.y_dtype, (int64_t)P.y_off + r, sum * h2f(P.row_scale[r]));
+    }
+}
+
+// d = 4, 12-bit tags, one codebook, no column orders, rows of whole segments, at most SEG_MAX_WAVES * 4 segments per row
+bool segs_shape(const sq_matrix& m) {
+    if (!m.tags || m.d != 4 || m.bits != 12 || m.G != 1 || m.perms || m.R <= 0) return false;
+    const int U = m.C / m.d;
+    if (m.C % m.d || U % 128 || U / 128 > SEG_MAX_WAVES * 4) return false;
+    if ((int64_t)U * 12 != (int64_t)m.W * 32) return false;
+    return (((uintptr_t)m.tags & 3) | ((uintptr_t)m.table & 15)) == 0;
+}
+
+template <int NB>
+static int segs_launch_as(const SegArgs& a, int grid, int threads, size_t smem, hipStream_t s) {
+    static std::atomic<bool> raised{false};
+    if (!raised.load(std::memory_order_acquire)) {
+        (void)hipFuncSetAttribute((const void*)segs_kernel<NB>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipGetLastError();
+        raised.store(true, std::memory_order_release);
+    }
+    hipLaunchKernelGGL((segs_kernel<NB>), dim3((unsigned)grid), dim3((unsigned)threads), smem, s, a);
+    return check_launch("sq_linear_small(segs)");
+}
+
+// How pieces [0, cnt) are launched together: false when the workgroups' partial sums would not fit LDS beside the
+// codebook (matrices of several hundred thousand rows).
+struct SegPlan { int nseg, rps, waves, per_cu, grid, rows_max, NB; int wg_begin[SEG_MAX_PIECES], wg_count[SEG_MAX_PIECES]; size_t smem; };
+
+static bool segs_plan(const sq_matrix* mats, int cnt, int B, int cus, SegPlan& pl) {
+    pl.nseg = mats[0].C / mats[0].d / 128;
+    // rows per step: about 32 groups of 16 lanes per workgroup
+    pl.rps = 8;
+    while (pl.rps > 1 && pl.nseg * pl.rps > 32) pl.rps >>= 1;
+    pl.waves = (pl.nseg * pl.rps + 3) / 4;
+    pl.NB = B;
+    int64_t rows_total = 0;
+    for (int k = 0; k < cnt; ++k) rows_total += mats[k].R;
+    for (pl.per_cu = pl.waves <= 8 ? 2 : 1; pl.per_cu >= 1; --pl.per_cu) {   // workgroups a CU holds (128 registers per lane)
+        pl.grid = 0;
+        pl.rows_max = 1;
+        for (int k = 0; k < cnt; ++k) {
+            const int R = mats[k].R;
+            int64_t n = ((int64_t)R * cus * pl.per_cu + rows_total - 1) / rows_total;
+            const int64_t most = (R + pl.rps - 1) / pl.rps;      // a workgroup has at least one full step
+            if (n > most) n = most;
+            if (n < 1) n = 1;
+            pl.wg_begin[k] = pl.grid;
+            pl.wg_count[k] = (int)n;
+            pl.grid += (int)n;
+            pl.rows_max = std::max(pl.rows_max, (int)((R + n - 1) / n));
+        }
+        pl.smem = (size_t)SEG_TABLE_BYTES + (((size_t)pl.NB * pl.rows_max * pl.nseg * 4 + 15) & ~(size_t)15) + (size_t)pl.NB * pl.nseg * 1024;
+        if (pl.smem <= (size_t)(160 * 1024) / pl.per_cu) return true;
+    }
+    return false;
+}
+
+bool segs_fits(const sq_matrix* mats, int cnt, int B, int cus) {
+    SegPlan pl;
+    return cnt >= 1 && cnt <= SEG_MAX_PIECES && B >= 1 && B <= SEG_MAX_ROWS && segs_plan(mats, cnt, B, cus, pl);
+}
+
+// Pieces [0, cnt) pass segs_shape and share C, and segs_fits() holds (B <= SEG_MAX_ROWS); x is 16-byte aligned with ldx % 8 == 0.
+int launch_segs_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
+                      int64_t ldy, int B, int cus, hipStream_t s) {
+    SegPlan pl;
+    if (!segs_fits(mats, cnt, B, cus) || !segs_plan(mats, cnt, B, cus, pl)) return fail(SQ_ELAUNCH, "sq_linear_small(segs): no plan");
+    SegArgs a;
+    a.n = cnt;
+    a.x = (const uint16_t*)x; a.y = y; a.ldx = ldx; a.ldy = ldy; a.nb = B; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+    a.W = mats[0].W;
+    a.nseg = pl.nseg;
+    a.rps = pl.rps;
+    a.rows_max = pl.rows_max;
+    a.table_bytes = SEG_TABLE_BYTES;
+    for (int k = 0; k < cnt; ++k) {
+        const sq_matrix& m = mats[k];
+        SegPiece& P = a.p[k];
+        P.tags = (const uint32_t*)m.tags; P.table = m.table; P.row_scale = m.row_scale; P.R = m.R; P.y_off = m.y_off;
+        P.wg_begin = pl.wg_begin[k];
+        P.wg_count = pl.wg_count[k];
+    }
+    for (int k = cnt; k < SEG_MAX_PIECES; ++k) a.p[k] = a.p[0];
+    return pl.NB == 1 ? segs_launch_as<1>(a, pl.grid, pl.waves * 64, pl.smem, s) : segs_launch_as<2>(a, pl.grid, pl.waves * 64, pl.smem, s);
+}
+
+}  // namespace sq

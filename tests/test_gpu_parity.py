@@ -966,6 +966,47 @@ def test_full_7b_d4_stacks_at_small_batches_against_c_oracle(launch):
         _check_lowp(yb, ref)
 
 
+@pytest.mark.parametrize("shapes", [[(70, 512)], [(1, 512)], [(3, 1024), (9, 1024)], [(300, 3584), (64, 3584), (65, 3584)],
+                                    [(40, 18944)], [(129, 8192), (2, 8192), (2, 8192), (31, 8192)], [(9000, 512)]],
+                         ids=lambda c: "+".join(f"{r}x{k}" for r, k in c))
+def test_row_segment_kernel_of_the_12_bit_format(shapes):
+    """d = 4 / 12-bit pieces whose rows are whole segments of 128 tags run on the row-segment kernel at 1 and 2
+    activation rows (one segment per row up to 37, fewer rows than a workgroup takes per step, shares of rows that
+    do not divide, four stacked pieces, several thousand rows; 3 and 4 rows take the matrix-core kernel): against the
+    C oracle in fp32 and bf16 / fp16 output, with strided x and y; row 1 of a two-row call has the bits of the one-row
+    call; a one-hot input reads a weight column back exactly."""
+    from quantexperiments_amd.kernels import linear_small
+    pieces, ws = _stack(shapes, 4, 12, 1, 200 + len(shapes))
+    C, Rt = shapes[0][1], sum(r for r, _ in shapes)
+    w = np.concatenate(ws, axis=0)
+    one = {}
+    for B in (1, 2, 3, 4):
+        for dt in (torch.bfloat16, torch.float16):
+            x = rand_x(B, C, dt, seed=B)
+            ref = c_oracle.linear(_xf(x), w)
+            xd = torch.zeros(B, C + 8, dtype=dt, device="cuda")                # row stride C + 8
+            xd[:, :C] = x.cuda()
+            y = torch.full((B, Rt + 5), 7.0, dtype=torch.float32, device="cuda")
+            linear_small(pieces, xd[:, :C], y[:, :Rt])
+            assert rel_max_err(y[:, :Rt].cpu().numpy(), ref) < TOL, (B, dt)
+            assert bool((y[:, Rt:] == 7.0).all())
+            one[(B, dt)] = y[:, :Rt].clone()
+            yl = torch.empty(B, Rt, dtype=dt, device="cuda")
+            linear_small(pieces, xd[:, :C], yl)
+            _check_lowp(yl, ref)
+    # the same activation row alone and as row 1 of 2
+    x2 = rand_x(2, C, torch.bfloat16, seed=2)
+    y1 = torch.empty(1, Rt, dtype=torch.float32, device="cuda")
+    linear_small(pieces, x2[1:2].cuda(), y1)
+    assert torch.equal(y1[0], one[(2, torch.bfloat16)][1])
+    # one-hot input: every other product is an exact zero
+    col = C - 3
+    xo = torch.zeros(1, C, dtype=torch.float16)
+    xo[0, col] = 1.0
+    linear_small(pieces, xo.cuda(), y1)
+    assert np.array_equal(y1.cpu().numpy()[0], w[:, col].astype(np.float32))
+
+
 @pytest.mark.parametrize("shape", [(18944, 3584, 1), (3584, 18944, 1), (5120, 5120, 16)], ids=lambda c: "x".join(map(str, c)))
 def test_full_size_gemm_rows_against_gemv(shape):
     """M = 2048 prefill at the 7B gate/up and down sizes and at a 27B-class matrix with 16 column orders: every
