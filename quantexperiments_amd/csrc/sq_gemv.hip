@@ -211,7 +211,12 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
     a.ks = pl.ks;
     a.table_bytes = (int)mma_table_bytes(m0);
     const int threads = pl.KW * 64;
-    const size_t smem = (size_t)a.table_bytes + 16 + (pl.KW > 1 ? (size_t)MMA_TT * pl.KW * 64 * pl.NT * 16 : 0);
+    // LDS behind the codebook: the waves' accumulators of the tiles between two barriers (MMA_TT tiles when the codebook
+    // is read through the cache; with the codebook in LDS as many as the workgroup walks, if they fit: sized below)
+    const size_t red_tile = (size_t)pl.KW * 64 * pl.NT * 16;
+    const int pft = mma_pft(pl.RW);
+    a.tg = a.table_bytes ? pft : 0;
+    size_t smem = (size_t)a.table_bytes + 16 + (a.table_bytes ? (size_t)a.tg * red_tile : pl.KW > 1 ? (size_t)MMA_TT * red_tile : 0);
     int rc = SQ_EUNSUPPORTED;
 #define SQ_CASE(BI, DD) if (m0.bits == BI && m0.d == DD) rc = launch_mma_b##BI##d##DD(OP, a, pl.RW, pl.NT, GRID, threads, smem, s)
 #define OP 1
@@ -244,6 +249,17 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
         wg += P.wg_count;
     }
     for (int k = cnt; k < GEMV_MAX_PIECES; ++k) a.p[k] = a.p[0];
+    if (a.table_bytes) {
+        int most = 1;                                            // most tiles one workgroup walks
+        for (int k = 0; k < cnt; ++k) {
+            const int ntiles = (mats[k].R + 15) / 16, nshare = a.p[k].wg_count / pl.ks;
+            most = std::max(most, (ntiles + nshare - 1) / nshare);
+        }
+        const size_t room = (size_t)(160 * 1024) / rc - a.table_bytes - 16;
+        int fit = (int)(room / red_tile) / pft * pft;
+        a.tg = std::min((most + pft - 1) / pft * pft, std::max(fit, pft));
+        smem = (size_t)a.table_bytes + 16 + (size_t)a.tg * red_tile;
+    }
 #define OP 0
 #define GRID wg
     rc = SQ_EUNSUPPORTED;

@@ -11,12 +11,15 @@
 //
 // Work split.  A wave owns a slice of the columns for its whole life, so its B operands (the
 // activations of that slice, converted bf16 -> fp16 once) are loaded once and stay in registers; it
-// walks over 16-row tiles, prefetching the next tile's tags while it multiplies the current one.
+// walks over 16-row tiles with the tags of the next tiles in flight (one tile ahead when the codewords come
+// through the cache, which is then the bound; two or three tiles when the codebook sits in LDS).
 // The tag stream is read in lane units (UD dwords = TPU whole tags = UK columns): in round n the four
 // lane groups g = 0..3 of a row read units 4n + g, one wide load each, and the round's SPU matrix
 // instructions consume the units chunk pair by chunk pair.  The KW waves of a workgroup split the
-// columns of a tile; their accumulators are added through LDS by one wave per tile (round robin, two
-// buffers, one barrier per tile).  Rows longer than KW * RW rounds are split over `ks` workgroups whose
+// columns of a tile; their accumulators are added through LDS by one wave per tile (round robin): after
+// every MMA_TT tiles when the codebook is read through the cache, after all the tiles of the workgroup (as
+// many as LDS holds accumulators for: MmaArgs.tg) when it sits in LDS, so that the waves of a launch of the
+// 7B shapes meet once.  Rows longer than KW * RW rounds are split over `ks` workgroups whose
 // partial sums go to a workspace and are added, in slice order, by splitk_reduce_kernel.
 #pragma once
 #include <mutex>
@@ -45,9 +48,13 @@ struct MmaArgs {
     int U;                // lane units per row
     int ks;               // workgroup-level column slices
     int table_bytes;      // bytes of codebook staged in LDS (0 = read through cache)
+    int tg;               // codebook in LDS: 16-row tiles whose accumulators LDS holds between two barriers (a multiple of mma_pft(RW))
 };
 
-constexpr int MMA_TT = 4;     // 16-row tiles multiplied between two workgroup barriers
+constexpr int MMA_TT = 4;     // 16-row tiles multiplied between two workgroup barriers (codebook read through the cache)
+// codebook in LDS: tiles of tags in flight per lane (fewer when a lane's part of a tile is long: registers)
+// (2 to 5 tiles in flight measure alike on the 7B shapes)
+constexpr int mma_pft(int RW) { return RW >= 8 ? 2 : 3; }
 
 // Optional timeline of the first wave of every workgroup (debug builds define SQ_TRACE_POINT).
 #ifndef SQ_TRACE_POINT
@@ -83,7 +90,6 @@ __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
 
     // LDS: [codebook][one all-zero codeword][reduction buffer: TT tiles x KW waves x 64 lanes x NT x 16 bytes]
     const int zero_off = a.table_bytes;                                 // units past the row's end gather this entry
-    const uint32_t zero_idx = (uint32_t)(a.table_bytes / ESZ);
     float4v* red = reinterpret_cast<float4v*>(smem + a.table_bytes + 16);
 
     // ---- this wave's rounds
@@ -182,18 +188,19 @@ __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
         auto gather = [&](int k) {
             const int n = k / SPU, s = k - n * SPU;
             const bool dead = !all_live && !live[n];
-            const uint32_t bo = ((LDS_TAB && dead) ? zero_idx : cur.boff) * ESZ;      // byte offset of the row's codebook
+            const uint32_t bo = cur.boff * ESZ;                 // byte offset of the row's codebook
+            // (codebook in LDS: a unit past the row's end gathers the all-zero entry, whatever its tags are)
             if (D == 8) {
                 const uint32_t tag = unit_tag<BITS, UD>(cur.t[n], s);
-                if (LDS_TAB) av[k] = *reinterpret_cast<const u32x4*>(smem + (tag * ESZ + bo));
+                if (LDS_TAB) av[k] = *reinterpret_cast<const u32x4*>(smem + (dead ? (uint32_t)zero_off : tag * ESZ + bo));
                 else av[k] = *reinterpret_cast<const u32x4*>(table + ((size_t)tag * ESZ + bo));
             } else {
                 const uint32_t g0 = unit_tag<BITS, UD>(cur.t[n], 2 * s);
                 const uint32_t g1 = unit_tag<BITS, UD>(cur.t[n], 2 * s + 1);
                 u32x2 c0, c1;
                 if (LDS_TAB) {
-                    c0 = *reinterpret_cast<const u32x2*>(smem + (g0 * ESZ + bo));
-                    c1 = *reinterpret_cast<const u32x2*>(smem + (g1 * ESZ + bo));
+                    c0 = *reinterpret_cast<const u32x2*>(smem + (dead ? (uint32_t)zero_off : g0 * ESZ + bo));
+                    c1 = *reinterpret_cast<const u32x2*>(smem + (dead ? (uint32_t)zero_off : g1 * ESZ + bo));
                 } else {
                     c0 = *reinterpret_cast<const u32x2*>(table + ((size_t)g0 * ESZ + bo));
                     c1 = *reinterpret_cast<const u32x2*>(table + ((size_t)g1 * ESZ + bo));
@@ -216,67 +223,150 @@ __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
         }
     };
 
-    // ---- groups of TT tiles: multiply them one after the other (the next tile's tags load meanwhile), then
-    // add the KW waves' accumulators through LDS, each tile of the group by a different wave
-    for (int tg = t0, grp = 0; tg < t1; tg += TT, ++grp) {
-        float4v acc[TT][NT];
-        if (grp > 0) {
+    if constexpr (LDS_TAB) {
+        // ---- codebook in LDS.  Nothing here waits for the cache, so what bounds the kernel is how many bytes of tags it
+        // keeps in flight and how often its waves meet: every lane holds mma_pft(RW) tiles of tags (a tile's registers are
+        // refilled as soon as its last codeword has been gathered), a tile's accumulator goes straight to its place in
+        // LDS, and the waves meet once per a.tg tiles (once per launch when the workgroup's tiles all fit), after which
+        // each tile is added up by one wave (round robin), scaled and stored.
+        constexpr int PFT = mma_pft(RW);
+        if (t0 >= t1) return;                                 // (uniform in the workgroup; the launcher gives every one a tile)
+        // a tile's tags without a branch around the loads (the waits then count loads exactly): the two layouts differ
+        // in a base and a stride, chosen once
+        const bool til = P.tiled != nullptr;
+        const uint32_t* fbase = til ? P.tiled + li * UD : tags;
+        uint32_t fo[RW];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) sc[0][v] = sc[TT][v];
-        }
-#pragma unroll
-        for (int tt = 0; tt < TT; tt += 2) {
-            if (tg + tt < t1) {
-                if (tg + tt + 1 < t1) fetch(tg + tt + 1, tB, sc[tt + 1]);
-                multiply(tA, acc[tt]);
-            }
-            if (tg + tt + 1 < t1) {
-                if (tg + tt + 2 < t1) fetch(tg + tt + 2, tA, sc[tt + 2]);
-                multiply(tB, acc[tt + 1]);
-            }
-        }
-        SQ_TRACE_POINT(3 + 3 * (grp < 4 ? grp : 4));
-        if (KW > 1) {
-            if (grp > 0) __syncthreads();                     // the previous group's reducers are done reading
-#pragma unroll
-            for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) red[((tt * KW + wave) * 64 + lane) * NT + nt] = acc[tt][nt];
-            __syncthreads();
-        }
-        SQ_TRACE_POINT(4 + 3 * (grp < 4 ? grp : 4));
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-            const int t = tg + tt;
-            if (t >= t1) continue;
-            if (KW > 1 && wave != (tt + grp) % KW) continue;   // this tile's reducer
-            float4v tot[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                if (KW > 1) {
-                    float4v s4 = red[((tt * KW) * 64 + lane) * NT + nt];
-                    for (int k = 1; k < KW; ++k) {
-                        const float4v o = red[((tt * KW + k) * 64 + lane) * NT + nt];
-                        s4.x += o.x; s4.y += o.y; s4.z += o.z; s4.w += o.w;
-                    }
-                    tot[nt] = s4;
-                } else tot[nt] = acc[tt][nt];
-            }
+        for (int n = 0; n < RW; ++n) fo[n] = til ? uoff[n] * 16u : uoff[n];
+        auto fetch_tags = [&](int t, Tile& T) {
             const int row0 = t << 4;
+            const int r = row0 + li < m.R ? row0 + li : m.R - 1;
+            const uint32_t* bp = fbase + (til ? (size_t)t * a.U * 16 * UD : (size_t)r * m.W);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int tok = nt * 16 + li;
-                if (tok >= a.B) continue;
+            for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(bp + fo[n]);
+            T.boff = m.row_book ? (uint32_t)m.row_book[r] << BITS : 0u;
+        };
+        Tile ring[PFT];
+        ring[0] = tA;
+#pragma unroll
+        for (int q = 1; q < PFT; ++q) fetch_tags(min(t0 + q, t1 - 1), ring[q]);
+        auto tile_done = [&](int tl, const float4v (&acc)[NT]) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) red[((tl * KW + wave) * 64 + lane) * NT + nt] = acc[nt];
+        };
+        for (int tg = t0; tg < t1; tg += a.tg) {
+            const int te = min(tg + a.tg, t1);
+            if (tg > t0) __syncthreads();                     // the previous group's sums have been read
+            int t = tg;
+            for (; t + PFT <= te; t += PFT) {
+#pragma unroll
+                for (int q = 0; q < PFT; ++q) {
+                    float4v acc[NT];
+                    multiply(ring[q], acc);
+                    __builtin_amdgcn_sched_barrier(0);
+                    fetch_tags(min(t + q + PFT, t1 - 1), ring[q]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    tile_done(t + q - tg, acc);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < PFT; ++q)
+                if (t + q < te) {                             // (the last group's last tiles: nothing left to fetch)
+                    float4v acc[NT];
+                    multiply(ring[q], acc);
+                    tile_done(t + q - tg, acc);
+                }
+            __syncthreads();
+            for (int tl = wave; tl < te - tg; tl += KW) {
+                const int row0 = (tg + tl) << 4;
+                float scl[4];
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const int r = row0 + 4 * lg + v;
-                    if (r >= m.R) continue;
-                    if (a.ks > 1) P.part[((int64_t)slice * a.B + tok) * m.R + r] = tot[nt][v];
-                    else store_y(a.y, a.y_dtype, (int64_t)tok * a.ldy + m.y_off + r, tot[nt][v] * sc[tt][v]);
+                    const int ro = row0 + 4 * lg + v;
+                    scl[v] = h2f(m.row_scale[ro < m.R ? ro : m.R - 1]);
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    float4v s4 = red[((tl * KW) * 64 + lane) * NT + nt];
+                    for (int k = 1; k < KW; ++k) {
+                        const float4v o = red[((tl * KW + k) * 64 + lane) * NT + nt];
+                        s4.x += o.x; s4.y += o.y; s4.z += o.z; s4.w += o.w;
+                    }
+                    const int tok = nt * 16 + li;
+                    if (tok >= a.B) continue;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int r = row0 + 4 * lg + v;
+                        if (r >= m.R) continue;
+                        if (a.ks > 1) P.part[((int64_t)slice * a.B + tok) * m.R + r] = s4[v];
+                        else store_y(a.y, a.y_dtype, (int64_t)tok * a.ldy + m.y_off + r, s4[v] * scl[v]);
+                    }
                 }
             }
         }
-        SQ_TRACE_POINT(5 + 3 * (grp < 4 ? grp : 4));
+    } else {
+        // ---- groups of TT tiles: multiply them one after the other (the next tile's tags load meanwhile), then
+        // add the KW waves' accumulators through LDS, each tile of the group by a different wave
+        for (int tg = t0, grp = 0; tg < t1; tg += TT, ++grp) {
+            float4v acc[TT][NT];
+            if (grp > 0) {
+    #pragma unroll
+                for (int v = 0; v < 4; ++v) sc[0][v] = sc[TT][v];
+            }
+    #pragma unroll
+            for (int tt = 0; tt < TT; tt += 2) {
+                if (tg + tt < t1) {
+                    if (tg + tt + 1 < t1) fetch(tg + tt + 1, tB, sc[tt + 1]);
+                    multiply(tA, acc[tt]);
+                }
+                if (tg + tt + 1 < t1) {
+                    if (tg + tt + 2 < t1) fetch(tg + tt + 2, tA, sc[tt + 2]);
+                    multiply(tB, acc[tt + 1]);
+                }
+            }
+            SQ_TRACE_POINT(3 + 3 * (grp < 4 ? grp : 4));
+            if (KW > 1) {
+                if (grp > 0) __syncthreads();                     // the previous group's reducers are done reading
+    #pragma unroll
+                for (int tt = 0; tt < TT; ++tt)
+    #pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) red[((tt * KW + wave) * 64 + lane) * NT + nt] = acc[tt][nt];
+                __syncthreads();
+            }
+            SQ_TRACE_POINT(4 + 3 * (grp < 4 ? grp : 4));
+    #pragma unroll
+            for (int tt = 0; tt < TT; ++tt) {
+                const int t = tg + tt;
+                if (t >= t1) continue;
+                if (KW > 1 && wave != (tt + grp) % KW) continue;   // this tile's reducer
+                float4v tot[NT];
+    #pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    if (KW > 1) {
+                        float4v s4 = red[((tt * KW) * 64 + lane) * NT + nt];
+                        for (int k = 1; k < KW; ++k) {
+                            const float4v o = red[((tt * KW + k) * 64 + lane) * NT + nt];
+                            s4.x += o.x; s4.y += o.y; s4.z += o.z; s4.w += o.w;
+                        }
+                        tot[nt] = s4;
+                    } else tot[nt] = acc[tt][nt];
+                }
+                const int row0 = t << 4;
+    #pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int tok = nt * 16 + li;
+                    if (tok >= a.B) continue;
+    #pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int r = row0 + 4 * lg + v;
+                        if (r >= m.R) continue;
+                        if (a.ks > 1) P.part[((int64_t)slice * a.B + tok) * m.R + r] = tot[nt][v];
+                        else store_y(a.y, a.y_dtype, (int64_t)tok * a.ldy + m.y_off + r, tot[nt][v] * sc[tt][v]);
+                    }
+                }
+            }
+            SQ_TRACE_POINT(5 + 3 * (grp < 4 ? grp : 4));
+        }
     }
     SQ_TRACE_POINT(19);
 }
