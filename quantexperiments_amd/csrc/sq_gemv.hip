@@ -316,7 +316,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
             // d = 4 / 12-bit rows of whole 128-tag segments at 1 or 2 activation rows: the row-segment kernel (7B-shaped
             // layer: 45-46 us at one row, 56 at two, against 65-67 on the matrix-core kernel)
             int j = i + 1;
-            while (j < n && j - i < 4 && segs_shape(mats[j]) && mats[j].W == m0.W) ++j;
+            while (j < n && j - i < 4 && segs_shape(mats[j]) && mats[j].W == m0.W && mats[j].G == m0.G) ++j;
             if (segs_fits(mats + i, j - i, B, cus)) {
                 int rc = launch_segs_group(mats + i, j - i, x, x_dtype, ldx, y, y_dtype, ldy, B, cus, s);
                 if (rc) return rc;

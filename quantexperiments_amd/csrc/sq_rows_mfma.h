@@ -146,6 +146,14 @@ __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
     // tags, the activations of this wave's columns (raw), the codebook
     Tile tA, tB;
     float sc[TT + 1][4];                                      // [TT]: first tile of the next group, fetched early
+    // (a codebook of whole KB goes memory -> LDS without passing through registers, a wave instruction per KB)
+    const bool table_dma = LDS_TAB && (a.table_bytes & 1023) == 0;
+    if (table_dma) {
+        typedef const __attribute__((address_space(1))) void* gptr_t;
+        typedef __attribute__((address_space(3))) void* lptr_t;
+        for (int c = wave; c < (a.table_bytes >> 10); c += KW)
+            __builtin_amdgcn_global_load_lds((gptr_t)(table + (size_t)c * 1024 + lane * 16), (lptr_t)(smem + c * 1024), 16, 0, 0);
+    }
     if (t0 < t1) fetch(t0, tA, sc[0]);
     u32x4 xraw[RW][SPU][NT];
 #pragma unroll
@@ -158,7 +166,7 @@ __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
                 xraw[n][s][nt] = *reinterpret_cast<const u32x4*>(a.x + (int64_t)(tok < a.B ? tok : a.B - 1) * a.ldx + ucol[n] + 8 * s);
             }
     if (LDS_TAB) {
-        stage_table(m.table, a.table_bytes, smem);
+        if (!table_dma) stage_table(m.table, a.table_bytes, smem);
         if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0u;
     }
     // the B operands: this wave's activations as fp16, in registers for the whole kernel
@@ -175,7 +183,10 @@ __global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
                 xb[n][s][nt] = __builtin_bit_cast(half8v, v);
             }
     SQ_TRACE_POINT(1);
-    if (LDS_TAB) __syncthreads();
+    if (LDS_TAB) {
+        if (table_dma) __builtin_amdgcn_s_waitcnt(0);         // the codebook has landed (and the first tile's tags with it)
+        __syncthreads();
+    }
     SQ_TRACE_POINT(2);
 
     // One tile: NS = RW * SPU matrix instructions.  The codeword gathers run PD instructions ahead of the

@@ -1,5 +1,5 @@
-// Decode-time product of the d = 4 / 12-bit format (one codebook of 4096 entries, no column orders) at 1 or 2
-// activation rows, straight from the file's row-major tags.
+// Decode-time product of the d = 4 / 12-bit format (codebooks of 4096 entries, up to four per matrix, no column
+// orders) at 1 or 2 activation rows, straight from the file's row-major tags.
 //
 // A row is cut into segments of 128 tags = 192 bytes = 512 columns; 16 lanes own a segment, lane j its tags
 // 8 j .. 8 j + 7 (three dwords).  A workgroup's 16-lane groups are bound to (row slot, segment) pairs for the whole
@@ -26,12 +26,14 @@ constexpr int SEG_MAX_WAVES = 16;
 // measured on the 7B-shaped layer, two rows cost 56 us against 46 for one, four rows 85 (the matrix-core kernel: 67-69
 // at any of them).
 constexpr int SEG_MAX_ROWS = 2;
-constexpr int SEG_TABLE_BYTES = 4096 * 4 * 2;   // the codebook: 4096 entries of 4 fp16
+constexpr int SEG_TABLE_BYTES = 4096 * 4 * 2;   // one codebook: 4096 entries of 4 fp16
+constexpr int SEG_MAX_BOOKS = 4;                // codebooks per matrix (128 KB of the CU's 160 KB of LDS)
 
 struct SegPiece {
     const uint32_t* tags;
     const uint16_t* table;
     const uint16_t* row_scale;
+    const uint8_t* row_book;             // codebook of every row (several codebooks per matrix) or NULL
     int R, y_off, wg_begin, wg_count;
 };
 
@@ -48,14 +50,16 @@ struct SegArgs {
     int rps;                             // rows per step of a workgroup
     int rows_max;                        // most rows in one workgroup's share: the LDS sums are [NB][rows_max][nseg]; the
                                          // activation rows follow them as fp16 [NB][C]
-    int table_bytes;
+    int table_bytes;                     // all codebooks of a piece: G x 32 KB
+    int xdirect;                         // 1: no room in LDS for the activation rows, every lane fetches its own
 };
 
 typedef __attribute__((address_space(3))) void* seg_lptr_t;
 typedef const __attribute__((address_space(1))) void* seg_gptr_t;
 typedef __attribute__((address_space(3))) u32x2 seg_lds_u32x2;
 
-template <int NB>
+// NB activation rows; MB: rows name one of several codebooks (row_book), all of them in LDS
+template <int NB, bool MB>
 __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -79,10 +83,11 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
     const int g2 = active ? gidx : 0;
     const int rsub = g2 / nseg, seg = g2 - rsub * nseg;
     const uint32_t* tg = P.tags + seg * 48 + j * 3;
+    auto row_of = [&](int t) { return min(p0 + min(t, nsteps - 1) * rps + rsub, p1 - 1); };
     auto load_step = [&](int t) {
-        const int row = min(p0 + min(t, nsteps - 1) * rps + rsub, p1 - 1);
-        return __builtin_nontemporal_load(reinterpret_cast<const u32x3*>(tg + (size_t)row * a.W));
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x3*>(tg + (size_t)row_of(t) * a.W));
     };
+
     // everything this workgroup needs from memory is requested before anything waits: the codebook (memory to LDS
     // without passing through registers), the first steps of tags, the activation rows
     {
@@ -98,7 +103,16 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
     constexpr int XT = 4;                                        // turns requested together
     const int xchunks = nseg * 64;                               // 16-byte pieces of a row
     unsigned char* xs = lds + a.table_bytes + (((size_t)NB * a.rows_max * nseg * 4 + 15) & ~(size_t)15);   // [NB][C] fp16
-    for (int i0 = tid; i0 < NB * xchunks; i0 += XT * (int)blockDim.x) {
+    u32x4 xown[NB][4];                                           // (xdirect) this lane's activations as loaded
+    if (a.xdirect) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint16_t* xp = a.x + (int64_t)min(b, a.nb - 1) * a.ldx + seg * 512 + j * 32;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xown[b][i] = reinterpret_cast<const u32x4*>(xp)[i];
+        }
+    }
+    for (int i0 = tid; !a.xdirect && i0 < NB * xchunks; i0 += XT * (int)blockDim.x) {
         u32x4 v[XT];
 #pragma unroll
         for (int k = 0; k < XT; ++k) {
@@ -114,27 +128,41 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
         }
     }
     float* psum = reinterpret_cast<float*>(lds + a.table_bytes);   // [NB][rows_max][nseg]
+    // several codebooks: the codebook ids of this workgroup's rows, one byte each, behind everything else in LDS
+    unsigned char* lbooks = xs + (a.xdirect ? 0 : (size_t)NB * xchunks * 16);
+    if (MB)
+        for (int i = tid; i < nrows; i += (int)blockDim.x) lbooks[i] = P.row_book[p0 + i];
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    // LDS offset of the codebook of step t's row (32 KB apiece), read one step ahead of its use
+    auto book_at = [&](int t) { return MB ? (uint32_t)lbooks[row_of(t) - p0] << 15 : 0u; };
+    uint32_t bo = book_at(0);
     uint32_t xr[NB][16];                                         // this lane's 32 activations per row, as fp16 pairs
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const u32x4 q = reinterpret_cast<const u32x4*>(xs + ((size_t)b * xchunks + seg * 64 + j * 4) * 16)[i];
+            u32x4 q;
+            if (a.xdirect) {
+                q = xown[b][i];
+                if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
+            } else {
+                q = reinterpret_cast<const u32x4*>(xs + ((size_t)b * xchunks + seg * 64 + j * 4) * 16)[i];
+            }
             xr[b][4 * i] = q.x; xr[b][4 * i + 1] = q.y; xr[b][4 * i + 2] = q.z; xr[b][4 * i + 3] = q.w;
         }
 
     // LDS byte addresses of the codewords of a lane's eight tags: tag k sits at bit 12 k of the lane's 96
-    auto addresses = [](const u32x3& w, uint32_t (&ad)[8]) {
-        ad[0] = (w.x << 3) & 0x7FF8u;
-        ad[1] = (w.x >> 9) & 0x7FF8u;
-        ad[2] = __builtin_amdgcn_alignbit(w.y, w.x, 21) & 0x7FF8u;
-        ad[3] = (w.y >> 1) & 0x7FF8u;
-        ad[4] = (w.y >> 13) & 0x7FF8u;
-        ad[5] = __builtin_amdgcn_alignbit(w.z, w.y, 25) & 0x7FF8u;
-        ad[6] = (w.z >> 5) & 0x7FF8u;
-        ad[7] = (w.z >> 17) & 0x7FF8u;
+    // (plus the LDS offset of the row's codebook, 32 KB apiece: `(v & mask) | offset` is one instruction)
+    auto addresses = [](const u32x3& w, uint32_t bo, uint32_t (&ad)[8]) {
+        ad[0] = ((w.x << 3) & 0x7FF8u) | bo;
+        ad[1] = ((w.x >> 9) & 0x7FF8u) | bo;
+        ad[2] = (__builtin_amdgcn_alignbit(w.y, w.x, 21) & 0x7FF8u) | bo;
+        ad[3] = ((w.y >> 1) & 0x7FF8u) | bo;
+        ad[4] = ((w.y >> 13) & 0x7FF8u) | bo;
+        ad[5] = (__builtin_amdgcn_alignbit(w.z, w.y, 25) & 0x7FF8u) | bo;
+        ad[6] = ((w.z >> 5) & 0x7FF8u) | bo;
+        ad[7] = ((w.z >> 17) & 0x7FF8u) | bo;
     };
     // the rest of a step: the eight codewords, their products, the group's sum to its place
     auto finish = [&](int t, const uint32_t (&ad)[8]) {
@@ -168,9 +196,10 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
 #pragma unroll
         for (int q = 0; q < SEG_PF; ++q) {
             uint32_t ad[8];
-            addresses(ring[q], ad);
+            addresses(ring[q], bo, ad);
             __builtin_amdgcn_sched_barrier(0);
             ring[q] = load_step(t0 + q + SEG_PF);
+            bo = book_at(t0 + q + 1);
             __builtin_amdgcn_sched_barrier(0);
             finish(t0 + q, ad);
         }
@@ -179,7 +208,8 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
     for (int q = 0; q < SEG_PF; ++q)
         if (t0 + q < nsteps) {                                   // uniform in the workgroup
             uint32_t ad[8];
-            addresses(ring[q], ad);
+            addresses(ring[q], bo, ad);
+            bo = book_at(t0 + q + 1);
             finish(t0 + q, ad);
         }
     __syncthreads();
@@ -194,46 +224,55 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
     }
 }
 
-// d = 4, 12-bit tags, one codebook, no column orders, rows of whole segments, at most SEG_MAX_WAVES * 4 segments per row
+// d = 4, 12-bit tags, codebooks of 4096 entries (up to 4: all of them fit LDS), no column orders, rows of whole
+// segments, at most SEG_MAX_WAVES * 4 segments per row
 bool segs_shape(const sq_matrix& m) {
-    if (!m.tags || m.d != 4 || m.bits != 12 || m.G != 1 || m.perms || m.R <= 0) return false;
+    if (!m.tags || m.d != 4 || m.bits != 12 || m.G < 1 || m.G > SEG_MAX_BOOKS || m.perms || m.R <= 0) return false;
+    if (m.G > 1 && !m.row_book) return false;
     const int U = m.C / m.d;
     if (m.C % m.d || U % 128 || U / 128 > SEG_MAX_WAVES * 4) return false;
     if ((int64_t)U * 12 != (int64_t)m.W * 32) return false;
     return (((uintptr_t)m.tags & 3) | ((uintptr_t)m.table & 15)) == 0;
 }
 
-template <int NB>
+template <int NB, bool MB>
 static int segs_launch_as(const SegArgs& a, int grid, int threads, size_t smem, hipStream_t s) {
     static std::atomic<bool> raised{false};
     if (!raised.load(std::memory_order_acquire)) {
-        (void)hipFuncSetAttribute((const void*)segs_kernel<NB>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)segs_kernel<NB, MB>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         (void)hipGetLastError();
         raised.store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((segs_kernel<NB>), dim3((unsigned)grid), dim3((unsigned)threads), smem, s, a);
+    hipLaunchKernelGGL((segs_kernel<NB, MB>), dim3((unsigned)grid), dim3((unsigned)threads), smem, s, a);
     return check_launch("sq_linear_small(segs)");
 }
 
-// How pieces [0, cnt) are launched together: false when the workgroups' partial sums would not fit LDS beside the
-// codebook (matrices of several hundred thousand rows).
-struct SegPlan { int nseg, rps, waves, per_cu, grid, rows_max, NB; int wg_begin[SEG_MAX_PIECES], wg_count[SEG_MAX_PIECES]; size_t smem; };
+// How pieces [0, cnt) (same C, same number of codebooks) are launched together: false when the workgroups' partial
+// sums would not fit LDS beside the codebooks (matrices of several hundred thousand rows).
+struct SegPlan {
+    int nseg, rps, waves, per_cu, grid, rows_max, NB, table_bytes, xdirect;
+    int wg_begin[SEG_MAX_PIECES], wg_count[SEG_MAX_PIECES];
+    size_t smem;
+};
 
 static bool segs_plan(const sq_matrix* mats, int cnt, int B, int cus, SegPlan& pl) {
     pl.nseg = mats[0].C / mats[0].d / 128;
-    // rows per step: about 32 groups of 16 lanes per workgroup
+    pl.table_bytes = mats[0].G * SEG_TABLE_BYTES;
+    // 16-lane groups per workgroup: about 32 in 8 waves, two workgroups per CU, when the codebooks leave room for two;
+    // about 64 in one workgroup of 16 waves otherwise
+    const bool two = pl.table_bytes <= 64 * 1024;
     pl.rps = 8;
-    while (pl.rps > 1 && pl.nseg * pl.rps > 32) pl.rps >>= 1;
+    while (pl.rps > 1 && pl.nseg * pl.rps > (two ? 32 : 64)) pl.rps >>= 1;
     pl.waves = (pl.nseg * pl.rps + 3) / 4;
     pl.NB = B;
     int64_t rows_total = 0;
     for (int k = 0; k < cnt; ++k) rows_total += mats[k].R;
-    for (pl.per_cu = pl.waves <= 8 ? 2 : 1; pl.per_cu >= 1; --pl.per_cu) {   // workgroups a CU holds (128 registers per lane)
+    for (pl.per_cu = two && pl.waves <= 8 ? 2 : 1; pl.per_cu >= 1; --pl.per_cu) {   // workgroups a CU holds (128 registers per lane)
         pl.grid = 0;
         pl.rows_max = 1;
         for (int k = 0; k < cnt; ++k) {
             const int R = mats[k].R;
-            int64_t n = ((int64_t)R * cus * pl.per_cu + rows_total - 1) / rows_total;
+            int64_t n = (int64_t)R * cus * pl.per_cu / rows_total;   // (rounded down: one workgroup too many is a second round)
             const int64_t most = (R + pl.rps - 1) / pl.rps;      // a workgroup has at least one full step
             if (n > most) n = most;
             if (n < 1) n = 1;
@@ -242,8 +281,13 @@ static bool segs_plan(const sq_matrix* mats, int cnt, int B, int cus, SegPlan& p
             pl.grid += (int)n;
             pl.rows_max = std::max(pl.rows_max, (int)((R + n - 1) / n));
         }
-        pl.smem = (size_t)SEG_TABLE_BYTES + (((size_t)pl.NB * pl.rows_max * pl.nseg * 4 + 15) & ~(size_t)15) + (size_t)pl.NB * pl.nseg * 1024;
-        if (pl.smem <= (size_t)(160 * 1024) / pl.per_cu) return true;
+        const size_t room = (size_t)(160 * 1024) / pl.per_cu;
+        const size_t base = (size_t)pl.table_bytes + (((size_t)pl.NB * pl.rows_max * pl.nseg * 4 + 15) & ~(size_t)15);
+        const size_t xs = (size_t)pl.NB * pl.nseg * 1024;        // the activation rows as fp16
+        const size_t ids = mats[0].G > 1 ? (((size_t)pl.rows_max + 15) & ~(size_t)15) : 0;   // codebook ids of the rows
+        pl.xdirect = base + xs + ids > room ? 1 : 0;
+        pl.smem = base + (pl.xdirect ? 0 : xs) + ids;
+        if (pl.smem <= room) return true;
     }
     return false;
 }
@@ -253,7 +297,8 @@ bool segs_fits(const sq_matrix* mats, int cnt, int B, int cus) {
     return cnt >= 1 && cnt <= SEG_MAX_PIECES && B >= 1 && B <= SEG_MAX_ROWS && segs_plan(mats, cnt, B, cus, pl);
 }
 
-// Pieces [0, cnt) pass segs_shape and share C, and segs_fits() holds (B <= SEG_MAX_ROWS); x is 16-byte aligned with ldx % 8 == 0.
+// Pieces [0, cnt) pass segs_shape, share C and G, and segs_fits() holds (B <= SEG_MAX_ROWS); x is 16-byte aligned with
+// ldx % 8 == 0.
 int launch_segs_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                       int64_t ldy, int B, int cus, hipStream_t s) {
     SegPlan pl;
@@ -265,16 +310,21 @@ int launch_segs_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype
     a.nseg = pl.nseg;
     a.rps = pl.rps;
     a.rows_max = pl.rows_max;
-    a.table_bytes = SEG_TABLE_BYTES;
+    a.table_bytes = pl.table_bytes;
+    a.xdirect = pl.xdirect;
     for (int k = 0; k < cnt; ++k) {
         const sq_matrix& m = mats[k];
         SegPiece& P = a.p[k];
-        P.tags = (const uint32_t*)m.tags; P.table = m.table; P.row_scale = m.row_scale; P.R = m.R; P.y_off = m.y_off;
+        P.tags = (const uint32_t*)m.tags; P.table = m.table; P.row_scale = m.row_scale; P.row_book = m.G > 1 ? m.row_book : nullptr;
+        P.R = m.R; P.y_off = m.y_off;
         P.wg_begin = pl.wg_begin[k];
         P.wg_count = pl.wg_count[k];
     }
     for (int k = cnt; k < SEG_MAX_PIECES; ++k) a.p[k] = a.p[0];
-    return pl.NB == 1 ? segs_launch_as<1>(a, pl.grid, pl.waves * 64, pl.smem, s) : segs_launch_as<2>(a, pl.grid, pl.waves * 64, pl.smem, s);
+    const int threads = pl.waves * 64;
+    if (mats[0].G > 1)
+        return pl.NB == 1 ? segs_launch_as<1, true>(a, pl.grid, threads, pl.smem, s) : segs_launch_as<2, true>(a, pl.grid, threads, pl.smem, s);
+    return pl.NB == 1 ? segs_launch_as<1, false>(a, pl.grid, threads, pl.smem, s) : segs_launch_as<2, false>(a, pl.grid, threads, pl.smem, s);
 }
 
 }  // namespace sq

@@ -1026,6 +1026,38 @@ def test_row_segment_kernel_of_the_12_bit_format(shapes):
     assert np.array_equal(y1.cpu().numpy()[0], w[:, col].astype(np.float32))
 
 
+@pytest.mark.parametrize("shapes,G", [([(300, 3584)], 4), ([(130, 5120), (64, 5120), (3, 5120)], 4), ([(40, 17408)], 4), ([(77, 1024)], 2),
+                                      ([(2100, 512)], 3)], ids=lambda c: str(c))
+def test_row_segment_kernel_with_several_codebooks(shapes, G):
+    """The same kernel on matrices whose rows name one of G codebooks of 4096 entries (the 27B recipe: G = 4, all four
+    in LDS), including rows so long that the activation rows no longer fit LDS beside the codebooks: 1 to 4 activation
+    rows against the C oracle (3 and 4 run on the matrix cores), row 1 of two equal to the single-row call."""
+    from quantexperiments_amd.kernels import linear_small, prepare_stack
+    pieces, ws = [], []
+    for k, (R, C) in enumerate(shapes):
+        sy = synth(R, C, 4, 12, G, 1, seed=300 + 7 * k + G)
+        pieces.append(to_device(sy, stream="later"))
+        ws.append(c_oracle.decode(sy.words, 12, C, 4, sy.K, sy.table, sy.row_scale, sy.row_book, None, None))
+    prepare_stack(pieces)
+    w = np.concatenate(ws, axis=0)
+    C, Rt = shapes[0][1], w.shape[0]
+    ys = {}
+    for B in (1, 2, 3, 4):
+        x = rand_x(B, C, torch.bfloat16, seed=10 + B)
+        ref = c_oracle.linear(_xf(x), w)
+        y = torch.full((B, Rt), 7.0, dtype=torch.float32, device="cuda")
+        linear_small(pieces, x.cuda(), y)
+        assert rel_max_err(y.cpu().numpy(), ref) < TOL, B
+        ys[B] = y
+        yb = torch.empty(B, Rt, dtype=torch.float16, device="cuda")
+        linear_small(pieces, x.to(torch.float16).cuda(), yb)
+        _check_lowp(yb, c_oracle.linear(_xf(x.to(torch.float16)), w))
+    x2 = rand_x(2, C, torch.bfloat16, seed=12)
+    y1 = torch.empty(1, Rt, dtype=torch.float32, device="cuda")
+    linear_small(pieces, x2[1:2].cuda(), y1)
+    assert torch.equal(y1[0], ys[2][1])
+
+
 @pytest.mark.parametrize("shape", [(18944, 3584, 1), (3584, 18944, 1), (5120, 5120, 16)], ids=lambda c: "x".join(map(str, c)))
 def test_full_size_gemm_rows_against_gemv(shape):
     """M = 2048 prefill at the 7B gate/up and down sizes and at a 27B-class matrix with 16 column orders: every
