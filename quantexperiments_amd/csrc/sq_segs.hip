@@ -22,9 +22,10 @@ namespace sq {
 constexpr int SEG_PF = 8;                // steps of tags in flight per lane
 constexpr int SEG_MAX_PIECES = 4;
 constexpr int SEG_MAX_WAVES = 16;
-// Activation rows per launch.  The products are vector-ALU dot instructions, 16 per lane, step and activation row:
-// measured on the 7B-shaped layer, two rows cost 56 us against 46 for one, four rows 85 (the matrix-core kernel: 67-69
-// at any of them).
+// Activation rows per launch.  Measured on the 7B-shaped layer: two rows cost 55 us against 45 for one, four rows 85 (the
+// matrix-core kernel: 58-60 at four).  The same products on the matrix cores (v_mfma_f32_4x4x4_16b_f16, one instruction
+// per tag and activation row instead of two v_dot2c, element j of lane j's result) measured no faster at one or two rows
+// (gate|up 17.0-17.5 / 21.0 against 16.8 / 20.6 us).
 constexpr int SEG_MAX_ROWS = 2;
 constexpr int SEG_TABLE_BYTES = 4096 * 4 * 2;   // one codebook: 4096 entries of 4 fp16
 constexpr int SEG_MAX_BOOKS = 4;                // codebooks per matrix (128 KB of the CU's 160 KB of LDS)
