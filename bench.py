@@ -269,9 +269,10 @@ def lm_head(torch, dev, rows=(1, 4, 8, 16, 32, 64)):
 
 def neighbours(torch, dev, layers, x, y):
     """One decoder layer with the three elementwise neighbours of its products (add + RMS norm before q|k|v and
-    before gate|up, SiLU * up before down), as separate launches and fused into the consuming products; and the
-    two stand-alone kernels by themselves.  Microseconds per layer / per launch inside a HIP graph."""
-    from quantexperiments_amd.kernels import addnorm, linear_small, linear_small_from, silu_mul
+    before gate|up, SiLU * up before down), as separate launches and fused (add + norm into the product that consumes
+    it, SiLU * up into the gate|up product that feeds it: four launches per layer); and the two stand-alone kernels by
+    themselves.  Microseconds per layer / per launch inside a HIP graph."""
+    from quantexperiments_amd.kernels import addnorm, linear_small, linear_small_from, linear_small_silu, silu_mul
     L, I = LAUNCHES, SHAPES_7B["gate"][0]
     h = [torch.randn(1, 3584, device=dev), torch.empty(1, 3584, device=dev)]
     w = torch.ones(3584, device=dev, dtype=torch.bfloat16)
@@ -293,8 +294,8 @@ def neighbours(torch, dev, layers, x, y):
         for Ly in layers:
             linear_small_from([Ly[n] for n in L[0]], y[L[0]], x1, h_in=h[1], add=y[L[3]], w=w, eps=1e-6, h_out=h[0])
             linear_small([Ly[n] for n in L[1]], x[3584], y[L[1]])
-            linear_small_from([Ly[n] for n in L[2]], y[L[2]], x1, h_in=h[0], add=y[L[1]], w=w, eps=1e-6, h_out=h[1])
-            linear_small_from([Ly[n] for n in L[3]], y[L[3]], act, gate=gate, up=up)
+            linear_small_silu([Ly[n] for n in L[2]], None, act, x_out=x1, h_in=h[0], add=y[L[1]], w=w, eps=1e-6, h_out=h[1])
+            linear_small([Ly[n] for n in L[3]], act, y[L[3]])
 
     res = {}
     for name, fn, per in (("layer_separate_us", separate, len(layers)), ("layer_fused_us", fused, len(layers)),

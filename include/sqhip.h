@@ -297,6 +297,21 @@ typedef struct sq_producer {
 int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_producer* from, int x_dtype, void* y, int y_dtype,
                          int64_t ldy, int32_t B, void* workspace, size_t ws_bytes, void* stream);
 
+/* The stacked gate | up product with SiLU * up on the way out: mats[0] = the gate piece, mats[1] = the up piece (same
+ * R and C), out[b * ld_out + r] = silu(Y[b, r]) * Y[b, R + r] with Y the stacked product rounded to `dtype` (SQ_F16 /
+ * SQ_BF16, also x's type): the same results, bit for bit, as sq_linear_small into a `dtype` y followed by sq_silu_mul
+ * (gate = y, up = y + R, perms = NULL).  One launch: the workgroup that adds a row's partial sums up reads the gate
+ * row's and the up row's and writes their product, so Y never goes to memory.  This is the reference's EPI 2 epilogue
+ * (reference shapequant/kernels/proto_runs.py:223-237,269-287, the epi argument of gemv at :505-571) without its
+ * launch-wide ticket: there the last blocks of the launch compute the whole next input once every block has written y,
+ * here every row is finished where its sums meet.  `from` (NULL, or mode SQ_FROM_ADDNORM as in sq_linear_small_from,
+ * one activation row; x and ldx are then ignored and from->x_out is the row the launch computes and reads) lets the
+ * same launch produce its own input too.  For pieces on the tag-stream kernel without column orders whose streams are
+ * cut into the same runs (sq_stream_build with the same `runs`), 1 to 8 activation rows; any other stack returns
+ * SQ_EUNSUPPORTED and the caller makes the two calls.  Needs the workspace of sq_linear_small (its header). */
+int sq_linear_small_silu(const sq_matrix* mats, int32_t n_mats, const sq_producer* from, const void* x, int dtype, int64_t ldx,
+                         void* out, int64_t ld_out, int32_t B, void* workspace, size_t ws_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

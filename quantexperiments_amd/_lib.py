@@ -98,8 +98,9 @@ def lib() -> ctypes.CDLL:
                                  ctypes.c_int, vp]
         L.sq_silu_mul.argtypes = [vp, vp, ctypes.c_int, i64, vp, i32, i32, i32, vp, vp]
         L.sq_linear_small_from.argtypes = [mp, i32, ctypes.POINTER(SqProducer), ctypes.c_int, vp, ctypes.c_int, i64, i32, vp, sz, vp]
+        L.sq_linear_small_silu.argtypes = [mp, i32, ctypes.POINTER(SqProducer), vp, ctypes.c_int, i64, vp, i64, i32, vp, sz, vp]
         for f in (L.sq_dequant, L.sq_linear_small, L.sq_linear_gemm, L.sq_gemm_dense, L.sq_q8_linear, L.sq_q8_dequant,
-                  L.sq_q4_embed, L.sq_addnorm, L.sq_silu_mul, L.sq_linear_small_from, L.sq_workspace_status,
+                  L.sq_q4_embed, L.sq_addnorm, L.sq_silu_mul, L.sq_linear_small_from, L.sq_linear_small_silu, L.sq_workspace_status,
                   L.sq_workspace_reset, L.sq_noalloc_reset):
             f.restype = ctypes.c_int
         _lib = L
@@ -109,7 +110,7 @@ def lib() -> ctypes.CDLL:
 EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_linear_gemm", "sq_gemm_dense",
            "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build", "sq_stream_bytes_balanced", "sq_stream_build_balanced", "sq_q8_linear", "sq_q8_workspace_bytes",
            "sq_q8_dequant", "sq_q4_embed", "sq_addnorm", "sq_silu_mul",
-           "sq_linear_small_from", "sq_gemm_dense_ws", "sq_gemm_dense_workspace_bytes", "sq_linear_small_noalloc",
+           "sq_linear_small_from", "sq_linear_small_silu", "sq_gemm_dense_ws", "sq_gemm_dense_workspace_bytes", "sq_linear_small_noalloc",
            "sq_workspace_status", "sq_workspace_reset", "sq_noalloc_reset", "sq_stream_spin_limit", "sq_codebook_balance")
 
 

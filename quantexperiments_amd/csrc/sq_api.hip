@@ -76,7 +76,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 107; }
+int sq_version(void) { return 108; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -212,6 +212,28 @@ int sq_linear_small_from(const sq_matrix* mats, int32_t n_mats, const sq_produce
     if (small_takes_gemm_route(mats, n_mats, B, from->x_out, C))
         return launch_gemm(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, has_ws ? workspace : nullptr, s);
     return launch_small(mats, n_mats, from->x_out, x_dtype, C, y, y_dtype, ldy, B, ws, wsb, has_ws ? workspace : nullptr, s);
+}
+
+int sq_linear_small_silu(const sq_matrix* mats, int32_t n_mats, const sq_producer* from, const void* x, int dtype, int64_t ldx,
+                         void* out, int64_t ld_out, int32_t B, void* workspace, size_t ws_bytes, void* stream) {
+    const char* who = "sq_linear_small_silu";
+    if (n_mats != 2 || !mats) return fail(SQ_EINVAL, "%s: the gate and the up piece, n_mats %d", who, n_mats);
+    if (from && from->mode != SQ_FROM_ADDNORM) return fail(SQ_EINVAL, "%s: producer mode %d", who, from->mode);
+    const void* xin = from ? from->x_out : x;
+    const int64_t ldxin = from ? mats[0].C : ldx;
+    // (check_xy's bound on ldy is for the stacked y, which is not written here: ld_out is checked below)
+    int rc = check_xy(who, mats, n_mats, xin, dtype, ldxin, out, dtype, (int64_t)1 << 40, B);
+    if (rc) return rc;
+    if (mats[0].R != mats[1].R) return fail(SQ_EINVAL, "%s: gate has %d rows, up %d", who, mats[0].R, mats[1].R);
+    if (B > 1 && ld_out < mats[0].R) return fail(SQ_EINVAL, "%s: ld_out %lld < %d", who, (long long)ld_out, mats[0].R);
+    if (B == 0) return SQ_OK;
+    if (from && (B != 1 || !from->h_in || !from->w || from->h_out == from->h_in || (mats[0].C % 8) || ((uintptr_t)from->x_out & 15)))
+        return fail(SQ_EINVAL, "%s: a fused producer takes one activation row, h_in and w, h_out != h_in, a 16-byte aligned x_out", who);
+    if ((rc = refuse_if_poisoned(who, mats, n_mats))) return rc;
+    const WsParts wp = split_workspace(workspace, ws_bytes);
+    hipStream_t s = (hipStream_t)stream;
+    if (wp.sums) (void)stream_host_flag(s, true);
+    return launch_small_silu(mats, n_mats, xin, dtype, ldxin, out, ld_out, B, wp.sums ? workspace : nullptr, s, from);
 }
 
 int sq_linear_gemm(const sq_matrix* mats, int32_t n_mats, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,

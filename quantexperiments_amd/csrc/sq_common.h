@@ -119,6 +119,10 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
                  const sq_producer* from = nullptr);
 // one activation row of these pieces is a single launch of the tag-stream kernel, which can produce its own x
 bool small_fuses_producer(const sq_matrix* mats, int n, int B);
+// the two pieces are a gate and an up projection whose launch can write SiLU(gate) * up itself
+bool small_fuses_silu(const sq_matrix* mats, int n, int B);
+int launch_small_silu(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* act, int64_t ld_act, int B,
+                      void* sums, hipStream_t s, const sq_producer* from = nullptr);
 size_t small_workspace(const sq_matrix* mats, int n, int B);
 // some piece runs the tag-stream kernel, whose partial sums live in the workspace header (`sums` above)
 bool small_uses_sums(const sq_matrix* mats, int n);

@@ -289,6 +289,29 @@ bool small_fuses_producer(const sq_matrix* mats, int n, int B) {
     return true;
 }
 
+// SiLU(gate) * up written by the product itself: the two pieces are a gate and an up projection of one shape on the
+// tag-stream kernel (no column orders, cut into the same runs), at most 8 activation rows (one pass)
+bool small_fuses_silu(const sq_matrix* mats, int n, int B) {
+    if (n != 2 || B < 1 || B > 8) return false;
+    const sq_matrix &g = mats[0], &u = mats[1];
+    if (g.R <= 0 || g.R != u.R || g.C != u.C || g.bits != u.bits || g.perms || u.perms) return false;
+    // (the same cut into runs; the other fields of stream_runs describe each piece's own buffer and may differ)
+    if (!stream_rows(g, B) || !stream_rows(u, B) || stream_runs_of(g) != stream_runs_of(u) || stream_run_max_of(g) != stream_run_max_of(u) ||
+        g.stream_groups != u.stream_groups)
+        return false;
+    if (stream_geom_of(g).NV > 16 || stream_group_len(mats, 2) != 2) return false;
+    return stream_pass_rows(B) >= B;
+}
+
+int launch_small_silu(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* act, int64_t ld_act, int B,
+                      void* sums, hipStream_t s, const sq_producer* from) {
+    const bool x_ok = (B == 1 || ldx % 8 == 0) && (((uintptr_t)x & 15) == 0);
+    if (!small_fuses_silu(mats, n, B) || !(x_ok || from) || (from && !small_fuses_producer(mats, n, B)))
+        return fail(SQ_EUNSUPPORTED, "sq_linear_small_silu: no fused kernel for this stack (run sq_linear_small, then sq_silu_mul)");
+    if (!sums) return fail(SQ_EWORKSPACE, "sq_linear_small_silu: these pieces need a workspace (its header holds their partial sums)");
+    return launch_stream_group(mats, 2, x, x_dtype, ldx, nullptr, x_dtype, 0, B, (char*)sums, s, from, act, ld_act);
+}
+
 int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
                  int64_t ldy, int B, void* ws, size_t ws_bytes, void* sums, hipStream_t s, const sq_producer* from) {
     if (from && !small_fuses_producer(mats, n, B)) return fail(SQ_EUNSUPPORTED, "sq_linear_small_from: no fused kernel for this stack");

@@ -86,10 +86,15 @@ bool stream_shape(const sq_matrix& m);
 size_t stream_part_bytes(const sq_matrix& m, int rows);   // partial sums of one pass of `rows` activation rows
 // dense rows [r0, r1) of a matrix that is held as its tag stream only (sq_matrix.tags == NULL)
 int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t ld_out, int r0, int r1, hipStream_t s, bool raw);
+// act != NULL (two pieces of one shape, gate and up, no column orders, a 16-bit y_dtype): y is not written, act[b * ld_act + r]
+// = silu(Y[b, r]) * Y[b, R + r] is
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                        int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from = nullptr);
+                        int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from = nullptr, void* act = nullptr,
+                        int64_t ld_act = 0);
 // pieces [0, n) a single launch can take: their partial sums of one activation row fit the workspace header together
 int stream_group_len(const sq_matrix* mats, int n);
+// activation rows the kernel takes per pass for B of them (1, 2, 4 or 8)
+int stream_pass_rows(int B);
 // Polls of an item's partial sums before a workgroup gives up (sq_stream_spin_limit); and this device's host-visible
 // copy of the error word, which a workgroup that gives up also sets so that the next call can refuse without a
 // synchronisation: its device address (NULL when there is none and `may_allocate` is false, or under stream capture),

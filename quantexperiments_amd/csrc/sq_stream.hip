@@ -647,6 +647,11 @@ struct StreamArgs {
     const uint16_t* w;
     uint16_t* x_out;
     float eps;
+    // Consumer of the output (pieces 0 and 1 = the gate and the up projection, same shape, no column orders): instead of
+    // y the launch writes act[b * ld_act + r] = silu(round(Y[b, r])) * round(Y[b, R + r]) in y_dtype, the arithmetic of
+    // silu_mul_kernel on the rounded outputs.  NULL: y is written.
+    uint16_t* act;
+    int64_t ld_act;
     uint32_t* err;                    // the workspace header's error word (SQ_WS_ERR_OFF)
     uint32_t* host_err;               // its host-visible copy (pinned host memory) or NULL
     int spin_max;                     // polls of an item's partial sums before it gives up
@@ -1229,8 +1234,66 @@ __global__ __launch_bounds__(STREAM_NW * 64) void stream_kernel(StreamArgs a) {
     // y and zeroes the words.  The NV workgroups of a run are neighbours in the grid and workgroups are dispatched in
     // grid order, so a workgroup only ever waits for workgroups that are already running or done; the wait is bounded
     // all the same (an item that gives up is written as NaN).
-    const uint32_t* rows0 = reinterpret_cast<const uint32_t*>(P.stream + P.off_rows) + (size_t)g0 * 64;
     const int nl = ng * 64, items = nl * a.nb;
+    if constexpr (ORD == 0) {
+        if (a.act != nullptr) {
+            // SiLU * up on the way out.  The gate and the up piece have the same runs, and a row's partial sums sit at
+            // the same place of both pieces' areas, so the 2 NV workgroups of run `wi` of both pieces share the run's
+            // rows: each reads the NV sums of the gate row and the NV sums of the up row, finishes both as above, and
+            // writes their SiLU product.  (Workgroups of the gate piece then wait for workgroups up to half a launch
+            // behind them in the grid: running or done when the launch fits the machine in one round, which the
+            // caller's run counts see to; the wait is bounded all the same.)
+            const int nf = 2 * P.NV, f = pi * P.NV + v;
+            const int e_lo = (int)((int64_t)items * f / nf), e_hi = (int)((int64_t)items * (f + 1) / nf);
+            uint32_t* pg = reinterpret_cast<uint32_t*>(a.p[0].part) + (size_t)g0 * 64;
+            uint32_t* pu = reinterpret_cast<uint32_t*>(a.p[1].part) + (size_t)g0 * 64;
+            const size_t bs = (size_t)NB * np;
+            for (int it = e_lo + tid; it < e_hi; it += NTH) {
+                const int b = it / nl, i = it - b * nl;
+                const uint32_t r = g0 * 64 + i < P.R ? (uint32_t)(g0 * 64 + i) : STREAM_NO_ROW;
+                const float rg = h2f(a.p[0].row_scale[r != STREAM_NO_ROW ? r : 0u]), ru = h2f(a.p[1].row_scale[r != STREAM_NO_ROW ? r : 0u]);
+                uint32_t* qg = pg + (size_t)b * np + i;
+                uint32_t* qu = pu + (size_t)b * np + i;
+                uint32_t ug[16], uu[16];
+                bool ok = true;
+                for (int spin = 0;; ++spin) {
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) {
+                        ug[k] = __hip_atomic_load(qg + (size_t)min(k, P.NV - 1) * bs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        uu[k] = __hip_atomic_load(qu + (size_t)min(k, P.NV - 1) * bs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    ok = true;
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) ok = ok && ug[k] != 0u && uu[k] != 0u;
+                    if (ok || spin >= a.spin_max) break;
+                    __builtin_amdgcn_s_sleep(2);
+                }
+                float sg = 0.f, su = 0.f;
+#pragma unroll
+                for (int k = 0; k < 16; ++k)
+                    if (k < P.NV) {
+                        sg += ug[k] == STREAM_ZERO_SUM ? 0.f : __builtin_bit_cast(float, ug[k]);
+                        su += uu[k] == STREAM_ZERO_SUM ? 0.f : __builtin_bit_cast(float, uu[k]);
+                    }
+                for (int k = 0; k < P.NV; ++k) {
+                    __hip_atomic_store(qg + (size_t)k * bs, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(qu + (size_t)k * bs, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (!ok) {
+                    __hip_atomic_store(a.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (a.host_err) __hip_atomic_store(a.host_err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+                if (r != STREAM_NO_ROW) {
+                    const bool good = ok && err0 == 0u;
+                    const uint16_t g16 = round16(good ? sg * rg : __builtin_nanf(""), a.y_dtype);
+                    const uint16_t u16 = round16(good ? su * ru : __builtin_nanf(""), a.y_dtype);
+                    a.act[(int64_t)b * a.ld_act + r] = silu_mul_one(g16, u16, a.y_dtype);
+                }
+            }
+            return;
+        }
+    }
+    const uint32_t* rows0 = reinterpret_cast<const uint32_t*>(P.stream + P.off_rows) + (size_t)g0 * 64;
     const int i_lo = (int)((int64_t)items * v / P.NV), i_hi = (int)((int64_t)items * (v + 1) / P.NV);
     uint32_t* pp = reinterpret_cast<uint32_t*>(P.part) + (size_t)g0 * 64;
     const size_t ysz = a.y_dtype == SQ_F32 ? 4 : 2;
@@ -1494,8 +1557,16 @@ int stream_group_len(const sq_matrix* mats, int n) {
 // sums of that many rows do not fit LDS beside the slice, or the pieces' partial sums of that many rows the workspace
 // header): one launch per pass.  `sums` is the workspace header; every pass uses it from its start (a pass leaves it zeroed).
 int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dtype, int64_t ldx, void* y, int y_dtype,
-                        int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from) {
+                        int64_t ldy, int B, char* sums, hipStream_t s, const sq_producer* from, void* act, int64_t ld_act) {
     StreamArgs a;
+    a.act = (uint16_t*)act;
+    a.ld_act = ld_act;
+    if (act) {
+        // (what stream_fuses_silu() promises; checked again where the kernel depends on it)
+        if (cnt != 2 || mats[0].perms || mats[1].perms || mats[0].R != mats[1].R || stream_runs_of(mats[0]) != stream_runs_of(mats[1]) ||
+            mats[0].stream_groups != mats[1].stream_groups || y_dtype == SQ_F32 || stream_geom_of(mats[0]).NV > 16)
+            return fail(SQ_EINVAL, "sq_linear_small_silu: the two pieces must be a gate and an up projection of one shape");
+    }
     a.h_in = nullptr; a.h_out = nullptr; a.add = a.w = nullptr; a.x_out = nullptr; a.eps = 0.f;
     if (from) {
         a.h_in = from->h_in; a.h_out = from->h_out; a.add = (const uint16_t*)from->add;
@@ -1579,7 +1650,8 @@ int launch_stream_group(const sq_matrix* mats, int cnt, const void* x, int x_dty
     const size_t ysz = y_dtype == SQ_F32 ? 4 : 2;
     for (int b0 = 0; b0 < B; b0 += rows) {
         a.x = (const uint16_t*)((const char*)x + (size_t)b0 * ldx * 2);
-        a.y = (char*)y + (size_t)b0 * ldy * ysz;
+        a.y = y ? (char*)y + (size_t)b0 * ldy * ysz : nullptr;
+        a.act = act ? (uint16_t*)act + (size_t)b0 * ld_act : nullptr;
         a.nb = std::min(rows, B - b0);
         int rc;
         switch (rows) {

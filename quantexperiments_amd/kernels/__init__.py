@@ -531,3 +531,54 @@ def linear_small_from(pieces, y: torch.Tensor, x_out: torch.Tensor, *, h_in=None
                                           ldy, x_out.shape[0], None if ws is None else ws.data_ptr(),
                                           0 if ws is None else ws.numel(), _lib.stream_ptr(dev)))
     return y
+
+
+def linear_small_silu(pieces, x: torch.Tensor, out: torch.Tensor, *, x_out=None, h_in=None, add=None, w=None, eps: float = 0.0,
+                      h_out=None) -> torch.Tensor:
+    """out[b, r] = silu(Y[b, r]) * Y[b, R + r] for the stacked product Y of pieces = [gate, up] (sq_linear_small_silu):
+    the same bits as linear_small into a y of x's dtype followed by silu_mul(y[:, :R], y[:, R:], out).  One launch
+    where the library has a fused kernel for the stack (the tag-stream kernel writes the SiLU product where a row's
+    partial sums meet), else the two calls through a temporary y.  With h_in / w (and add, eps, h_out, x_out as in
+    linear_small_from) the launch also computes its own input, rmsnorm(h_in + add) * w, into x_out; x is then ignored.
+    The reference's EPI 2 epilogue of proto_runs.gemv (shapequant/kernels/proto_runs.py:269-287, 505-571)."""
+    if len(pieces) != 2 or pieces[0].R != pieces[1].R:
+        raise ValueError("linear_small_silu: pieces = [gate, up] of one shape")
+    R = pieces[0].R
+    norm = h_in is not None
+    xin = x_out if norm else x
+    if xin is None or xin.dim() != 2 or xin.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("linear_small_silu: x (or x_out with a producer) must be fp16 / bf16 [B, C]")
+    B, dt, dev = xin.shape[0], xin.dtype, xin.device
+    if out.dtype != dt or out.dim() != 2 or out.shape != (B, R) or out.stride(1) != 1:
+        raise ValueError("linear_small_silu: out must be [B, R] of x's dtype with unit column stride")
+    offs = (0, R)
+    mats = _lib.matrix_array([p.descriptor(o) for p, o in zip(pieces, offs)])
+    L = _lib.lib()
+    pr = None
+    if norm:
+        if B != 1 or not xin.is_contiguous() or h_in.dtype != torch.float32 or h_in.shape != xin.shape or w is None or w.dtype != dt:
+            raise ValueError("linear_small_silu: a fused producer takes one row: fp32 h_in, w of x_out's dtype, contiguous x_out")
+        pr = _lib.SqProducer()
+        pr.mode, pr.x_out, pr.eps, pr.h_in, pr.ld_h, pr.w = _lib.SQ_FROM_ADDNORM, xin.data_ptr(), float(eps), h_in.data_ptr(), _row_ld(h_in), w.data_ptr()
+        pr.h_out = None if h_out is None else h_out.data_ptr()
+        if add is not None:
+            pr.add, pr.ld_in = add.data_ptr(), _row_ld(add)
+    with torch.cuda.device(dev):
+        need = L.sq_workspace_bytes(mats, 2, B, 0)
+        ws = _Workspace.get(need, dev) if need else None
+        rc = L.sq_linear_small_silu(mats, 2, None if pr is None else ctypes.byref(pr), None if norm else xin.data_ptr(), _lib.DTYPES[dt],
+                                    0 if norm else _row_ld(xin), out.data_ptr(), _row_ld(out), B,
+                                    None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), _lib.stream_ptr(dev))
+    if rc == _lib.SQ_EUNSUPPORTED:
+        y = torch.empty(B, 2 * R, dtype=dt, device=dev)
+        if norm:
+            linear_small_from(pieces, y, xin, h_in=h_in, add=add, w=w, eps=eps, h_out=h_out)
+        else:
+            linear_small(pieces, xin, y)
+        if out.is_contiguous():
+            return silu_mul(y[:, :R], y[:, R:], out)
+        out.copy_(silu_mul(y[:, :R], y[:, R:], torch.empty(B, R, dtype=dt, device=dev)))
+        return out
+    _lib.check(rc)
+    return out
+

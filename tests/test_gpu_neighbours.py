@@ -248,6 +248,80 @@ def test_linear_small_from_equals_two_calls(case, dtype, B):
     assert float(np.abs(y_ref.cpu().numpy() - ref).max() / np.abs(ref).max()) < 1e-3
 
 
+SILU_OUT = [  # rows of the gate and of the up piece, C, tag bits, M, d, fused?
+    (260, 3584, 16, 1, 8, True), (130, 896, 16, 1, 8, True), (333, 2048, 14, 1, 8, True), (65, 18944, 16, 1, 8, True),
+    (300, 5120, 16, 16, 8, False), (96, 512, 12, 1, 4, False),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", SILU_OUT, ids=lambda c: f"{c[0]}x{c[1]}_b{c[2]}_M{c[3]}_d{c[4]}")
+def test_linear_small_silu_equals_two_calls(case, dtype):
+    """The gate | up product that writes SiLU(gate) * up itself against linear_small + silu_mul, bit for bit, at 1 to 8
+    activation rows (and 9: two calls inside the wrapper), with and without the add + norm producer in the same launch;
+    stacks the library has no fused kernel for (column orders, d = 4) fall back inside the wrapper and must agree too."""
+    from quantexperiments_amd import _lib
+    from quantexperiments_amd.kernels import addnorm, linear_small, linear_small_silu, silu_mul
+    R, C, bits, M, d, fused = case
+    ss, lins = _stack([(R, C), (R, C)], bits, M, seed=R + C, d=d)
+    mats = _lib.matrix_array([lins[0].descriptor(0), lins[1].descriptor(R)])
+    assert bool(_lib.lib().sq_linear_small_silu(mats, 2, None, None, _lib.DTYPES[dtype], 0, None, 0, 0, None, 0, None) == 0)
+    for B in (1, 2, 3, 8, 9):
+        x = rand_x(B, C, dtype, seed=B).cuda()
+        y = torch.empty(B, 2 * R, dtype=dtype, device="cuda")
+        linear_small(lins, x, y)
+        want = torch.empty(B, R, dtype=dtype, device="cuda")
+        silu_mul(y[:, :R], y[:, R:], want)
+        got = torch.full((B, R + 3), 5.0, dtype=dtype, device="cuda")
+        linear_small_silu(lins, x, got[:, :R])
+        assert torch.equal(got[:, :R], want), B
+        assert bool((got[:, R:] == 5.0).all())
+    # the launch also computing its input
+    g = torch.Generator().manual_seed(C)
+    h = (torch.randn(1, C, generator=g) * 2).cuda()
+    add = rand_x(1, C, dtype, seed=1).cuda()
+    w = (torch.rand(C, generator=g) + 0.5).to(dtype).cuda()
+    x_ref = torch.empty(1, C, dtype=dtype, device="cuda")
+    h_ref = torch.empty(1, C, device="cuda")
+    addnorm(h, add, w, 1e-6, x_ref, h_out=h_ref)
+    y = torch.empty(1, 2 * R, dtype=dtype, device="cuda")
+    linear_small(lins, x_ref, y)
+    want = torch.empty(1, R, dtype=dtype, device="cuda")
+    silu_mul(y[:, :R], y[:, R:], want)
+    x_out = torch.full((1, C), float("nan"), dtype=dtype, device="cuda")
+    h_out = torch.full((1, C), float("nan"), device="cuda")
+    got = torch.full((1, R), float("nan"), dtype=dtype, device="cuda")
+    linear_small_silu(lins, None, got, x_out=x_out, h_in=h, add=add, w=w, eps=1e-6, h_out=h_out)
+    assert torch.equal(got, want) and torch.equal(x_out, x_ref) and torch.equal(h_out, h_ref)
+    # the C entry point says whether it fused
+    ws = torch.zeros(_lib.lib().sq_workspace_bytes(mats, 2, 1, 0), dtype=torch.uint8, device="cuda")
+    x = rand_x(1, C, dtype, seed=77).cuda()
+    rc = _lib.lib().sq_linear_small_silu(mats, 2, None, x.data_ptr(), _lib.DTYPES[dtype], C, got.data_ptr(), R, 1, ws.data_ptr(), ws.numel(),
+                                         _lib.stream_ptr(x.device))
+    torch.cuda.synchronize()
+    assert rc == (0 if fused else _lib.SQ_EUNSUPPORTED)
+
+
+def test_full_size_gate_up_with_silu_on_the_way_out():
+    """The 7B gate | up launch (2 x 18944 x 3584) as bench.py builds it, writing SiLU(gate) * up: equal to the two calls,
+    and the workspace header is left zero."""
+    from quantexperiments_amd.kernels import linear_small, linear_small_silu, silu_mul, _Workspace
+    ss, lins = _stack([(18944, 3584), (18944, 3584)], 16, 1, seed=5)
+    R = 18944
+    for B, dtype in ((1, torch.bfloat16), (4, torch.float16)):
+        x = rand_x(B, 3584, dtype, seed=B).cuda()
+        y = torch.empty(B, 2 * R, dtype=dtype, device="cuda")
+        linear_small(lins, x, y)
+        want = torch.empty(B, R, dtype=dtype, device="cuda")
+        silu_mul(y[:, :R], y[:, R:], want)
+        got = torch.empty(B, R, dtype=dtype, device="cuda")
+        linear_small_silu(lins, x, got)
+        assert torch.equal(got, want), B
+        assert float(got.float().abs().max()) > 0
+    ws = _Workspace.get(0, torch.device("cuda", 0))
+    assert int(ws[:(32 << 20) - 4096].view(torch.int32).abs().max()) == 0
+
+
 def test_linear_small_from_rejects_bad_arguments():
     from quantexperiments_amd import _lib
     from quantexperiments_amd.kernels import linear_small_from
