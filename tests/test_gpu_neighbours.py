@@ -385,3 +385,53 @@ def test_decode_layer_with_fused_producers_under_graph():
         gr.replay()
         torch.cuda.synchronize()
         assert torch.equal(yd, eager[0]) and torch.equal(h1, eager[1]) and torch.equal(act, eager[2])
+
+
+def test_four_launch_decoder_layer_under_graph():
+    """o -> gate|up (add + norm in, SiLU * up out) -> down as three launches, captured in a HIP graph and replayed with
+    other work in between: every replay equals the eager chain of separate kernels; and the same for a d = 4 / 12-bit
+    layer, whose one-row products run on the row-segment kernel (the SiLU call then makes its two calls inside)."""
+    from quantexperiments_amd.kernels import addnorm, linear_small, linear_small_silu, silu_mul
+    for bits, d in ((16, 8), (12, 4)):
+        C, I = 512, 1024
+        _, o = _stack([(C, C)], bits, 1, seed=1, d=d)
+        _, gu = _stack([(I, C), (I, C)], bits, 1, seed=2, d=d)
+        _, dn = _stack([(C, I)], bits, 1, seed=3, d=d)
+        g = torch.Generator().manual_seed(4)
+        attn = rand_x(1, C, torch.bfloat16, seed=5).cuda()
+        h0 = torch.randn(1, C, generator=g).cuda()
+        w = (torch.rand(C, generator=g) + 0.5).bfloat16().cuda()
+        yo = torch.empty(1, C, dtype=torch.bfloat16, device="cuda")
+        ygu = torch.empty(1, 2 * I, dtype=torch.bfloat16, device="cuda")
+        yd = torch.empty(1, C, dtype=torch.bfloat16, device="cuda")
+        x1 = torch.empty(1, C, dtype=torch.bfloat16, device="cuda")
+        act = torch.empty(1, I, dtype=torch.bfloat16, device="cuda")
+        h1 = torch.empty_like(h0)
+        # the chain of separate kernels
+        linear_small(o, attn, yo)
+        addnorm(h0, yo, w, 1e-6, x1, h_out=h1)
+        linear_small(gu, x1, ygu)
+        silu_mul(ygu[:, :I], ygu[:, I:], act)
+        linear_small(dn, act, yd)
+        torch.cuda.synchronize()
+        want = (yd.clone(), h1.clone(), act.clone())
+
+        def step():
+            linear_small(o, attn, yo)
+            linear_small_silu(gu, None, act, x_out=x1, h_in=h0, add=yo, w=w, eps=1e-6, h_out=h1)
+            linear_small(dn, act, yd)
+
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(yd, want[0]) and torch.equal(h1, want[1]) and torch.equal(act, want[2]), bits
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            step()
+        for _ in range(3):
+            yd.zero_(); h1.zero_(); act.zero_()
+            torch.cuda.synchronize()
+            gr.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(yd, want[0]) and torch.equal(h1, want[1]) and torch.equal(act, want[2]), bits
+        del gr
+
