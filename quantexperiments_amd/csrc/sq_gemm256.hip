@@ -298,11 +298,21 @@ static Gemm256Plan gemm256_plan(int T, int R, int C, int cus) {
     if (cus < 8) return p;
     const int main = tiles / cus * cus, tail = tiles - main;          // cus is a multiple of 8 on this hardware
     if (tail == 0 || main % 8) return p;
-    int kt = cus / tail;
-    if (kt > 4) kt = 4;
-    while (kt > 1 && (C / G_BK) / kt < 16) --kt;
-    if (kt < 2) return p;
-    return Gemm256Plan{main, tail, kt};
+    // kt = the split with the least estimated time of the last round: rounds of workgroups x slabs per part, plus the
+    // partial tiles written and read back (256 KB each way per part; a slab of a round takes about 1.45 us, a part's
+    // reduction traffic about 0.12 us of the chip's memory bandwidth).  5120 x 17408 at 2048 rows (160 tiles): kt = 3
+    // makes 480 workgroups, 1.9 rounds of a third of the slabs, 391 -> 318 us by this estimate.
+    const int slabs = C / G_BK;
+    int best = 1;
+    double best_t = 1e30;
+    for (int kt = 1; kt <= 4; ++kt) {
+        if (kt > 1 && slabs / kt < 16) break;
+        const int wgs = tail * kt, rounds = (wgs + cus - 1) / cus;
+        const double t = rounds * (double)((slabs + kt - 1) / kt) * 1.45 + (kt > 1 ? wgs * 0.12 : 0.0);
+        if (t < best_t - 1e-9) { best_t = t; best = kt; }
+    }
+    if (best < 2) return p;
+    return Gemm256Plan{main, tail, best};
 }
 
 size_t gemm256_part_bytes(int T, int R, int C, int cus) {
