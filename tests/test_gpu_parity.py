@@ -1026,18 +1026,23 @@ def test_row_segment_kernel_of_the_12_bit_format(shapes):
     assert np.array_equal(y1.cpu().numpy()[0], w[:, col].astype(np.float32))
 
 
-@pytest.mark.parametrize("shapes,G", [([(300, 3584)], 4), ([(130, 5120), (64, 5120), (3, 5120)], 4), ([(40, 17408)], 4), ([(77, 1024)], 2),
-                                      ([(2100, 512)], 3)], ids=lambda c: str(c))
-def test_row_segment_kernel_with_several_codebooks(shapes, G):
-    """The same kernel on matrices whose rows name one of G codebooks of 4096 entries (the 27B recipe: G = 4, all four
-    in LDS), including rows so long that the activation rows no longer fit LDS beside the codebooks: 1 to 4 activation
-    rows against the C oracle (3 and 4 run on the matrix cores), row 1 of two equal to the single-row call."""
+@pytest.mark.parametrize("shapes,G,bits", [([(300, 3584)], 4, 12), ([(130, 5120), (64, 5120), (3, 5120)], 4, 12), ([(40, 17408)], 4, 12),
+                                           ([(77, 1024)], 2, 12), ([(2100, 512)], 3, 12),
+                                           ([(300, 5120)], 4, 10), ([(130, 5120), (64, 5120), (3, 5120)], 4, 10), ([(40, 17408)], 4, 10),
+                                           ([(77, 1024)], 1, 10), ([(9000, 256)], 2, 10),
+                                           ([(300, 5120)], 4, 8), ([(40, 17408), (24, 17408)], 4, 8), ([(130, 3584)], 1, 8),
+                                           ([(77, 512), (5, 512)], 3, 8), ([(4864, 896)], 1, 8)], ids=lambda c: str(c))
+def test_row_segment_kernel_with_several_codebooks(shapes, G, bits):
+    """The same kernel on 8-, 10- and 12-bit tags (segments of 128 or 256 tags) and on matrices whose rows name one of G
+    codebooks (the 27B recipe: d = 4, 256 / 1024 / 4096 entries, G = 4, all of them in LDS), including rows so long that
+    the activation rows no longer fit LDS beside the codebooks: 1 to 4 activation rows against the C oracle (3 and 4
+    run on the matrix cores), row 1 of two equal to the single-row call."""
     from quantexperiments_amd.kernels import linear_small, prepare_stack
     pieces, ws = [], []
     for k, (R, C) in enumerate(shapes):
-        sy = synth(R, C, 4, 12, G, 1, seed=300 + 7 * k + G)
+        sy = synth(R, C, 4, bits, G, 1, seed=300 + 7 * k + G + bits)
         pieces.append(to_device(sy, stream="later"))
-        ws.append(c_oracle.decode(sy.words, 12, C, 4, sy.K, sy.table, sy.row_scale, sy.row_book, None, None))
+        ws.append(c_oracle.decode(sy.words, bits, C, 4, sy.K, sy.table, sy.row_scale, sy.row_book, None, None))
     prepare_stack(pieces)
     w = np.concatenate(ws, axis=0)
     C, Rt = shapes[0][1], w.shape[0]
