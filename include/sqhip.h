@@ -153,7 +153,7 @@ int sq_noalloc_reset(void* stream);
 void sq_stream_spin_limit(int32_t polls);
 
 /* Load-time regrouping of a matrix' tags for codebooks that do not fit LDS (d = 8, K = 8192..65,536, one
- * codebook): the decode-time product (up to 4 activation rows, up to 8 of rows with at most 1024 chunks, any
+ * codebook; several: sq_stream_build_books below): the decode-time product (up to 4 activation rows, up to 8 of rows with at most 1024 chunks, any
  * B <= 32 with column orders) then gathers codewords from a 64 KB LDS slice instead of from L2.
  * HOST pointers: `tags_host` is the file's tag tensor in host memory, `row_mask_host` the file's row_mask
  * (NULL when the matrix has one column order), `out_host` receives sq_stream_bytes() bytes that the caller
@@ -206,6 +206,27 @@ int sq_stream_build_balanced(const int32_t* tags_host, int32_t R, int32_t W, int
  * own, and the relabelled table serves every other entry point too. */
 int sq_codebook_balance(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits,
                         uint16_t* remap_out);
+
+/* The three calls above for a matrix with G codebooks (G a power of two, `row_book_host` [R] names each row's; the
+ * file's row_book tensor, reference shapequant/packed.py:30-40).  The G codebooks lie behind each other in sq_matrix.table,
+ * so a row's tags are labels of that one long codebook, book * 2^bits + tag, and the stream is cut into slices of 4096
+ * of those labels: d = 8, more than 4096 and at most 64 * 4096 codewords over all codebooks (4 MiB).  A workgroup then
+ * finds entries only in the rows of its slice's codebook, so the work is even when the codebooks have about the same
+ * number of rows.  The buffer is handed to the library exactly like a single-codebook stream (sq_matrix.stream,
+ * stream_runs, stream_groups, with G and row_book set as usual); each run becomes G * 2^bits / 4096 * ceil(C / 8 / 4064)
+ * workgroups.  sq_codebook_balance_books writes remap_out[book * 2^bits + k] = the new label, within its codebook, of
+ * the file's codeword k of that codebook (every codebook is balanced over its own slices; one of at most 4096 codewords
+ * keeps its labels).  A stream with a relabelled codebook of its own (sq_stream_build_balanced) is for one codebook
+ * only.  G == 1, and the d = 4 formats whose buffer is the tile-major copy of the tags (which does not depend on the
+ * codebooks), forward to the calls above.  The reference groups its tiles by (codebook, column order) at load time
+ * for the same purpose (shapequant/kernels/proto_runs.py:352-366 book_tiles). */
+size_t sq_stream_bytes_books(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t G,
+                             const uint8_t* row_book_host, const uint8_t* row_mask_host, int32_t runs);
+int sq_stream_build_books(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t G,
+                          const uint8_t* row_book_host, const uint8_t* row_mask_host, int32_t runs, void* out_host,
+                          size_t out_bytes, int32_t* runs_out, int32_t* groups_out);
+int sq_codebook_balance_books(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t G,
+                              const uint8_t* row_book_host, uint16_t* remap_out);
 
 /* ---- The packed file's block-32 side formats (reference shapequant/packed.py:30-40): the 8-bit output head
  * `aux.lm_head` (q int8 [V, C], scale fp16 [V, C/32], w = q * scale of the row's 32-column block) and the 4-bit

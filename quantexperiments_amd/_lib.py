@@ -89,6 +89,12 @@ def lib() -> ctypes.CDLL:
         L.sq_stream_build_balanced.restype = ctypes.c_int
         L.sq_codebook_balance.argtypes = [vp, i32, i32, i32, i32, i32, vp]
         L.sq_codebook_balance.restype = ctypes.c_int
+        L.sq_stream_bytes_books.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp, i32]
+        L.sq_stream_bytes_books.restype = sz
+        L.sq_stream_build_books.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp, i32, vp, sz, ip, ip]
+        L.sq_stream_build_books.restype = ctypes.c_int
+        L.sq_codebook_balance_books.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
+        L.sq_codebook_balance_books.restype = ctypes.c_int
         L.sq_q8_linear.argtypes = [vp, vp, i32, i32, vp, ctypes.c_int, i64, vp, ctypes.c_int, i64, i32, vp, sz, vp]
         L.sq_q8_workspace_bytes.argtypes = [i32, i32, i32]
         L.sq_q8_workspace_bytes.restype = sz
@@ -111,7 +117,8 @@ EXPORTS = ("sq_version", "sq_last_error", "sq_dequant", "sq_linear_small", "sq_l
            "sq_workspace_bytes", "sq_stream_bytes", "sq_stream_build", "sq_stream_bytes_balanced", "sq_stream_build_balanced", "sq_q8_linear", "sq_q8_workspace_bytes",
            "sq_q8_dequant", "sq_q4_embed", "sq_addnorm", "sq_silu_mul",
            "sq_linear_small_from", "sq_linear_small_silu", "sq_gemm_dense_ws", "sq_gemm_dense_workspace_bytes", "sq_linear_small_noalloc",
-           "sq_workspace_status", "sq_workspace_reset", "sq_noalloc_reset", "sq_stream_spin_limit", "sq_codebook_balance")
+           "sq_workspace_status", "sq_workspace_reset", "sq_noalloc_reset", "sq_stream_spin_limit", "sq_codebook_balance",
+           "sq_stream_bytes_books", "sq_stream_build_books", "sq_codebook_balance_books")
 
 
 def check(rc: int) -> None:

@@ -76,7 +76,7 @@ using namespace sq;
 
 extern "C" {
 
-int sq_version(void) { return 108; }
+int sq_version(void) { return 109; }
 
 const char* sq_last_error(void) { return g_err; }
 
@@ -354,6 +354,51 @@ int sq_codebook_balance(const int32_t* tags_host, int32_t R, int32_t W, int32_t 
     if (d <= 0 || !stream_format_ok(R, C, d, bits)) return fail(SQ_EUNSUPPORTED, "sq_codebook_balance: d %d bits %d R %d not covered", d, bits, R);
     if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_codebook_balance: W %d too small", W);
     stream_balance_host((const uint32_t*)tags_host, R, W, C, d, bits, remap_out);
+    return SQ_OK;
+}
+
+// ---- several codebooks per matrix: the labels of the tag stream are book << bits | tag (sq_stream.h)
+static int books_check(const char* who, int32_t R, int32_t G, const uint8_t* row_book_host) {
+    if (G < 1 || G > 256 || (G & (G - 1)) != 0) return fail(SQ_EUNSUPPORTED, "%s: %d codebooks (a power of two is needed)", who, G);
+    if (G > 1 && !row_book_host) return fail(SQ_EINVAL, "%s: G %d needs row_book", who, G);
+    if (G > 1)
+        for (int32_t r = 0; r < R; ++r)
+            if (row_book_host[r] >= G) return fail(SQ_EINVAL, "%s: row %d names codebook %d of %d", who, r, (int)row_book_host[r], G);
+    return SQ_OK;
+}
+
+size_t sq_stream_bytes_books(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t G,
+                             const uint8_t* row_book_host, const uint8_t* row_mask_host, int32_t runs) {
+    // (one codebook, and the formats whose buffer is the tile-major copy of the tags, which does not depend on the codebooks)
+    if (G <= 1 || (d > 0 && !stream_format_ok(R, C, d, bits, G) && !row_mask_host && tiled_format_ok(R, W, C, d, bits)))
+        return sq_stream_bytes_balanced(tags_host, R, W, C, d, bits, row_mask_host, runs, nullptr);
+    if (!tags_host || d <= 0 || R <= 0 || (int64_t)W * 32 < (int64_t)(C / d) * bits) return 0;
+    if (!stream_format_ok(R, C, d, bits, G) || books_check("sq_stream_bytes_books", R, G, row_book_host) != SQ_OK) return 0;
+    return stream_bytes_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs, nullptr, G, row_book_host);
+}
+
+int sq_stream_build_books(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t G,
+                          const uint8_t* row_book_host, const uint8_t* row_mask_host, int32_t runs, void* out_host,
+                          size_t out_bytes, int32_t* runs_out, int32_t* groups_out) {
+    if (G <= 1 || (d > 0 && !stream_format_ok(R, C, d, bits, G) && !row_mask_host && tiled_format_ok(R, W, C, d, bits)))
+        return sq_stream_build_balanced(tags_host, R, W, C, d, bits, row_mask_host, runs, nullptr, out_host, out_bytes, runs_out, groups_out);
+    if (!tags_host || !out_host || !runs_out || !groups_out) return fail(SQ_EINVAL, "sq_stream_build_books: null pointer");
+    if (d <= 0 || !stream_format_ok(R, C, d, bits, G))
+        return fail(SQ_EUNSUPPORTED, "sq_stream_build_books: d %d bits %d G %d R %d not covered", d, bits, G, R);
+    if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_stream_build_books: W %d too small", W);
+    if (int rc = books_check("sq_stream_build_books", R, G, row_book_host)) return rc;
+    return stream_build_host((const uint32_t*)tags_host, R, W, C, d, bits, row_mask_host, runs, (unsigned char*)out_host,
+                             out_bytes, runs_out, groups_out, nullptr, G, row_book_host);
+}
+
+int sq_codebook_balance_books(const int32_t* tags_host, int32_t R, int32_t W, int32_t C, int32_t d, int32_t bits, int32_t G,
+                              const uint8_t* row_book_host, uint16_t* remap_out) {
+    if (!tags_host || !remap_out) return fail(SQ_EINVAL, "sq_codebook_balance_books: null pointer");
+    if (d <= 0 || !stream_format_ok(R, C, d, bits, G))
+        return fail(SQ_EUNSUPPORTED, "sq_codebook_balance_books: d %d bits %d G %d R %d not covered", d, bits, G, R);
+    if ((int64_t)W * 32 < (int64_t)(C / d) * bits) return fail(SQ_EINVAL, "sq_codebook_balance_books: W %d too small", W);
+    if (int rc = books_check("sq_codebook_balance_books", R, G, row_book_host)) return rc;
+    stream_balance_host((const uint32_t*)tags_host, R, W, C, d, bits, remap_out, G, G > 1 ? row_book_host : nullptr);
     return SQ_OK;
 }
 

@@ -285,7 +285,7 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
 bool small_fuses_producer(const sq_matrix* mats, int n, int B) {
     if (B != 1 || n < 1 || n > GEMV_MAX_PIECES_STREAM) return false;
     for (int i = 0; i < n; ++i)
-        if (mats[i].R <= 0 || !stream_rows(mats[i], 1) || mats[i].bits != mats[0].bits || mats[i].perms) return false;
+        if (mats[i].R <= 0 || !stream_rows(mats[i], 1) || mats[i].bits != mats[0].bits || mats[i].G != mats[0].G || mats[i].perms) return false;
     return true;
 }
 
@@ -294,7 +294,7 @@ bool small_fuses_producer(const sq_matrix* mats, int n, int B) {
 bool small_fuses_silu(const sq_matrix* mats, int n, int B) {
     if (n != 2 || B < 1 || B > 8) return false;
     const sq_matrix &g = mats[0], &u = mats[1];
-    if (g.R <= 0 || g.R != u.R || g.C != u.C || g.bits != u.bits || g.perms || u.perms) return false;
+    if (g.R <= 0 || g.R != u.R || g.C != u.C || g.bits != u.bits || g.G != u.G || g.perms || u.perms) return false;
     // (the same cut into runs; the other fields of stream_runs describe each piece's own buffer and may differ)
     if (!stream_rows(g, B) || !stream_rows(u, B) || stream_runs_of(g) != stream_runs_of(u) || stream_run_max_of(g) != stream_run_max_of(u) ||
         g.stream_groups != u.stream_groups)
@@ -328,7 +328,7 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
         if (stream_rows(m0, B) && (x_ok || from)) {
             if (!sums) return fail(SQ_EWORKSPACE, "sq_linear_small: these pieces need a workspace (its header holds their partial sums)");
             int j = i + 1;
-            while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_rows(mats[j], B) && mats[j].bits == m0.bits && mats[j].R > 0) ++j;
+            while (j < n && j - i < GEMV_MAX_PIECES_STREAM && stream_rows(mats[j], B) && mats[j].bits == m0.bits && mats[j].G == m0.G && mats[j].R > 0) ++j;
             j = i + stream_group_len(mats + i, j - i);
             int rc = launch_stream_group(mats + i, j - i, x, x_dtype, ldx, y, y_dtype, ldy, B, (char*)sums, s, from);
             if (rc) return rc;

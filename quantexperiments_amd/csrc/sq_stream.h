@@ -59,17 +59,31 @@ struct StreamGeom {
     uint64_t total_steps;                    // filled by the builder only
 };
 
-StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanced = false, int fs = 0);
-bool stream_format_ok(int R, int C, int d, int bits);
-// table: the matrix' codebook (fp16 [2^bits, d], host memory) or NULL.  With it the codewords are relabelled so that
-// every slice of 4096 carries the same share of the tags whatever their distribution, and the buffer holds the
-// relabelled copy of the codebook that the kernels then read their slices from.
+// Several codebooks per matrix (G, a power of two; row_book[r] names the row's): the G codebooks lie behind each other in
+// the table, so a row's tags become labels of that one long codebook, book << bits | tag, and everything below (slices,
+// buckets, the kernels) sees a matrix with one codebook of G << bits codewords: `label_bits` = bits + log2 G.  The
+// workgroups of a slice then find entries only in the rows of that slice's codebook.
+constexpr int STREAM_SLICES_MAX = 64;        // most slices of one matrix (4 MiB of codebooks): the workgroups of a run wait for
+                                             // each other and must be resident together
+inline int stream_label_bits(int bits, int G) {
+    int lb = bits;
+    while (G > 1) { G >>= 1; ++lb; }
+    return lb;
+}
+StreamGeom stream_geom(int C, int d, int label_bits, int groups, int runs, bool balanced = false, int fs = 0);
+bool stream_format_ok(int R, int C, int d, int bits, int G = 1);
+// table: the matrix' codebook (fp16 [2^bits, d], host memory; one codebook only) or NULL.  With it the codewords are
+// relabelled so that every slice of 4096 carries the same share of the tags whatever their distribution, and the buffer
+// holds the relabelled copy of the codebook that the kernels then read their slices from.
 size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                         const uint16_t* table = nullptr);
+                         const uint16_t* table = nullptr, int G = 1, const uint8_t* row_book = nullptr);
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table = nullptr);
-// remap_out[file label] = new label (2^bits entries): the relabelling a balanced stream applies, by itself
-void stream_balance_host(const uint32_t* tags, int R, int W, int C, int d, int bits, uint16_t* remap_out);
+                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table = nullptr,
+                      int G = 1, const uint8_t* row_book = nullptr);
+// remap_out[book << bits | file label] = new label within the book (G << bits entries): the relabelling a balanced stream
+// applies, by itself; every codebook is balanced over its own slices (one of at most 4096 codewords keeps its labels)
+void stream_balance_host(const uint32_t* tags, int R, int W, int C, int d, int bits, uint16_t* remap_out, int G = 1,
+                         const uint8_t* row_book = nullptr);
 // sq_matrix.stream_runs is sq_stream_build's runs_out: the run count in the low 16 bits, the groups of the longest run
 // in the next 8, the most column orders in one run (less one) in bits 24-26, the steps per unit of the first-steps region
 // (less one) in bits 27-28, bit 30 = the stream carries a relabelled codebook
@@ -80,7 +94,7 @@ inline int stream_run_max_of(const sq_matrix& m) { return (int)(((uint32_t)m.str
 inline int stream_run_orders_of(const sq_matrix& m) { return (int)(((uint32_t)m.stream_runs >> 24) & 7u) + 1; }
 inline bool stream_balanced_of(const sq_matrix& m) { return (m.stream_runs & STREAM_BALANCED) != 0; }
 inline StreamGeom stream_geom_of(const sq_matrix& m) {
-    return stream_geom(m.C, m.d, m.bits, m.stream_groups, stream_runs_of(m), stream_balanced_of(m), stream_fs_of(m));
+    return stream_geom(m.C, m.d, stream_label_bits(m.bits, m.G), m.stream_groups, stream_runs_of(m), stream_balanced_of(m), stream_fs_of(m));
 }
 bool stream_shape(const sq_matrix& m);
 size_t stream_part_bytes(const sq_matrix& m, int rows);   // partial sums of one pass of `rows` activation rows

@@ -1,4 +1,5 @@
-// Bucketed tag stream: the batch-1 product for codebooks too large for LDS (K = 8192 .. 65,536 at d = 8).
+// Bucketed tag stream: the batch-1 product for codebooks too large for LDS (K = 8192 .. 65,536 at d = 8; several
+// codebooks per matrix count as one long codebook, see sq_stream.h).
 //
 // A 65,536 x 8 fp16 codebook is 1 MiB; gathering 16-byte codewords from it through L2 is what bounds the
 // row-major kernels.  Here the tags of a matrix are regrouped once, at load time, by the part of the
@@ -79,8 +80,11 @@ StreamGeom stream_geom(int C, int d, int bits, int groups, int runs, bool balanc
 }
 
 // (R + 64 * 256 bounds the places: every column order can leave one group short)
-bool stream_format_ok(int R, int C, int d, int bits) {
-    return d == 8 && bits > STREAM_SLICE_BITS && bits <= 16 && C % d == 0 && R > 0 && R + 64 * 256 < (int)STREAM_NO_ROW;
+bool stream_format_ok(int R, int C, int d, int bits, int G) {
+    if (G < 1 || (G & (G - 1)) != 0 || bits < 1 || bits > 16) return false;
+    const int lb = stream_label_bits(bits, G);
+    return d == 8 && lb > STREAM_SLICE_BITS && (1 << (lb - STREAM_SLICE_BITS)) <= (G > 1 ? STREAM_SLICES_MAX : 16) && C % d == 0 &&
+           R > 0 && R + 64 * 256 < (int)STREAM_NO_ROW;
 }
 
 static inline uint32_t host_tag(const uint32_t* row, int W, int bits, int j) {
@@ -130,31 +134,46 @@ struct StreamPlan {
 // whichever slice of 4096 carries the fewest tags so far and still has room, so every slice ends up with the same
 // share of the tags (a slice is one workgroup's work) whatever the distribution of the tags is, and a slice's popular
 // codewords get consecutive places, i.e. different LDS bank groups.
-static void balance_codewords(const uint32_t* tags, int R, int W, int U, int bits, std::vector<uint16_t>& remap) {
+// With several codebooks (row_book names a row's) every codebook is relabelled by itself, over its own slices:
+// remap[book << bits | label] is the new label within the book; a codebook of at most one slice keeps its labels.
+static void balance_codewords(const uint32_t* tags, int R, int W, int U, int bits, std::vector<uint16_t>& remap, int G = 1,
+                              const uint8_t* row_book = nullptr) {
     const int K = 1 << bits, NS = K >> STREAM_SLICE_BITS, SL = 1 << STREAM_SLICE_BITS;
-    std::vector<uint64_t> count(K, 0);
+    remap.assign((size_t)G * K, 0);
+    if (NS < 2) {
+        for (size_t k = 0; k < remap.size(); ++k) remap[k] = (uint16_t)(k & (size_t)(K - 1));
+        return;
+    }
+    std::vector<uint64_t> count((size_t)G * K, 0);
     for (int r = 0; r < R; ++r) {
         const uint32_t* row = tags + (size_t)r * W;
-        for (int j = 0; j < U; ++j) ++count[host_tag(row, W, bits, j)];
+        uint64_t* cb = count.data() + (size_t)(row_book ? row_book[r] & (G - 1) : 0) * K;
+        for (int j = 0; j < U; ++j) ++cb[host_tag(row, W, bits, j)];
     }
     std::vector<uint32_t> ids(K);
-    for (int k = 0; k < K; ++k) ids[k] = (uint32_t)k;
-    std::stable_sort(ids.begin(), ids.end(), [&count](uint32_t a, uint32_t b) { return count[a] > count[b]; });
-    std::vector<uint64_t> load(NS, 0);
-    std::vector<int> fill(NS, 0);
-    remap.assign(K, 0);
-    for (int k = 0; k < K; ++k) {
-        int best = -1;
-        for (int sl = 0; sl < NS; ++sl)
-            if (fill[sl] < SL && (best < 0 || load[sl] < load[best])) best = sl;
-        remap[ids[k]] = (uint16_t)(best * SL + fill[best]);
-        ++fill[best];
-        load[best] += count[ids[k]];
+    std::vector<uint64_t> load(NS);
+    std::vector<int> fill(NS);
+    for (int b = 0; b < G; ++b) {
+        const uint64_t* cb = count.data() + (size_t)b * K;
+        for (int k = 0; k < K; ++k) ids[k] = (uint32_t)k;
+        std::stable_sort(ids.begin(), ids.end(), [cb](uint32_t x, uint32_t y) { return cb[x] > cb[y]; });
+        std::fill(load.begin(), load.end(), 0);
+        std::fill(fill.begin(), fill.end(), 0);
+        for (int k = 0; k < K; ++k) {
+            int best = -1;
+            for (int sl = 0; sl < NS; ++sl)
+                if (fill[sl] < SL && (best < 0 || load[sl] < load[best])) best = sl;
+            remap[(size_t)b * K + ids[k]] = (uint16_t)(best * SL + fill[best]);
+            ++fill[best];
+            load[best] += cb[ids[k]];
+        }
     }
 }
 
+// (G > 1: the labels a row's tags become are book << bits | tag, see sq_stream.h; `balanced` is for one codebook only)
 static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                        StreamPlan& P, bool balanced) {
+                        StreamPlan& P, bool balanced, int G, const uint8_t* row_book) {
+    const int lbits = stream_label_bits(bits, G);
     P.remap.clear();
     if (balanced) balance_codewords(tags, R, W, C / d, bits, P.remap);
     const uint16_t* remap = balanced ? P.remap.data() : nullptr;
@@ -163,7 +182,7 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     for (int r = 0; r < R; ++r) order[r] = (uint32_t)r;
     if (row_mask)
         std::stable_sort(order.begin(), order.end(), [row_mask](uint32_t a, uint32_t b) { return row_mask[a] < row_mask[b]; });
-    StreamGeom g0 = stream_geom(C, d, bits, 0, 0);
+    StreamGeom g0 = stream_geom(C, d, lbits, 0, 0);
     if (runs <= 0) runs = (STREAM_DEFAULT_WGS + g0.NV / 2) / g0.NV;
     if (runs < 1) runs = 1;
     // Groups per column order.  A run takes the groups of one order, GR at a time, or, when orders are small, the whole
@@ -239,7 +258,7 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
         const int a = first[i], b = first[i + 1];
         for (int k = 0; k < ngm[i] * 64; ++k) P.base.push_back(a + k < b ? order[a + k] : STREAM_NO_ROW);
     }
-    P.g = stream_geom(C, d, bits, (int)(P.base.size() / 64), (int)P.runs.size(), balanced);
+    P.g = stream_geom(C, d, lbits, (int)(P.base.size() / 64), (int)P.runs.size(), balanced);
     const StreamGeom& g = P.g;
     P.cnt.assign((size_t)g.NV * R, 0);
     P.pos.assign((size_t)g.NV * R, 0);
@@ -247,9 +266,11 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     parallel_rows(R, [&](int a, int b) {
         for (int r = a; r < b; ++r) {
             const uint32_t* row = tags + (size_t)r * W;
+            const uint32_t book = row_book ? (uint32_t)(row_book[r] & (G - 1)) << bits : 0u;
             for (int j = 0; j < g.U; ++j) {
                 uint32_t t = host_tag(row, W, bits, j);
                 if (remap) t = remap[t];
+                t |= book;
                 const int v = (j / g.PC) * g.NS + (int)(t >> STREAM_SLICE_BITS);
                 ++P.cnt[(size_t)v * R + r];
             }
@@ -314,16 +335,17 @@ static void plan_stream(const uint32_t* tags, int R, int W, int C, int d, int bi
     P.g.total_steps = at;
 }
 
-void stream_balance_host(const uint32_t* tags, int R, int W, int C, int d, int bits, uint16_t* remap_out) {
+void stream_balance_host(const uint32_t* tags, int R, int W, int C, int d, int bits, uint16_t* remap_out, int G,
+                         const uint8_t* row_book) {
     std::vector<uint16_t> remap;
-    balance_codewords(tags, R, W, C / d, bits, remap);
+    balance_codewords(tags, R, W, C / d, bits, remap, G, row_book);
     memcpy(remap_out, remap.data(), remap.size() * sizeof(uint16_t));
 }
 
 size_t stream_bytes_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                         const uint16_t* table) {
+                         const uint16_t* table, int G, const uint8_t* row_book) {
     StreamPlan P;
-    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr);
+    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr, G, row_book);
     return P.g.off_steps + (size_t)P.g.total_steps * P.g.fmt.step_bytes;
 }
 
@@ -499,9 +521,10 @@ static void encode_step(const uint32_t* e, const StreamFmt& f, unsigned char* ou
 }
 
 int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits, const uint8_t* row_mask, int runs,
-                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table) {
+                      unsigned char* out, size_t bytes, int* runs_out, int* groups_out, const uint16_t* table, int G,
+                      const uint8_t* row_book) {
     StreamPlan P;
-    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr);
+    plan_stream(tags, R, W, C, d, bits, row_mask, runs, P, table != nullptr, G, row_book);
     const uint16_t* remap = table ? P.remap.data() : nullptr;
     const StreamGeom& g = P.g;
     const StreamFmt f = g.fmt;
@@ -534,6 +557,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
         std::vector<uint32_t> q(g.NV), last(g.NV);
         for (int r = a; r < b; ++r) {
             const uint32_t* row = tags + (size_t)r * W;
+            const uint32_t book = row_book ? (uint32_t)(row_book[r] & (G - 1)) << bits : 0u;
             std::fill(q.begin(), q.end(), 0u);
             std::fill(last.begin(), last.end(), 0u);
             for (int v = 0; v < g.NV; ++v) {
@@ -543,6 +567,7 @@ int stream_build_host(const uint32_t* tags, int R, int W, int C, int d, int bits
             for (int j = 0; j < g.U; ++j) {
                 uint32_t t = host_tag(row, W, bits, j);
                 if (remap) t = remap[t];
+                t |= book;
                 const int kp = j / g.PC, v = kp * g.NS + (int)(t >> STREAM_SLICE_BITS);
                 const uint32_t k = P.pos[(size_t)v * R + r], n = q[v]++;
                 const uint32_t e = (t & ((1u << STREAM_SLICE_BITS) - 1u)) | ((uint32_t)(j - kp * g.PC) << STREAM_SLICE_BITS);
@@ -1482,7 +1507,8 @@ int launch_stream_dequant(const sq_matrix& m, void* out, int out_dtype, int64_t 
 }
 
 bool stream_shape(const sq_matrix& m) {
-    return m.stream && stream_runs_of(m) > 0 && m.stream_groups > 0 && m.G == 1 && stream_format_ok(m.R, m.C, m.d, m.bits) &&
+    return m.stream && stream_runs_of(m) > 0 && m.stream_groups > 0 && stream_format_ok(m.R, m.C, m.d, m.bits, m.G) &&
+           !(m.G > 1 && stream_balanced_of(m)) &&
            (m.M <= 1 || m.perms) && (((uintptr_t)m.table | (uintptr_t)m.stream | (uintptr_t)m.perms) & 15) == 0 &&
            stream_part_bytes(m, 1) <= SQ_WS_SUMS;
 }

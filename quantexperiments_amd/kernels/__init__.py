@@ -120,7 +120,10 @@ class PackedLinear(torch.nn.Module):
         self.relabelled = False
         # stream: True builds now, cut for a launch of this matrix alone; "later" leaves the build to prepare_stack
         # (pieces that will be launched together are cut for the joint launch, and built once); False: never
-        self.wants_stream = bool(stream) and self.G == 1 and table.numel() * 2 > 128 * 1024 and d == 8 and 12 < self.bits <= 16
+        # (several codebooks: they lie behind each other in the table and the stream's labels are book * K + tag, so what
+        # counts is the table as a whole: more than one slice of 4096 codewords, at most 64)
+        self.wants_stream = (bool(stream) and table.numel() * 2 > 128 * 1024 and d == 8 and self.bits <= 16 and
+                             self.G & (self.G - 1) == 0 and (self.G == 1 or self.G * K <= 64 * 4096))
         if self.wants_stream:
             if stream != "later":
                 self.build_stream(0)
@@ -138,7 +141,8 @@ class PackedLinear(torch.nn.Module):
         if self.wants_stream and self.balance and not self.relabelled:
             self._relabel()
         self.stream, self.stream_runs, self.stream_groups = build_stream(
-            self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs)
+            self.words, self.C, self.d, self.bits, self.row_mask if self.has_mask else None, runs,
+            row_book=None if self.row_book is None else (self.row_book, self.G))
         self.stream_asked = runs
         if self.stream is None:
             self.wants_stream = False
@@ -149,24 +153,31 @@ class PackedLinear(torch.nn.Module):
         relabelled pair: the tags are rewritten through the map and row k of the table moves to row map[k].  Every
         weight decodes to the same bits as before, the tag-stream kernel's workgroups (one per slice) get equal work
         whatever the distribution of the tags, and the matrix keeps ONE codebook (a stream that carries its own
-        relabelled copy, sq_stream_build_balanced, costs another 1.1 MiB per matrix)."""
+        relabelled copy, sq_stream_build_balanced, costs another 1.1 MiB per matrix).  With several codebooks each is
+        relabelled by itself, over its own slices (sq_codebook_balance_books)."""
         from ..packed import pack_bits, unpack_bits
         host = self.words.detach().to("cpu", torch.int32).contiguous()
-        remap = torch.empty(1 << self.bits, dtype=torch.int16)
-        rc = _lib.lib().sq_codebook_balance(host.data_ptr(), self.R, self.W, self.C, self.d, self.bits, remap.data_ptr())
+        remap = torch.empty(self.G << self.bits, dtype=torch.int16)
+        book = None if self.row_book is None else self.row_book.detach().to("cpu", torch.uint8).contiguous()
+        rc = _lib.lib().sq_codebook_balance_books(host.data_ptr(), self.R, self.W, self.C, self.d, self.bits, self.G,
+                                                  None if book is None else book.data_ptr(), remap.data_ptr())
         if rc == _lib.SQ_EUNSUPPORTED:                  # a shape the slice stream does not cover: nothing to balance
             self.relabelled = True
             return
         _lib.check(rc)
-        new_of = (remap.to(torch.int32) & 0xFFFF).to(torch.int64)            # file label -> new label
+        new_of = (remap.to(torch.int32) & 0xFFFF).to(torch.int64)            # book * K + file label -> new label in the book
         dev = self.words.device
-        if self.bits == 16:
+        if self.bits == 16 and self.G == 1:
             old = (self.words.view(torch.int16).to(torch.int32) & 0xFFFF).to(torch.int64)
             self.words = remap.to(dev)[old].view(torch.int32).reshape(self.R, self.W).contiguous()
         else:
-            self.words = pack_bits(new_of[unpack_bits(host, self.bits, self.nch)], self.bits).to(dev)
+            old = unpack_bits(host, self.bits, self.nch).to(torch.int64)
+            if book is not None:
+                old = old + (book.to(torch.int64) << self.bits)[:, None]
+            self.words = pack_bits(new_of[old], self.bits).to(dev)
         table = torch.empty_like(self.table)
-        table[new_of.to(dev)] = self.table
+        at = new_of + ((torch.arange(self.G << self.bits) >> self.bits) << self.bits)      # row of the table a codeword moves to
+        table[at.to(dev)] = self.table
         self.table = table
         self.relabelled = True
 
@@ -249,13 +260,15 @@ class PackedLinear(torch.nn.Module):
             self.words = None
 
 
-def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, runs: int = 0, table=None):
+def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, runs: int = 0, table=None, row_book=None):
     """(stream, runs, groups): the bucketed tag stream of one matrix (sq_stream_build) as a uint8 tensor on
     words' device with the library's runs_out (opaque: run count, longest run, flags) and group count, to be handed
     back in sq_matrix, or (None, 0, 0) when the format is not covered.  The regrouping itself is the library's host
     routine; the tags make one trip to host memory at load time.  With `table` (the matrix' fp16 codebook) the library
     relabels the codewords so that every slice of the codebook carries the same share of the tags, whatever their
-    distribution, and the stream holds the relabelled codebook (sq_stream_build_balanced)."""
+    distribution, and the stream holds the relabelled codebook (sq_stream_build_balanced).  `row_book` (uint8 [R], values
+    below a power of two G = its maximum rounded up; or a (row_book, G) pair): the matrix has G codebooks behind each
+    other in its table (sq_stream_build_books; not together with `table`)."""
     L = _lib.lib()
     host = words.detach().to("cpu", torch.int32).contiguous()
     mask = None if row_mask is None else row_mask.detach().to("cpu", torch.uint8).contiguous()
@@ -265,11 +278,25 @@ def build_stream(words: torch.Tensor, C: int, d: int, bits: int, row_mask=None, 
         raise ValueError(f"codebook of {tab.numel()} values for {bits}-bit tags of {d}")
     tp = None if tab is None else tab.data_ptr()
     R, W = host.shape
+    r, g = ctypes.c_int32(0), ctypes.c_int32(0)
+    if row_book is not None:
+        if tab is not None:
+            raise ValueError("a stream with a codebook of its own is for matrices with one codebook")
+        book, G = row_book if isinstance(row_book, tuple) else (row_book, None)
+        book = book.detach().to("cpu", torch.uint8).contiguous()
+        if G is None:
+            G = 1 << int(book.max()).bit_length() if R else 1
+        n = L.sq_stream_bytes_books(host.data_ptr(), R, W, C, d, bits, G, book.data_ptr(), mp, runs)
+        if n == 0:
+            return None, 0, 0
+        out = torch.empty(n, dtype=torch.uint8)
+        _lib.check(L.sq_stream_build_books(host.data_ptr(), R, W, C, d, bits, G, book.data_ptr(), mp, runs, out.data_ptr(), n,
+                                           ctypes.byref(r), ctypes.byref(g)))
+        return out.to(words.device), r.value, g.value
     n = L.sq_stream_bytes_balanced(host.data_ptr(), R, W, C, d, bits, mp, runs, tp)
     if n == 0:
         return None, 0, 0
     out = torch.empty(n, dtype=torch.uint8)
-    r, g = ctypes.c_int32(0), ctypes.c_int32(0)
     _lib.check(L.sq_stream_build_balanced(host.data_ptr(), R, W, C, d, bits, mp, runs, tp, out.data_ptr(), n, ctypes.byref(r),
                                           ctypes.byref(g)))
     return out.to(words.device), r.value, g.value
@@ -294,7 +321,7 @@ def prepare_stack(pieces, workgroups: int | None = None) -> None:
     # still fits the device in one round of workgroups.
     rows = sum(p.R for p in ps)
     for p in sorted(ps, key=lambda q: q.R):
-        buckets = (1 << (p.bits - 12)) * -(-(p.C // p.d) // STREAM_PART_MAX)
+        buckets = ((p.G << p.bits) >> 12) * -(-(p.C // p.d) // STREAM_PART_MAX)
         runs = max(1, round(workgroups * p.R / rows / buckets))
         if p.words is not None and (p.stream is None or (runs != p.stream_asked and not (default and len(ps) == 1 and p.stream_asked == 0))):
             p.build_stream(runs)

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     for name in _declared():
         assert getattr(L, name) is not None, name
-    assert L.sq_version() == 108
+    assert L.sq_version() == 109
 
 
 def test_struct_layout_matches_header():

@@ -277,6 +277,84 @@ def test_stream_gemv_matches_oracle_and_row_path(case, dtype):
                 assert rel_max_err(yb[:, :R].cpu().numpy(), _ref(s, xb)) < TOL and (yb[:, R:] == 5.0).all()
 
 
+STREAM_BOOKS = [  # R, C, bits, G, M
+    (200, 512, 14, 4, 1), (260, 3584, 16, 2, 1), (130, 3584, 16, 4, 1), (300, 1024, 12, 8, 4), (90, 1024, 11, 8, 1),
+    (333, 5376, 13, 2, 1), (70, 5120, 15, 2, 16),
+]
+
+
+@pytest.mark.parametrize("case", STREAM_BOOKS, ids=lambda c: "x".join(map(str, c)))
+def test_stream_with_several_codebooks_matches_oracle(case):
+    """Matrices with G codebooks of d = 8 whose table is beyond LDS (the file's row_book names each row's): the tag
+    stream's labels are book * K + tag, so its slices are slices of the table as a whole (up to 64 of them) and a
+    workgroup finds entries only in its codebook's rows.  Against the oracle at 1 to 8 rows and beyond (other kernels),
+    against the kernels that read the file's tags, twice for the same bits, after another cut into runs, and with the
+    tags dropped (dense rows and products from the stream alone)."""
+    from quantexperiments_amd.kernels import linear_small, linear_gemm
+    R, C, bits, G, M = case
+    s = synth(R, C, 8, bits, G, M, seed=sum(case))
+    s.tags[5] = 7                                       # a row whose tags all sit in one slice
+    s.words = O.pack_bits(s.tags, bits)
+    lin, plain = to_device(s), to_device(s, stream=False)
+    assert lin.stream is not None and lin.G == G and plain.stream is None
+    ref_w = O.decode_tensors(s.tags, s.table, s.row_scale, s.row_book, s.row_mask if M > 1 else np.zeros(R, np.uint8), s.perms, 1 << bits)
+    assert np.array_equal(lin.dense(torch.float32).cpu().numpy().view(np.uint32), ref_w.view(np.uint32))   # relabelled pair, same weights
+    for dtype in (torch.bfloat16, torch.float16):
+        x = rand_x(1, C, dtype, seed=R)
+        ref = _ref(s, x)
+        y32 = torch.full((1, R), 9.0, dtype=torch.float32, device="cuda")
+        linear_small([lin], x.cuda(), y32)
+        assert rel_max_err(y32.cpu().numpy(), ref) < TOL
+        yp = torch.empty(1, R, dtype=torch.float32, device="cuda")
+        linear_small([plain], x.cuda(), yp)
+        assert rel_max_err(y32.cpu().numpy(), yp.cpu().numpy().astype(np.float64)) < 1e-5
+        _check_lowp(lin.gemv(x.cuda()[0])[None], ref)
+        y2 = torch.empty_like(y32)
+        linear_small([lin], x.cuda(), y2)
+        assert torch.equal(y2, y32)
+        for B in (2, 3, 8, 17):
+            xb = rand_x(B, C, dtype, seed=R + B)
+            yb = torch.full((B, R + 3), 5.0, dtype=torch.float32, device="cuda")
+            linear_small([lin], xb.cuda(), yb[:, :R])
+            assert rel_max_err(yb[:, :R].cpu().numpy(), _ref(s, xb)) < TOL and (yb[:, R:] == 5.0).all()
+            if B <= 3:                                  # (the tag-stream kernel at any shape: a row's sums in one order)
+                for b in range(B):
+                    linear_small([lin], xb[b:b + 1].cuda(), y2)
+                    assert torch.equal(y2[0], yb[b, :R]), (B, b)
+    for runs in (1, 3):
+        lin.build_stream(runs)
+        linear_small([lin], x.cuda(), y2)
+        assert rel_max_err(y2.cpu().numpy(), y32.cpu().numpy().astype(np.float64)) < 1e-5
+    # one copy: the tags dropped, everything from the stream
+    lin.make_compact()
+    assert lin.words is None
+    assert np.array_equal(lin.dense(torch.float32).cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
+    linear_small([lin], x.cuda(), y2)
+    assert rel_max_err(y2.cpu().numpy(), ref) < TOL
+    xb = rand_x(40, C, torch.float16, seed=3)
+    yb = torch.empty(40, R, dtype=torch.float32, device="cuda")
+    linear_gemm([lin], xb.cuda(), yb)
+    assert rel_max_err(yb.cpu().numpy(), _ref(s, xb)) < TOL
+
+
+def test_stacked_pieces_with_several_codebooks_share_a_launch():
+    """A q|k|v-like stack of pieces with four codebooks of 16,384 each through PackedShards (streams cut for the joint
+    launch), and the header left zero."""
+    from quantexperiments_amd import _lib
+    from quantexperiments_amd.vllm_ext.core import PackedShards
+    from quantexperiments_amd.kernels import _Workspace
+    C = 1024
+    ss = [synth(R, C, 8, 14, 4, 1, seed=40 + i) for i, R in enumerate((448, 128, 130))]
+    sh = PackedShards([to_device(s, stream="later") for s in ss])
+    assert all(rl.stream is not None for rl in sh.rls)
+    for B in (1, 2, 5):
+        x = rand_x(B, C, torch.bfloat16, seed=B)
+        _check_lowp(sh.forward(x.cuda()), np.concatenate([_ref(s, x) for s in ss], 1))
+    torch.cuda.synchronize()
+    ws = [b for (_, kind), b in _Workspace.bufs.items() if kind == "kernels"]
+    assert ws and all(not b[:_lib.WS_HEADER - 4096].any() for b in ws)
+
+
 def test_workspace_header_is_zero_after_every_stream_launch():
     # The header of a workspace holds the partial sums the workgroups of the tag-stream kernel exchange; a word is its
     # own arrival flag, so every launch must leave all of them zero, whatever runs between two launches writes behind

@@ -178,8 +178,9 @@ def test_neutral_defaults_and_registry():
 
 # ---------------------------------------------------------------------------- bucketed tag stream (host builder)
 
-def _build_stream(words, R, C, bits, row_mask, runs, table=None):
-    """Bytes of the stream, its run count and its group count; with `table` (fp16 [2^bits, 8]) the balanced form."""
+def _build_stream(words, R, C, bits, row_mask, runs, table=None, books=None):
+    """Bytes of the stream, its run count and its group count; with `table` (fp16 [2^bits, 8]) the balanced form; with
+    `books` = (row_book uint8 [R], G) the stream of a matrix with G codebooks."""
     import ctypes
     from quantexperiments_amd import _lib
     L = _lib.lib()
@@ -187,7 +188,17 @@ def _build_stream(words, R, C, bits, row_mask, runs, table=None):
     ptr = words.ctypes.data_as(ctypes.c_void_p)
     mp = None if row_mask is None else row_mask.ctypes.data_as(ctypes.c_void_p)
     r, g = ctypes.c_int32(0), ctypes.c_int32(0)
-    if table is None:
+    if books is not None:
+        book, G = books
+        bp = book.ctypes.data_as(ctypes.c_void_p)
+        n = L.sq_stream_bytes_books(ptr, R, W, C, 8, bits, G, bp, mp, runs)
+        assert n > 0
+        out = np.zeros(n, np.uint8)
+        args = (ptr, R, W, C, 8, bits, G, bp, mp, runs, out.ctypes.data_as(ctypes.c_void_p))
+        assert L.sq_stream_build_books(*args, n, ctypes.byref(r), ctypes.byref(g)) == 0
+        assert L.sq_stream_build_books(*args, n - 1, ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EINVAL
+        assert not r.value & (1 << 30)
+    elif table is None:
         n = L.sq_stream_bytes(ptr, R, W, C, 8, bits, mp, runs)
         assert n > 0
         out = np.zeros(n, np.uint8)
@@ -233,6 +244,7 @@ class _Fmt:
 
 
 def _geom(C, bits):
+    """(bits: of the stream's labels, i.e. the tag width plus log2 of the number of codebooks)"""
     U, NS = C // 8, 1 << (bits - 12)
     KP = -(-U // PART_MAX)
     PC = -(-U // KP)
@@ -415,6 +427,86 @@ def test_stream_builder_keeps_every_tag(R, C, bits, runs, M):
     buf, eff, NG = _build_stream(words, R, C, bits, row_mask, runs)
     assert NG >= -(-R // 64) and 1 <= eff <= NG
     assert np.array_equal(_walk_stream(buf, R, C, 8, bits, eff, NG, row_mask), tags)
+
+
+@pytest.mark.parametrize("R,C,bits,G,runs,M", [(200, 512, 14, 4, 0, 1),      # 4 books of 4 slices: 16 buckets
+                                                (130, 3584, 16, 2, 2, 1),     # 32 buckets, narrow entries at their widest rows
+                                                (300, 256, 12, 8, 3, 4),      # a book is exactly one slice; column orders
+                                                (90, 1024, 11, 4, 0, 1),      # two books share a slice
+                                                (70, 512, 16, 4, 1, 1),       # 64 buckets
+                                                (100, 5376, 13, 2, 2, 1)])    # wide entries
+def test_stream_builder_with_several_codebooks(R, C, bits, G, runs, M):
+    """sq_stream_build_books: the stream's labels are book << bits | tag, every one of them is kept, a slice holds
+    entries of its own codebook's rows only, and the kernel's reads stay inside the buffer."""
+    rng = np.random.default_rng(R + C + G)
+    U = C // 8
+    tags = rng.integers(0, 1 << bits, (R, U))
+    book = rng.integers(0, G, R).astype(np.uint8)
+    book[:min(R, G)] = np.arange(min(R, G))
+    row_mask = rng.integers(0, M, R).astype(np.uint8) if M > 1 else None
+    words = np.ascontiguousarray(O.pack_bits(tags, bits))
+    buf, eff, NG = _build_stream(words, R, C, bits, row_mask, runs, books=(book, G))
+    lbits = bits + G.bit_length() - 1
+    labels = tags + (book.astype(np.int64) << bits)[:, None]
+    assert np.array_equal(_walk_stream(buf, R, C, 8, lbits, eff, NG, row_mask), labels)
+    for what, a, b in _stream_reads(buf, R, C, lbits, _build_stream.runs_out, NG, row_mask):   # (defined below)
+        assert 0 <= a < b <= len(buf), (what, a, b)
+    # one codebook through the same entry point: the same buffer as sq_stream_build
+    one, e1, g1 = _build_stream(words, R, C, bits, row_mask, runs, books=(np.zeros(R, np.uint8), 1)) if lbits - (G.bit_length() - 1) > 12 else (None, 0, 0)
+    if one is not None:
+        assert (one, e1, g1) == _build_stream(words, R, C, bits, row_mask, runs)
+
+
+def test_several_codebooks_argument_checks_and_balance():
+    """sq_stream_*_books refuse what they do not cover; sq_codebook_balance_books relabels every codebook by itself:
+    a permutation within each, even slices within each, an equivalent matrix."""
+    import ctypes
+    from quantexperiments_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(11)
+    R, C, bits, G = 240, 256, 14, 4
+    K, U = 1 << bits, C // 8
+    w = 1.0 / np.arange(1, K + 1)
+    tags = rng.choice(K, size=(R, U), p=w / w.sum())                       # popular codewords first, in every book
+    book = (np.arange(R) % G).astype(np.uint8)
+    words = np.ascontiguousarray(O.pack_bits(tags, bits))
+    wp, bp = words.ctypes.data_as(ctypes.c_void_p), book.ctypes.data_as(ctypes.c_void_p)
+    W = words.shape[1]
+    assert L.sq_stream_bytes_books(wp, R, W, C, 8, bits, 3, bp, None, 0) == 0             # not a power of two
+    assert L.sq_stream_bytes_books(wp, R, W, C, 8, bits, 32, bp, None, 0) == 0            # 128 slices
+    assert L.sq_stream_bytes_books(wp, R, W, C, 8, bits, 4, None, None, 0) == 0           # no row_book
+    assert L.sq_stream_bytes_books(wp, R, W, C, 8, bits, 2, bp, None, 0) == 0             # a row names book 2 or 3
+    r, g = ctypes.c_int32(0), ctypes.c_int32(0)
+    out = np.zeros(1 << 20, np.uint8)
+    assert L.sq_stream_build_books(wp, R, W, C, 8, bits, 2, bp, None, 0, out.ctypes.data_as(ctypes.c_void_p), out.size,
+                                   ctypes.byref(r), ctypes.byref(g)) == _lib.SQ_EINVAL
+    assert b"codebook" in L.sq_last_error()
+    remap = np.zeros(G * K, np.uint16)
+    assert L.sq_codebook_balance_books(wp, R, W, C, 8, bits, G, bp, remap.ctypes.data_as(ctypes.c_void_p)) == 0
+    remap = remap.astype(np.int64).reshape(G, K)
+    for b in range(G):
+        assert sorted(remap[b].tolist()) == list(range(K))
+        t = tags[book == b]
+        before, after = np.bincount((t >> 12).ravel(), minlength=K >> 12), np.bincount((remap[b][t] >> 12).ravel(), minlength=K >> 12)
+        assert before.max() > 2 * before.mean()
+        top = int(np.bincount(t.ravel(), minlength=K).max())
+        assert after.max() <= max(1.02 * after.mean() + 1, top)
+    # the relabelled pair decodes to the same weights
+    table = rng.standard_normal((G * K, 8)).astype(np.float16)
+    rs = (rng.random(R) * 0.02 + 0.01).astype(np.float16)
+    tags2 = remap[book.astype(np.int64)[:, None], tags]
+    table2 = np.empty_like(table)
+    for b in range(G):
+        table2[b * K + remap[b]] = table[b * K:(b + 1) * K]
+    ident = np.arange(C)[None]
+    w1 = O.decode_tensors(tags, table, rs, book, np.zeros(R, np.uint8), ident, K)
+    w2 = O.decode_tensors(tags2, table2, rs, book, np.zeros(R, np.uint8), ident, K)
+    assert np.array_equal(np.asarray(w1).view(np.uint32), np.asarray(w2).view(np.uint32))
+    # one codebook: the same map as sq_codebook_balance
+    r1, r2 = np.zeros(K, np.uint16), np.zeros(K, np.uint16)
+    assert L.sq_codebook_balance(wp, R, W, C, 8, bits, r1.ctypes.data_as(ctypes.c_void_p)) == 0
+    assert L.sq_codebook_balance_books(wp, R, W, C, 8, bits, 1, None, r2.ctypes.data_as(ctypes.c_void_p)) == 0
+    assert np.array_equal(r1, r2)
 
 
 @pytest.mark.parametrize("R,C,bits,runs,M", [(300, 512, 16, 3, 1), (130, 3584, 14, 2, 1), (200, 256, 16, 0, 4)])
