@@ -156,7 +156,15 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
     }
     for (int rw = NT == 1 ? r1 : r1 / 2; rw >= 1 && rw >= r1 / 4; rw /= 2) {
         const int need = (rounds + rw - 1) / rw;
-        const int ks = (need + max_kw - 1) / max_kw, kw = (need + ks - 1) / ks;
+        // (the variants with few activation operands per lane fit four waves per SIMD: up to 16 waves per workgroup.  Long rows
+        // then take more, shorter column slices: 7B down, 148 rounds, at 4 rows: 15.1 us with 15 waves x 2 rounds x 5 slices
+        // against 18.4 with 7 x 8 x 3, reduction launch included)
+        int mk = max_kw;
+        if (tab && mma_waves_max(rw * spu * NT, true) == 16) {
+            const size_t room = 160 * 1024 - tab - 16, per_wave = (size_t)64 * NT * 16 * mma_pft(rw);
+            mk = (int)std::min<size_t>(16, room / per_wave);
+        }
+        const int ks = (need + mk - 1) / mk, kw = (need + ks - 1) / ks;
         const double cost = (double)rw * kw * ks / rounds + 0.03 * (ks - 1) + 0.002 * kw;
         if (cost < best_cost - 1e-9) { best_cost = cost; best = MmaPlan{rw, NT, kw, ks}; }
     }

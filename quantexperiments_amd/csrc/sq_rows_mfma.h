@@ -66,8 +66,13 @@ constexpr int mma_pft(int RW) { return RW >= 8 ? 2 : 3; }
 // kernel differ from the batch-1 one on the same input)
 __device__ __forceinline__ uint32_t bf2h_pk(uint32_t v) { return bf2h_x2(v); }
 
+// Waves per workgroup: up to 16 for the variants whose lanes hold at most 8 activation operands (32 registers) beside a
+// codebook in LDS, which fit four waves per SIMD; 8 otherwise.
+constexpr int mma_waves_max(int x_operands, bool lds_tab) { return lds_tab && x_operands <= 8 ? 16 : 8; }
+
 template <int BITS, int D, int RW, int NT, bool LDS_TAB>
-__global__ __launch_bounds__(512) void rows_mfma_kernel(MmaArgs a) {
+__global__ __launch_bounds__(64 * mma_waves_max(RW * ((unit_of<BITS>::UD * 32 / BITS) / (8 / D)) * NT, LDS_TAB))
+void rows_mfma_kernel(MmaArgs a) {
     constexpr int UD = unit_of<BITS>::UD;
     constexpr int TPU = UD * 32 / BITS;      // tags per lane unit
     constexpr int CPS = 8 / D;               // codewords a lane feeds into one matrix instruction
