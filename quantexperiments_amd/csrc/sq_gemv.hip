@@ -151,7 +151,7 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
     const size_t tab = mma_table_bytes(m);
     int max_kw = 8;
     if (tab) {
-        const size_t room = 160 * 1024 - tab - 16, per_wave = (size_t)MMA_TT * 64 * NT * 16;
+        const size_t room = 160 * 1024 - tab - 16, per_wave = std::max((size_t)MMA_TT * 64 * NT * 16, (size_t)mma_x_stage_bytes(tpu * m.d));
         if (room / per_wave < 8) max_kw = (int)(room / per_wave);
     }
     for (int rw = NT == 1 ? r1 : r1 / 2; rw >= 1 && rw >= r1 / 4; rw /= 2) {
@@ -161,7 +161,7 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
         // against 18.4 with 7 x 8 x 3, reduction launch included)
         int mk = max_kw;
         if (tab && mma_waves_max(rw * spu * NT, true) == 16) {
-            const size_t room = 160 * 1024 - tab - 16, per_wave = (size_t)64 * NT * 16 * mma_pft(rw);
+            const size_t room = 160 * 1024 - tab - 16, per_wave = std::max((size_t)64 * NT * 16 * mma_pft(rw), (size_t)mma_x_stage_bytes(tpu * m.d));
             mk = (int)std::min<size_t>(16, room / per_wave);
         }
         const int ks = (need + mk - 1) / mk, kw = (need + ks - 1) / ks;
@@ -224,7 +224,9 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
     const size_t red_tile = (size_t)pl.KW * 64 * pl.NT * 16;
     const int pft = mma_pft(pl.RW);
     a.tg = a.table_bytes ? pft : 0;
-    size_t smem = (size_t)a.table_bytes + 16 + (a.table_bytes ? (size_t)a.tg * red_tile : pl.KW > 1 ? (size_t)MMA_TT * red_tile : 0);
+    const int tpu = unit_dwords(m0.bits) * 32 / m0.bits;
+    const size_t xstage = (size_t)pl.KW * mma_x_stage_bytes(tpu * m0.d);      // the waves' activation staging areas (same LDS)
+    size_t smem = (size_t)a.table_bytes + 16 + std::max(xstage, a.table_bytes ? (size_t)a.tg * red_tile : pl.KW > 1 ? (size_t)MMA_TT * red_tile : 0);
     int rc = SQ_EUNSUPPORTED;
 #define SQ_CASE(BI, DD) if (m0.bits == BI && m0.d == DD) rc = launch_mma_b##BI##d##DD(OP, a, pl.RW, pl.NT, GRID, threads, smem, s)
 #define OP 1
@@ -266,7 +268,7 @@ static int launch_mma_group(const sq_matrix* mats, int cnt, const void* x, int x
         const size_t room = (size_t)(160 * 1024) / rc - a.table_bytes - 16;
         int fit = (int)(room / red_tile) / pft * pft;
         a.tg = std::min((most + pft - 1) / pft * pft, std::max(fit, pft));
-        smem = (size_t)a.table_bytes + 16 + (size_t)a.tg * red_tile;
+        smem = (size_t)a.table_bytes + 16 + std::max(xstage, (size_t)a.tg * red_tile);
     }
 #define OP 0
 #define GRID wg

@@ -55,6 +55,9 @@ constexpr int MMA_TT = 4;     // 16-row tiles multiplied between two workgroup b
 // codebook in LDS: tiles of tags in flight per lane (fewer when a lane's part of a tile is long: registers)
 // (2 to 5 tiles in flight measure alike on the 7B shapes)
 constexpr int mma_pft(int RW) { return RW >= 8 ? 2 : 3; }
+// LDS per wave in which a round's activations (16 tokens x 4 lane units of UK columns, fp16) pass from whole-line loads
+// to the lanes that use them; it lies where the accumulators are added afterwards
+constexpr int mma_x_stage_bytes(int UK) { return 16 * (4 * UK * 2 + 16); }
 
 // Optional timeline of the first wave of every workgroup (debug builds define SQ_TRACE_POINT).
 #ifndef SQ_TRACE_POINT
@@ -160,15 +163,28 @@ void rows_mfma_kernel(MmaArgs a) {
             __builtin_amdgcn_global_load_lds((gptr_t)(table + (size_t)c * 1024 + lane * 16), (lptr_t)(smem + c * 1024), 16, 0, 0);
     }
     if (t0 < t1) fetch(t0, tA, sc[0]);
-    u32x4 xraw[RW][SPU][NT];
+    // The activations.  In the matrix instruction a lane supplies one token's 8 columns, so loading the operands where
+    // they are used makes every load instruction touch 64 different cache lines (16 tokens x 4 lane units, 16 bytes of
+    // each).  Instead the wave fetches the columns of a round, 16 tokens x XRB contiguous bytes, with whole-line loads
+    // (1 KB per instruction: 8 lines), and the lanes pick their operands out of LDS: a staging area per wave that lies
+    // where the accumulators are added later, which nobody writes before the barrier below.
+    constexpr int XRB = 4 * UK * 2;                          // bytes of one token's columns in one round of a wave
+    constexpr int XROW = XRB + 16;                           // a token's row in the staging area (the 16 tokens' reads spread over the banks)
+    constexpr int XTPI = 1024 / XRB;                         // tokens per load instruction
+    static_assert(16 / XTPI == SPU, "a round's activations are SPU loads per token tile");
+    unsigned char* xst = smem + a.table_bytes + 16 + wave * mma_x_stage_bytes(UK);
+    const int xtl = lane / (XRB / 16), xob = (lane % (XRB / 16)) * 16;    // this lane's token (within an instruction) and byte in the round
+    u32x4 xraw[RW][NT][SPU];
 #pragma unroll
     for (int n = 0; n < RW; ++n)
 #pragma unroll
-        for (int s = 0; s < SPU; ++s)
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int tok = nt * 16 + li;
-                xraw[n][s][nt] = *reinterpret_cast<const u32x4*>(a.x + (int64_t)(tok < a.B ? tok : a.B - 1) * a.ldx + ucol[n] + 8 * s);
+            for (int j = 0; j < SPU; ++j) {
+                const int tok = nt * 16 + j * XTPI + xtl;
+                int col = 4 * (rbase + n) * UK + (xob >> 1);
+                col = col < m.C ? col : m.C - 8;             // (columns past the row's end: any valid address, the operand is zeroed)
+                xraw[n][nt][j] = *reinterpret_cast<const u32x4*>(a.x + (int64_t)(tok < a.B ? tok : a.B - 1) * a.ldx + col);
             }
     if (LDS_TAB) {
         if (!table_dma) stage_table(m.table, a.table_bytes, smem);
@@ -179,19 +195,33 @@ void rows_mfma_kernel(MmaArgs a) {
 #pragma unroll
     for (int n = 0; n < RW; ++n)
 #pragma unroll
-        for (int s = 0; s < SPU; ++s)
+        for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                u32x4 v = xraw[n][s][nt];
+            for (int j = 0; j < SPU; ++j) {
+                u32x4 v = xraw[n][nt][j];
                 if (a.x_dtype == SQ_BF16) { v.x = bf2h_pk(v.x); v.y = bf2h_pk(v.y); v.z = bf2h_pk(v.z); v.w = bf2h_pk(v.w); }
+                *reinterpret_cast<u32x4*>(xst + (j * XTPI + xtl) * XROW + xob) = v;
+            }
+            // (the lanes of a wave exchange data here: its LDS instructions run in order, the fences keep the compiler from
+            // moving a lane's reads before its writes)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int s = 0; s < SPU; ++s) {
+                u32x4 v = *reinterpret_cast<const u32x4*>(xst + li * XROW + lg * (UK * 2) + s * 16);
                 if (!(live[n] && nt * 16 + li < a.B)) v = u32x4{0u, 0u, 0u, 0u};
                 xb[n][s][nt] = __builtin_bit_cast(half8v, v);
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
     SQ_TRACE_POINT(1);
-    if (LDS_TAB) {
-        if (table_dma) __builtin_amdgcn_s_waitcnt(0);         // the codebook has landed (and the first tile's tags with it)
-        __syncthreads();
-    }
+    // every wave has taken its operands out of the staging area (and, with the codebook in LDS, the codebook has landed
+    // and the first tile's tags with it)
+    __builtin_amdgcn_s_waitcnt(0);
+    if (LDS_TAB || KW > 1) __syncthreads();
     SQ_TRACE_POINT(2);
 
     // One tile: NS = RW * SPU matrix instructions.  The codeword gathers run PD instructions ahead of the
