@@ -194,7 +194,7 @@ def layer_times(torch, dev, layers, shapes, B, fn, gen):
 def small_batch_crossover(torch, dev, gen, n_layers):
     """cfg3: the 7B shapes in the d = 4, K = 4096, 12-bit format (3 bits per weight) from 1 to 256 activation rows, on
     the two routes PackedShards.forward can take: "direct" = the library's own choice (sq_linear_small up to 32 rows;
-    sq_linear_gemm above: passes of 32 rows through the decode-time kernel up to 160 rows, then decode + 256 x 256
+    sq_linear_gemm above: passes of 32 rows through the decode-time kernel up to 224 rows, then decode + 256 x 256
     tile GEMM) and "dequant" = decode to fp16 + dense GEMM (the reference's large-M route).  Per M: both times, the
     faster route and its fractions of the HBM roofline (packed bytes + x + y) and of the MFMA roofline (2 M R C).
     crossover_M = the first M at which the MFMA fraction exceeds the HBM fraction: where the product stops being
@@ -225,7 +225,7 @@ def small_batch_crossover(torch, dev, gen, n_layers):
         res[f"M{M}"] = r
     return {"workload": "cfg3: 7B shapes, d=4, K=4096, 12-bit tags (3 bpw), bf16 rows", "layers_rotated": n_layers,
             "flops_per_row": flops1, "rows": res, "crossover_M": cross, "route_change_M": change,
-            "note": "direct = sq_linear_small (M <= 32) / sq_linear_gemm (passes of 32 rows up to 160, then decode + tile GEMM); "
+            "note": "direct = sq_linear_small (M <= 32) / sq_linear_gemm (passes of 32 rows up to 224, then decode + tile GEMM); "
                     "dequant = sq_dequant to fp16 + sq_gemm_dense; crossover_M = first M whose MFMA fraction exceeds its HBM "
                     "fraction; route_change_M = first M at which the dequant route is faster (null: never up to 256)"}
 

@@ -91,7 +91,7 @@ int sq_linear_small_noalloc(const sq_matrix* mats, int32_t n_mats, const void* x
  * accumulation, row scale applied to the accumulator.  Same argument meaning as sq_linear_small.
  * Replaces runs_gemm.gemm (reference shapequant/kernels/runs_gemm.py:471-514).  Pieces with
  * M > 1 are decoded with their column orders into workspace and multiplied from there.  Between
- * SQ_SMALL_BMAX + 1 and 160 rows (64 when the codebook does not fit LDS) pieces without column orders
+ * SQ_SMALL_BMAX + 1 and 224 rows (64 when the codebook does not fit LDS) pieces without column orders
  * run as passes of SQ_SMALL_BMAX rows through sq_linear_small's kernels, which is cheaper than decoding
  * the matrix first, and up to SQ_SMALL_BMAX rows the call is sq_linear_small; sq_workspace_bytes(which = 1)
  * accounts for whichever route T takes. */

@@ -146,23 +146,20 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
     MmaPlan best{0, 0, 0, 0};
     double best_cost = 1e30;
     const int NT = B > 16 ? 2 : 1;
-    // waves per workgroup: 8, or as many as leave room in the CU's 160 KB of LDS for their reduction buffers
-    // next to a codebook that is staged there (4 books of 4096 d = 4 entries fill 128 KB)
+    // waves per workgroup: 8 (16 for the variants with few activation operands per lane, which fit four waves per SIMD),
+    // or as many as leave room in the CU's 160 KB of LDS, next to a codebook that is staged there (4 books of 4096 d = 4
+    // entries fill 128 KB), for their accumulators of the tiles in flight and their activation staging areas.  Long rows
+    // then take more, shorter column slices: 7B down, 148 rounds, at 4 rows: 15.1 us with 15 waves x 2 rounds x 5 slices
+    // against 18.4 with 7 x 8 x 3, reduction launch included.
     const size_t tab = mma_table_bytes(m);
-    int max_kw = 8;
-    if (tab) {
-        const size_t room = 160 * 1024 - tab - 16, per_wave = std::max((size_t)MMA_TT * 64 * NT * 16, (size_t)mma_x_stage_bytes(tpu * m.d));
-        if (room / per_wave < 8) max_kw = (int)(room / per_wave);
-    }
     for (int rw = NT == 1 ? r1 : r1 / 2; rw >= 1 && rw >= r1 / 4; rw /= 2) {
         const int need = (rounds + rw - 1) / rw;
-        // (the variants with few activation operands per lane fit four waves per SIMD: up to 16 waves per workgroup.  Long rows
-        // then take more, shorter column slices: 7B down, 148 rounds, at 4 rows: 15.1 us with 15 waves x 2 rounds x 5 slices
-        // against 18.4 with 7 x 8 x 3, reduction launch included)
-        int mk = max_kw;
-        if (tab && mma_waves_max(rw * spu * NT, true) == 16) {
-            const size_t room = 160 * 1024 - tab - 16, per_wave = std::max((size_t)64 * NT * 16 * mma_pft(rw), (size_t)mma_x_stage_bytes(tpu * m.d));
-            mk = (int)std::min<size_t>(16, room / per_wave);
+        int mk = 8;
+        if (tab) {
+            const size_t room = 160 * 1024 - tab - 16;
+            const size_t per_wave = std::max((size_t)64 * NT * 16 * mma_pft(rw), (size_t)mma_x_stage_bytes(tpu * m.d));
+            mk = (int)std::min<size_t>(mma_waves_max(rw * spu * NT, true), room / per_wave);
+            if (mk < 1) continue;
         }
         const int ks = (need + mk - 1) / mk, kw = (need + ks - 1) / ks;
         const double cost = (double)rw * kw * ks / rounds + 0.03 * (ks - 1) + 0.002 * kw;
@@ -171,16 +168,16 @@ static MmaPlan mma_plan(const sq_matrix& m, int B) {
     return best;
 }
 
-// Passes of 32 rows through the matrix-core decode kernel against decode + tile GEMM (7B layer): 104 us per pass
+// Passes of 32 rows through the matrix-core decode kernel against decode + tile GEMM (7B layer): 77 us per pass
 // against 600-640 us when the codebook sits in LDS (d = 4), 201 us per pass when its gathers go to L2.  A
 // codebook that fills most of LDS leaves room for fewer waves per workgroup and doubles the cost of a pass
 // (27B layer, 4 books of 4096: 246 us per pass against 800 us).
 int small_pass_limit(const sq_matrix* mats, int n) {
-    int limit = 160;
+    int limit = 224;
     for (int i = 0; i < n; ++i) {
         if (!mma_shape(mats[i])) return 0;
         const size_t tab = mma_table_bytes(mats[i]);
-        const int li = tab == 0 ? 64 : tab > 64 * 1024 ? 96 : 160;
+        const int li = tab == 0 ? 64 : tab > 64 * 1024 ? 96 : 224;
         if (li < limit) limit = li;
     }
     return n > 0 ? limit : 0;

@@ -76,8 +76,8 @@ def test_workspace_sizes_are_host_arithmetic():
     # 33 .. 64 rows of a matrix the matrix-core decode kernel takes: passes of 32 rows, its workspace (none here)
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 64, 1) == 0
     lds = _lib.SqMatrix(0x1000, 0x2000, 0x3000, None, None, None, None, 64, 512, 4, 12, 1, 1, 48, 0)
-    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 160, 1) == 0          # codebook in LDS: up to 160 rows
-    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 161, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 161 * 512 * 2
+    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 224, 1) == 0          # codebook in LDS: up to 224 rows
+    assert L.sq_workspace_bytes(_lib.matrix_array([lds]), 1, 225, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 225 * 512 * 2
     # beyond: raw fp16 codewords of the largest piece + an fp16 copy of the activations
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 100, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 100 * 512 * 2
     assert L.sq_workspace_bytes(_lib.matrix_array([plain]), 1, 2048, 1) == _lib.WS_HEADER + 64 * 512 * 2 + 2048 * 512 * 2

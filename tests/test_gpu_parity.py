@@ -525,9 +525,9 @@ GEMM = [  # R, C, d, bits, G, M, T
     (96, 256, 4, 10, 4, 16, 70), (140, 5120, 8, 16, 1, 16, 129), (50, 96, 2, 5, 3, 1, 40), (64, 200, 4, 8, 1, 1, 35),
     # 256 activation rows and more: the 256 x 256 tile route (ragged row / token counts, mixture books, column orders)
     (300, 1280, 4, 10, 4, 1, 260), (140, 5120, 8, 16, 1, 16, 300), (513, 640, 4, 8, 1, 1, 256), (257, 3584, 8, 16, 1, 1, 511),
-    # 33 .. 255 rows: passes of 32 rows through the decode-time kernel (up to 160 rows with the codebook in LDS, up
+    # 33 .. 255 rows: passes of 32 rows through the decode-time kernel (up to 224 rows with the codebook in LDS, up
     # to 64 otherwise, never with column orders), the 256 x 256 tile route beyond; C % 64 != 0 keeps the fused kernel
-    (200, 1280, 4, 12, 1, 1, 160), (200, 1280, 4, 12, 1, 1, 161), (130, 3584, 8, 16, 1, 1, 64), (130, 3584, 8, 16, 1, 1, 65), (2100, 4096, 8, 16, 1, 1, 33),
+    (200, 1280, 4, 12, 1, 1, 224), (200, 1280, 4, 12, 1, 1, 225), (130, 3584, 8, 16, 1, 1, 64), (130, 3584, 8, 16, 1, 1, 65), (2100, 4096, 8, 16, 1, 1, 33),
     (300, 1280, 4, 10, 4, 1, 97), (96, 256, 4, 10, 4, 16, 200), (64, 200, 4, 8, 1, 1, 130),
     # few tiles, long rows: K split over 3 and 4 workgroups with fp32 partial products
     (260, 3584, 8, 16, 1, 1, 511), (512, 4096, 8, 14, 1, 1, 256),
