@@ -64,6 +64,21 @@ constexpr int mma_x_stage_bytes(int UK) { return 16 * (4 * UK * 2 + 16); }
 #define SQ_TRACE_POINT(k)
 #endif
 
+// LDS byte offset of the codeword of tag t of a unit, counted from the start of the dynamic LDS: the tag times 2^SH (the
+// codeword size) plus `bo`, the byte offset of the row's codebook, whose bits lie above the tag's: one shift (or
+// v_alignbit_b32 for a tag that straddles two dwords, which starts past bit SH) and one v_and_or_b32
+template <int BITS, int UD, int SH>
+__device__ __forceinline__ uint32_t unit_lds_offset(const dwords<UD>& u, int t, uint32_t bo) {
+    const int p = t * BITS, w = p >> 5, s = p & 31;
+    constexpr uint32_t MASK = ((1u << BITS) - 1u) << SH;
+    uint32_t v;
+    if (s + BITS <= 32) v = s >= SH ? u.v[w] >> (s - SH) : u.v[w] << (SH - s);
+    else v = __builtin_amdgcn_alignbit(u.v[w + 1 < UD ? w + 1 : w], u.v[w], s - SH);
+    return (v & MASK) | bo;
+}
+typedef __attribute__((address_space(3))) u32x2 mma_lds_u32x2;
+typedef __attribute__((address_space(3))) u32x4 mma_lds_u32x4;
+
 // two packed bf16 -> two packed fp16: round to nearest even like every other kernel of the library (exact for every
 // fp16-normal value, +-inf beyond 65,504; a round-toward-zero conversion would clamp to 65,504 instead and make this
 // kernel differ from the batch-1 one on the same input)
@@ -96,8 +111,10 @@ void rows_mfma_kernel(MmaArgs a) {
     const int t0 = (int)((int64_t)ntiles * share / nshare), t1 = (int)((int64_t)ntiles * (share + 1) / nshare);
     SQ_TRACE_POINT(0);
 
-    // LDS: [codebook][one all-zero codeword][reduction buffer: TT tiles x KW waves x 64 lanes x NT x 16 bytes]
-    const int zero_off = a.table_bytes;                                 // units past the row's end gather this entry
+    // LDS: [codebook][16 bytes][reduction buffer: TT tiles x KW waves x 64 lanes x NT x 16 bytes]
+    // (the codeword gathers form LDS addresses as numbers counted from the start of the dynamic LDS, which is address 0 in a
+    // kernel without static LDS; a build in which it is not leaves y unwritten, which no test survives)
+    if (LDS_TAB && (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)smem != 0u) return;
     float4v* red = reinterpret_cast<float4v*>(smem + a.table_bytes + 16);
 
     // ---- this wave's rounds
@@ -115,19 +132,23 @@ void rows_mfma_kernel(MmaArgs a) {
         uoff[n] = (uint32_t)uc * UD;
         ucol[n] = uc * UK;
     }
-    // Units past the row's end (only in waves that cover the tail of the columns) must contribute exact
-    // zeros even if codeword 0 is not finite: their tags are zeroed and their codebook offset points at the
-    // all-zero LDS entry (or, without LDS, their operand is zeroed).  Interior waves skip all of that.
+    // Units past the row's end (only in waves that cover the tail of the columns) contribute exact zeros: their
+    // activation operands are zero, and what they multiply with is the row's own last unit again (with the codebook in
+    // LDS; a codeword that is not finite is already part of the row's sum) or a zeroed operand (without).
     const bool all_live = __builtin_amdgcn_readfirstlane(__all(lane_live) ? 1 : 0) != 0;
     const uint32_t* tags = reinterpret_cast<const uint32_t*>(m.tags);
     const unsigned char* table = reinterpret_cast<const unsigned char*>(m.table);
 
     // ---- a tile's memory: tags of this lane's row, its codebook offset, the scales of its four output rows
-    struct Tile { dwords<UD> t[RW]; uint32_t boff; };
+    // (book: the byte of row_book as loaded; without codebook ids a byte of valid memory that `bkmask` turns into 0 where it is
+    // used: a branch around the load, or a use right behind it, would make every wait of the loop a wait for all loads)
+    struct Tile { dwords<UD> t[RW]; uint32_t book; };
+    const uint8_t* bkp = m.row_book ? m.row_book : reinterpret_cast<const uint8_t*>(m.row_scale);
+    const uint32_t bkmask = m.row_book ? 0xFFu : 0u;
     auto fetch = [&](int t, Tile& T, float (&sc)[4]) {
         const int row0 = t << 4;
         const int r = row0 + li < m.R ? row0 + li : m.R - 1;
-        T.boff = m.row_book ? (uint32_t)m.row_book[r] << BITS : 0u;
+        T.book = bkp[r];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int ro = row0 + 4 * lg + v;
@@ -142,7 +163,7 @@ void rows_mfma_kernel(MmaArgs a) {
 #pragma unroll
             for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(rp + uoff[n]);
         }
-        if (!all_live) {
+        if (!LDS_TAB && !all_live) {
 #pragma unroll
             for (int n = 0; n < RW; ++n)
 #pragma unroll
@@ -188,7 +209,6 @@ void rows_mfma_kernel(MmaArgs a) {
             }
     if (LDS_TAB) {
         if (!table_dma) stage_table(m.table, a.table_bytes, smem);
-        if (tid < 4) reinterpret_cast<uint32_t*>(smem + zero_off)[tid] = 0u;
     }
     // the B operands: this wave's activations as fp16, in registers for the whole kernel
     half8v xb[RW][SPU][NT];
@@ -234,20 +254,22 @@ void rows_mfma_kernel(MmaArgs a) {
         auto gather = [&](int k) {
             const int n = k / SPU, s = k - n * SPU;
             const bool dead = !all_live && !live[n];
-            const uint32_t bo = cur.boff * ESZ;                 // byte offset of the row's codebook
-            // (codebook in LDS: a unit past the row's end gathers the all-zero entry, whatever its tags are)
+            const uint32_t bo = ((cur.book & bkmask) << BITS) * ESZ;    // byte offset of the row's codebook
             if (D == 8) {
-                const uint32_t tag = unit_tag<BITS, UD>(cur.t[n], s);
-                if (LDS_TAB) av[k] = *reinterpret_cast<const u32x4*>(smem + (dead ? (uint32_t)zero_off : tag * ESZ + bo));
-                else av[k] = *reinterpret_cast<const u32x4*>(table + ((size_t)tag * ESZ + bo));
+                if (LDS_TAB) {
+                    av[k] = *reinterpret_cast<const mma_lds_u32x4*>((uintptr_t)unit_lds_offset<BITS, UD, 4>(cur.t[n], s, bo));
+                } else {
+                    const uint32_t tag = unit_tag<BITS, UD>(cur.t[n], s);
+                    av[k] = *reinterpret_cast<const u32x4*>(table + ((size_t)tag * ESZ + bo));
+                }
             } else {
-                const uint32_t g0 = unit_tag<BITS, UD>(cur.t[n], 2 * s);
-                const uint32_t g1 = unit_tag<BITS, UD>(cur.t[n], 2 * s + 1);
                 u32x2 c0, c1;
                 if (LDS_TAB) {
-                    c0 = *reinterpret_cast<const u32x2*>(smem + (dead ? (uint32_t)zero_off : g0 * ESZ + bo));
-                    c1 = *reinterpret_cast<const u32x2*>(smem + (dead ? (uint32_t)zero_off : g1 * ESZ + bo));
+                    c0 = *reinterpret_cast<const mma_lds_u32x2*>((uintptr_t)unit_lds_offset<BITS, UD, 3>(cur.t[n], 2 * s, bo));
+                    c1 = *reinterpret_cast<const mma_lds_u32x2*>((uintptr_t)unit_lds_offset<BITS, UD, 3>(cur.t[n], 2 * s + 1, bo));
                 } else {
+                    const uint32_t g0 = unit_tag<BITS, UD>(cur.t[n], 2 * s);
+                    const uint32_t g1 = unit_tag<BITS, UD>(cur.t[n], 2 * s + 1);
                     c0 = *reinterpret_cast<const u32x2*>(table + ((size_t)g0 * ESZ + bo));
                     c1 = *reinterpret_cast<const u32x2*>(table + ((size_t)g1 * ESZ + bo));
                 }
@@ -288,9 +310,9 @@ void rows_mfma_kernel(MmaArgs a) {
             const int row0 = t << 4;
             const int r = row0 + li < m.R ? row0 + li : m.R - 1;
             const uint32_t* bp = fbase + (til ? (size_t)t * a.U * 16 * UD : (size_t)r * m.W);
+            T.book = bkp[r];                                  // (first: loads return in order, the tags' waits then cover it)
 #pragma unroll
             for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(bp + fo[n]);
-            T.boff = m.row_book ? (uint32_t)m.row_book[r] << BITS : 0u;
         };
         Tile ring[PFT];
         ring[0] = tA;
