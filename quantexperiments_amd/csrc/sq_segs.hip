@@ -28,6 +28,12 @@ constexpr int SEG_MAX_WAVES = 16;
 // four rows 85 (the matrix-core kernel: 58-60 at four).  The same products on the matrix cores
 // (v_mfma_f32_4x4x4_16b_f16, one instruction per tag and activation row instead of two v_dot2c, element j of lane j's
 // result) measured no faster at one or two rows (gate|up 17.0-17.5 / 21.0 against 16.8 / 20.6 us).
+// Nor did a variant of this kernel for 3 to 8 rows that uses the whole instruction (the four lanes of a block take the same
+// tags of four consecutive weight rows and one activation row each: four weight rows x four activation rows per
+// instruction, a lane's registers hold one activation row's chunks as here): correct, and 53.3 / 55.3 / 60.8 us per
+// 7B-shaped layer at 3 / 4 / 8 rows against 54.0 / 54.5 / 55.4 for the matrix-core kernel (gate|up 18.6 against 19.2, down
+// 16.4-17.9 against 15.6).  With neither gathers, products nor sums (timing only) its gate|up launch still takes 16.9 us:
+// what these launches wait for is the tags, which arrive at 4.2 TB/s.
 constexpr int SEG_MAX_ROWS = 2;
 constexpr int SEG_MAX_BOOKS = 4;                // codebooks per matrix (4 x 32 KB of the CU's 160 KB of LDS at 12 bits)
 

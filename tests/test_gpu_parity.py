@@ -1069,17 +1069,18 @@ def test_full_7b_d4_stacks_at_small_batches_against_c_oracle(launch):
 def test_row_segment_kernel_of_the_12_bit_format(shapes):
     """d = 4 / 12-bit pieces whose rows are whole segments of 128 tags run on the row-segment kernel at 1 and 2
     activation rows (one segment per row up to 37, fewer rows than a workgroup takes per step, shares of rows that
-    do not divide, four stacked pieces, several thousand rows; 3 and 4 rows take the matrix-core kernel): against the
+    do not divide, four stacked pieces, several thousand rows; 3 to 8 rows take the matrix-core kernel): against the
     C oracle in fp32 and bf16 / fp16 output, with strided x and y; row 1 of a two-row call has the bits of the one-row
-    call; a one-hot input reads a weight column back exactly."""
+    call, the rows of a three-row call those of the four-row call; a one-hot input reads a weight column back exactly
+    at 1 and at 4 rows."""
     from quantexperiments_amd.kernels import linear_small
     pieces, ws = _stack(shapes, 4, 12, 1, 200 + len(shapes))
     C, Rt = shapes[0][1], sum(r for r, _ in shapes)
     w = np.concatenate(ws, axis=0)
     one = {}
-    for B in (1, 2, 3, 4):
+    for B in (1, 2, 3, 4, 5, 8):
         for dt in (torch.bfloat16, torch.float16):
-            x = rand_x(B, C, dt, seed=B)
+            x = rand_x(8, C, dt, seed=dt.itemsize)[:B]                      # (the same rows at every count)
             ref = c_oracle.linear(_xf(x), w)
             xd = torch.zeros(B, C + 8, dtype=dt, device="cuda")                # row stride C + 8
             xd[:, :C] = x.cuda()
@@ -1092,16 +1093,23 @@ def test_row_segment_kernel_of_the_12_bit_format(shapes):
             linear_small(pieces, xd[:, :C], yl)
             _check_lowp(yl, ref)
     # the same activation row alone and as row 1 of 2
-    x2 = rand_x(2, C, torch.bfloat16, seed=2)
     y1 = torch.empty(1, Rt, dtype=torch.float32, device="cuda")
+    x2 = rand_x(8, C, torch.bfloat16, seed=torch.bfloat16.itemsize)
     linear_small(pieces, x2[1:2].cuda(), y1)
     assert torch.equal(y1[0], one[(2, torch.bfloat16)][1])
+    assert torch.equal(one[(3, torch.bfloat16)], one[(4, torch.bfloat16)][:3])
+    assert torch.equal(one[(5, torch.bfloat16)], one[(8, torch.bfloat16)][:5])
     # one-hot input: every other product is an exact zero
     col = C - 3
-    xo = torch.zeros(1, C, dtype=torch.float16)
+    xo = torch.zeros(4, C, dtype=torch.float16)
     xo[0, col] = 1.0
-    linear_small(pieces, xo.cuda(), y1)
+    xo[3, 5] = 1.0
+    linear_small(pieces, xo[:1].cuda(), y1)
     assert np.array_equal(y1.cpu().numpy()[0], w[:, col].astype(np.float32))
+    y4 = torch.empty(4, Rt, dtype=torch.float32, device="cuda")
+    linear_small(pieces, xo.cuda(), y4)
+    assert np.array_equal(y4.cpu().numpy()[0], w[:, col].astype(np.float32)) and np.array_equal(y4.cpu().numpy()[3], w[:, 5].astype(np.float32))
+    assert not y4[1:3].any()
 
 
 @pytest.mark.parametrize("shapes,G,bits", [([(300, 3584)], 4, 12), ([(130, 5120), (64, 5120), (3, 5120)], 4, 12), ([(40, 17408)], 4, 12),
@@ -1113,7 +1121,7 @@ def test_row_segment_kernel_of_the_12_bit_format(shapes):
 def test_row_segment_kernel_with_several_codebooks(shapes, G, bits):
     """The same kernel on 8-, 10- and 12-bit tags (segments of 128 or 256 tags) and on matrices whose rows name one of G
     codebooks (the 27B recipe: d = 4, 256 / 1024 / 4096 entries, G = 4, all of them in LDS), including rows so long that
-    the activation rows no longer fit LDS beside the codebooks: 1 to 4 activation rows against the C oracle (3 and 4
+    the activation rows no longer fit LDS beside the codebooks: 1 to 8 activation rows against the C oracle (3 to 8
     run on the matrix cores), row 1 of two equal to the single-row call."""
     from quantexperiments_amd.kernels import linear_small, prepare_stack
     pieces, ws = [], []
@@ -1125,7 +1133,7 @@ def test_row_segment_kernel_with_several_codebooks(shapes, G, bits):
     w = np.concatenate(ws, axis=0)
     C, Rt = shapes[0][1], w.shape[0]
     ys = {}
-    for B in (1, 2, 3, 4):
+    for B in (1, 2, 3, 4, 5, 8):
         x = rand_x(B, C, torch.bfloat16, seed=10 + B)
         ref = c_oracle.linear(_xf(x), w)
         y = torch.full((B, Rt), 7.0, dtype=torch.float32, device="cuda")
