@@ -342,9 +342,10 @@ int launch_small(const sq_matrix* mats, int n, const void* x, int x_dtype, int64
             i = j;
             continue;
         }
-        if (B <= 2 && x_ok && segs_shape(m0)) {
-            // d = 4 / 12-bit rows of whole 128-tag segments at 1 or 2 activation rows: the row-segment kernel (7B-shaped
-            // layer: 45-46 us at one row, 56 at two, against 65-67 on the matrix-core kernel)
+        if (B <= 2 && x_ok && segs_shape(m0) && (B == 1 || mma_table_bytes(m0) > 64 * 1024)) {
+            // d = 4 rows of whole segments at one activation row, and at two when the codebooks leave a CU room for one
+            // workgroup only: the row-segment kernel (7B-shaped layer, 12-bit tags: 41.7 us at one row against 50 on the
+            // matrix-core kernel, 52.4 against 49.8 at two; four codebooks of 4096: 71-73 against 78-83 at two)
             int j = i + 1;
             while (j < n && j - i < 4 && segs_shape(mats[j]) && mats[j].W == m0.W && mats[j].G == m0.G) ++j;
             if (segs_fits(mats + i, j - i, B, cus)) {

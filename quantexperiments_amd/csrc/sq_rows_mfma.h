@@ -171,19 +171,13 @@ void rows_mfma_kernel(MmaArgs a) {
         }
     };
 
-    // ---- start-up: every load the first product needs is requested before anything waits: the first tile's
-    // tags, the activations of this wave's columns (raw), the codebook
+    // ---- start-up: every load the first products need is requested before anything waits, in the order in which it
+    // can come back (a wave's loads return in the order of their issue): the activations of this wave's columns, which
+    // the cache holds; the tags of the first tiles, which come from memory; then, once the activations have been handed
+    // to the lanes (a wait for them alone), the codebook.
     Tile tA, tB;
     float sc[TT + 1][4];                                      // [TT]: first tile of the next group, fetched early
-    // (a codebook of whole KB goes memory -> LDS without passing through registers, a wave instruction per KB)
     const bool table_dma = LDS_TAB && (a.table_bytes & 1023) == 0;
-    if (table_dma) {
-        typedef const __attribute__((address_space(1))) void* gptr_t;
-        typedef __attribute__((address_space(3))) void* lptr_t;
-        for (int c = wave; c < (a.table_bytes >> 10); c += KW)
-            __builtin_amdgcn_global_load_lds((gptr_t)(table + (size_t)c * 1024 + lane * 16), (lptr_t)(smem + c * 1024), 16, 0, 0);
-    }
-    if (t0 < t1) fetch(t0, tA, sc[0]);
     // The activations.  In the matrix instruction a lane supplies one token's 8 columns, so loading the operands where
     // they are used makes every load instruction touch 64 different cache lines (16 tokens x 4 lane units, 16 bytes of
     // each).  Instead the wave fetches the columns of a round, 16 tokens x XRB contiguous bytes, with whole-line loads
@@ -207,8 +201,28 @@ void rows_mfma_kernel(MmaArgs a) {
                 col = col < m.C ? col : m.C - 8;             // (columns past the row's end: any valid address, the operand is zeroed)
                 xraw[n][nt][j] = *reinterpret_cast<const u32x4*>(a.x + (int64_t)(tok < a.B ? tok : a.B - 1) * a.ldx + col);
             }
-    if (LDS_TAB) {
-        if (!table_dma) stage_table(m.table, a.table_bytes, smem);
+    fetch(t0 < t1 ? t0 : ntiles - 1, tA, sc[0]);             // (no branch around the loads; a workgroup without tiles reads the last one)
+    // (codebook in LDS: the tags of the first tiles in flight, without a branch around the loads so that the waits count
+    // them exactly: the two layouts differ in a base and a stride, chosen once)
+    constexpr int PFT = LDS_TAB ? mma_pft(RW) : 1;
+    const bool til = P.tiled != nullptr;
+    const uint32_t* fbase = til ? P.tiled + li * UD : tags;
+    uint32_t fo[RW];
+#pragma unroll
+    for (int n = 0; n < RW; ++n) fo[n] = til ? uoff[n] * 16u : uoff[n];
+    auto fetch_tags = [&](int t, Tile& T) {
+        const int row0 = t << 4;
+        const int r = row0 + li < m.R ? row0 + li : m.R - 1;
+        const uint32_t* bp = fbase + (til ? (size_t)t * a.U * 16 * UD : (size_t)r * m.W);
+        T.book = bkp[r];                                  // (first: loads return in order, the tags' waits then cover it)
+#pragma unroll
+        for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(bp + fo[n]);
+    };
+    Tile ring[PFT];
+    if constexpr (LDS_TAB) {
+        ring[0] = tA;
+#pragma unroll
+        for (int q = 1; q < PFT; ++q) fetch_tags(min(t0 + q, max(t1 - 1, t0)), ring[q]);
     }
     // the B operands: this wave's activations as fp16, in registers for the whole kernel
     half8v xb[RW][SPU][NT];
@@ -237,6 +251,15 @@ void rows_mfma_kernel(MmaArgs a) {
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
+    // (a codebook of whole KB goes memory -> LDS without passing through registers, a wave instruction per KB)
+    if (table_dma) {
+        typedef const __attribute__((address_space(1))) void* gptr_t;
+        typedef __attribute__((address_space(3))) void* lptr_t;
+        for (int c = wave; c < (a.table_bytes >> 10); c += KW)
+            __builtin_amdgcn_global_load_lds((gptr_t)(table + (size_t)c * 1024 + lane * 16), (lptr_t)(smem + c * 1024), 16, 0, 0);
+    } else if (LDS_TAB) {
+        stage_table(m.table, a.table_bytes, smem);
+    }
     SQ_TRACE_POINT(1);
     // every wave has taken its operands out of the staging area (and, with the codebook in LDS, the codebook has landed
     // and the first tile's tags with it)
@@ -297,27 +320,7 @@ void rows_mfma_kernel(MmaArgs a) {
         // refilled as soon as its last codeword has been gathered), a tile's accumulator goes straight to its place in
         // LDS, and the waves meet once per a.tg tiles (once per launch when the workgroup's tiles all fit), after which
         // each tile is added up by one wave (round robin), scaled and stored.
-        constexpr int PFT = mma_pft(RW);
         if (t0 >= t1) return;                                 // (uniform in the workgroup; the launcher gives every one a tile)
-        // a tile's tags without a branch around the loads (the waits then count loads exactly): the two layouts differ
-        // in a base and a stride, chosen once
-        const bool til = P.tiled != nullptr;
-        const uint32_t* fbase = til ? P.tiled + li * UD : tags;
-        uint32_t fo[RW];
-#pragma unroll
-        for (int n = 0; n < RW; ++n) fo[n] = til ? uoff[n] * 16u : uoff[n];
-        auto fetch_tags = [&](int t, Tile& T) {
-            const int row0 = t << 4;
-            const int r = row0 + li < m.R ? row0 + li : m.R - 1;
-            const uint32_t* bp = fbase + (til ? (size_t)t * a.U * 16 * UD : (size_t)r * m.W);
-            T.book = bkp[r];                                  // (first: loads return in order, the tags' waits then cover it)
-#pragma unroll
-            for (int n = 0; n < RW; ++n) T.t[n] = load_unit<UD>(bp + fo[n]);
-        };
-        Tile ring[PFT];
-        ring[0] = tA;
-#pragma unroll
-        for (int q = 1; q < PFT; ++q) fetch_tags(min(t0 + q, t1 - 1), ring[q]);
         auto tile_done = [&](int tl, const float4v (&acc)[NT]) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) red[((tl * KW + wave) * 64 + lane) * NT + nt] = acc[nt];

@@ -139,19 +139,14 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
     auto row_of = [&](int t) { return min(p0 + min(t, nsteps - 1) * rps + rsub, p1 - 1); };
     auto load_step = [&](int t) { return seg_load<WPL>(tg + (size_t)row_of(t) * a.W); };
 
-    // everything this workgroup needs from memory is requested before anything waits: the codebooks (memory to LDS
-    // without passing through registers; the last, partial KB through registers), the first steps of tags, the
-    // activation rows
-    {
-        const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table);
-        for (int c = wave; c < a.table_bytes / 1024; c += nwaves)
-            __builtin_amdgcn_global_load_lds((seg_gptr_t)(src + (size_t)c * 1024 + lane * 16), (seg_lptr_t)(lds + c * 1024), 16, 0, 0);
-    }
-    dwords<WPL> ring[PF];
-#pragma unroll
-    for (int q = 0; q < PF; ++q) ring[q] = load_step(q);
-    // the activation rows go through LDS once per workgroup (every group of a segment needs the same ones; fetched by
-    // each lane for itself they would cost as much cache traffic as the tags): 16 bytes per thread and turn
+    // Everything this workgroup needs from memory is requested before anything waits, in the order in which it can come
+    // back (a wave's loads return in the order of their issue): the activation rows, which the cache holds, the
+    // codebooks (memory to LDS without passing through registers; the last, partial KB through registers), the first
+    // steps of tags, which come from memory.  (The activations requested behind the tags arrive behind them: 2.8 us of a
+    // 46.8 us layer at one row.)
+    // One activation row is fetched by every lane for itself (64 bytes, the 16 lanes of a group 1 KB in a row); two go
+    // through LDS once per workgroup, 16 bytes per thread and turn, where every group of a segment finds them (fetched
+    // per lane they would cost as much cache traffic as the tags).
     constexpr int XT = 4;                                        // turns requested together
     constexpr int XL = TPL / 2;                                  // 16-byte pieces of a row that one lane multiplies with
     const int xchunks = nseg * 16 * XL;                          // 16-byte pieces of a row
@@ -165,7 +160,33 @@ __global__ __launch_bounds__(SEG_MAX_WAVES * 64) void segs_kernel(SegArgs a) {
             for (int i = 0; i < XL; ++i) xown[b][i] = xp[i];
         }
     }
-    for (int i0 = tid; !a.xdirect && i0 < NB * xchunks; i0 += XT * (int)blockDim.x) {
+    const bool xearly = !a.xdirect && NB * xchunks <= XT * (int)blockDim.x;   // one turn serves the rows: its loads go out now
+    u32x4 xv[XT];
+    if (xearly) {
+#pragma unroll
+        for (int k = 0; k < XT; ++k) {
+            const int i = min(tid + k * (int)blockDim.x, NB * xchunks - 1), b = i / xchunks;
+            xv[k] = reinterpret_cast<const u32x4*>(a.x + (int64_t)min(b, a.nb - 1) * a.ldx)[i - b * xchunks];
+        }
+    }
+    {
+        const unsigned char* src = reinterpret_cast<const unsigned char*>(P.table);
+        for (int c = wave; c < a.table_bytes / 1024; c += nwaves)
+            __builtin_amdgcn_global_load_lds((seg_gptr_t)(src + (size_t)c * 1024 + lane * 16), (seg_lptr_t)(lds + c * 1024), 16, 0, 0);
+    }
+    dwords<WPL> ring[PF];
+#pragma unroll
+    for (int q = 0; q < PF; ++q) ring[q] = load_step(q);
+    if (xearly) {
+#pragma unroll
+        for (int k = 0; k < XT; ++k) {
+            const int i = tid + k * (int)blockDim.x;
+            u32x4 q = xv[k];
+            if (a.x_dtype == SQ_BF16) { q.x = bf2h_x2(q.x); q.y = bf2h_x2(q.y); q.z = bf2h_x2(q.z); q.w = bf2h_x2(q.w); }
+            if (i < NB * xchunks) reinterpret_cast<u32x4*>(xs)[i] = q;
+        }
+    }
+    for (int i0 = tid; !a.xdirect && !xearly && i0 < NB * xchunks; i0 += XT * (int)blockDim.x) {
         u32x4 v[XT];
 #pragma unroll
         for (int k = 0; k < XT; ++k) {
@@ -364,7 +385,7 @@ static bool segs_plan(const sq_matrix* mats, int cnt, int B, int cus, SegPlan& p
         const size_t base = (size_t)pl.table_bytes + (((size_t)pl.NB * pl.rows_max * pl.nseg * 4 + 15) & ~(size_t)15);
         const size_t xs = (size_t)pl.NB * mats[0].C * 2;         // the activation rows as fp16
         const size_t ids = mats[0].G > 1 ? (((size_t)pl.rows_max + 15) & ~(size_t)15) : 0;   // codebook ids of the rows
-        pl.xdirect = base + xs + ids > room ? 1 : 0;
+        pl.xdirect = base + xs + ids > room || B == 1 ? 1 : 0;  // (one row: fetched per lane, 41.8 against 43.2 us per 7B-shaped layer)  // (one row: 45.0 against 46.8 us per 7B-shaped layer fetched per lane)
         pl.smem = base + (pl.xdirect ? 0 : xs) + ids;
         if (pl.smem <= room) return true;
     }

@@ -1067,12 +1067,12 @@ def test_full_7b_d4_stacks_at_small_batches_against_c_oracle(launch):
                                     [(40, 18944)], [(129, 8192), (2, 8192), (2, 8192), (31, 8192)], [(9000, 512)]],
                          ids=lambda c: "+".join(f"{r}x{k}" for r, k in c))
 def test_row_segment_kernel_of_the_12_bit_format(shapes):
-    """d = 4 / 12-bit pieces whose rows are whole segments of 128 tags run on the row-segment kernel at 1 and 2
-    activation rows (one segment per row up to 37, fewer rows than a workgroup takes per step, shares of rows that
-    do not divide, four stacked pieces, several thousand rows; 3 to 8 rows take the matrix-core kernel): against the
-    C oracle in fp32 and bf16 / fp16 output, with strided x and y; row 1 of a two-row call has the bits of the one-row
-    call, the rows of a three-row call those of the four-row call; a one-hot input reads a weight column back exactly
-    at 1 and at 4 rows."""
+    """d = 4 / 12-bit pieces whose rows are whole segments of 128 tags run on the row-segment kernel at one activation
+    row (one segment per row up to 37, fewer rows than a workgroup takes per step, shares of rows that do not divide,
+    four stacked pieces, several thousand rows; 2 to 8 rows of a codebook this small take the matrix-core kernel):
+    against the C oracle in fp32 and bf16 / fp16 output, with strided x and y; the rows of a two- and a three-row call
+    have the bits of the four-row call's, the one-row call agrees to the order of additions; a one-hot input reads a
+    weight column back exactly at 1 and at 4 rows."""
     from quantexperiments_amd.kernels import linear_small
     pieces, ws = _stack(shapes, 4, 12, 1, 200 + len(shapes))
     C, Rt = shapes[0][1], sum(r for r, _ in shapes)
@@ -1096,7 +1096,8 @@ def test_row_segment_kernel_of_the_12_bit_format(shapes):
     y1 = torch.empty(1, Rt, dtype=torch.float32, device="cuda")
     x2 = rand_x(8, C, torch.bfloat16, seed=torch.bfloat16.itemsize)
     linear_small(pieces, x2[1:2].cuda(), y1)
-    assert torch.equal(y1[0], one[(2, torch.bfloat16)][1])
+    assert rel_max_err(y1[0].cpu().numpy(), one[(2, torch.bfloat16)][1].cpu().numpy().astype(np.float64)) < 1e-5
+    assert torch.equal(one[(2, torch.bfloat16)], one[(4, torch.bfloat16)][:2])
     assert torch.equal(one[(3, torch.bfloat16)], one[(4, torch.bfloat16)][:3])
     assert torch.equal(one[(5, torch.bfloat16)], one[(8, torch.bfloat16)][:5])
     # one-hot input: every other product is an exact zero
@@ -1122,7 +1123,8 @@ def test_row_segment_kernel_with_several_codebooks(shapes, G, bits):
     """The same kernel on 8-, 10- and 12-bit tags (segments of 128 or 256 tags) and on matrices whose rows name one of G
     codebooks (the 27B recipe: d = 4, 256 / 1024 / 4096 entries, G = 4, all of them in LDS), including rows so long that
     the activation rows no longer fit LDS beside the codebooks: 1 to 8 activation rows against the C oracle (3 to 8
-    run on the matrix cores), row 1 of two equal to the single-row call."""
+    run on the matrix cores, and so do 2 when the codebooks take at most 64 KB), row 1 of two equal to the single-row
+    call where one kernel serves both."""
     from quantexperiments_amd.kernels import linear_small, prepare_stack
     pieces, ws = [], []
     for k, (R, C) in enumerate(shapes):
@@ -1146,7 +1148,10 @@ def test_row_segment_kernel_with_several_codebooks(shapes, G, bits):
     x2 = rand_x(2, C, torch.bfloat16, seed=12)
     y1 = torch.empty(1, Rt, dtype=torch.float32, device="cuda")
     linear_small(pieces, x2[1:2].cuda(), y1)
-    assert torch.equal(y1[0], ys[2][1])
+    if G * (8 << bits) > 64 * 1024:
+        assert torch.equal(y1[0], ys[2][1])
+    else:
+        assert rel_max_err(y1[0].cpu().numpy(), ys[2][1].cpu().numpy().astype(np.float64)) < 1e-5
 
 
 @pytest.mark.parametrize("shape", [(18944, 3584, 1), (3584, 18944, 1), (5120, 5120, 16)], ids=lambda c: "x".join(map(str, c)))
