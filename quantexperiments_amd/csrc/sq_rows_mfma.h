@@ -111,7 +111,7 @@ void rows_mfma_kernel(MmaArgs a) {
     const int t0 = (int)((int64_t)ntiles * share / nshare), t1 = (int)((int64_t)ntiles * (share + 1) / nshare);
     SQ_TRACE_POINT(0);
 
-    // LDS: [codebook][16 bytes][reduction buffer: TT tiles x KW waves x 64 lanes x NT x 16 bytes]
+    // LDS: [codebook][16 bytes, unused][reduction buffer: TT tiles x KW waves x 64 lanes x NT x 16 bytes]
     // (the codeword gathers form LDS addresses as numbers counted from the start of the dynamic LDS, which is address 0 in a
     // kernel without static LDS; a build in which it is not leaves y unwritten, which no test survives)
     if (LDS_TAB && (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)smem != 0u) return;
