@@ -1209,3 +1209,33 @@ def test_random_large_codebook_shapes_match_oracle():
         linear_small(pair, x.cuda(), y)
         ref = np.concatenate(refs, axis=1)
         assert rel_max_err(y.cpu().numpy(), ref) < TOL, (it, C, bits, B, [p.R for p in pair], [p.M for p in pair])
+
+
+def test_random_lds_codebook_shapes_match_oracle():
+    """48 seeded random stacks with d = 4 and 8-, 10- or 12-bit tags, 1 to 4 codebooks, with and without the tile-major
+    copy: row counts around the 16-row tile and the 4 x 16 tiles of a group, column counts that are and are not whole
+    segments (so both decode kernels and the generic one are met), long rows that are split over workgroups, 1 to 32
+    activation rows and beyond (passes of 32 through sq_linear_gemm)."""
+    from quantexperiments_amd.kernels import linear_small, linear_gemm, prepare_stack
+    rng = np.random.default_rng(4096)
+    for it in range(48):
+        bits = int(rng.choice([8, 10, 12]))
+        C = int(rng.choice([128, 512, 640, 1024, 1280, 3584, 5120, 8192, 18944]))
+        G = int(rng.choice([1, 1, 2, 4]))
+        B = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 40, 70]))
+        n = int(rng.integers(1, 4))
+        x = rand_x(B, C, torch.bfloat16 if it % 3 else torch.float16, seed=it)
+        pieces, refs = [], []
+        for k in range(n):
+            R = int(rng.choice([1, 15, 16, 17, 63, 64, 65, 130, 257, 1100])) if C < 8192 else int(rng.choice([1, 17, 70]))
+            s = synth(R, C, 4, bits, G, 1, seed=1000 * it + k)
+            pieces.append(to_device(s, stream=("later" if it % 2 else False)))
+            refs.append(_ref(s, x))
+        if it % 2:
+            prepare_stack(pieces)
+        Rt = sum(p.R for p in pieces)
+        y = torch.full((B, Rt + 3), 3.0, dtype=torch.float32, device="cuda")
+        (linear_small if B <= 32 else linear_gemm)(pieces, x.cuda(), y[:, :Rt])
+        ref = np.concatenate(refs, axis=1)
+        assert rel_max_err(y[:, :Rt].cpu().numpy(), ref) < TOL, (it, C, bits, G, B, [p.R for p in pieces])
+        assert bool((y[:, Rt:] == 3.0).all()), it
