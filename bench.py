@@ -154,22 +154,24 @@ def cpu_baseline(torch, layer, x, d, bits, shapes):
             "us_per_layer": total * 1e6, "decode_s": dec, "matmul_s": mm}
 
 
-def prefill(torch, dev, layer, shapes, names=("gate", "down"), T=2048, dense=True):
-    """T-row prefill GEMM of single matrices: ms (median of REPS graph replays) and TFLOP/s; with `dense`, also the
-    time of a dense bf16 GEMM of the same shape in PyTorch."""
+def prefill(torch, dev, layers, shapes, names=("gate", "down"), T=2048, dense=True, calls=20):
+    """T-row prefill GEMM of single matrices: ms per product and TFLOP/s, from HIP-graph replays of `calls` products
+    that rotate over the same matrix of up to 7 distinct layers (median of REPS replays); with `dense`, also the time
+    of a dense bf16 GEMM of the same shape in PyTorch, timed the same way."""
     from quantexperiments_amd.kernels import linear_gemm
     res = {}
     for nm in names:
         R, C = shapes[nm]
+        mats = [L[nm] for L in layers[:7]]
         x = torch.randn(T, C, device=dev).to(torch.bfloat16)
         y = torch.empty(T, R, device=dev, dtype=torch.bfloat16)
-        ms = timed_graph(torch, lambda: linear_gemm([layer[nm]], x, y))
-        res[nm] = {"ms": ms, "tflops": 2.0 * T * R * C / (ms * 1e-3) / 1e12}
+        ms = timed_graph(torch, lambda: [linear_gemm([mats[i % len(mats)]], x, y) for i in range(calls)]) / calls
+        res[nm] = {"ms": ms, "tflops": 2.0 * T * R * C / (ms * 1e-3) / 1e12, "products_per_replay": calls, "matrices_rotated": len(mats)}
         if dense:
             # for scale: the same product on a dense bf16 copy of the weights through PyTorch (the vendor GEMM library),
             # timed the same way; it reads 4x the bytes and decodes nothing
             w = (torch.randn(R, C, device=dev) * 0.02).to(torch.bfloat16)
-            lib = timed_graph(torch, lambda: torch.matmul(x, w.t(), out=y))
+            lib = timed_graph(torch, lambda: [torch.matmul(x, w.t(), out=y) for _ in range(calls)]) / calls
             res[nm].update(library_dense_ms=lib, library_dense_tflops=2.0 * T * R * C / (lib * 1e-3) / 1e12, speed_vs_library_dense=lib / ms)
             del w
     return res
@@ -360,6 +362,7 @@ def main():
     ap.add_argument("--layers", type=int, default=28, help="distinct layers the steps rotate over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prefill-calls", type=int, default=20, help="prefill products per timed graph replay (1: short profiler runs)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant launch (gate|up) and print only its roofline object: the command "
                          "the rocprofv3 summaries under profiles/ are made with")
@@ -485,7 +488,7 @@ def main():
     if args.copy_probe:
         out["copy_probe"] = copy_probe(torch, dev)
     if not args.no_prefill:
-        pf = prefill(torch, dev, layers[0], SHAPES_7B)
+        pf = prefill(torch, dev, layers, SHAPES_7B, calls=max(1, args.prefill_calls))
         out["prefill"] = {"M": 2048, "gate_18944x3584": pf["gate"], "down_3584x18944": pf["down"],
                           "peak_tflops": MFMA_PEAK_TFLOPS,
                           "frac_of_peak": min(pf["gate"]["tflops"], pf["down"]["tflops"]) / MFMA_PEAK_TFLOPS}
