@@ -177,8 +177,9 @@ def prefill(torch, dev, layers, shapes, names=("gate", "down"), T=2048, dense=Tr
     return res
 
 
-def layer_times(torch, dev, layers, shapes, B, fn, gen):
-    """us per launch and per layer of fn(pieces, x, y) over the 4 launches of `layers` rotated inside one graph."""
+def layer_times(torch, dev, layers, shapes, B, fn, gen, rounds=1):
+    """us per launch and per layer of fn(pieces, x, y) over the 4 launches of `layers` rotated inside one graph
+    (`rounds` times over the layers: few layers of long products still make a graph of many calls)."""
     xs = {C: torch.randn(B, C, generator=gen).to(torch.bfloat16).to(dev) for C in sorted({c for _, c in shapes.values()})}
     per, tot = {}, 0.0
     for l in LAUNCHES:
@@ -186,9 +187,10 @@ def layer_times(torch, dev, layers, shapes, B, fn, gen):
         y = torch.empty(B, sum(shapes[n][0] for n in l), device=dev, dtype=torch.bfloat16)
 
         def run():
-            for L in layers:
-                fn([L[n] for n in l], xs[C], y)
-        per["|".join(l)] = timed_graph(torch, run) * 1e3 / len(layers)
+            for _ in range(rounds):
+                for L in layers:
+                    fn([L[n] for n in l], xs[C], y)
+        per["|".join(l)] = timed_graph(torch, run) * 1e3 / (len(layers) * rounds)
         tot += per["|".join(l)]
     return tot, per
 
@@ -210,7 +212,8 @@ def small_batch_crossover(torch, dev, gen, n_layers):
     res, cross, change = {}, None, None
     for M in (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256):
         nbytes = sum(launch_bytes(SHAPES_7B, l, d, bits, B=M) for l in LAUNCHES)
-        direct, per = layer_times(torch, dev, layers if M <= 32 else layers[:2], SHAPES_7B, M, linear_small if M <= 32 else linear_gemm, gen)
+        direct, per = layer_times(torch, dev, layers if M <= 32 else layers[:2], SHAPES_7B, M, linear_small if M <= 32 else linear_gemm, gen,
+                                  rounds=1 if M <= 32 else 4)
         r = {"direct_us_per_layer": direct, "per_launch_us": per}
         best, route = direct, "direct"
         if M > 1:
@@ -241,7 +244,7 @@ def masked_27b(torch, dev, gen, n_layers):
     nbytes = sum(launch_bytes(SHAPES_27B, l, d, bits, 1, M) for l in LAUNCHES)
     flops1 = 2.0 * sum(R * C for R, C in SHAPES_27B.values())
     us1, per1 = layer_times(torch, dev, layers, SHAPES_27B, 1, linear_small, gen)
-    us2k, per2k = layer_times(torch, dev, layers[:2], SHAPES_27B, 2048, linear_gemm, gen)
+    us2k, per2k = layer_times(torch, dev, layers[:2], SHAPES_27B, 2048, linear_gemm, gen, rounds=5)
     return {"workload": "cfg5: 27B-class layer (hidden 5120, intermediate 17408), d=8, K=65536, 16 column orders, 4-bit order index per row",
             "layers_rotated": n_layers, "bytes_per_layer": nbytes,
             "bs1": {"us_per_layer": us1, "per_launch_us": per1, "GBps_packed": nbytes / us1 / 1e3, "frac_hbm": nbytes / us1 / 1e3 / HBM_PEAK_GBS},
