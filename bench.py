@@ -177,21 +177,23 @@ def prefill(torch, dev, layers, shapes, names=("gate", "down"), T=2048, dense=Tr
     return res
 
 
-def layer_times(torch, dev, layers, shapes, B, fn, gen, rounds=1):
-    """us per launch and per layer of fn(pieces, x, y) over the 4 launches of `layers` rotated inside one graph
-    (`rounds` times over the layers: few layers of long products still make a graph of many calls)."""
+def layer_times(torch, dev, layers, shapes, B, fn, gen, rounds=None):
+    """us per layer and per launch of fn(pieces, x, y).  Per layer: one HIP graph of whole layers (the 4 launches of
+    every layer in turn, `rounds` times over `layers`), so that the weights walked between two uses of a matrix exceed
+    the last-level cache and a replay holds about a hundred calls; per launch: a graph of that launch alone over the
+    same layers and rounds.  `rounds` defaults to what makes 24 calls of every launch."""
+    if rounds is None:
+        rounds = max(1, -(-24 // len(layers)))
     xs = {C: torch.randn(B, C, generator=gen).to(torch.bfloat16).to(dev) for C in sorted({c for _, c in shapes.values()})}
-    per, tot = {}, 0.0
-    for l in LAUNCHES:
-        C = shapes[l[0]][1]
-        y = torch.empty(B, sum(shapes[n][0] for n in l), device=dev, dtype=torch.bfloat16)
+    ys = {l: torch.empty(B, sum(shapes[n][0] for n in l), device=dev, dtype=torch.bfloat16) for l in LAUNCHES}
 
-        def run():
-            for _ in range(rounds):
-                for L in layers:
-                    fn([L[n] for n in l], xs[C], y)
-        per["|".join(l)] = timed_graph(torch, run) * 1e3 / (len(layers) * rounds)
-        tot += per["|".join(l)]
+    def run(launches):
+        for _ in range(rounds):
+            for L in layers:
+                for l in launches:
+                    fn([L[n] for n in l], xs[shapes[l[0]][1]], ys[l])
+    per = {"|".join(l): timed_graph(torch, lambda: run((l,))) * 1e3 / (len(layers) * rounds) for l in LAUNCHES}
+    tot = timed_graph(torch, lambda: run(LAUNCHES)) * 1e3 / (len(layers) * rounds)
     return tot, per
 
 
@@ -213,7 +215,7 @@ def small_batch_crossover(torch, dev, gen, n_layers):
     for M in (1, 2, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256):
         nbytes = sum(launch_bytes(SHAPES_7B, l, d, bits, B=M) for l in LAUNCHES)
         direct, per = layer_times(torch, dev, layers if M <= 32 else layers[:2], SHAPES_7B, M, linear_small if M <= 32 else linear_gemm, gen,
-                                  rounds=1 if M <= 32 else 4)
+                                  rounds=None if M <= 32 else 4)
         r = {"direct_us_per_layer": direct, "per_launch_us": per}
         best, route = direct, "direct"
         if M > 1:
