@@ -419,12 +419,15 @@ def main():
     gu = LAUNCHES[2]
     gu_bytes = launch_bytes(SHAPES_7B, gu, D, BITS)
 
+    rounds = max(1, -(-96 // len(layers)))       # a graph of one launch holds about a hundred calls, like a graph of layers
+
     def gate_up_all():
-        for L in layers:
-            linear_small([L[n] for n in gu], x[3584], y[gu])
+        for _ in range(rounds):
+            for L in layers:
+                linear_small([L[n] for n in gu], x[3584], y[gu])
 
     def roofline():
-        dur_us = timed_graph(torch, gate_up_all) * 1e3 / len(layers)
+        dur_us = timed_graph(torch, gate_up_all) * 1e3 / (len(layers) * rounds)
         achieved = gu_bytes / (dur_us * 1e-6) / 1e9
         return {"bound": "hbm", "kernel": "sq::stream_kernel (gate|up launch, 2 x 18944x3584)",
                 "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
@@ -467,10 +470,11 @@ def main():
     per_launch = {}
     for l in LAUNCHES:
         def one(l=l):
-            for L in layers:
-                linear_small([L[n] for n in l], x[SHAPES_7B[l[0]][1]], y[l])
+            for _ in range(rounds):
+                for L in layers:
+                    linear_small([L[n] for n in l], x[SHAPES_7B[l[0]][1]], y[l])
         nb = launch_bytes(SHAPES_7B, l, D, BITS)
-        us = timed_graph(torch, one) * 1e3 / len(layers)
+        us = timed_graph(torch, one) * 1e3 / (len(layers) * rounds)
         per_launch["|".join(l)] = {"us": us, "bytes": nb, "frac_hbm": nb / us / 1e3 / HBM_PEAK_GBS}
 
     out = {
